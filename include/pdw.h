@@ -1,0 +1,94 @@
+/*
+ * pdw.h - C ABI of libpdw.so: hand-written gfx950 (MI355X) kernels for the pyramid
+ * depthwise-convolution block.
+ *
+ * The reference (IrisRainbowNeko/PyramidConvBlock) has no FFI: its device code is reached
+ * through Triton's `kernel[grid](...)` launches inside Python autograd Functions.  Each
+ * entry point below replaces one such launch site (cited per function, paths relative to
+ * the reference tree) and is what a binding for that site would call.
+ *
+ * Conventions
+ *   - All tensors are dense channels-last: x[B][H][W][C] with C fastest; depthwise
+ *     weights are w[KH][KW][C]  (dwconv_triton.py:413-416).
+ *   - Every pointer is a DEVICE pointer borrowed for the duration of the call; nothing is
+ *     allocated, freed or synchronised inside the library.  Work is enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the null stream) of the current device.
+ *   - `dtype` is one of PDW_F32 / PDW_F16 / PDW_BF16 and applies to every tensor of the
+ *     call.  Arithmetic is fp32 (bf16/fp16 products are exact in fp32), one rounding on store.
+ *   - Return value: 0 on success; non-zero on invalid arguments or a failed launch, with a
+ *     message available from pdw_last_error() (thread-local).
+ *   - Re-entrant; no global mutable state except the per-thread error text.
+ */
+#ifndef PDW_H_
+#define PDW_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { PDW_F32 = 0, PDW_F16 = 1, PDW_BF16 = 2 };
+
+/* ABI version of the library (bumped when a signature changes). */
+int pdw_version(void);
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *pdw_last_error(void);
+
+/* Output extent of a convolution axis: (in + 2p - d(k-1) - 1)/s + 1, 0 if empty.
+ * dwconv_triton.py:311-312. */
+int pdw_conv_out_size(int in, int k, int stride, int pad, int dil);
+
+/* Depthwise cross-correlation  y[b,i,j,c] = sum_{kh,kw} x[b, i*sh-ph+kh*dh, j*sw-pw+kw*dw, c] * w[kh,kw,c],
+ * zero outside the image.  x[B,H,W,C] -> y[B,OH,OW,C].
+ * Replaces the launch of _depthwise_conv_kernel_optimized, dwconv_triton.py:325-333 (kernel :20-104). */
+int pdw_dwconv_fwd(const void *x, const void *w, void *y, int B, int H, int W, int C, int KH, int KW,
+                   int SH, int SW, int PH, int PW, int DH, int DW, int dtype, void *stream);
+
+/* Input gradient (exact adjoint of pdw_dwconv_fwd in x): gy[B,OH,OW,C] -> dx[B,H,W,C]; H,W are
+ * the forward INPUT extents.  Fully overwrites dx (no pre-zeroing needed).
+ * Replaces the launch of _depthwise_conv_backward_input_kernel, dwconv_triton.py:358-366
+ * (kernel :119-203), which is only correct for stride 1 and 2*pad == dil*(k-1); this entry
+ * point is correct for every stride/pad/dilation. */
+int pdw_dwconv_dgrad(const void *gy, const void *w, void *dx, int B, int H, int W, int C, int KH, int KW,
+                     int SH, int SW, int PH, int PW, int DH, int DW, int dtype, void *stream);
+
+/* Bytes of device scratch pdw_dwconv_wgrad needs for these extents (fp32 partial sums). */
+size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW,
+                                        int PH, int PW, int DH, int DW, int dtype);
+
+/* Weight gradient dw[kh,kw,c] = sum_{b,i,j} gy[b,i,j,c] * x[b, i*sh-ph+kh*dh, j*sw-pw+kw*dw, c].
+ * Two deterministic passes (per-block fp32 partials in `workspace`, then a fixed-order sum);
+ * no atomics, so results are bit-reproducible.  Fully overwrites dw.
+ * Replaces the launch of _depthwise_conv_weight_grad_kernel, dwconv_triton.py:377-385
+ * (kernel :219-296). */
+int pdw_dwconv_wgrad(const void *x, const void *gy, void *dw, void *workspace, size_t workspace_bytes,
+                     int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW, int DH,
+                     int DW, int dtype, void *stream);
+
+/* Adaptive average pooling x[B,H,W,C] -> y[B,h,w,C]; bin i covers [floor(i*H/h), ceil((i+1)*H/h)).
+ * Replaces F.adaptive_avg_pool2d at conv_block.py:16 and the launch at avgpool_triton.py:225-229
+ * (kernel :14-107; integer bin arithmetic here instead of the fp16 one at :42-47). */
+int pdw_avgpool_fwd(const void *x, void *y, int B, int H, int W, int C, int h, int w, int dtype, void *stream);
+
+/* Its gradient gy[B,h,w,C] -> gx[B,H,W,C], gather form (no atomics, fully overwrites gx).
+ * Replaces avgpool_triton.py:253-257 (kernel :118-203). */
+int pdw_avgpool_bwd(const void *gy, void *gx, int B, int H, int W, int C, int h, int w, int dtype, void *stream);
+
+/* Bilinear resize, align_corners=False, no explicit scale factor: x[B,h,w,C] -> y[B,H,W,C].
+ * Replaces F.interpolate at conv_block.py:21 and the launch at up_triton.py:157-161 (kernel :14-125). */
+int pdw_bilinear_fwd(const void *x, void *y, int B, int h, int w, int C, int H, int W, int dtype, void *stream);
+
+/* Its gradient gy[B,H,W,C] -> gx[B,h,w,C] (transpose of the above, gather form).  The reference
+ * has no backward for up_triton.py; inside ConvBlock autograd supplies upsample_bilinear2d_backward. */
+int pdw_bilinear_bwd(const void *gy, void *gx, int B, int h, int w, int C, int H, int W, int dtype, void *stream);
+
+/* Gate  y[m,c] = x[m,c] * x[m,G+c] * sqrt(G),  G = I/2,  x[M,I] -> y[M,G]   (conv_block.py:10,18-19). */
+int pdw_gate_fwd(const void *x, void *y, long long M, int I, int dtype, void *stream);
+/* gx[m,c] = gy*x[m,G+c]*sqrt(G);  gx[m,G+c] = gy*x[m,c]*sqrt(G). */
+int pdw_gate_bwd(const void *x, const void *gy, void *gx, long long M, int I, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PDW_H_ */

@@ -1,0 +1,101 @@
+"""ctypes binding of libpdw.so, the C-ABI library of hand-written gfx950 kernels.
+
+There is deliberately no fallback: if the library is missing and cannot be built, or a
+tensor is not on a HIP device, the operators raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_longlong, c_size_t, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpdw.so")
+
+PDW_F32, PDW_F16, PDW_BF16 = 0, 1, 2
+_DTYPES = {torch.float32: PDW_F32, torch.float16: PDW_F16, torch.bfloat16: PDW_BF16}
+
+_lib = None
+
+_CONV = [c_int] * 12  # B,H,W,C,KH,KW,SH,SW,PH,PW,DH,DW
+_SIGS = {
+    "pdw_version": (c_int, []),
+    "pdw_last_error": (c_char_p, []),
+    "pdw_conv_out_size": (c_int, [c_int] * 5),
+    "pdw_dwconv_fwd": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
+    "pdw_dwconv_dgrad": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
+    "pdw_dwconv_wgrad_workspace_bytes": (c_size_t, _CONV + [c_int]),
+    "pdw_dwconv_wgrad": (c_int, [c_void_p] * 4 + [c_size_t] + _CONV + [c_int, c_void_p]),
+    "pdw_avgpool_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
+    "pdw_avgpool_bwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
+    "pdw_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
+    "pdw_bilinear_bwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
+    "pdw_gate_fwd": (c_int, [c_void_p] * 2 + [c_longlong, c_int, c_int, c_void_p]),
+    "pdw_gate_bwd": (c_int, [c_void_p] * 3 + [c_longlong, c_int, c_int, c_void_p]),
+}
+EXPORTS = tuple(_SIGS)
+
+
+def lib():
+    """Loads libpdw.so (building it with hipcc only if it has never been built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            from . import build as _build
+
+            _build.build()
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(L, name)  # AttributeError if the library lacks a declared symbol
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def check(status: int, what: str = "libpdw") -> None:
+    if status != 0:
+        raise RuntimeError(f"{what}: {lib().pdw_last_error().decode()} (status {status})")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError(f"pyramid dwconv kernels support float32/float16/bfloat16, got {dtype}") from None
+
+
+def require_device(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("pyramid dwconv kernels run on a HIP device only (tensor is on %s); "
+                               "there is no CPU path" % t.device)
+        if t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} vs {t.device}")
+    return dev
+
+
+def stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+class on_device:
+    """Makes `dev` the current HIP device for the duration of a launch (no-op when it already is)."""
+
+    def __init__(self, dev: torch.device):
+        self.dev, self.prev = dev, None
+
+    def __enter__(self):
+        idx = self.dev.index if self.dev.index is not None else torch.cuda.current_device()
+        cur = torch.cuda.current_device()
+        if idx != cur:
+            self.prev = cur
+            torch.cuda.set_device(idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False

@@ -1,0 +1,136 @@
+// C ABI of libpdw.so (declared in include/pdw.h): argument validation and dispatch to
+// the kernel launchers.  No allocation, no synchronisation, no global mutable state
+// besides the per-thread error text.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/pdw.h"
+#include "common.h"
+#include "kernels.h"
+
+namespace pdw {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+        return 2;
+    }
+    return 0;
+}
+
+static bool valid_dtype(int dtype) { return dtype == kF32 || dtype == kF16 || dtype == kBF16; }
+
+static int check_conv(const char* fn, const void* a, const void* b, const void* c, int B, int H, int W, int C, int KH,
+                      int KW, int SH, int SW, int PH, int PW, int DH, int DW, int dtype) {
+    if (!valid_dtype(dtype)) return set_error("%s: unknown dtype %d", fn, dtype), 1;
+    if (B < 0 || H < 1 || W < 1 || C < 1 || KH < 1 || KW < 1)
+        return set_error("%s: bad extents B=%d H=%d W=%d C=%d KH=%d KW=%d", fn, B, H, W, C, KH, KW), 1;
+    if (SH < 1 || SW < 1 || DH < 1 || DW < 1 || PH < 0 || PW < 0)
+        return set_error("%s: bad stride/padding/dilation (%d,%d)/(%d,%d)/(%d,%d)", fn, SH, SW, PH, PW, DH, DW), 1;
+    if (B > 0 && (!a || !b || !c)) return set_error("%s: null pointer", fn), 1;
+    return 0;
+}
+
+static int check_resample(const char* fn, const void* a, const void* b, int B, int H, int W, int C, int h, int w,
+                          int dtype) {
+    if (!valid_dtype(dtype)) return set_error("%s: unknown dtype %d", fn, dtype), 1;
+    if (B < 0 || H < 1 || W < 1 || C < 1 || h < 1 || w < 1)
+        return set_error("%s: bad extents B=%d H=%d W=%d C=%d h=%d w=%d", fn, B, H, W, C, h, w), 1;
+    if (B > 0 && (!a || !b)) return set_error("%s: null pointer", fn), 1;
+    return 0;
+}
+
+}  // namespace pdw
+
+using namespace pdw;
+
+extern "C" {
+
+int pdw_version(void) { return 1; }
+
+const char* pdw_last_error(void) { return g_err; }
+
+int pdw_conv_out_size(int in, int k, int stride, int pad, int dil) {
+    if (in < 1 || k < 1 || stride < 1 || dil < 1 || pad < 0) return 0;
+    return conv_out_size(in, k, stride, pad, dil);
+}
+
+int pdw_dwconv_fwd(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int SH, int SW,
+                   int PH, int PW, int DH, int DW, int dtype, void* stream) {
+    if (int e = check_conv("pdw_dwconv_fwd", x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
+    if (B == 0 || conv_out_size(H, KH, SH, PH, DH) == 0 || conv_out_size(W, KW, SW, PW, DW) == 0) return 0;
+    return dwconv_fwd_direct_launch(x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype, (hipStream_t)stream);
+}
+
+int pdw_dwconv_dgrad(const void* gy, const void* w, void* dx, int B, int H, int W, int C, int KH, int KW, int SH,
+                     int SW, int PH, int PW, int DH, int DW, int dtype, void* stream) {
+    if (int e = check_conv("pdw_dwconv_dgrad", gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
+    if (B == 0) return 0;
+    return dwconv_dgrad_direct_launch(gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype,
+                                      (hipStream_t)stream);
+}
+
+size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW,
+                                        int DH, int DW, int dtype) {
+    if (check_conv("pdw_dwconv_wgrad_workspace_bytes", "", "", "", B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype))
+        return 0;
+    return dwconv_wgrad_direct_workspace(B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW);
+}
+
+int pdw_dwconv_wgrad(const void* x, const void* gy, void* dw, void* workspace, size_t workspace_bytes, int B, int H,
+                     int W, int C, int KH, int KW, int SH, int SW, int PH, int PW, int DH, int DW, int dtype,
+                     void* stream) {
+    if (int e = check_conv("pdw_dwconv_wgrad", x, gy, dw, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
+    if (!dw) return set_error("pdw_dwconv_wgrad: null dw"), 1;
+    const size_t need = pdw_dwconv_wgrad_workspace_bytes(B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype);
+    if (!workspace || workspace_bytes < need)
+        return set_error("pdw_dwconv_wgrad: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
+    return dwconv_wgrad_direct_launch(x, gy, dw, workspace, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype,
+                                      (hipStream_t)stream);
+}
+
+int pdw_avgpool_fwd(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
+    if (int e = check_resample("pdw_avgpool_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
+    return avgpool_fwd_launch(x, y, B, H, W, C, h, w, dtype, (hipStream_t)stream);
+}
+
+int pdw_avgpool_bwd(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
+    if (int e = check_resample("pdw_avgpool_bwd", gy, gx, B, H, W, C, h, w, dtype)) return e;
+    return avgpool_bwd_launch(gy, gx, B, H, W, C, h, w, dtype, (hipStream_t)stream);
+}
+
+int pdw_bilinear_fwd(const void* x, void* y, int B, int h, int w, int C, int H, int W, int dtype, void* stream) {
+    if (int e = check_resample("pdw_bilinear_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
+    return bilinear_fwd_launch(x, y, B, h, w, C, H, W, dtype, (hipStream_t)stream);
+}
+
+int pdw_bilinear_bwd(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int dtype, void* stream) {
+    if (int e = check_resample("pdw_bilinear_bwd", gy, gx, B, H, W, C, h, w, dtype)) return e;
+    return bilinear_bwd_launch(gy, gx, B, h, w, C, H, W, dtype, (hipStream_t)stream);
+}
+
+int pdw_gate_fwd(const void* x, void* y, long long M, int I, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_gate_fwd: unknown dtype %d", dtype), 1;
+    if (M < 0 || I < 2 || (I & 1)) return set_error("pdw_gate_fwd: need M >= 0 and even I >= 2 (M=%lld I=%d)", M, I), 1;
+    if (M > 0 && (!x || !y)) return set_error("pdw_gate_fwd: null pointer"), 1;
+    return gate_fwd_launch(x, y, M, I, dtype, (hipStream_t)stream);
+}
+
+int pdw_gate_bwd(const void* x, const void* gy, void* gx, long long M, int I, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_gate_bwd: unknown dtype %d", dtype), 1;
+    if (M < 0 || I < 2 || (I & 1)) return set_error("pdw_gate_bwd: need M >= 0 and even I >= 2 (M=%lld I=%d)", M, I), 1;
+    if (M > 0 && (!x || !gy || !gx)) return set_error("pdw_gate_bwd: null pointer"), 1;
+    return gate_bwd_launch(x, gy, gx, M, I, dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,34 @@
+// Internal launcher interface between the C ABI (api.hip) and the kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+namespace pdw {
+
+inline int conv_out_size(int in, int k, int s, int p, int d) {
+    const int num = in + 2 * p - d * (k - 1) - 1;
+    return num < 0 ? 0 : num / s + 1;
+}
+
+// dwconv_direct.hip: any stride / padding / dilation
+int dwconv_fwd_direct_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW,
+                             int SH, int SW, int PH, int PW, int DH, int DW, int dtype, hipStream_t s);
+int dwconv_dgrad_direct_launch(const void* gy, const void* w, void* dx, int B, int H, int W, int C, int KH, int KW,
+                               int SH, int SW, int PH, int PW, int DH, int DW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_direct_workspace(int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW,
+                                     int DH, int DW);
+int dwconv_wgrad_direct_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C,
+                               int KH, int KW, int SH, int SW, int PH, int PW, int DH, int DW, int dtype,
+                               hipStream_t s);
+template <typename T>
+int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s);
+
+// resample.hip: adaptive average pool, bilinear resize, gate
+int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
+int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
+int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s);
+int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s);
+int gate_fwd_launch(const void* x, void* y, long long M, int I, int dtype, hipStream_t s);
+int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int dtype, hipStream_t s);
+
+}  // namespace pdw

@@ -1,0 +1,321 @@
+// HBM-bound helpers around the depthwise conv: adaptive average pooling, bilinear
+// resize (align_corners=False) and the multiplicative gate, forward and backward.
+// Channels-last; one thread owns VEC consecutive channels of one pixel (up to 16 bytes),
+// so every wavefront access is a contiguous run.  Both backward kernels are gathers:
+// each input element sums the few outputs that touch it, in a fixed order, so there are
+// no atomics and results are bit-reproducible.
+#include "common.h"
+#include "kernels.h"
+
+namespace pdw {
+
+// ---------------------------------------------------------------- adaptive average pool
+__device__ __forceinline__ int bin_start(int i, int in, int out) { return (int)(((long long)i * in) / out); }
+__device__ __forceinline__ int bin_end(int i, int in, int out) {
+    return (int)(((long long)(i + 1) * in + out - 1) / out);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void avgpool_fwd_k(const T* __restrict__ x, T* __restrict__ y, int H, int W, int C,
+                                                     int h, int w, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC;
+    const int c = (int)(idx % CV) * VEC;
+    long long t = idx / CV;
+    const int j = (int)(t % w);
+    t /= w;
+    const int i = (int)(t % h);
+    const long long b = t / h;
+    const int hs = bin_start(i, H, h), he = bin_end(i, H, h);
+    const int ws = bin_start(j, W, w), we = bin_end(j, W, w);
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    for (int ih = hs; ih < he; ++ih)
+        for (int iw = ws; iw < we; ++iw) {
+            float xv[VEC];
+            load_f32<T, VEC>(x + ((b * H + ih) * W + iw) * C + c, xv);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] += xv[v];
+        }
+    const float inv = 1.f / (float)((he - hs) * (we - ws));
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] *= inv;
+    store_f32<T, VEC>(y + ((b * h + i) * w + j) * C + c, acc);
+}
+
+// Input row ih lies in bins i with floor(ih*h/H) <= i <= ceil((ih+1)*h/H) - 1.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int H, int W,
+                                                     int C, int h, int w, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC;
+    const int c = (int)(idx % CV) * VEC;
+    long long t = idx / CV;
+    const int iw = (int)(t % W);
+    t /= W;
+    const int ih = (int)(t % H);
+    const long long b = t / H;
+    const int i0 = (int)(((long long)ih * h) / H), i1 = (int)((((long long)(ih + 1)) * h + H - 1) / H) - 1;
+    const int j0 = (int)(((long long)iw * w) / W), j1 = (int)((((long long)(iw + 1)) * w + W - 1) / W) - 1;
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    for (int i = i0; i <= i1; ++i) {
+        const int kh = bin_end(i, H, h) - bin_start(i, H, h);
+        for (int j = j0; j <= j1; ++j) {
+            const int kw = bin_end(j, W, w) - bin_start(j, W, w);
+            const float inv = 1.f / (float)(kh * kw);
+            float gv[VEC];
+            load_f32<T, VEC>(gy + ((b * h + i) * w + j) * C + c, gv);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] = fmaf(gv[v], inv, acc[v]);
+        }
+    }
+    store_f32<T, VEC>(gx + ((b * H + ih) * W + iw) * C + c, acc);
+}
+
+// ---------------------------------------------------------------- bilinear, align_corners=False
+// src = max(scale*(dst+0.5)-0.5, 0), i0 = floor(src), i1 = min(i0+1, in-1), lam = src - i0 (fp32, as ATen does
+// for every element type up to float).
+__device__ __forceinline__ void bl_src(int dst, float scale, int in, int& i0, int& i1, float& lam) {
+    float src = scale * ((float)dst + 0.5f) - 0.5f;
+    src = src < 0.f ? 0.f : src;
+    int lo = (int)src;
+    lo = lo > in - 1 ? in - 1 : lo;
+    i0 = lo;
+    i1 = lo + (lo < in - 1 ? 1 : 0);
+    lam = src - (float)lo;
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
+                                                      int C, int H, int W, float sy, float sx, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC;
+    const int c = (int)(idx % CV) * VEC;
+    long long t = idx / CV;
+    const int j = (int)(t % W);
+    t /= W;
+    const int i = (int)(t % H);
+    const long long b = t / H;
+    int y0, y1, x0, x1;
+    float ly, lx;
+    bl_src(i, sy, h, y0, y1, ly);
+    bl_src(j, sx, w, x0, x1, lx);
+    const T* xb = x + b * h * w * C + c;
+    float a[VEC], bb[VEC], cc[VEC], d[VEC], o[VEC];
+    load_f32<T, VEC>(xb + ((long long)y0 * w + x0) * C, a);
+    load_f32<T, VEC>(xb + ((long long)y0 * w + x1) * C, bb);
+    load_f32<T, VEC>(xb + ((long long)y1 * w + x0) * C, cc);
+    load_f32<T, VEC>(xb + ((long long)y1 * w + x1) * C, d);
+    const float hy = 1.f - ly, hx = 1.f - lx;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[v] = hy * (hx * a[v] + lx * bb[v]) + ly * (hx * cc[v] + lx * d[v]);
+    store_f32<T, VEC>(y + ((b * H + i) * W + j) * C + c, o);
+}
+
+// Weight with which destination index `dst` reads source index m along one axis.
+__device__ __forceinline__ float bl_weight(int dst, float scale, int in, int m) {
+    int i0, i1;
+    float lam;
+    bl_src(dst, scale, in, i0, i1, lam);
+    return (i0 == m ? 1.f - lam : 0.f) + (i1 == m ? lam : 0.f);
+}
+
+// Destination indices whose taps can include source m: src in [m-1, m+1), padded by 2 for fp rounding.
+__device__ __forceinline__ void bl_dst_range(int m, float scale, int out, int& lo, int& hi) {
+    const float inv = 1.f / scale;
+    lo = (int)floorf(((float)m - 0.5f) * inv - 0.5f) - 2;
+    hi = (int)ceilf(((float)m + 1.5f) * inv - 0.5f) + 2;
+    if (lo < 0 || m == 0) lo = 0;
+    if (hi > out - 1) hi = out - 1;
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w,
+                                                      int C, int H, int W, float sy, float sx, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC;
+    const int c = (int)(idx % CV) * VEC;
+    long long t = idx / CV;
+    const int n = (int)(t % w);
+    t /= w;
+    const int m = (int)(t % h);
+    const long long b = t / h;
+    int ilo, ihi, jlo, jhi;
+    bl_dst_range(m, sy, H, ilo, ihi);
+    bl_dst_range(n, sx, W, jlo, jhi);
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    const T* gb = gy + b * H * W * C + c;
+    for (int i = ilo; i <= ihi; ++i) {
+        const float wy = bl_weight(i, sy, h, m);
+        if (wy == 0.f) continue;
+        for (int j = jlo; j <= jhi; ++j) {
+            const float wx = bl_weight(j, sx, w, n);
+            if (wx == 0.f) continue;
+            float gv[VEC];
+            load_f32<T, VEC>(gb + ((long long)i * W + j) * C, gv);
+            const float ww = wy * wx;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, gv[v], acc[v]);
+        }
+    }
+    store_f32<T, VEC>(gx + ((b * h + m) * w + n) * C + c, acc);
+}
+
+// ---------------------------------------------------------------- gate
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __restrict__ y, int I, float s,
+                                                  long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int G = I / 2, GV = G / VEC;
+    const int c = (int)(idx % GV) * VEC;
+    const long long m = idx / GV;
+    float a[VEC], b[VEC], o[VEC];
+    load_f32<T, VEC>(x + m * I + c, a);
+    load_f32<T, VEC>(x + m * I + G + c, b);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o[v] = a[v] * b[v] * s;
+    store_f32<T, VEC>(y + m * G + c, o);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const T* __restrict__ gy,
+                                                  T* __restrict__ gx, int I, float s, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int G = I / 2, GV = G / VEC;
+    const int c = (int)(idx % GV) * VEC;
+    const long long m = idx / GV;
+    float a[VEC], b[VEC], g[VEC], ga[VEC], gb[VEC];
+    load_f32<T, VEC>(x + m * I + c, a);
+    load_f32<T, VEC>(x + m * I + G + c, b);
+    load_f32<T, VEC>(gy + m * G + c, g);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        ga[v] = g[v] * b[v] * s;
+        gb[v] = g[v] * a[v] * s;
+    }
+    store_f32<T, VEC>(gx + m * I + c, ga);
+    store_f32<T, VEC>(gx + m * I + G + c, gb);
+}
+
+// ---------------------------------------------------------------- launch plumbing
+// Instantiates KERNEL<T, VEC> for the element type and the widest legal channel vector.
+#define PDW_VEC_SWITCH(T, vec, CALL)                       \
+    switch (vec) {                                         \
+        case 8: if constexpr (sizeof(T) == 2) { CALL(T, 8) } break; \
+        case 4: CALL(T, 4) break;                          \
+        case 2: CALL(T, 2) break;                          \
+        default: CALL(T, 1) break;                         \
+    }
+#define PDW_TYPE_SWITCH(dtype, vec, CALL)                  \
+    switch (dtype) {                                       \
+        case kF32: PDW_VEC_SWITCH(float, vec, CALL) break; \
+        case kF16: PDW_VEC_SWITCH(f16_t, vec, CALL) break; \
+        default: PDW_VEC_SWITCH(bf16_t, vec, CALL) break;  \
+    }
+
+static inline size_t esize(int dtype) { return dtype == kF32 ? 4 : 2; }
+
+static bool grid_for(long long total, unsigned* blocks) {
+    const long long nb = (total + 255) / 256;
+    if (nb > 0x7fffffffLL) {
+        set_error("problem too large for one launch (%lld threads)", total);
+        return false;
+    }
+    *blocks = (unsigned)nb;
+    return true;
+}
+
+int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s) {
+    const void* ptrs[2] = {x, y};
+    const int vec = pick_vec(C, esize(dtype), ptrs, 2);
+    const long long total = (long long)B * h * w * (C / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+#define CALL(T, V) hipLaunchKernelGGL((avgpool_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, H, W, C, h, w, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("avgpool_fwd");
+}
+
+int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s) {
+    const void* ptrs[2] = {gy, gx};
+    const int vec = pick_vec(C, esize(dtype), ptrs, 2);
+    const long long total = (long long)B * H * W * (C / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+#define CALL(T, V) hipLaunchKernelGGL((avgpool_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, H, W, C, h, w, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("avgpool_bwd");
+}
+
+int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s) {
+    const void* ptrs[2] = {x, y};
+    const int vec = pick_vec(C, esize(dtype), ptrs, 2);
+    const long long total = (long long)B * H * W * (C / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+    const float sy = (float)h / (float)H, sx = (float)w / (float)W;
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, h, w, C, H, W, sy, sx, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("bilinear_fwd");
+}
+
+int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s) {
+    const void* ptrs[2] = {gy, gx};
+    const int vec = pick_vec(C, esize(dtype), ptrs, 2);
+    const long long total = (long long)B * h * w * (C / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+    const float sy = (float)h / (float)H, sx = (float)w / (float)W;
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, h, w, C, H, W, sy, sx, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("bilinear_bwd");
+}
+
+int gate_fwd_launch(const void* x, void* y, long long M, int I, int dtype, hipStream_t s) {
+    const void* ptrs[2] = {x, y};
+    const int vec = pick_vec(I / 2, esize(dtype), ptrs, 2);
+    const long long total = M * (I / 2 / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+    const float sc = sqrtf((float)(I / 2));
+#define CALL(T, V) hipLaunchKernelGGL((gate_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, I, sc, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("gate_fwd");
+}
+
+int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int dtype, hipStream_t s) {
+    const void* ptrs[3] = {x, gy, gx};
+    const int vec = pick_vec(I / 2, esize(dtype), ptrs, 3);
+    const long long total = M * (I / 2 / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+    const float sc = sqrtf((float)(I / 2));
+#define CALL(T, V) hipLaunchKernelGGL((gate_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (const T*)gy, (T*)gx, I, sc, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("gate_bwd");
+}
+
+}  // namespace pdw

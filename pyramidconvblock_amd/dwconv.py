@@ -1,0 +1,133 @@
+"""Depthwise conv2d on channels-last tensors, backed by libpdw.so.
+
+Mirrors the reference operator API: ``DepthwiseConv2DFunction``
+(pyramid_dwconv/dwconv_triton.py:299-387) and ``OptimizedDepthwiseConv2d``
+(pyramid_dwconv/dwconv_triton.py:389-426).  Same call signatures, parameter name, weight
+layout ``[k1,k2,C]`` and default initialisation.  Differences, all in the direction of
+correctness: inputs are made contiguous and moved to the weight dtype, arguments are
+checked, the backward is the exact adjoint for every stride/padding/dilation, and the
+weight gradient is accumulated in fp32 without atomics (bit-reproducible).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, int) else (int(v[0]), int(v[1]))
+
+
+def _conv_args(x_shape, w_shape, stride, padding, dilation):
+    B, H, W, C = x_shape
+    KH, KW = w_shape[0], w_shape[1]
+    return (B, H, W, C, KH, KW, stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1])
+
+
+def dwconv_forward(x, weight, stride, padding, dilation):
+    """y[B,OH,OW,C] = depthwise cross-correlation of x[B,H,W,C] with weight[k1,k2,C]."""
+    dev = _lib.require_device(x, weight)
+    L = _lib.lib()
+    args = _conv_args(x.shape, weight.shape, stride, padding, dilation)
+    OH = L.pdw_conv_out_size(args[1], args[4], stride[0], padding[0], dilation[0])
+    OW = L.pdw_conv_out_size(args[2], args[5], stride[1], padding[1], dilation[1])
+    y = torch.empty((x.shape[0], OH, OW, x.shape[3]), device=dev, dtype=x.dtype)
+    if y.numel():
+        with _lib.on_device(dev):
+            _lib.check(L.pdw_dwconv_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), *args,
+                                        _lib.dtype_code(x.dtype), _lib.stream_ptr(dev)), "pdw_dwconv_fwd")
+    return y
+
+
+def dwconv_dgrad(gy, weight, in_shape, stride, padding, dilation):
+    dev = _lib.require_device(gy, weight)
+    L = _lib.lib()
+    dx = torch.empty(in_shape, device=dev, dtype=gy.dtype)
+    if dx.numel():
+        if gy.numel() == 0:
+            return dx.zero_()
+        args = _conv_args(in_shape, weight.shape, stride, padding, dilation)
+        with _lib.on_device(dev):
+            _lib.check(L.pdw_dwconv_dgrad(gy.data_ptr(), weight.data_ptr(), dx.data_ptr(), *args,
+                                          _lib.dtype_code(gy.dtype), _lib.stream_ptr(dev)), "pdw_dwconv_dgrad")
+    return dx
+
+
+def dwconv_wgrad(x, gy, w_shape, stride, padding, dilation):
+    dev = _lib.require_device(x, gy)
+    L = _lib.lib()
+    dw = torch.empty(tuple(w_shape), device=dev, dtype=x.dtype)
+    if x.numel() == 0 or gy.numel() == 0:
+        return dw.zero_()
+    args = _conv_args(x.shape, w_shape, stride, padding, dilation)
+    code = _lib.dtype_code(x.dtype)
+    nbytes = L.pdw_dwconv_wgrad_workspace_bytes(*args, code)
+    ws = torch.empty(max(nbytes, 4) // 4 + 1, device=dev, dtype=torch.float32)
+    with _lib.on_device(dev):
+        _lib.check(L.pdw_dwconv_wgrad(x.data_ptr(), gy.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel() * 4,
+                                      *args, code, _lib.stream_ptr(dev)), "pdw_dwconv_wgrad")
+    return dw
+
+
+class DepthwiseConv2DFunction(torch.autograd.Function):
+    """apply(input[B,H,W,C], weight[k1,k2,C], stride, padding, dilation, dtype) -> output[B,OH,OW,C] of `dtype`.
+
+    backward returns (grad_input like input, grad_weight like weight, None, None, None, None),
+    as dwconv_triton.py:387 does.
+    """
+
+    @staticmethod
+    def forward(ctx, input, weight, stride, padding, dilation, dtype):
+        stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+        if input.dim() != 4 or weight.dim() != 3 or input.shape[3] != weight.shape[2]:
+            raise ValueError(f"expected input [B,H,W,C] and weight [k1,k2,C], got {tuple(input.shape)} and "
+                             f"{tuple(weight.shape)}")
+        dtype = dtype if dtype is not None else weight.dtype
+        ctx.stride, ctx.padding, ctx.dilation = stride, padding, dilation
+        ctx.in_dtype, ctx.w_dtype = input.dtype, weight.dtype
+        x = input.detach().to(dtype).contiguous()
+        w = weight.detach().to(dtype).contiguous()
+        y = dwconv_forward(x, w, stride, padding, dilation)
+        ctx.save_for_backward(x, w)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, w = ctx.saved_tensors
+        gy = grad_output.to(x.dtype).contiguous()
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = dwconv_dgrad(gy, w, x.shape, ctx.stride, ctx.padding, ctx.dilation).to(ctx.in_dtype)
+        if ctx.needs_input_grad[1]:
+            dw = dwconv_wgrad(x, gy, w.shape, ctx.stride, ctx.padding, ctx.dilation).to(ctx.w_dtype)
+        return dx, dw, None, None, None, None
+
+
+class OptimizedDepthwiseConv2d(torch.nn.Module):
+    """Depthwise conv layer with weight ``[k1,k2,C]`` on ``[B,H,W,C]`` input.
+
+    As in the reference (dwconv_triton.py:390-416) the ``dtype`` argument is accepted and
+    ignored: the weight is created in float16 and filled by ``kaiming_uniform_``; callers move
+    the module with ``.to(dtype)``.  There is no bias.
+    """
+
+    def __init__(self, channels, kernel_size, stride=1, padding=0, dilation=1, dtype=None):
+        super().__init__()
+        self.channels = channels
+        self.kernel_size = _pair(kernel_size)
+        self.stride = _pair(stride)
+        self.padding = _pair(padding)
+        self.dilation = _pair(dilation)
+        self.weight = torch.nn.Parameter(torch.empty(self.kernel_size[0], self.kernel_size[1], channels,
+                                                     dtype=torch.float16))
+        torch.nn.init.kaiming_uniform_(self.weight)
+
+    def forward(self, x):
+        assert x.dim() == 4 and x.shape[3] == self.channels, "input must be [B,H,W,C] with matching channels"
+        return DepthwiseConv2DFunction.apply(x, self.weight, self.stride, self.padding, self.dilation,
+                                             self.weight.dtype)
+
+    def extra_repr(self):
+        return (f"channels={self.channels}, kernel_size={self.kernel_size}, stride={self.stride}, "
+                f"padding={self.padding}, dilation={self.dilation}")

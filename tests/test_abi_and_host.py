@@ -1,0 +1,75 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares,
+and the host-side mirror keeps the reference's module structure, names and init."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from pyramidconvblock_amd import _lib
+
+    header = open(os.path.join(ROOT, "include", "pdw.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(pdw_\w+)\s*\(", header))
+    assert len(declared) >= 13
+    L = _lib.lib()  # loads libpdw.so (built in-tree); no compute call is made here
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(raw, name), f"libpdw.so does not export {name}"
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    assert L.pdw_version() >= 1
+    assert L.pdw_conv_out_size(56, 13, 1, 6, 1) == 56
+    assert L.pdw_conv_out_size(5, 9, 1, 0, 1) == 0
+    assert L.pdw_conv_out_size(32, 7, 2, 3, 1) == 16
+
+
+def test_argument_validation_without_gpu():
+    from pyramidconvblock_amd import _lib
+
+    L = _lib.lib()
+    # invalid arguments are rejected before any HIP call
+    assert L.pdw_dwconv_fwd(None, None, None, 1, 4, 4, 8, 3, 3, 1, 1, 1, 1, 1, 1, 7, None) != 0
+    assert b"dtype" in L.pdw_last_error()
+    assert L.pdw_dwconv_fwd(None, None, None, 1, 4, 4, 8, 3, 3, 0, 1, 1, 1, 1, 1, 0, None) != 0
+    assert b"stride" in L.pdw_last_error()
+    assert L.pdw_gate_fwd(None, None, 4, 7, 0, None) != 0
+    assert L.pdw_dwconv_wgrad_workspace_bytes(2, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 0) > 0
+    assert L.pdw_dwconv_wgrad(1, 1, 1, None, 0, 2, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 0, None) != 0
+    assert b"workspace" in L.pdw_last_error()
+
+
+def test_module_structure_and_seeded_init_match_reference_recipe():
+    import pyramid_dwconv
+    from oracle import torch_path
+
+    torch.manual_seed(0)
+    m = pyramid_dwconv.ConvBlock(dim=64, kernel_size=7)
+    torch.manual_seed(0)
+    P = torch_path.default_params(64, 7)
+    sd = m.state_dict()
+    assert list(sd.keys()) == list(P.keys())
+    for k in P:
+        assert sd[k].dtype == P[k].dtype and torch.equal(sd[k], P[k]), k
+    assert tuple(sd["gates.1.conv_spatial.weight"].shape) == (7, 7, 32)
+    assert sd["gates.0.conv_spatial.weight"].dtype == torch.float16
+    assert m.gates[1].scale_factor == 0.5 and abs(m.gates[0].scale - 16 ** -0.5) < 1e-12
+    mb = m.to(torch.bfloat16)
+    assert all(v.dtype == torch.bfloat16 for v in mb.state_dict().values())
+
+
+def test_no_cpu_path():
+    import pyramidconvblock_amd as P
+
+    conv = P.OptimizedDepthwiseConv2d(8, 3, padding=1, dtype=torch.float32)
+    assert conv.weight.dtype == torch.float16  # dtype argument ignored, as in the reference
+    with pytest.raises(RuntimeError, match="HIP device"):
+        conv(torch.zeros(1, 4, 4, 8, dtype=torch.float16))
+    with pytest.raises(AssertionError):
+        conv(torch.zeros(1, 4, 4, 9))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        P.ConvBlock(8, kernel_size=3)(torch.zeros(1, 4, 4, 8))

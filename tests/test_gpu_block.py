@@ -1,0 +1,56 @@
+"""Parity of the full ConvBlock (forward, dx and every parameter gradient) with the float64
+block oracle at the BASELINE configurations."""
+import pytest
+import torch
+
+from parity import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+
+
+def _block_case(oracle, dim, k, shape, dtype, dist="normal", seed=0, scale=1.0):
+    import pyramid_dwconv
+
+    torch.manual_seed(seed)  # module first, then x, then grad (the order the configs state)
+    m = pyramid_dwconv.ConvBlock(dim=dim, kernel_size=k)
+    gen = torch.Generator().manual_seed(seed)
+    x = randn(gen, *shape) if dist == "normal" else torch.rand(*shape, generator=gen) * 4 - 2
+    g = randn(gen, *shape)
+    m = m.to(dtype)
+    params = {n: p.detach().double().numpy() for n, p in m.state_dict().items()}
+    xr, gr = x.to(dtype), g.to(dtype)
+    yo, cache = oracle.convblock_fwd(xr.double().numpy(), params)
+    dxo, go = oracle.convblock_bwd(cache, gr.double().numpy())
+    m = m.cuda()
+    xd = xr.cuda().requires_grad_()
+    y = m(xd)
+    assert y.dtype == dtype and y.shape == xd.shape
+    errs = {"y": assert_close(y, yo, dtype, "y", scale)}
+    torch.autograd.backward(y, gr.cuda())
+    errs["dx"] = assert_close(xd.grad, dxo, dtype, "dx", scale)
+    for n, p in m.named_parameters():
+        errs[n] = assert_close(p.grad, go[n], dtype, "grad " + n, scale)
+    return errs
+
+
+def test_config1_fp32(oracle):
+    _block_case(oracle, 64, 7, (2, 32, 32, 64), torch.float32)
+
+
+def test_config3_bf16(oracle):
+    _block_case(oracle, 128, 13, (32, 56, 56, 128), torch.bfloat16)
+
+
+@pytest.mark.parametrize("k", [9, 17])
+def test_metric_sweep_bf16(oracle, k):
+    _block_case(oracle, 128, k, (8, 56, 56, 128), torch.bfloat16)
+
+
+def test_config4_fp16(oracle):
+    _block_case(oracle, 96, 17, (8, 112, 112, 96), torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k", [9, 15])
+def test_config5_ragged(oracle, dtype, k):
+    _block_case(oracle, 200, k, (3, 57, 61, 200), dtype, dist="uniform")

@@ -1,0 +1,135 @@
+"""Parity of the HIP depthwise conv (fwd, dgrad, wgrad) with the float64 oracle, called
+through the C ABI of libpdw.so via the operator mirror."""
+import numpy as np
+import pytest
+import torch
+
+from parity import TOL, assert_close, randn, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+
+
+def _run(oracle, shape, k, dtype, stride=1, padding=None, dilation=1, seed=0, dist="normal", wscale=None):
+    import pyramidconvblock_amd as P
+
+    B, H, W, C = shape
+    kh, kw = (k, k) if isinstance(k, int) else k
+    pad = (kh // 2, kw // 2) if padding is None else padding
+    gen = torch.Generator().manual_seed(seed)
+    x = randn(gen, B, H, W, C) if dist == "normal" else torch.rand(B, H, W, C, generator=gen) * 4 - 2
+    w = randn(gen, kh, kw, C) * (wscale if wscale is not None else 1.0 / max(kh, kw))
+    xr, wr = x.to(dtype), w.to(dtype)
+    xd = xr.cuda().requires_grad_()
+    wd = wr.cuda().requires_grad_()
+    y = P.DepthwiseConv2DFunction.apply(xd, wd, stride, pad, dilation, dtype)
+    yo = oracle.dwconv_fwd(xr.double().numpy(), wr.double().numpy(), stride, pad, dilation)
+    assert y.dtype == dtype and tuple(y.shape) == yo.shape
+    errs = [assert_close(y, yo, dtype, "y")]
+    g = randn(gen, *y.shape).to(dtype)
+    y.backward(g.cuda())
+    go = g.double().numpy()
+    errs.append(assert_close(xd.grad, oracle.dwconv_dgrad(go, wr.double().numpy(), (H, W), stride, pad, dilation), dtype, "dx"))
+    errs.append(assert_close(wd.grad, oracle.dwconv_wgrad(xr.double().numpy(), go, (kh, kw), stride, pad, dilation), dtype, "dW"))
+    assert xd.grad.dtype == dtype and wd.grad.dtype == dtype and wd.grad.shape == wd.shape
+    return errs
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [3, 7, 9, 13, 17])
+def test_same_padding_small(oracle, dtype, k):
+    _run(oracle, (2, 20, 23, 24), k, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [1, 3, 10, 50, 100, 136])
+def test_channel_counts_and_vector_widths(oracle, dtype, C):
+    _run(oracle, (2, 11, 9, C), 5, dtype, seed=C)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geom", [
+    dict(k=(3, 5), stride=(2, 1), padding=(0, 2), dilation=(1, 2)),
+    dict(k=(4, 2), stride=(2, 3), padding=(2, 1), dilation=(2, 1)),
+    dict(k=(5, 5), stride=1, padding=(0, 0)),
+    dict(k=(5, 7), stride=1, padding=(4, 1)),
+    dict(k=(9, 9), stride=1, padding=(4, 4)),
+])
+def test_general_stride_padding_dilation(oracle, dtype, geom):
+    _run(oracle, (2, 14, 15, 12), dtype=dtype, **geom)
+
+
+def test_kernel_larger_than_image(oracle):
+    _run(oracle, (1, 6, 5, 8), 13, torch.float32)
+    _run(oracle, (1, 6, 5, 8), 13, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k", [9, 15])
+def test_config5_ragged(oracle, dtype, k):
+    """[3,57,61,100] is the conv the ragged ConvBlock(200) runs; U(-2,2) input."""
+    _run(oracle, (3, 57, 61, 100), k, dtype, dist="uniform")
+    _run(oracle, (3, 28, 30, 100), k, dtype, dist="uniform")
+
+
+@pytest.mark.parametrize("k", [9, 13, 17])
+def test_config2_full_size_bf16(oracle, k):
+    """x [32,56,56,128] ~ N(0,1), w ~ N(0, 1/k^2), bf16 (forward is the benchmarked op; grads checked too)."""
+    _run(oracle, (32, 56, 56, 128), k, torch.bfloat16)
+
+
+def test_config4_conv_fp16(oracle):
+    _run(oracle, (8, 112, 112, 48), 17, torch.float16)
+
+
+def test_empty_batch_and_empty_output():
+    import pyramidconvblock_amd as P
+
+    w = torch.randn(3, 3, 8, device="cuda")
+    y = P.DepthwiseConv2DFunction.apply(torch.zeros(0, 5, 5, 8, device="cuda"), w, 1, 1, 1, torch.float32)
+    assert tuple(y.shape) == (0, 5, 5, 8)
+    x = torch.randn(2, 2, 2, 8, device="cuda", requires_grad=True)
+    wp = w.clone().requires_grad_()
+    y = P.DepthwiseConv2DFunction.apply(x, wp, 1, 0, 1, torch.float32)  # 3x3 valid conv on 2x2: empty
+    assert tuple(y.shape) == (2, 0, 0, 8)
+    y.sum().backward()
+    assert torch.all(x.grad == 0) and torch.all(wp.grad == 0)
+
+
+def test_wgrad_is_deterministic():
+    import pyramidconvblock_amd as P
+
+    gen = torch.Generator().manual_seed(1)
+    x = randn(gen, 4, 33, 31, 40).to(torch.bfloat16).cuda()
+    g = randn(gen, 4, 33, 31, 40).to(torch.bfloat16).cuda()
+    from pyramidconvblock_amd.dwconv import dwconv_wgrad
+    a = dwconv_wgrad(x, g, (9, 9, 40), (1, 1), (4, 4), (1, 1))
+    b = dwconv_wgrad(x, g, (9, 9, 40), (1, 1), (4, 4), (1, 1))
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_full_size_properties(dtype):
+    """Size-independent checks at the benchmark shape: delta kernel = identity, linearity in w,
+    and the adjoint identity <conv(x,w), g> = <x, dgrad(g,w)> = <w, wgrad(x,g)>."""
+    from pyramidconvblock_amd.dwconv import dwconv_dgrad, dwconv_forward, dwconv_wgrad
+
+    B, H, W, C, k = 32, 56, 56, 128, 13
+    gen = torch.Generator().manual_seed(3)
+    x = randn(gen, B, H, W, C).to(dtype).cuda()
+    g = randn(gen, B, H, W, C).to(dtype).cuda()
+    w = (randn(gen, k, k, C) / k).to(dtype).cuda()
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    delta = torch.zeros(k, k, C, dtype=dtype, device="cuda")
+    delta[k // 2, k // 2] = 1
+    assert torch.equal(dwconv_forward(x, delta, *geo), x)
+    y = dwconv_forward(x, w, *geo)
+    y2 = dwconv_forward(x, (2 * w), *geo)
+    assert rel_err(y2, 2 * y.double().cpu().numpy()) <= TOL[dtype]
+    lhs = float((y.double() * g.double()).sum())
+    dx = dwconv_dgrad(g, w, x.shape, *geo)
+    dw = dwconv_wgrad(x, g, w.shape, *geo)
+    tol = 5e-3 if dtype != torch.float32 else 1e-4
+    assert abs(float((dx.double() * x.double()).sum()) - lhs) <= tol * abs(lhs)
+    assert abs(float((dw.double() * w.double()).sum()) - lhs) <= tol * abs(lhs)

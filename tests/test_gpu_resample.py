@@ -1,0 +1,79 @@
+"""Parity of the HIP adaptive average pool, bilinear resize and gate (forward and
+backward) with the float64 oracle, through the C ABI."""
+import pytest
+import torch
+
+from parity import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+
+POOL = [((8, 10), (4, 5), 16), ((57, 61), (28, 30), 100), ((9, 7), (4, 3), 3), ((5, 5), (5, 5), 8), ((7, 9), (1, 1), 6),
+        ((6, 6), (4, 4), 2), ((56, 56), (28, 28), 64), ((4, 5), (9, 11), 4)]
+UP = [((4, 5), (8, 10), 16), ((28, 30), (57, 61), 50), ((3, 4), (7, 9), 3), ((5, 5), (5, 5), 8), ((1, 1), (4, 3), 6),
+      ((8, 8), (5, 6), 2), ((28, 28), (56, 56), 32), ((56, 56), (112, 112), 24)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hw,out,C", POOL)
+def test_avgpool(oracle, dtype, hw, out, C):
+    import pyramidconvblock_amd as P
+
+    gen = torch.Generator().manual_seed(C)
+    x = randn(gen, 3, *hw, C).to(dtype)
+    xd = x.cuda().requires_grad_()
+    y = P.AdaptiveAvgPool2dFunction.apply(xd, out)
+    assert_close(y, oracle.avgpool_fwd(x.double().numpy(), out), dtype, "pool y")
+    g = randn(gen, *y.shape).to(dtype)
+    y.backward(g.cuda())
+    assert_close(xd.grad, oracle.avgpool_bwd(g.double().numpy(), hw), dtype, "pool dx")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hw,out,C", UP)
+def test_bilinear(oracle, dtype, hw, out, C):
+    import pyramidconvblock_amd as P
+
+    gen = torch.Generator().manual_seed(C + 100)
+    x = randn(gen, 2, *hw, C).to(dtype)
+    xd = x.cuda().requires_grad_()
+    y = P.BilinearInterp2dFunction.apply(xd, out)
+    assert_close(y, oracle.bilinear_fwd(x.double().numpy(), out), dtype, "bilinear y")
+    g = randn(gen, *y.shape).to(dtype)
+    y.backward(g.cuda())
+    assert_close(xd.grad, oracle.bilinear_bwd(g.double().numpy(), hw), dtype, "bilinear dx")
+
+
+def test_bilinear_exact_2x_is_exact_in_fp32():
+    """At exact 2x the weights are 0.25/0.75 (and 1 at the border), representable exactly."""
+    import pyramidconvblock_amd as P
+
+    x = torch.tensor([1.0, 5.0, 2.0, 8.0]).reshape(1, 1, 4, 1).repeat(1, 1, 1, 4).cuda()
+    y = P.OptimizedBilinearInterp2d((1, 8))(x)[0, 0, :, 0].cpu()
+    ref = torch.tensor([1.0, 2.0, 4.0, 4.25, 2.75, 3.5, 6.5, 8.0])
+    assert torch.equal(y, ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("I", [2, 6, 32, 64, 100, 48])
+def test_gate(oracle, dtype, I):
+    import pyramidconvblock_amd as P
+
+    gen = torch.Generator().manual_seed(I)
+    x = randn(gen, 2, 5, 7, I).to(dtype)
+    xd = x.cuda().requires_grad_()
+    y = P.GateFunction.apply(xd)
+    assert_close(y, oracle.gate_fwd(x.double().numpy()), dtype, "gate y")
+    g = randn(gen, *y.shape).to(dtype)
+    y.backward(g.cuda())
+    assert_close(xd.grad, oracle.gate_bwd(x.double().numpy(), g.double().numpy()), dtype, "gate dx")
+
+
+def test_modules_and_empty():
+    import pyramidconvblock_amd as P
+
+    x = torch.randn(2, 8, 8, 16, device="cuda")
+    assert tuple(P.OptimizedAdaptiveAvgPool2d(4)(x).shape) == (2, 4, 4, 16)
+    assert tuple(P.OptimizedBilinearInterp2d(12)(x).shape) == (2, 12, 12, 16)
+    e = torch.zeros(0, 8, 8, 16, device="cuda")
+    assert tuple(P.OptimizedAdaptiveAvgPool2d((3, 2))(e).shape) == (0, 3, 2, 16)
