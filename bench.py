@@ -128,6 +128,37 @@ def kernel_rooflines(B, H, W, D, k, dtype):
     return out
 
 
+def run_single_kernel(name, iters, B, H, W, D, k, dtype):
+    """Launches one hot kernel `iters` times at its shape inside the headline block (for rocprofv3 runs).
+    name: {fwd,dgrad,wgrad}_{full,half} | avgpool_fwd | avgpool_bwd | bilinear_fwd | bilinear_bwd"""
+    from pyramidconvblock_amd import avgpool, dwconv, up
+
+    I, G = D // 2, D // 4
+    h, w = H // 2, W // 2
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    op, _, res = name.partition("_")
+    if op in ("fwd", "dgrad", "wgrad"):
+        hh, ww = (H, W) if res == "full" else (h, w)
+        x = torch.randn(B, hh, ww, I, device="cuda").to(dtype)
+        g = torch.randn(B, hh, ww, I, device="cuda").to(dtype)
+        wt = (torch.randn(k, k, I, device="cuda") / k).to(dtype)
+        fn = {"fwd": lambda: dwconv.dwconv_forward(x, wt, *geo),
+              "dgrad": lambda: dwconv.dwconv_dgrad(g, wt, x.shape, *geo),
+              "wgrad": lambda: dwconv.dwconv_wgrad(x, g, wt.shape, *geo)}[op]
+    else:
+        a = torch.randn(B, H, W, I, device="cuda").to(dtype)
+        p = torch.randn(B, h, w, I, device="cuda").to(dtype)
+        gs = torch.randn(B, h, w, G, device="cuda").to(dtype)
+        gb = torch.randn(B, H, W, G, device="cuda").to(dtype)
+        fn = {"avgpool_fwd": lambda: avgpool.avgpool_forward(a, (h, w)),
+              "avgpool_bwd": lambda: avgpool.avgpool_backward(p, (H, W)),
+              "bilinear_fwd": lambda: up.bilinear_forward(gs, (H, W)),
+              "bilinear_bwd": lambda: up.bilinear_backward(gb, (h, w))}[name]
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+
+
 def cpu_baseline(B, H, W, D, k, dtype, threads, iters=3):
     """The reference's PyTorch path (F.conv2d groups=C, adaptive_avg_pool2d, interpolate, linear) on
     the host cores: forward+backward of the same block on the same seeded inputs."""
@@ -165,6 +196,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep and forward-only timings")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel event timings")
+    ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
+                    "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}")
+    ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (pure data parallel over B; "
@@ -177,6 +211,9 @@ def main():
     _lib.lib()
     dtype = torch.bfloat16
     B, H, W, D, k = (WORKLOAD[n] for n in ("B", "H", "W", "D", "k"))
+    if args.kernel:
+        run_single_kernel(args.kernel, args.steps, B, H, W, D, args.k, dtype)
+        return
     gen = torch.Generator().manual_seed(0)
     x = torch.randn(B, H, W, D, generator=gen).to(dtype).cuda().requires_grad_()
     g = torch.randn(B, H, W, D, generator=gen).to(dtype).cuda()

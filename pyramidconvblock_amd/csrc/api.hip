@@ -69,6 +69,10 @@ int pdw_dwconv_fwd(const void* x, const void* w, void* y, int B, int H, int W, i
                    int PH, int PW, int DH, int DW, int dtype, void* stream) {
     if (int e = check_conv("pdw_dwconv_fwd", x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
     if (B == 0 || conv_out_size(H, KH, SH, PH, DH) == 0 || conv_out_size(W, KW, SW, PW, DW) == 0) return 0;
+    if (SH == 1 && SW == 1 && DH == 1 && DW == 1) {
+        const int r = dwconv_tiled_launch(x, w, y, B, H, W, C, KH, KW, PH, PW, false, dtype, (hipStream_t)stream);
+        if (r != -1) return r;
+    }
     return dwconv_fwd_direct_launch(x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype, (hipStream_t)stream);
 }
 
@@ -76,6 +80,15 @@ int pdw_dwconv_dgrad(const void* gy, const void* w, void* dx, int B, int H, int 
                      int SW, int PH, int PW, int DH, int DW, int dtype, void* stream) {
     if (int e = check_conv("pdw_dwconv_dgrad", gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
     if (B == 0) return 0;
+    if (SH == 1 && SW == 1 && DH == 1 && DW == 1 && PH <= KH - 1 && PW <= KW - 1) {
+        // dx = correlation of gy with the 180-degree rotated filter at padding k-1-p
+        const int OH = conv_out_size(H, KH, 1, PH, 1), OW = conv_out_size(W, KW, 1, PW, 1);
+        if (OH > 0 && OW > 0) {
+            const int r = dwconv_tiled_launch(gy, w, dx, B, OH, OW, C, KH, KW, KH - 1 - PH, KW - 1 - PW, true, dtype,
+                                              (hipStream_t)stream);
+            if (r != -1) return r;
+        }
+    }
     return dwconv_dgrad_direct_launch(gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype,
                                       (hipStream_t)stream);
 }

@@ -1,0 +1,45 @@
+// Dispatch of the LDS-tiled depthwise convolution (stride 1, dilation 1) by filter width.
+// The kernel template and its description live in dwconv_tiled.h; each width is instantiated
+// in its own translation unit (dwconv_tiled_kw*.hip).
+#include "common.h"
+#include "kernels.h"
+
+namespace pdw {
+
+int dwconv_tiled_kw3(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw5(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw7(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw9(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw11(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw13(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw15(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+int dwconv_tiled_kw17(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
+                      bool flip, int dtype, hipStream_t s);
+
+// Returns -1 when the tiled kernel does not cover the case (the caller then uses the direct
+// kernel), otherwise the launch status.  With flip the 180-degree rotated filter is used: the
+// caller passes gy as x with padding k-1-p, which yields the input gradient.
+int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
+                        int PW, bool flip, int dtype, hipStream_t s) {
+    if (KH > 31 || H + 2 * PH - KH + 1 < 1 || W + 2 * PW - KW + 1 < 1) return -1;
+    switch (KW) {
+        case 3: return dwconv_tiled_kw3(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 5: return dwconv_tiled_kw5(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 7: return dwconv_tiled_kw7(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 9: return dwconv_tiled_kw9(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 11: return dwconv_tiled_kw11(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 13: return dwconv_tiled_kw13(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 15: return dwconv_tiled_kw15(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        case 17: return dwconv_tiled_kw17(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
+        default: return -1;
+    }
+}
+
+}  // namespace pdw

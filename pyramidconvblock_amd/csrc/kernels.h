@@ -23,6 +23,11 @@ int dwconv_wgrad_direct_launch(const void* x, const void* gy, void* dw, void* ws
 template <typename T>
 int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s);
 
+// dwconv_tiled.hip: LDS-tiled forward / input gradient for stride 1, dilation 1, odd KW <= 17.
+// Returns -1 if the case is not covered (the caller then uses the direct kernel).
+int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
+                        int PW, bool flip, int dtype, hipStream_t s);
+
 // resample.hip: adaptive average pool, bilinear resize, gate
 int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
 int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
