@@ -97,7 +97,12 @@ size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int 
                                         int DH, int DW, int dtype) {
     if (check_conv("pdw_dwconv_wgrad_workspace_bytes", "", "", "", B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype))
         return 0;
-    return dwconv_wgrad_direct_workspace(B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW);
+    size_t need = dwconv_wgrad_direct_workspace(B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW);
+    if (SH == 1 && SW == 1 && DH == 1 && DW == 1) {
+        const size_t t = dwconv_wgrad_tiled_workspace(B, H, W, C, KH, KW, PH, PW, dtype);
+        if (t > need) need = t;
+    }
+    return need;
 }
 
 int pdw_dwconv_wgrad(const void* x, const void* gy, void* dw, void* workspace, size_t workspace_bytes, int B, int H,
@@ -108,6 +113,11 @@ int pdw_dwconv_wgrad(const void* x, const void* gy, void* dw, void* workspace, s
     const size_t need = pdw_dwconv_wgrad_workspace_bytes(B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype);
     if (!workspace || workspace_bytes < need)
         return set_error("pdw_dwconv_wgrad: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
+    if (B > 0 && SH == 1 && SW == 1 && DH == 1 && DW == 1) {
+        const int r = dwconv_wgrad_tiled_launch(x, gy, dw, workspace, B, H, W, C, KH, KW, PH, PW, dtype,
+                                                (hipStream_t)stream);
+        if (r != -1) return r;
+    }
     return dwconv_wgrad_direct_launch(x, gy, dw, workspace, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype,
                                       (hipStream_t)stream);
 }

@@ -23,6 +23,7 @@
 
 #include "common.h"
 #include "kernels.h"
+#include "tile_common.h"
 
 namespace pdw {
 
@@ -38,35 +39,6 @@ struct TiledGeom {
     int flip;         // 1: use the 180-degree rotated filter (input gradient)
     int ulog;         // log2 of the staging threads laid along a row of LDS units
 };
-
-template <typename T>
-struct PackOf {
-    static constexpr int PK = 2;
-};
-template <>
-struct PackOf<float> {
-    static constexpr int PK = 1;
-};
-
-__device__ __forceinline__ float dot2acc(uint32_t a, uint32_t b, float c, bf16_t) {
-    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
-}
-__device__ __forceinline__ float dot2acc(uint32_t a, uint32_t b, float c, f16_t) {
-    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
-}
-
-__device__ __forceinline__ uint32_t bits16(bf16_t v) { return (uint32_t)__builtin_bit_cast(unsigned short, v); }
-__device__ __forceinline__ uint32_t bits16(f16_t v) { return (uint32_t)__builtin_bit_cast(unsigned short, v); }
-
-// XCD-aware work order: consecutive workgroup ids go to the 8 XCDs round-robin, so give each
-// XCD a contiguous range of work items (neighbouring tiles of one image share an L2).
-__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
-    const int per = nblocks >> 3;
-    if (bid >= (per << 3)) return bid;  // tail that does not fill all 8
-    return (bid & 7) * per + (bid >> 3);
-}
 
 template <typename T, int KW, int R, int Q, int CS, int V>
 __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, const T* __restrict__ w,
@@ -137,67 +109,9 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
         }
     }
 
-    // ---- stage the input tile with its halo (zeros outside the image / channel range).
-    // Thread (cv, u, rs): channel vector cv of LDS unit u in rows rs, rs+RS, ...; no divisions.
-    {
-        constexpr int CV = CS / V;
-        constexpr int UT = 256 / CV;
-        constexpr int SU = 4;
-        constexpr int NL = PK;  // pixels loaded per LDS unit
-        const T* xb = x + (long long)b * g.H * g.W * g.C;
-        const int cv = tid % CV, tu = tid / CV;
-        const int u0 = tu & ((1 << g.ulog) - 1), rs = tu >> g.ulog;
-        const int US = 1 << g.ulog, RS = UT >> g.ulog;
-        const int ch = c0 + cv * V;
-        const bool chok = ch < g.C;
-        const int chc = chok ? ch : 0;
-        for (int u = u0; u < g.CPn; u += US) {
-            int coff[NL];
-            bool cok[NL];
-#pragma unroll
-            for (int l = 0; l < NL; ++l) {
-                const int iw = icol0 + NL * u + l;
-                cok[l] = chok && iw >= 0 && iw < g.W;
-                coff[l] = min(max(iw, 0), g.W - 1) * g.C + chc;
-            }
-            for (int rb = rs; rb < g.rows_in; rb += RS * SU) {
-                ChanVec<T, V> ld[SU][NL];
-#pragma unroll
-                for (int s = 0; s < SU; ++s) {
-                    const int ih = min(max(irow0 + rb + s * RS, 0), g.H - 1);
-                    const T* xr = xb + (long long)ih * g.W * g.C;
-#pragma unroll
-                    for (int l = 0; l < NL; ++l) ld[s][l] = *reinterpret_cast<const ChanVec<T, V>*>(xr + coff[l]);
-                }
-#pragma unroll
-                for (int s = 0; s < SU; ++s) {
-                    const int r = rb + s * RS;
-                    if (r < g.rows_in) {
-                        const int ih = irow0 + r;
-                        const bool rok = ih >= 0 && ih < g.H;
-                        uint32_t out[V];
-#pragma unroll
-                        for (int i = 0; i < V; ++i) {
-                            if constexpr (PK == 2)
-                                out[i] = ((rok && cok[0]) ? bits16(ld[s][0].v[i]) : 0u) |
-                                         (((rok && cok[1]) ? bits16(ld[s][1].v[i]) : 0u) << 16);
-                            else
-                                out[i] = (rok && cok[0]) ? __builtin_bit_cast(uint32_t, ld[s][0].v[i]) : 0u;
-                        }
-                        uint32_t* dst = xl + (r * g.CPn + u) * CS + cv * V;
-                        if constexpr (V % 4 == 0) {
-#pragma unroll
-                            for (int i = 0; i < V; i += 4)
-                                *reinterpret_cast<uint4*>(dst + i) = make_uint4(out[i], out[i + 1], out[i + 2], out[i + 3]);
-                        } else {
-#pragma unroll
-                            for (int i = 0; i < V; ++i) dst[i] = out[i];
-                        }
-                    }
-                }
-            }
-        }
-    }
+    // ---- stage the input tile with its halo (zeros outside the image / channel range)
+    stage_tile<T, CS, V>(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, irow0, icol0, g.rows_in, g.CPn,
+                         g.ulog, c0, tid);
     __syncthreads();
 
     // ---- compute: each (wave, lane group) slot walks the tile's patches
@@ -337,8 +251,7 @@ static int launch_tiled(const TiledPlan& plan, const void* x, const void* w, voi
 #define PDW_GO(V)                                                                                            \
     {                                                                                                        \
         auto kern = dwconv_tiled_k<T, KW, R, Q, CS, V>;                                                      \
-        const int ut = 256 / (CS / V);                                                                       \
-        while ((1 << g.ulog) < g.CPn && (2 << g.ulog) <= ut) ++g.ulog;                                       \
+        g.ulog = stage_ulog(g.CPn, CS, V);                                                                   \
         static bool attr_done = false;                                                                       \
         if (!attr_done) {                                                                                    \
             (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \

@@ -1,0 +1,67 @@
+// Dispatch of the LDS-tiled depthwise-convolution weight gradient (stride 1, dilation 1, odd
+// square filters up to 17x17) by filter size.  The kernel template and its description live in
+// dwconv_wgrad_tiled.h; each size is instantiated in its own translation unit.
+#include "common.h"
+#include "kernels.h"
+
+namespace pdw {
+
+size_t dwconv_wgrad_tiled_ws_k3(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k3(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k5(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k5(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k7(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k7(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k9(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k9(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k11(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k11(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k13(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k13(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k15(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k15(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_tiled_ws_k17(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_k17(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                           int PW, int dtype, hipStream_t s);
+
+// Bytes of fp32 workspace the tiled weight gradient needs; 0 when it does not cover the case.
+size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype) {
+    if (KH != KW) return 0;
+    switch (KH) {
+        case 3: return dwconv_wgrad_tiled_ws_k3(B, H, W, C, PH, PW, dtype);
+        case 5: return dwconv_wgrad_tiled_ws_k5(B, H, W, C, PH, PW, dtype);
+        case 7: return dwconv_wgrad_tiled_ws_k7(B, H, W, C, PH, PW, dtype);
+        case 9: return dwconv_wgrad_tiled_ws_k9(B, H, W, C, PH, PW, dtype);
+        case 11: return dwconv_wgrad_tiled_ws_k11(B, H, W, C, PH, PW, dtype);
+        case 13: return dwconv_wgrad_tiled_ws_k13(B, H, W, C, PH, PW, dtype);
+        case 15: return dwconv_wgrad_tiled_ws_k15(B, H, W, C, PH, PW, dtype);
+        case 17: return dwconv_wgrad_tiled_ws_k17(B, H, W, C, PH, PW, dtype);
+        default: return 0;
+    }
+}
+
+// Returns -1 when the case is not covered (the caller then uses the direct kernel).
+int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int KH,
+                              int KW, int PH, int PW, int dtype, hipStream_t s) {
+    if (KH != KW) return -1;
+    switch (KH) {
+        case 3: return dwconv_wgrad_tiled_k3(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 5: return dwconv_wgrad_tiled_k5(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 7: return dwconv_wgrad_tiled_k7(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 9: return dwconv_wgrad_tiled_k9(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 11: return dwconv_wgrad_tiled_k11(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 13: return dwconv_wgrad_tiled_k13(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 15: return dwconv_wgrad_tiled_k15(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 17: return dwconv_wgrad_tiled_k17(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        default: return -1;
+    }
+}
+
+}  // namespace pdw

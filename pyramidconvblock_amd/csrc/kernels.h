@@ -28,6 +28,11 @@ int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStrea
 int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
                         int PW, bool flip, int dtype, hipStream_t s);
 
+// dwconv_wgrad_tiled.hip: LDS-tiled weight gradient for stride 1, dilation 1, odd square filters <= 17.
+size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype);
+int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int KH,
+                              int KW, int PH, int PW, int dtype, hipStream_t s);
+
 // resample.hip: adaptive average pool, bilinear resize, gate
 int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
 int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
