@@ -71,22 +71,41 @@ int pdw_dwconv_wgrad(const void *x, const void *gy, void *dw, void *workspace, s
  * (kernel :14-107; integer bin arithmetic here instead of the fp16 one at :42-47). */
 int pdw_avgpool_fwd(const void *x, void *y, int B, int H, int W, int C, int h, int w, int dtype, void *stream);
 
-/* Its gradient gy[B,h,w,C] -> gx[B,H,W,C], gather form (no atomics, fully overwrites gx).
+/* Its gradient gy[B,h,w,C] -> gx[B,H,W,C], gather form (no atomics).  With accumulate != 0 the result
+ * is added to gx (fp32 add, one rounding), otherwise gx is fully overwritten.
  * Replaces avgpool_triton.py:253-257 (kernel :118-203). */
-int pdw_avgpool_bwd(const void *gy, void *gx, int B, int H, int W, int C, int h, int w, int dtype, void *stream);
+int pdw_avgpool_bwd(const void *gy, void *gx, int B, int H, int W, int C, int h, int w, int accumulate, int dtype,
+                    void *stream);
 
-/* Bilinear resize, align_corners=False, no explicit scale factor: x[B,h,w,C] -> y[B,H,W,C].
+/* Bilinear resize, align_corners=False, no explicit scale factor: x[B,h,w,C] -> y[B,H,W,C].  Output pixels are
+ * ldy elements apart (0 = dense, ldy = C), so the result can be written into a channel slice of a wider tensor
+ * (the torch.cat of conv_block.py:43).
  * Replaces F.interpolate at conv_block.py:21 and the launch at up_triton.py:157-161 (kernel :14-125). */
-int pdw_bilinear_fwd(const void *x, void *y, int B, int h, int w, int C, int H, int W, int dtype, void *stream);
+int pdw_bilinear_fwd(const void *x, void *y, int B, int h, int w, int C, int H, int W, int ldy, int dtype,
+                     void *stream);
 
-/* Its gradient gy[B,H,W,C] -> gx[B,h,w,C] (transpose of the above, gather form).  The reference
- * has no backward for up_triton.py; inside ConvBlock autograd supplies upsample_bilinear2d_backward. */
-int pdw_bilinear_bwd(const void *gy, void *gx, int B, int h, int w, int C, int H, int W, int dtype, void *stream);
+/* Its gradient gy[B,H,W,C] (pixels ldgy elements apart, 0 = dense) -> gx[B,h,w,C], transpose of the above in
+ * gather form.  The reference has no backward for up_triton.py; inside ConvBlock autograd supplies
+ * upsample_bilinear2d_backward. */
+int pdw_bilinear_bwd(const void *gy, void *gx, int B, int h, int w, int C, int H, int W, int ldgy, int dtype,
+                     void *stream);
 
-/* Gate  y[m,c] = x[m,c] * x[m,G+c] * sqrt(G),  G = I/2,  x[M,I] -> y[M,G]   (conv_block.py:10,18-19). */
-int pdw_gate_fwd(const void *x, void *y, long long M, int I, int dtype, void *stream);
-/* gx[m,c] = gy*x[m,G+c]*sqrt(G);  gx[m,G+c] = gy*x[m,c]*sqrt(G). */
-int pdw_gate_bwd(const void *x, const void *gy, void *gx, long long M, int I, int dtype, void *stream);
+/* Gate  y[m,c] = x[m,c] * x[m,G+c] * sqrt(G),  G = I/2,  x[M,I] -> y[M,G] with rows ldy elements apart
+ * (0 = dense)   (conv_block.py:10,18-19). */
+int pdw_gate_fwd(const void *x, void *y, long long M, int I, int ldy, int dtype, void *stream);
+/* gx[m,c] = gy*x[m,G+c]*sqrt(G);  gx[m,G+c] = gy*x[m,c]*sqrt(G); gy rows ldgy elements apart (0 = dense). */
+int pdw_gate_bwd(const void *x, const void *gy, void *gx, long long M, int I, int ldgy, int dtype, void *stream);
+
+/* Per-image sum over positions: x[B,P,C] -> out[B,C] (fp32), two deterministic passes through `workspace`.
+ * Replaces x.mean(dim=(1,2)) at conv_block.py:46 (divide by P on the host side) and, in the backward, the
+ * reduction of the broadcast add at conv_block.py:49. */
+size_t pdw_spatial_sum_workspace_bytes(int B, int P, int C);
+int pdw_spatial_sum(const void *x, float *out, void *workspace, size_t workspace_bytes, int B, int P, int C,
+                    int dtype, void *stream);
+
+/* In place y[b,p,c] += v[b,c] (v fp32 [B,C]): the broadcast add of the pooled branch, conv_block.py:49,
+ * and its mirror in the backward (the gradient of the mean, conv_block.py:46). */
+int pdw_add_rowbias(void *y, const float *v, int B, int P, int C, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

@@ -29,11 +29,14 @@ _SIGS = {
     "pdw_dwconv_wgrad_workspace_bytes": (c_size_t, _CONV + [c_int]),
     "pdw_dwconv_wgrad": (c_int, [c_void_p] * 4 + [c_size_t] + _CONV + [c_int, c_void_p]),
     "pdw_avgpool_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
-    "pdw_avgpool_bwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
-    "pdw_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
-    "pdw_bilinear_bwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
-    "pdw_gate_fwd": (c_int, [c_void_p] * 2 + [c_longlong, c_int, c_int, c_void_p]),
-    "pdw_gate_bwd": (c_int, [c_void_p] * 3 + [c_longlong, c_int, c_int, c_void_p]),
+    "pdw_avgpool_bwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
+    "pdw_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
+    "pdw_bilinear_bwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
+    "pdw_gate_fwd": (c_int, [c_void_p] * 2 + [c_longlong, c_int, c_int, c_int, c_void_p]),
+    "pdw_gate_bwd": (c_int, [c_void_p] * 3 + [c_longlong, c_int, c_int, c_int, c_void_p]),
+    "pdw_spatial_sum_workspace_bytes": (c_size_t, [c_int] * 3),
+    "pdw_spatial_sum": (c_int, [c_void_p] * 3 + [c_size_t] + [c_int] * 4 + [c_void_p]),
+    "pdw_add_rowbias": (c_int, [c_void_p] * 2 + [c_int] * 4 + [c_void_p]),
 }
 EXPORTS = tuple(_SIGS)
 

@@ -7,29 +7,7 @@ from __future__ import annotations
 
 import torch
 
-from . import _lib
-
-
-def _pool_call(fn_name, src, dst, B, H, W, C, h, w):
-    dev = _lib.require_device(src, dst)
-    if src.numel() and dst.numel():
-        with _lib.on_device(dev):
-            fn = getattr(_lib.lib(), fn_name)
-            _lib.check(fn(src.data_ptr(), dst.data_ptr(), B, H, W, C, h, w, _lib.dtype_code(src.dtype),
-                          _lib.stream_ptr(dev)), fn_name)
-    return dst
-
-
-def avgpool_forward(x, out_hw):
-    B, H, W, C = x.shape
-    h, w = int(out_hw[0]), int(out_hw[1])
-    return _pool_call("pdw_avgpool_fwd", x, torch.empty((B, h, w, C), device=x.device, dtype=x.dtype), B, H, W, C, h, w)
-
-
-def avgpool_backward(gy, in_hw):
-    B, h, w, C = gy.shape
-    H, W = int(in_hw[0]), int(in_hw[1])
-    return _pool_call("pdw_avgpool_bwd", gy, torch.empty((B, H, W, C), device=gy.device, dtype=gy.dtype), B, H, W, C, h, w)
+from .ops import avgpool_backward, avgpool_forward  # noqa: F401  (re-exported)
 
 
 class AdaptiveAvgPool2dFunction(torch.autograd.Function):

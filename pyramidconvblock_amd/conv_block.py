@@ -4,16 +4,23 @@ names, parameter shapes and ``[B,H,W,C]`` in/out contract
 
 ``state_dict`` keys match the reference: ``conv_up.weight``, ``gates.{i}.conv_spatial.weight``
 (``[k,k,inter_dim]``), ``conv_out.{weight,bias}``, ``conv_pool.{weight,bias}``.
+
+``ConvBlock.forward`` runs as ONE autograd node (``ConvBlockFunction``): the pooling, depthwise
+convolutions, gates and upsampling go through libpdw.so, the gate outputs are written straight
+into the halves of the concatenated buffer (no ``torch.cat``), the pooled branch is added in
+place, and the backward reuses one per-image column sum for both bias gradients and the
+gradient of the mean.  The three dense layers stay library GEMMs (hipBLASLt through torch);
+their weight gradients, whose reduction dimension is B*H*W, are computed as a batched
+split-K product because the library's single GEMM for that shape is ~10x slower.
 """
 from __future__ import annotations
 
 import torch
 from torch import nn
+from torch.nn import functional as F
 
-from . import _lib
-from .avgpool import AdaptiveAvgPool2dFunction
-from .dwconv import OptimizedDepthwiseConv2d
-from .up import BilinearInterp2dFunction
+from . import _lib, ops
+from .dwconv import OptimizedDepthwiseConv2d, dwconv_dgrad, dwconv_forward, dwconv_wgrad
 
 
 class GateFunction(torch.autograd.Function):
@@ -22,30 +29,13 @@ class GateFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x):
         x = x.detach().contiguous()
-        dev = _lib.require_device(x)
-        I = x.shape[-1]
-        if I % 2:
-            raise ValueError("gate needs an even channel count")
-        y = torch.empty(x.shape[:-1] + (I // 2,), device=dev, dtype=x.dtype)
-        if y.numel():
-            with _lib.on_device(dev):
-                _lib.check(_lib.lib().pdw_gate_fwd(x.data_ptr(), y.data_ptr(), x.numel() // I, I,
-                                                   _lib.dtype_code(x.dtype), _lib.stream_ptr(dev)), "pdw_gate_fwd")
         ctx.save_for_backward(x)
-        return y
+        return ops.gate_forward(x)
 
     @staticmethod
     def backward(ctx, gy):
         (x,) = ctx.saved_tensors
-        gy = gy.contiguous()
-        dev = x.device
-        I = x.shape[-1]
-        gx = torch.empty_like(x)
-        if gx.numel():
-            with _lib.on_device(dev):
-                _lib.check(_lib.lib().pdw_gate_bwd(x.data_ptr(), gy.data_ptr(), gx.data_ptr(), x.numel() // I, I,
-                                                   _lib.dtype_code(x.dtype), _lib.stream_ptr(dev)), "pdw_gate_bwd")
-        return gx
+        return ops.gate_backward(x, gy.contiguous())
 
 
 class SimpleGate(nn.Module):
@@ -59,6 +49,9 @@ class SimpleGate(nn.Module):
         self.conv_spatial = OptimizedDepthwiseConv2d(dim, kernel_size=kernel_size, padding=kernel_size // 2)
 
     def forward(self, x):
+        from .avgpool import AdaptiveAvgPool2dFunction
+        from .up import BilinearInterp2dFunction
+
         B, H, W, C = x.shape
         if self.scale_factor != 1.:
             x = AdaptiveAvgPool2dFunction.apply(x, (int(H * self.scale_factor), int(W * self.scale_factor)))
@@ -66,6 +59,133 @@ class SimpleGate(nn.Module):
         if self.scale_factor != 1.:
             x = BilinearInterp2dFunction.apply(x, (H, W))
         return x
+
+
+_BMM_FP32_OUT = [True]
+
+
+def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
+    """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I], as a batched product over S slabs of N summed in fp32."""
+    N = g2d.shape[0]
+    S = 1
+    while S < 256 and N % (2 * S) == 0 and N // (2 * S) >= 128:
+        S *= 2
+    if S == 1 or g2d.dtype == torch.float32:
+        return g2d.float().t() @ x2d.float() if N else g2d.new_zeros((g2d.shape[1], x2d.shape[1]), dtype=torch.float32)
+    a = g2d.view(S, N // S, -1).transpose(1, 2)
+    b = x2d.view(S, N // S, -1)
+    if _BMM_FP32_OUT[0]:
+        try:
+            return torch.bmm(a, b, out_dtype=torch.float32).sum(0)
+        except (TypeError, RuntimeError):
+            _BMM_FP32_OUT[0] = False
+    return torch.bmm(a, b).float().sum(0)
+
+
+class ConvBlockFunction(torch.autograd.Function):
+    """The whole block of conv_block.py:36-49 as one differentiable op.
+
+    apply(x, scales, kernel_sizes, w_up, b_up, w_out, b_out, w_pool, b_pool, *dw_weights)"""
+
+    @staticmethod
+    def forward(ctx, x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, *w_dw):
+        dev = _lib.require_device(x)
+        x = x.detach().contiguous()
+        B, H, W, D = x.shape
+        dt = x.dtype
+        a = F.linear(x, w_up, b_up)
+        I = a.shape[-1]
+        G = I // 2
+        ns = len(scales)
+        cat = torch.empty((B, H, W, G * ns), device=dev, dtype=dt)
+        convs, pooled = [], []
+        for i, s in enumerate(scales):
+            w = w_dw[i].detach().to(dt).contiguous()
+            k1, k2 = w.shape[0], w.shape[1]
+            geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
+            dst = cat[..., i * G:(i + 1) * G]
+            if s != 1.:
+                p = ops.avgpool_forward(a, (int(H * s), int(W * s)))
+                c = dwconv_forward(p, w, *geo)
+                ops.bilinear_forward(ops.gate_forward(c), (H, W), out=dst)
+            else:
+                p = None
+                c = dwconv_forward(a, w, *geo)
+                ops.gate_forward(c, out=dst)
+            convs.append(c)
+            pooled.append(p)
+        y = F.linear(cat, w_out)
+        m = (ops.spatial_sum(x) / float(H * W)).to(dt)          # x.mean(dim=(1,2))
+        yp = F.linear(m, w_pool, b_pool).float()
+        if b_out is not None:
+            yp = yp + b_out.float()
+        ops.add_rowbias_(y, yp.contiguous())                     # conv_out bias + broadcast pooled branch
+        ctx.scales = tuple(scales)
+        ctx.has_bias = (b_up is not None, b_out is not None, b_pool is not None)
+        ctx.save_for_backward(x, a, cat, m, w_up, w_out, w_pool, *w_dw, *convs, *[p for p in pooled if p is not None])
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        scales = ctx.scales
+        ns = len(scales)
+        saved = ctx.saved_tensors
+        x, a, cat, m, w_up, w_out, w_pool = saved[:7]
+        w_dw = saved[7:7 + ns]
+        convs = saved[7 + ns:7 + 2 * ns]
+        pooled_it = iter(saved[7 + 2 * ns:])
+        pooled = [next(pooled_it) if s != 1. else None for s in scales]
+        B, H, W, D = x.shape
+        dt = x.dtype
+        I = a.shape[-1]
+        G = I // 2
+        N = B * H * W
+        gy = gy.to(dt).contiguous()
+        g2d = gy.view(N, D)
+
+        gs = ops.spatial_sum(gy)                                 # [B, D] fp32: column sums per image
+        gbias = gs.sum(0)
+        grad_b_out = gbias.to(w_out.dtype) if ctx.has_bias[1] else None
+        grad_b_pool = gbias.to(w_pool.dtype) if ctx.has_bias[2] else None
+        grad_w_pool = (gs.t() @ m.float()).to(w_pool.dtype)
+        dm = gs @ w_pool.float()                                 # gradient of the per-image mean
+
+        dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
+        grad_w_out = _weight_grad(g2d, cat.view(N, G * ns)).to(w_out.dtype)
+
+        da = None
+        grad_w_dw = [None] * ns
+        order = sorted(range(ns), key=lambda i: scales[i] != 1.)   # dense gates first: they initialise da
+        for i in order:
+            s = scales[i]
+            w = w_dw[i].detach().to(dt).contiguous()
+            k1, k2 = w.shape[0], w.shape[1]
+            geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
+            dslice = dcat[..., i * G:(i + 1) * G]
+            c = convs[i]
+            if s != 1.:
+                gc = ops.gate_backward(c, ops.bilinear_backward(dslice, (c.shape[1], c.shape[2])))
+                src = pooled[i]
+            else:
+                gc = ops.gate_backward(c, dslice)
+                src = a
+            grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo).to(w_dw[i].dtype)
+            dp = dwconv_dgrad(gc, w, src.shape, *geo)
+            if s != 1.:
+                if da is None:
+                    da = ops.avgpool_backward(dp, (H, W))
+                else:
+                    ops.avgpool_backward(dp, (H, W), out=da, accumulate=True)
+            else:
+                da = dp if da is None else da.add_(dp)
+        a2d = da.view(N, I)
+        grad_w_up = _weight_grad(a2d, x.view(N, D)).to(w_up.dtype)
+        grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.matmul(a2d, w_up).view(B, H, W, D)
+            ops.add_rowbias_(dx, (dm / float(H * W)).contiguous())
+        return (dx, None, grad_w_up, grad_b_up, grad_w_out, grad_b_out, grad_w_pool, grad_b_pool, *grad_w_dw)
 
 
 class ConvBlock(nn.Module):
@@ -83,8 +203,9 @@ class ConvBlock(nn.Module):
 
     def forward(self, x):
         _lib.require_device(x)
-        x_conv = self.conv_up(x)
-        x_conv = torch.cat([gate(x_conv) for gate in self.gates], dim=-1)
-        x_conv = self.conv_out(x_conv)
-        x_pool = self.conv_pool(x.mean(dim=(1, 2), keepdim=True))
-        return x_conv + x_pool
+        if x.dim() != 4 or x.shape[3] != self.conv_up.in_features:
+            raise ValueError(f"expected [B,H,W,{self.conv_up.in_features}] input, got {tuple(x.shape)}")
+        scales = tuple(float(g.scale_factor) for g in self.gates)
+        return ConvBlockFunction.apply(x, scales, self.conv_up.weight, self.conv_up.bias, self.conv_out.weight,
+                                       self.conv_out.bias, self.conv_pool.weight, self.conv_pool.bias,
+                                       *[g.conv_spatial.weight for g in self.gates])

@@ -56,7 +56,7 @@ using namespace pdw;
 
 extern "C" {
 
-int pdw_version(void) { return 1; }
+int pdw_version(void) { return 2; }
 
 const char* pdw_last_error(void) { return g_err; }
 
@@ -127,33 +127,69 @@ int pdw_avgpool_fwd(const void* x, void* y, int B, int H, int W, int C, int h, i
     return avgpool_fwd_launch(x, y, B, H, W, C, h, w, dtype, (hipStream_t)stream);
 }
 
-int pdw_avgpool_bwd(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
+int pdw_avgpool_bwd(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int accumulate, int dtype,
+                    void* stream) {
     if (int e = check_resample("pdw_avgpool_bwd", gy, gx, B, H, W, C, h, w, dtype)) return e;
-    return avgpool_bwd_launch(gy, gx, B, H, W, C, h, w, dtype, (hipStream_t)stream);
+    return avgpool_bwd_launch(gy, gx, B, H, W, C, h, w, accumulate ? 1 : 0, dtype, (hipStream_t)stream);
 }
 
-int pdw_bilinear_fwd(const void* x, void* y, int B, int h, int w, int C, int H, int W, int dtype, void* stream) {
+int pdw_bilinear_fwd(const void* x, void* y, int B, int h, int w, int C, int H, int W, int ldy, int dtype,
+                     void* stream) {
     if (int e = check_resample("pdw_bilinear_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
-    return bilinear_fwd_launch(x, y, B, h, w, C, H, W, dtype, (hipStream_t)stream);
+    if (ldy == 0) ldy = C;
+    if (ldy < C) return set_error("pdw_bilinear_fwd: ldy=%d smaller than C=%d", ldy, C), 1;
+    return bilinear_fwd_launch(x, y, B, h, w, C, H, W, ldy, dtype, (hipStream_t)stream);
 }
 
-int pdw_bilinear_bwd(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int dtype, void* stream) {
+int pdw_bilinear_bwd(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int ldgy, int dtype,
+                     void* stream) {
     if (int e = check_resample("pdw_bilinear_bwd", gy, gx, B, H, W, C, h, w, dtype)) return e;
-    return bilinear_bwd_launch(gy, gx, B, h, w, C, H, W, dtype, (hipStream_t)stream);
+    if (ldgy == 0) ldgy = C;
+    if (ldgy < C) return set_error("pdw_bilinear_bwd: ldgy=%d smaller than C=%d", ldgy, C), 1;
+    return bilinear_bwd_launch(gy, gx, B, h, w, C, H, W, ldgy, dtype, (hipStream_t)stream);
 }
 
-int pdw_gate_fwd(const void* x, void* y, long long M, int I, int dtype, void* stream) {
+int pdw_gate_fwd(const void* x, void* y, long long M, int I, int ldy, int dtype, void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_gate_fwd: unknown dtype %d", dtype), 1;
     if (M < 0 || I < 2 || (I & 1)) return set_error("pdw_gate_fwd: need M >= 0 and even I >= 2 (M=%lld I=%d)", M, I), 1;
     if (M > 0 && (!x || !y)) return set_error("pdw_gate_fwd: null pointer"), 1;
-    return gate_fwd_launch(x, y, M, I, dtype, (hipStream_t)stream);
+    if (ldy == 0) ldy = I / 2;
+    if (ldy < I / 2) return set_error("pdw_gate_fwd: ldy=%d smaller than I/2=%d", ldy, I / 2), 1;
+    return gate_fwd_launch(x, y, M, I, ldy, dtype, (hipStream_t)stream);
 }
 
-int pdw_gate_bwd(const void* x, const void* gy, void* gx, long long M, int I, int dtype, void* stream) {
+int pdw_gate_bwd(const void* x, const void* gy, void* gx, long long M, int I, int ldgy, int dtype, void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_gate_bwd: unknown dtype %d", dtype), 1;
     if (M < 0 || I < 2 || (I & 1)) return set_error("pdw_gate_bwd: need M >= 0 and even I >= 2 (M=%lld I=%d)", M, I), 1;
     if (M > 0 && (!x || !gy || !gx)) return set_error("pdw_gate_bwd: null pointer"), 1;
-    return gate_bwd_launch(x, gy, gx, M, I, dtype, (hipStream_t)stream);
+    if (ldgy == 0) ldgy = I / 2;
+    if (ldgy < I / 2) return set_error("pdw_gate_bwd: ldgy=%d smaller than I/2=%d", ldgy, I / 2), 1;
+    return gate_bwd_launch(x, gy, gx, M, I, ldgy, dtype, (hipStream_t)stream);
+}
+
+size_t pdw_spatial_sum_workspace_bytes(int B, int P, int C) {
+    if (B < 1 || P < 1 || C < 1) return 0;
+    return spatial_sum_workspace(B, P, C);
+}
+
+int pdw_spatial_sum(const void* x, float* out, void* workspace, size_t workspace_bytes, int B, int P, int C, int dtype,
+                    void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_spatial_sum: unknown dtype %d", dtype), 1;
+    if (B < 0 || P < 1 || C < 1) return set_error("pdw_spatial_sum: bad extents B=%d P=%d C=%d", B, P, C), 1;
+    if (B == 0) return 0;
+    if (!x || !out) return set_error("pdw_spatial_sum: null pointer"), 1;
+    const size_t need = spatial_sum_workspace(B, P, C);
+    if (!workspace || workspace_bytes < need)
+        return set_error("pdw_spatial_sum: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
+    return spatial_sum_launch(x, out, (float*)workspace, B, P, C, dtype, (hipStream_t)stream);
+}
+
+int pdw_add_rowbias(void* y, const float* v, int B, int P, int C, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_add_rowbias: unknown dtype %d", dtype), 1;
+    if (B < 0 || P < 0 || C < 1) return set_error("pdw_add_rowbias: bad extents B=%d P=%d C=%d", B, P, C), 1;
+    if (B == 0 || P == 0) return 0;
+    if (!y || !v) return set_error("pdw_add_rowbias: null pointer"), 1;
+    return add_rowbias_launch(y, v, B, P, C, dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

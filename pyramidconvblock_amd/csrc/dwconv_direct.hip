@@ -119,22 +119,31 @@ __global__ __launch_bounds__(256) void dwconv_wgrad_direct(const T* __restrict__
     }
 }
 
-// Pass 2 of wgrad (shared with the tiled kernels): dw[e] = sum over parts, fixed order.
+// Pass 2 of wgrad (shared with the tiled kernels): dw[e] = sum over parts in a fixed order.
+// Block = 32 outputs x 8 part lanes; lane q adds parts q, q+8, ... and the 8 lanes are combined
+// through LDS, so the reads of one part are contiguous and many parts are in flight.
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restrict__ part, T* __restrict__ dw,
                                                           int nparts, int n) {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n) return;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    int p = 0;
-    for (; p + 4 <= nparts; p += 4) {
-        s0 += part[(long long)p * n + e];
-        s1 += part[(long long)(p + 1) * n + e];
-        s2 += part[(long long)(p + 2) * n + e];
-        s3 += part[(long long)(p + 3) * n + e];
+    __shared__ float red[8][32];
+    const int el = threadIdx.x & 31, q = threadIdx.x >> 5;
+    const int e = blockIdx.x * 32 + el;
+    float s0 = 0.f, s1 = 0.f;
+    if (e < n) {
+        int p = q;
+        for (; p + 8 < nparts; p += 16) {
+            s0 += part[(long long)p * n + e];
+            s1 += part[(long long)(p + 8) * n + e];
+        }
+        if (p < nparts) s0 += part[(long long)p * n + e];
     }
-    for (; p < nparts; ++p) s0 += part[(long long)p * n + e];
-    dw[e] = from_f32<T>((s0 + s1) + (s2 + s3));
+    red[q][el] = s0 + s1;
+    __syncthreads();
+    if (q == 0 && e < n) {
+        const float s = ((red[0][el] + red[1][el]) + (red[2][el] + red[3][el])) +
+                        ((red[4][el] + red[5][el]) + (red[6][el] + red[7][el]));
+        dw[e] = from_f32<T>(s);
+    }
 }
 
 static ConvGeom make_geom(int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW, int DH,
@@ -207,7 +216,7 @@ size_t dwconv_wgrad_direct_workspace(int B, int H, int W, int C, int KH, int KW,
 
 template <typename T>
 int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s) {
-    hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, 256)), dim3(256), 0, s, part, (T*)dw, nparts, n);
+    hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, 32)), dim3(256), 0, s, part, (T*)dw, nparts, n);
     return check_launch("wgrad_reduce_parts");
 }
 template int wgrad_reduce_launch<float>(const float*, void*, int, int, hipStream_t);

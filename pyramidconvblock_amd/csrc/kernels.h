@@ -35,10 +35,16 @@ int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws,
 
 // resample.hip: adaptive average pool, bilinear resize, gate
 int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
-int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);
-int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s);
-int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s);
-int gate_fwd_launch(const void* x, void* y, long long M, int I, int dtype, hipStream_t s);
-int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int dtype, hipStream_t s);
+int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int accumulate, int dtype,
+                       hipStream_t s);
+int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int ldy, int dtype,
+                        hipStream_t s);
+int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int ldg, int dtype,
+                        hipStream_t s);
+int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s);
+int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int ldg, int dtype, hipStream_t s);
+size_t spatial_sum_workspace(int B, int P, int C);
+int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C, int dtype, hipStream_t s);
+int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, hipStream_t s);
 
 }  // namespace pdw

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void avgpool_fwd_k(const T* __restrict__ x, T*
 // Input row ih lies in bins i with floor(ih*h/H) <= i <= ceil((ih+1)*h/H) - 1.
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int H, int W,
-                                                     int C, int h, int w, long long total) {
+                                                     int C, int h, int w, int accumulate, long long total) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
@@ -74,7 +74,14 @@ __global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T
             for (int v = 0; v < VEC; ++v) acc[v] = fmaf(gv[v], inv, acc[v]);
         }
     }
-    store_f32<T, VEC>(gx + ((b * H + ih) * W + iw) * C + c, acc);
+    T* dst = gx + ((b * H + ih) * W + iw) * C + c;
+    if (accumulate) {  // gx += pooled gradient (fp32 add, one rounding)
+        float old[VEC];
+        load_f32<T, VEC>(dst, old);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] += old[v];
+    }
+    store_f32<T, VEC>(dst, acc);
 }
 
 // ---------------------------------------------------------------- bilinear, align_corners=False
@@ -92,7 +99,8 @@ __device__ __forceinline__ void bl_src(int dst, float scale, int in, int& i0, in
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
-                                                      int C, int H, int W, float sy, float sx, long long total) {
+                                                      int C, int H, int W, int ldy, float sy, float sx,
+                                                      long long total) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
@@ -115,7 +123,7 @@ __global__ __launch_bounds__(256) void bilinear_fwd_k(const T* __restrict__ x, T
     const float hy = 1.f - ly, hx = 1.f - lx;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = hy * (hx * a[v] + lx * bb[v]) + ly * (hx * cc[v] + lx * d[v]);
-    store_f32<T, VEC>(y + ((b * H + i) * W + j) * C + c, o);
+    store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
 }
 
 // Weight with which destination index `dst` reads source index m along one axis.
@@ -137,7 +145,8 @@ __device__ __forceinline__ void bl_dst_range(int m, float scale, int out, int& l
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w,
-                                                      int C, int H, int W, float sy, float sx, long long total) {
+                                                      int C, int H, int W, int ldg, float sy, float sx,
+                                                      long long total) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
     float acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
-    const T* gb = gy + b * H * W * C + c;
+    const T* gb = gy + b * H * W * ldg + c;
     for (int i = ilo; i <= ihi; ++i) {
         const float wy = bl_weight(i, sy, h, m);
         if (wy == 0.f) continue;
@@ -161,7 +170,7 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
             const float wx = bl_weight(j, sx, w, n);
             if (wx == 0.f) continue;
             float gv[VEC];
-            load_f32<T, VEC>(gb + ((long long)i * W + j) * C, gv);
+            load_f32<T, VEC>(gb + ((long long)i * W + j) * ldg, gv);
             const float ww = wy * wx;
 #pragma unroll
             for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, gv[v], acc[v]);
@@ -172,7 +181,7 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
 
 // ---------------------------------------------------------------- gate
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __restrict__ y, int I, float s,
+__global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
                                                   long long total) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
@@ -184,12 +193,12 @@ __global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __
     load_f32<T, VEC>(x + m * I + G + c, b);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = a[v] * b[v] * s;
-    store_f32<T, VEC>(y + m * G + c, o);
+    store_f32<T, VEC>(y + m * ldy + c, o);
 }
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const T* __restrict__ gy,
-                                                  T* __restrict__ gx, int I, float s, long long total) {
+                                                  T* __restrict__ gx, int I, int ldg, float s, long long total) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int G = I / 2, GV = G / VEC;
@@ -198,7 +207,7 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
     float a[VEC], b[VEC], g[VEC], ga[VEC], gb[VEC];
     load_f32<T, VEC>(x + m * I + c, a);
     load_f32<T, VEC>(x + m * I + G + c, b);
-    load_f32<T, VEC>(gy + m * G + c, g);
+    load_f32<T, VEC>(gy + m * ldg + c, g);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
         ga[v] = g[v] * b[v] * s;
@@ -206,6 +215,68 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
     }
     store_f32<T, VEC>(gx + m * I + c, ga);
     store_f32<T, VEC>(gx + m * I + G + c, gb);
+}
+
+
+// ---------------------------------------------------------------- per-image column sums and broadcast add
+// Pass 1 of the spatial sum: block (chunk, b) adds its share of the P positions of image b for all C
+// channels; threads are (channel vector, position lane); position lanes are combined through LDS.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void spatial_sum_part_k(const T* __restrict__ x, float* __restrict__ part, int P, int C,
+                                                          int chunk_len) {
+    extern __shared__ float red[];  // [PL][CV*VEC]
+    const int CV = C / VEC;
+    const int PL = 256 / CV;  // position lanes (host guarantees CV <= 256)
+    const int cv = threadIdx.x % CV, pl = threadIdx.x / CV;
+    const int b = blockIdx.y, ch = blockIdx.x;
+    const int p0 = ch * chunk_len, p1 = min(p0 + chunk_len, P);
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    if (pl < PL) {
+        const T* xb = x + ((long long)b * P) * C + cv * VEC;
+        for (int p = p0 + pl; p < p1; p += PL) {
+            float xv[VEC];
+            load_f32<T, VEC>(xb + (long long)p * C, xv);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] += xv[v];
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) red[pl * C + cv * VEC + v] = acc[v];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float s = 0.f;
+        for (int q = 0; q < PL; ++q) s += red[q * C + c];
+        part[((long long)b * gridDim.x + ch) * C + c] = s;
+    }
+}
+
+__global__ __launch_bounds__(256) void spatial_sum_final_k(const float* __restrict__ part, float* __restrict__ out,
+                                                           int nchunks, int C, int total) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int c = idx % C, b = idx / C;
+    float s = 0.f;
+    for (int q = 0; q < nchunks; ++q) s += part[((long long)b * nchunks + q) * C + c];
+    out[idx] = s;
+}
+
+// y[b,p,c] += v[b,c]  (v in fp32, one rounding)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void add_rowbias_k(T* __restrict__ y, const float* __restrict__ v, int P, int C,
+                                                     long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC;
+    const int c = (int)(idx % CV) * VEC;
+    const long long bp = idx / CV;
+    const int b = (int)(bp / P);
+    float a[VEC];
+    load_f32<T, VEC>(y + bp * C + c, a);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) a[i] += v[(long long)b * C + c + i];
+    store_f32<T, VEC>(y + bp * C + c, a);
 }
 
 // ---------------------------------------------------------------- launch plumbing
@@ -225,6 +296,13 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
     }
 
 static inline size_t esize(int dtype) { return dtype == kF32 ? 4 : 2; }
+static inline int gcd_int(int a, int b) {
+    while (b) {
+        const int t = a % b;
+        a = b, b = t;
+    }
+    return a;
+}
 
 static bool grid_for(long long total, unsigned* blocks) {
     const long long nb = (total + 255) / 256;
@@ -249,73 +327,121 @@ int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h
     return check_launch("avgpool_fwd");
 }
 
-int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s) {
+int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int h, int w, int accumulate, int dtype,
+                       hipStream_t s) {
     const void* ptrs[2] = {gy, gx};
     const int vec = pick_vec(C, esize(dtype), ptrs, 2);
     const long long total = (long long)B * H * W * (C / vec);
     unsigned blocks;
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
-#define CALL(T, V) hipLaunchKernelGGL((avgpool_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, H, W, C, h, w, total);
+#define CALL(T, V) hipLaunchKernelGGL((avgpool_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, H, W, C, h, w, accumulate, total);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("avgpool_bwd");
 }
 
-int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s) {
+int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int ldy, int dtype,
+                        hipStream_t s) {
     const void* ptrs[2] = {x, y};
-    const int vec = pick_vec(C, esize(dtype), ptrs, 2);
+    const int vec = pick_vec(gcd_int(C, ldy), esize(dtype), ptrs, 2);
     const long long total = (long long)B * H * W * (C / vec);
     unsigned blocks;
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
     const float sy = (float)h / (float)H, sx = (float)w / (float)W;
-#define CALL(T, V) hipLaunchKernelGGL((bilinear_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, h, w, C, H, W, sy, sx, total);
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, h, w, C, H, W, ldy, sy, sx, total);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("bilinear_fwd");
 }
 
-int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int dtype, hipStream_t s) {
+int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int ldg, int dtype,
+                        hipStream_t s) {
     const void* ptrs[2] = {gy, gx};
-    const int vec = pick_vec(C, esize(dtype), ptrs, 2);
+    const int vec = pick_vec(gcd_int(C, ldg), esize(dtype), ptrs, 2);
     const long long total = (long long)B * h * w * (C / vec);
     unsigned blocks;
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
     const float sy = (float)h / (float)H, sx = (float)w / (float)W;
-#define CALL(T, V) hipLaunchKernelGGL((bilinear_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, h, w, C, H, W, sy, sx, total);
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, h, w, C, H, W, ldg, sy, sx, total);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("bilinear_bwd");
 }
 
-int gate_fwd_launch(const void* x, void* y, long long M, int I, int dtype, hipStream_t s) {
+int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s) {
     const void* ptrs[2] = {x, y};
-    const int vec = pick_vec(I / 2, esize(dtype), ptrs, 2);
+    const int vec = pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 2);
     const long long total = M * (I / 2 / vec);
     unsigned blocks;
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
     const float sc = sqrtf((float)(I / 2));
-#define CALL(T, V) hipLaunchKernelGGL((gate_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, I, sc, total);
+#define CALL(T, V) hipLaunchKernelGGL((gate_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, I, ldy, sc, total);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("gate_fwd");
 }
 
-int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int dtype, hipStream_t s) {
+int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int ldg, int dtype, hipStream_t s) {
     const void* ptrs[3] = {x, gy, gx};
-    const int vec = pick_vec(I / 2, esize(dtype), ptrs, 3);
+    const int vec = pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 3);
     const long long total = M * (I / 2 / vec);
     unsigned blocks;
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
     const float sc = sqrtf((float)(I / 2));
-#define CALL(T, V) hipLaunchKernelGGL((gate_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (const T*)gy, (T*)gx, I, sc, total);
+#define CALL(T, V) hipLaunchKernelGGL((gate_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (const T*)gy, (T*)gx, I, ldg, sc, total);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("gate_bwd");
+}
+
+static void spatial_sum_plan(int B, int P, int* nchunks, int* chunk_len) {
+    int n = cdiv(1024, B > 0 ? B : 1);  // about four workgroups per CU over the batch
+    if (n > cdiv(P, 64)) n = cdiv(P, 64);
+    if (n < 1) n = 1;
+    *chunk_len = cdiv(P, n);
+    *nchunks = cdiv(P, *chunk_len);
+}
+
+size_t spatial_sum_workspace(int B, int P, int C) {
+    int n, len;
+    spatial_sum_plan(B, P, &n, &len);
+    return (size_t)B * n * C * sizeof(float);
+}
+
+int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C, int dtype, hipStream_t s) {
+    int n, len;
+    spatial_sum_plan(B, P, &n, &len);
+    const void* ptrs[1] = {x};
+    int vec = pick_vec(C, esize(dtype), ptrs, 1);
+    if (C / vec > 256) return set_error("pdw_spatial_sum: more than %d channels not supported", 256 * vec), 1;
+    const int pl = 256 / (C / vec);
+    const size_t lds = (size_t)pl * C * sizeof(float);
+    if (lds > 64 * 1024) return set_error("pdw_spatial_sum: channel count %d too large", C), 1;
+#define CALL(T, V) hipLaunchKernelGGL((spatial_sum_part_k<T, V>), dim3(n, B), dim3(256), lds, s, (const T*)x, ws, P, C, len);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    if (int e = check_launch("spatial_sum_part")) return e;
+    const int total = B * C;
+    hipLaunchKernelGGL(spatial_sum_final_k, dim3(cdiv(total, 256)), dim3(256), 0, s, ws, out, n, C, total);
+    return check_launch("spatial_sum_final");
+}
+
+int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, hipStream_t s) {
+    const void* ptrs[1] = {y};
+    const int vec = pick_vec(C, esize(dtype), ptrs, 1);
+    const long long total = (long long)B * P * (C / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+#define CALL(T, V) hipLaunchKernelGGL((add_rowbias_k<T, V>), dim3(blocks), dim3(256), 0, s, (T*)y, v, P, C, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("add_rowbias");
 }
 
 }  // namespace pdw

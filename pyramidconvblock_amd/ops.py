@@ -1,0 +1,129 @@
+"""Thin tensor-level wrappers over the C ABI of libpdw.so (one call = one or two kernel
+launches on torch's current stream).  Outputs may be channel slices of wider tensors: a
+destination whose last dimension is contiguous and whose pixels are a fixed stride apart is
+passed to the kernels as (pointer, leading dimension)."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _pixel_stride(t: torch.Tensor) -> int:
+    """Element stride between consecutive pixels of a [..., C] tensor whose leading dims are
+    laid out densely over a (possibly wider) channels-last buffer."""
+    if t.stride(-1) != 1 and t.shape[-1] != 1:
+        raise ValueError("last dimension must be contiguous")
+    ld = t.stride(-2)
+    exp = ld
+    for d in range(t.dim() - 2, -1, -1):
+        if t.shape[d] != 1 and t.stride(d) != exp:
+            raise ValueError("tensor is not a channel slice of a dense channels-last buffer")
+        exp *= t.shape[d]
+    return ld
+
+
+def _launch(name, dev, *args):
+    with _lib.on_device(dev):
+        _lib.check(getattr(_lib.lib(), name)(*args, _lib.stream_ptr(dev)), name)
+
+
+def avgpool_forward(x, out_hw):
+    dev = _lib.require_device(x)
+    B, H, W, C = x.shape
+    h, w = int(out_hw[0]), int(out_hw[1])
+    y = torch.empty((B, h, w, C), device=dev, dtype=x.dtype)
+    if x.numel() and y.numel():
+        _launch("pdw_avgpool_fwd", dev, x.data_ptr(), y.data_ptr(), B, H, W, C, h, w, _lib.dtype_code(x.dtype))
+    return y
+
+
+def avgpool_backward(gy, in_hw, out=None, accumulate=False):
+    """gx[B,H,W,C] = transpose of the pool applied to gy[B,h,w,C]; with `out` and accumulate the
+    result is added to `out` in place."""
+    dev = _lib.require_device(gy)
+    B, h, w, C = gy.shape
+    H, W = int(in_hw[0]), int(in_hw[1])
+    if out is None:
+        out = torch.empty((B, H, W, C), device=dev, dtype=gy.dtype)
+        accumulate = False
+    if gy.numel() and out.numel():
+        _launch("pdw_avgpool_bwd", dev, gy.data_ptr(), out.data_ptr(), B, H, W, C, h, w, 1 if accumulate else 0,
+                _lib.dtype_code(gy.dtype))
+    return out
+
+
+def bilinear_forward(x, out_hw, out=None):
+    dev = _lib.require_device(x)
+    B, h, w, C = x.shape
+    H, W = int(out_hw[0]), int(out_hw[1])
+    if out is None:
+        out = torch.empty((B, H, W, C), device=dev, dtype=x.dtype)
+    if x.numel() and out.numel():
+        _launch("pdw_bilinear_fwd", dev, x.data_ptr(), out.data_ptr(), B, h, w, C, H, W, _pixel_stride(out),
+                _lib.dtype_code(x.dtype))
+    return out
+
+
+def bilinear_backward(gy, in_hw):
+    """gy may be a channel slice of a wider [B,H,W,*] tensor."""
+    dev = _lib.require_device(gy)
+    B, H, W, C = gy.shape
+    h, w = int(in_hw[0]), int(in_hw[1])
+    gx = torch.empty((B, h, w, C), device=dev, dtype=gy.dtype)
+    if gy.numel() and gx.numel():
+        _launch("pdw_bilinear_bwd", dev, gy.data_ptr(), gx.data_ptr(), B, h, w, C, H, W, _pixel_stride(gy),
+                _lib.dtype_code(gy.dtype))
+    return gx
+
+
+def gate_forward(x, out=None):
+    dev = _lib.require_device(x)
+    I = x.shape[-1]
+    if I % 2:
+        raise ValueError("gate needs an even channel count")
+    if out is None:
+        out = torch.empty(x.shape[:-1] + (I // 2,), device=dev, dtype=x.dtype)
+    if out.numel():
+        _launch("pdw_gate_fwd", dev, x.data_ptr(), out.data_ptr(), x.numel() // I, I, _pixel_stride(out),
+                _lib.dtype_code(x.dtype))
+    return out
+
+
+def gate_backward(x, gy):
+    """gy may be a channel slice of a wider tensor."""
+    dev = _lib.require_device(x, gy)
+    I = x.shape[-1]
+    gx = torch.empty_like(x)
+    if gx.numel():
+        _launch("pdw_gate_bwd", dev, x.data_ptr(), gy.data_ptr(), gx.data_ptr(), x.numel() // I, I, _pixel_stride(gy),
+                _lib.dtype_code(x.dtype))
+    return gx
+
+
+def spatial_sum(x):
+    """x [B, ..., C] -> fp32 [B, C]: sum over all middle dimensions."""
+    dev = _lib.require_device(x)
+    B, C = x.shape[0], x.shape[-1]
+    P = x.numel() // max(B * C, 1)
+    out = torch.empty((B, C), device=dev, dtype=torch.float32)
+    if B == 0:
+        return out
+    if P == 0:
+        return out.zero_()
+    nbytes = _lib.lib().pdw_spatial_sum_workspace_bytes(B, P, C)
+    ws = torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
+    _launch("pdw_spatial_sum", dev, x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, P, C,
+            _lib.dtype_code(x.dtype))
+    return out
+
+
+def add_rowbias_(y, v):
+    """In place y[b, ..., c] += v[b, c] with v fp32 [B, C]."""
+    dev = _lib.require_device(y, v)
+    B, C = y.shape[0], y.shape[-1]
+    P = y.numel() // max(B * C, 1)
+    assert v.dtype == torch.float32 and v.is_contiguous() and tuple(v.shape) == (B, C)
+    if y.numel():
+        _launch("pdw_add_rowbias", dev, y.data_ptr(), v.data_ptr(), B, P, C, _lib.dtype_code(y.dtype))
+    return y

@@ -8,29 +8,7 @@ from __future__ import annotations
 
 import torch
 
-from . import _lib
-
-
-def _call(fn_name, src, dst, B, h, w, C, H, W):
-    dev = _lib.require_device(src, dst)
-    if src.numel() and dst.numel():
-        with _lib.on_device(dev):
-            fn = getattr(_lib.lib(), fn_name)
-            _lib.check(fn(src.data_ptr(), dst.data_ptr(), B, h, w, C, H, W, _lib.dtype_code(src.dtype),
-                          _lib.stream_ptr(dev)), fn_name)
-    return dst
-
-
-def bilinear_forward(x, out_hw):
-    B, h, w, C = x.shape
-    H, W = int(out_hw[0]), int(out_hw[1])
-    return _call("pdw_bilinear_fwd", x, torch.empty((B, H, W, C), device=x.device, dtype=x.dtype), B, h, w, C, H, W)
-
-
-def bilinear_backward(gy, in_hw):
-    B, H, W, C = gy.shape
-    h, w = int(in_hw[0]), int(in_hw[1])
-    return _call("pdw_bilinear_bwd", gy, torch.empty((B, h, w, C), device=gy.device, dtype=gy.dtype), B, h, w, C, H, W)
+from .ops import bilinear_backward, bilinear_forward  # noqa: F401  (re-exported)
 
 
 class BilinearInterp2dFunction(torch.autograd.Function):

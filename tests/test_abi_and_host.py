@@ -37,7 +37,7 @@ def test_argument_validation_without_gpu():
     assert b"dtype" in L.pdw_last_error()
     assert L.pdw_dwconv_fwd(None, None, None, 1, 4, 4, 8, 3, 3, 0, 1, 1, 1, 1, 1, 0, None) != 0
     assert b"stride" in L.pdw_last_error()
-    assert L.pdw_gate_fwd(None, None, 4, 7, 0, None) != 0
+    assert L.pdw_gate_fwd(None, None, 4, 7, 0, 0, None) != 0
     assert L.pdw_dwconv_wgrad_workspace_bytes(2, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 0) > 0
     assert L.pdw_dwconv_wgrad(1, 1, 1, None, 0, 2, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 0, None) != 0
     assert b"workspace" in L.pdw_last_error()

@@ -77,3 +77,51 @@ def test_modules_and_empty():
     assert tuple(P.OptimizedBilinearInterp2d(12)(x).shape) == (2, 12, 12, 16)
     e = torch.zeros(0, 8, 8, 16, device="cuda")
     assert tuple(P.OptimizedAdaptiveAvgPool2d((3, 2))(e).shape) == (0, 3, 2, 16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_strided_outputs_and_accumulate(oracle, dtype):
+    """Gate / bilinear results written into (and gradients read from) a channel slice of a wider
+    buffer, and the pool gradient accumulated in place: the pieces the fused block uses."""
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(7)
+    B, H, W, I = 2, 10, 12, 24
+    G = I // 2
+    x = randn(gen, B, H, W, I).to(dtype)
+    wide = torch.full((B, H, W, 3 * G), 7.0, dtype=dtype, device="cuda")
+    ops.gate_forward(x.cuda(), out=wide[..., G:2 * G])
+    assert_close(wide[..., G:2 * G], oracle.gate_fwd(x.double().numpy()), dtype, "gate into slice")
+    assert torch.all(wide[..., :G] == 7) and torch.all(wide[..., 2 * G:] == 7)
+    small = randn(gen, B, 5, 6, G).to(dtype)
+    ops.bilinear_forward(small.cuda(), (H, W), out=wide[..., 2 * G:])
+    assert_close(wide[..., 2 * G:], oracle.bilinear_fwd(small.double().numpy(), (H, W)), dtype, "bilinear into slice")
+    assert torch.all(wide[..., :G] == 7)
+    gwide = randn(gen, B, H, W, 3 * G).to(dtype)
+    gd = gwide.cuda()
+    assert_close(ops.gate_backward(x.cuda(), gd[..., G:2 * G]),
+                 oracle.gate_bwd(x.double().numpy(), gwide[..., G:2 * G].double().numpy()), dtype, "gate bwd from slice")
+    assert_close(ops.bilinear_backward(gd[..., 2 * G:], (5, 6)),
+                 oracle.bilinear_bwd(gwide[..., 2 * G:].double().numpy(), (5, 6)), dtype, "bilinear bwd from slice")
+    base = randn(gen, B, H, W, G).to(dtype)
+    gp = randn(gen, B, 5, 6, G).to(dtype)
+    acc = base.cuda().clone()
+    ops.avgpool_backward(gp.cuda(), (H, W), out=acc, accumulate=True)
+    assert_close(acc, base.double().numpy() + oracle.avgpool_bwd(gp.double().numpy(), (H, W)), dtype, "pool bwd accumulate")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(3, 7, 9, 20), (32, 56, 56, 128), (2, 57, 61, 200), (1, 1, 1, 4), (5, 33, 2, 3)])
+def test_spatial_sum_and_rowbias(dtype, shape):
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(11)
+    x = randn(gen, *shape).to(dtype)
+    s = ops.spatial_sum(x.cuda())
+    ref = x.double().sum(dim=(1, 2)).numpy()
+    assert s.dtype == torch.float32
+    assert_close(s, ref, torch.float32, "spatial sum", scale=4.0)  # fp32 accumulation of up to 3136 terms
+    v = randn(gen, shape[0], shape[3])
+    y = x.cuda().clone()
+    ops.add_rowbias_(y, v.cuda())
+    assert_close(y, x.double().numpy() + v.double().numpy()[:, None, None, :], dtype, "rowbias")
