@@ -37,8 +37,14 @@ struct TiledGeom {
     int CPn;          // LDS column units per staged row
     int rows_in;      // staged rows = Q*NRG + KH - 1
     int flip;         // 1: use the 180-degree rotated filter (input gradient)
-    int ulog;         // log2 of the staging threads laid along a row of LDS units
+    int ntiles;       // tiles per channel slice = batch * tiles_h * tiles_w
+    int nchunks;      // workgroups per channel slice; workgroup q walks tiles q, q+nchunks, ...
+    int step_r, step_u;  // (row, unit) advance of a thread's staging item per pass of 256 threads
 };
+
+// Staging passes whose global loads are issued one tile ahead and held in registers while the
+// current tile is computed (software pipelining across the persistent tile loop).
+constexpr int kPrefetchPasses = 8;
 
 template <typename T, int KW, int R, int Q, int CS, int V>
 __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, const T* __restrict__ w,
@@ -48,22 +54,20 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
     constexpr int RU = R / PK;              // output units per patch row
     constexpr int XU = RU + NP - 1;         // staged units read per patch row
     constexpr int NG = 64 / CS;
+    constexpr int CV = CS / V;              // channel vectors per LDS unit
+    constexpr int UPP = 256 / CV;           // LDS units staged per pass of the workgroup
+    constexpr int NL = PK;                  // pixels loaded per LDS unit
+    constexpr int MAXIT = kPrefetchPasses;
     static_assert(R % 2 == 0 && 64 % CS == 0 && CS % V == 0, "bad tile parameters");
     extern __shared__ uint32_t smem[];
     uint32_t* xl = smem;                                  // [rows_in][CPn][CS]
     uint32_t* wl = smem + g.rows_in * g.CPn * CS;         // [KH][NP][CS]
 
-    int item = xcd_remap(blockIdx.x, gridDim.x);
-    const int tw = item % g.tiles_w;
-    item /= g.tiles_w;
-    const int th = item % g.tiles_h;
-    item /= g.tiles_h;
-    const int sl = item % g.slices;
-    const int b = item / g.slices;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int sl = bid % g.slices, chunk = bid / g.slices;
     const int c0 = sl * CS;
-    const int orow0 = th * (Q * g.NRG), ocol0 = tw * (R * g.NST);
-    const int irow0 = orow0 - g.PH, icol0 = ocol0 - g.PW;
     const int tid = threadIdx.x;
+    const int tiles_per_img = g.tiles_h * g.tiles_w;
 
     // ---- stage the filter slice: wl[kh][m][c] = unit m of (rotated) filter row kh.
     // Thread (c, mt) walks the filter rows; SU rows are loaded (clamped, always valid addresses)
@@ -109,17 +113,106 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
         }
     }
 
-    // ---- stage the input tile with its halo (zeros outside the image / channel range)
-    stage_tile<T, CS, V>(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, irow0, icol0, g.rows_in, g.CPn,
-                         g.ulog, c0, tid);
-    __syncthreads();
+    // ---- staging map of this thread (the same for every tile): channel vector cv of LDS unit
+    // (r, u) in pass 0, advancing by (step_r, step_u) units per pass.
+    const int scv = tid % CV;
+    const int sr0 = (tid / CV) / g.CPn, su0 = (tid / CV) % g.CPn;
+    const int sch = c0 + scv * V;
+    const bool schok = sch < g.C;
+    const int schc = schok ? sch : 0;
+    const int nunits = g.rows_in * g.CPn;
+    ChanVec<T, V> pre[MAXIT][NL];
 
-    // ---- compute: each (wave, lane group) slot walks the tile's patches
+    // Issues the global loads of a tile's first MAXIT staging passes (clamped, always valid addresses).
+    auto prefetch = [&](int tile) {
+        const int b = tile / tiles_per_img, rem = tile % tiles_per_img;
+        const int irow0 = (rem / g.tiles_w) * (Q * g.NRG) - g.PH, icol0 = (rem % g.tiles_w) * (R * g.NST) - g.PW;
+        const T* xb = x + (long long)b * g.H * g.W * g.C + schc;
+        int r = sr0, u = su0;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {
+            const int ih = min(max(irow0 + min(r, g.rows_in - 1), 0), g.H - 1);
+#pragma unroll
+            for (int l = 0; l < NL; ++l) {
+                const int iw = min(max(icol0 + NL * u + l, 0), g.W - 1);
+                pre[it][l] = *reinterpret_cast<const ChanVec<T, V>*>(xb + (ih * g.W + iw) * g.C);
+            }
+            r += g.step_r, u += g.step_u;
+            if (u >= g.CPn) u -= g.CPn, ++r;
+        }
+    };
+
+    // Packs one staged unit (zeros outside the image / channel range) and writes it to LDS.
+    auto put = [&](const ChanVec<T, V>* ld, int r, int u, int irow0, int icol0) {
+        const int ih = irow0 + r;
+        const bool rok = schok && ih >= 0 && ih < g.H;
+        const int iw0 = icol0 + NL * u;
+        const bool ok0 = rok && iw0 >= 0 && iw0 < g.W;
+        const bool ok1 = rok && iw0 + 1 >= 0 && iw0 + 1 < g.W;
+        uint32_t out[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            if constexpr (PK == 2)
+                out[i] = (ok0 ? bits16(ld[0].v[i]) : 0u) | ((ok1 ? bits16(ld[NL - 1].v[i]) : 0u) << 16);
+            else
+                out[i] = ok0 ? __builtin_bit_cast(uint32_t, ld[0].v[i]) : 0u;
+        }
+        uint32_t* dst = xl + (r * g.CPn + u) * CS + scv * V;
+        if constexpr (V % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < V; i += 4)
+                *reinterpret_cast<uint4*>(dst + i) = make_uint4(out[i], out[i + 1], out[i + 2], out[i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) dst[i] = out[i];
+        }
+    };
+
+    // Writes the prefetched passes to LDS and stages any remaining passes directly.
+    auto commit = [&](int tile) {
+        const int b = tile / tiles_per_img, rem = tile % tiles_per_img;
+        const int irow0 = (rem / g.tiles_w) * (Q * g.NRG) - g.PH, icol0 = (rem % g.tiles_w) * (R * g.NST) - g.PW;
+        int r = sr0, u = su0;
+#pragma unroll
+        for (int it = 0; it < MAXIT; ++it) {
+            if (r < g.rows_in) put(pre[it], r, u, irow0, icol0);
+            r += g.step_r, u += g.step_u;
+            if (u >= g.CPn) u -= g.CPn, ++r;
+        }
+        if (MAXIT * UPP < nunits) {  // tiles larger than the prefetch window (uniform branch)
+            const T* xb = x + (long long)b * g.H * g.W * g.C + schc;
+            for (; r < g.rows_in;) {
+                ChanVec<T, V> ld[NL];
+                const int ih = min(max(irow0 + r, 0), g.H - 1);
+#pragma unroll
+                for (int l = 0; l < NL; ++l) {
+                    const int iw = min(max(icol0 + NL * u + l, 0), g.W - 1);
+                    ld[l] = *reinterpret_cast<const ChanVec<T, V>*>(xb + (ih * g.W + iw) * g.C);
+                }
+                put(ld, r, u, irow0, icol0);
+                r += g.step_r, u += g.step_u;
+                if (u >= g.CPn) u -= g.CPn, ++r;
+            }
+        }
+    };
+
     const int lane = tid & 63, wv = tid >> 6;
     const int c = lane % CS, grp = lane / CS;
     const int slot = wv * NG + grp;
     const int npatch = g.NRG * g.NST;
     const int rowstride = g.CPn * CS;
+
+    int tile = chunk;
+    if (tile < g.ntiles) prefetch(tile);
+    for (; tile < g.ntiles; tile += g.nchunks) {
+    __syncthreads();  // the previous tile is fully consumed (and, first time, the filter is staged)
+    commit(tile);
+    __syncthreads();
+    if (tile + g.nchunks < g.ntiles) prefetch(tile + g.nchunks);  // in flight during the compute below
+    const int b = tile / tiles_per_img, rem = tile % tiles_per_img;
+    const int orow0 = (rem / g.tiles_w) * (Q * g.NRG), ocol0 = (rem % g.tiles_w) * (R * g.NST);
+
+    // ---- compute: each (wave, lane group) slot walks the tile's patches
     for (int p0 = 0; p0 < npatch; p0 += 4 * NG) {
         const bool valid = p0 + slot < npatch;
         const int p = valid ? p0 + slot : npatch - 1;
@@ -131,6 +224,50 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
             for (int r = 0; r < R; ++r) acc[q][r] = 0.f;
         const uint32_t* xbase = xl + (rg * Q) * rowstride + (st * RU) * CS + c;
         const uint32_t* wbase = wl + c;
+        if (g.KH == KW) {
+            // Square filter: walk the KW+Q-1 staged rows once, fully unrolled.  Row j feeds output row q
+            // through filter row j-q, so every LDS row segment is read once per patch and the
+            // scheduler is free to issue a row's reads while the previous row's dot products run.
+            uint32_t wa[KW][NP], wb[KW][NP];
+#pragma unroll
+            for (int j = 0; j < KW + Q - 1; ++j) {
+                if (j < KW) {
+#pragma unroll
+                    for (int m = 0; m < NP; ++m) wa[j][m] = wbase[(j * NP + m) * CS];
+                    if constexpr (PK == 2) {
+                        wb[j][0] = wa[j][0] << 16;
+#pragma unroll
+                        for (int m = 1; m < NP; ++m) wb[j][m] = __builtin_amdgcn_alignbit(wa[j][m], wa[j][m - 1], 16);
+                    }
+                }
+                const uint32_t* xr = xbase + j * rowstride;
+                uint32_t xp[XU];
+#pragma unroll
+                for (int i = 0; i < XU; ++i) xp[i] = xr[i * CS];
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    const int kh = j - q;
+                    if (kh >= 0 && kh < KW) {
+                        if constexpr (PK == 2) {
+#pragma unroll
+                            for (int t = 0; t < RU; ++t)
+#pragma unroll
+                                for (int m = 0; m < NP; ++m) {
+                                    acc[q][2 * t] = dot2acc(xp[t + m], wa[kh][m], acc[q][2 * t], T());
+                                    acc[q][2 * t + 1] = dot2acc(xp[t + m], wb[kh][m], acc[q][2 * t + 1], T());
+                                }
+                        } else {
+#pragma unroll
+                            for (int t = 0; t < R; ++t)
+#pragma unroll
+                                for (int m = 0; m < NP; ++m)
+                                    acc[q][t] = fmaf(__builtin_bit_cast(float, xp[t + m]),
+                                                     __builtin_bit_cast(float, wa[kh][m]), acc[q][t]);
+                        }
+                    }
+                }
+            }
+        } else {
 #pragma unroll 1
         for (int kh = 0; kh < g.KH; ++kh) {
             uint32_t wa[NP];
@@ -170,6 +307,7 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
                 }
             }
         }
+        }  // filter-shape branch
         // ---- store (one rounding to T)
         const int ch = c0 + c;
         if (valid && ch < g.C) {
@@ -189,6 +327,7 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
             }
         }
     }
+    }  // tile loop
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -241,17 +380,37 @@ static int launch_tiled(const TiledPlan& plan, const void* x, const void* w, voi
     g.tiles_h = cdiv(g.OH, Q * g.NRG), g.tiles_w = cdiv(g.OW, R * g.NST);
     g.rows_in = Q * g.NRG + KH - 1;
     g.CPn = (R * g.NST + KW - 1 + PK - 1) / PK;
-    g.ulog = 0;
     const size_t lds = ((size_t)g.rows_in * g.CPn + (size_t)KH * NP) * CS * 4;
-    const long long nblocks = (long long)g.tiles_h * g.tiles_w * g.slices * B;
-    if (nblocks > 0x7fffffffLL || (long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL)
+    const long long ntiles = (long long)g.tiles_h * g.tiles_w * B;
+    if (ntiles > 0x7fffffffLL || (long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL)
         return -1;
+    g.ntiles = (int)ntiles;
+    // Persistent workgroups: as many as fit on the chip at once (LDS-limited, at most 3 per CU), then
+    // trimmed so the tiles divide as evenly as possible among them.
+    int occ = (int)((160 * 1024) / (lds + 512));
+    const int occ_max = getenv("PDW_OCC") ? atoi(getenv("PDW_OCC")) : 3;
+    occ = occ < 1 ? 1 : (occ > occ_max ? occ_max : occ);
+    const int target = (256 * occ) / g.slices > 1 ? (256 * occ) / g.slices : 1;
+    int nch = (int)(ntiles < target ? ntiles : target);
+    {
+        double beste = -1;
+        for (int cand = (target + 1) / 2; cand <= target && cand <= ntiles; ++cand) {
+            const double rounds = (double)cdiv(ntiles, cand);
+            const long long blocks = (long long)cand * g.slices;
+            const double eff = ntiles / (rounds * cand) * blocks / (double)(cdiv(blocks, 256) * 256);
+            if (eff >= beste) beste = eff, nch = cand;
+        }
+    }
+    if (getenv("PDW_NCH")) nch = atoi(getenv("PDW_NCH"));
+    g.nchunks = nch < 1 ? 1 : nch;
+    const long long nblocks = (long long)g.nchunks * g.slices;
     const void* ptrs[1] = {x};
     const int vec = pick_vec(C, sizeof(T), ptrs, 1);
 #define PDW_GO(V)                                                                                            \
     {                                                                                                        \
         auto kern = dwconv_tiled_k<T, KW, R, Q, CS, V>;                                                      \
-        g.ulog = stage_ulog(g.CPn, CS, V);                                                                   \
+        const int upp = 256 / (CS / V);                                                                      \
+        g.step_r = upp / g.CPn, g.step_u = upp % g.CPn;                                                      \
         static bool attr_done = false;                                                                       \
         if (!attr_done) {                                                                                    \
             (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
@@ -282,7 +441,7 @@ static int launch_best(const void* x, const void* w, void* y, int B, int H, int 
     for (int i = 0; i < 3; ++i)
         if (ps[i]->cost >= 0 && (best < 0 || ps[i]->cost < best)) best = ps[i]->cost, pick = i;
     const char* force = getenv("PDW_PATCH");
-    if (force) pick = atoi(force);
+    if (force && atoi(force) >= 0 && atoi(force) < 3) pick = atoi(force);
     TiledPlan p = pick >= 0 ? *ps[pick] : p0;
     if (pick < 0 || p.cost < 0) return -1;
     if (getenv("PDW_NRG") && getenv("PDW_NST")) p.nrg = atoi(getenv("PDW_NRG")), p.nst = atoi(getenv("PDW_NST"));
