@@ -130,7 +130,8 @@ def kernel_rooflines(B, H, W, D, k, dtype):
 
 def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     """Launches one hot kernel `iters` times at its shape inside the headline block (for rocprofv3 runs).
-    name: {fwd,dgrad,wgrad}_{full,half} | avgpool_fwd | avgpool_bwd | bilinear_fwd | bilinear_bwd"""
+    name: {fwd,dgrad,wgrad}_{full,half} | avgpool_fwd | avgpool_bwd | bilinear_fwd | bilinear_bwd |
+    dense_{fwd,dgrad,wgrad} (the conv_up layer: [N,D] <-> [N,D/2])"""
     from pyramidconvblock_amd import avgpool, dwconv, up
 
     I, G = D // 2, D // 4
@@ -145,6 +146,16 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         fn = {"fwd": lambda: dwconv.dwconv_forward(x, wt, *geo),
               "dgrad": lambda: dwconv.dwconv_dgrad(g, wt, x.shape, *geo),
               "wgrad": lambda: dwconv.dwconv_wgrad(x, g, wt.shape, *geo)}[op]
+    elif op == "dense":
+        from pyramidconvblock_amd import ops
+
+        xin = torch.randn(B, H, W, D, device="cuda").to(dtype)
+        ain = torch.randn(B, H, W, I, device="cuda").to(dtype)
+        wup = (torch.randn(I, D, device="cuda") / D ** 0.5).to(dtype)
+        rb = torch.randn(B, D, device="cuda")
+        fn = {"fwd": lambda: ops.dense_forward(xin, wup),
+              "dgrad": lambda: ops.dense_forward(ain, wup, w_kmajor=True, rowbias=rb, rows_per_image=H * W),
+              "wgrad": lambda: ops.dense_wgrad(ain, xin)}[res]
     else:
         a = torch.randn(B, H, W, I, device="cuda").to(dtype)
         p = torch.randn(B, h, w, I, device="cuda").to(dtype)
@@ -197,7 +208,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep and forward-only timings")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel event timings")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
-                    "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}")
+                    "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, dense_{fwd,dgrad,wgrad}")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:

@@ -107,6 +107,38 @@ int pdw_spatial_sum(const void *x, float *out, void *workspace, size_t workspace
  * and its mirror in the backward (the gradient of the mean, conv_block.py:46). */
 int pdw_add_rowbias(void *y, const float *v, int B, int P, int C, int dtype, void *stream);
 
+/* Pooled branch of the block, forward (conv_block.py:46-47 plus the bias of :44): per image b,
+ *   m[b,:]       = mean over the P positions of x[b,:,:]            (rounded to the element type, kept for backward)
+ *   rowbias[b,o] = sum_c m[b,c] * w_pool[o,c] + b_pool[o] + b_out[o] (fp32; b_pool / b_out may be NULL)
+ * rowbias is what pdw_dense_fwd / pdw_add_rowbias then broadcast over the positions (conv_block.py:49). */
+size_t pdw_pool_branch_workspace_bytes(int B, int P, int D);
+int pdw_pool_branch_fwd(const void *x, const void *w_pool, const void *b_pool, const void *b_out, void *m,
+                        float *rowbias, void *workspace, size_t workspace_bytes, int B, int P, int D, int dtype,
+                        void *stream);
+/* Its backward from gy[B,P,D]: gbias[o] = sum over all positions of gy (the gradient of both biases),
+ * gw_pool[o,c] = sum_b gs[b,o] * m[b,c] with gs the per-image column sums of gy, and
+ * dmean[b,c] = (1/P) * sum_o gs[b,o] * w_pool[o,c] (fp32), the per-image term that the mean's gradient
+ * adds to every position of dx. */
+int pdw_pool_branch_bwd(const void *gy, const void *m, const void *w_pool, void *gbias, void *gw_pool, float *dmean,
+                        void *workspace, size_t workspace_bytes, int B, int P, int D, int dtype, void *stream);
+
+/* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 4 == 0;
+ * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).
+ *   y[n,o] = sum_k x[n,k] * W(o,k) + bias[o] + rowbias[n / P][o]        x[N,K] -> y[N,NO]
+ * W(o,k) = w[o*K + k] (w_kmajor == 0, the nn.Linear layout) or w[k*NO + o] (w_kmajor != 0, which gives the
+ * input gradient of a layer from its own weight without a transpose).  bias (element type) and rowbias
+ * (fp32 [ceil(N/P), NO]) may be NULL.  Replaces nn.Linear at conv_block.py:37 and :44 together with the
+ * broadcast add of conv_block.py:49, and the matching input-gradient GEMMs of the backward. */
+int pdw_dense_supported(int K, int NO, int dtype);
+int pdw_dense_fwd(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
+                  long long N, int K, int NO, int P, int dtype, void *stream);
+
+/* Weight gradient of such a layer: dw[m,o] = sum_n a[n,m] * b[n,o]  (a[N,M], b[N,NO] -> dw[M,NO]), fp32
+ * accumulation, two deterministic passes through `workspace` (no atomics). */
+size_t pdw_dense_wgrad_workspace_bytes(long long N, int M, int NO);
+int pdw_dense_wgrad(const void *a, const void *b, void *dw, void *workspace, size_t workspace_bytes, long long N,
+                    int M, int NO, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -37,6 +37,14 @@ _SIGS = {
     "pdw_spatial_sum_workspace_bytes": (c_size_t, [c_int] * 3),
     "pdw_spatial_sum": (c_int, [c_void_p] * 3 + [c_size_t] + [c_int] * 4 + [c_void_p]),
     "pdw_add_rowbias": (c_int, [c_void_p] * 2 + [c_int] * 4 + [c_void_p]),
+    "pdw_pool_branch_workspace_bytes": (c_size_t, [c_int] * 3),
+    "pdw_pool_branch_fwd": (c_int, [c_void_p] * 7 + [c_size_t] + [c_int] * 4 + [c_void_p]),
+    "pdw_pool_branch_bwd": (c_int, [c_void_p] * 7 + [c_size_t] + [c_int] * 4 + [c_void_p]),
+    "pdw_dense_supported": (c_int, [c_int] * 3),
+    "pdw_dense_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong] + [c_int] * 4
+                      + [c_void_p]),
+    "pdw_dense_wgrad_workspace_bytes": (c_size_t, [c_longlong, c_int, c_int]),
+    "pdw_dense_wgrad": (c_int, [c_void_p] * 4 + [c_size_t, c_longlong, c_int, c_int, c_int, c_void_p]),
 }
 EXPORTS = tuple(_SIGS)
 

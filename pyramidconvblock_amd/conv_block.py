@@ -9,9 +9,10 @@ names, parameter shapes and ``[B,H,W,C]`` in/out contract
 convolutions, gates and upsampling go through libpdw.so, the gate outputs are written straight
 into the halves of the concatenated buffer (no ``torch.cat``), the pooled branch is added in
 place, and the backward reuses one per-image column sum for both bias gradients and the
-gradient of the mean.  The three dense layers stay library GEMMs (hipBLASLt through torch);
-their weight gradients, whose reduction dimension is B*H*W, are computed as a batched
-split-K product because the library's single GEMM for that shape is ~10x slower.
+gradient of the mean.  For 16-bit types and widths up to 128 the dense layers run on the
+matrix-core kernels of libpdw.so (bias / broadcast add fused into the store, deterministic
+split reduction for the weight gradients); other shapes use library GEMMs, with the weight
+gradients as a batched split-K product.
 """
 from __future__ import annotations
 
@@ -93,8 +94,10 @@ class ConvBlockFunction(torch.autograd.Function):
         x = x.detach().contiguous()
         B, H, W, D = x.shape
         dt = x.dtype
-        a = F.linear(x, w_up, b_up)
-        I = a.shape[-1]
+        I = w_up.shape[0]
+        fast_up = (ops.dense_supported(D, I, dt) and ops.dense_supported(I, D, dt) and w_up.dtype == dt
+                   and (b_up is None or b_up.dtype == dt))
+        a = ops.dense_forward(x, w_up.detach().contiguous(), bias=b_up) if fast_up else F.linear(x, w_up, b_up)
         G = I // 2
         ns = len(scales)
         cat = torch.empty((B, H, W, G * ns), device=dev, dtype=dt)
@@ -114,12 +117,22 @@ class ConvBlockFunction(torch.autograd.Function):
                 ops.gate_forward(c, out=dst)
             convs.append(c)
             pooled.append(p)
-        y = F.linear(cat, w_out)
-        m = (ops.spatial_sum(x) / float(H * W)).to(dt)          # x.mean(dim=(1,2))
-        yp = F.linear(m, w_pool, b_pool).float()
-        if b_out is not None:
-            yp = yp + b_out.float()
-        ops.add_rowbias_(y, yp.contiguous())                     # conv_out bias + broadcast pooled branch
+        same_dt = w_pool.dtype == dt and all(b is None or b.dtype == dt for b in (b_pool, b_out))
+        if same_dt and B > 0:
+            # mean over positions -> conv_pool, plus conv_out's bias: one fp32 row per image
+            m, yp = ops.pool_branch_forward(x, w_pool.detach().contiguous(), b_pool, b_out)
+        else:
+            m = (ops.spatial_sum(x) / float(H * W)).to(dt)
+            yp = F.linear(m, w_pool, b_pool).float()
+            if b_out is not None:
+                yp = yp + b_out.float()
+            yp = yp.contiguous()
+        fast_out = ops.dense_supported(G * ns, D, dt) and ops.dense_supported(D, G * ns, dt) and w_out.dtype == dt
+        if fast_out:
+            y = ops.dense_forward(cat, w_out.detach().contiguous(), rowbias=yp, rows_per_image=H * W)
+        else:
+            y = ops.add_rowbias_(F.linear(cat, w_out), yp)
+        ctx.fast = (fast_up, fast_out)
         ctx.scales = tuple(scales)
         ctx.has_bias = (b_up is not None, b_out is not None, b_pool is not None)
         ctx.save_for_backward(x, a, cat, m, w_up, w_out, w_pool, *w_dw, *convs, *[p for p in pooled if p is not None])
@@ -143,15 +156,23 @@ class ConvBlockFunction(torch.autograd.Function):
         gy = gy.to(dt).contiguous()
         g2d = gy.view(N, D)
 
-        gs = ops.spatial_sum(gy)                                 # [B, D] fp32: column sums per image
-        gbias = gs.sum(0)
+        if w_pool.dtype == dt and B > 0:
+            gbias, grad_w_pool, dmean = ops.pool_branch_backward(gy, m, w_pool.detach().contiguous())
+        else:
+            gs = ops.spatial_sum(gy)                             # [B, D] fp32: column sums per image
+            gbias = gs.sum(0)
+            grad_w_pool = (gs.t() @ m.float()).to(w_pool.dtype)
+            dmean = ((gs @ w_pool.float()) / float(H * W)).contiguous()   # gradient of the per-image mean
         grad_b_out = gbias.to(w_out.dtype) if ctx.has_bias[1] else None
         grad_b_pool = gbias.to(w_pool.dtype) if ctx.has_bias[2] else None
-        grad_w_pool = (gs.t() @ m.float()).to(w_pool.dtype)
-        dm = gs @ w_pool.float()                                 # gradient of the per-image mean
 
-        dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
-        grad_w_out = _weight_grad(g2d, cat.view(N, G * ns)).to(w_out.dtype)
+        fast_up, fast_out = ctx.fast
+        if fast_out:
+            dcat = ops.dense_forward(gy, w_out.detach().contiguous(), w_kmajor=True)
+            grad_w_out = ops.dense_wgrad(gy, cat).to(w_out.dtype)
+        else:
+            dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
+            grad_w_out = _weight_grad(g2d, cat.view(N, G * ns)).to(w_out.dtype)
 
         da = None
         grad_w_dw = [None] * ns
@@ -179,12 +200,17 @@ class ConvBlockFunction(torch.autograd.Function):
             else:
                 da = dp if da is None else da.add_(dp)
         a2d = da.view(N, I)
-        grad_w_up = _weight_grad(a2d, x.view(N, D)).to(w_up.dtype)
         grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
         dx = None
-        if ctx.needs_input_grad[0]:
-            dx = torch.matmul(a2d, w_up).view(B, H, W, D)
-            ops.add_rowbias_(dx, (dm / float(H * W)).contiguous())
+        if fast_up:
+            grad_w_up = ops.dense_wgrad(da, x).to(w_up.dtype)
+            if ctx.needs_input_grad[0]:
+                dx = ops.dense_forward(da, w_up.detach().contiguous(), w_kmajor=True, rowbias=dmean,
+                                       rows_per_image=H * W)
+        else:
+            grad_w_up = _weight_grad(a2d, x.view(N, D)).to(w_up.dtype)
+            if ctx.needs_input_grad[0]:
+                dx = ops.add_rowbias_(torch.matmul(a2d, w_up).view(B, H, W, D), dmean)
         return (dx, None, grad_w_up, grad_b_up, grad_w_out, grad_b_out, grad_w_pool, grad_b_pool, *grad_w_dw)
 
 

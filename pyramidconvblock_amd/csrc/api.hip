@@ -47,6 +47,8 @@ static int check_resample(const char* fn, const void* a, const void* b, int B, i
     if (B < 0 || H < 1 || W < 1 || C < 1 || h < 1 || w < 1)
         return set_error("%s: bad extents B=%d H=%d W=%d C=%d h=%d w=%d", fn, B, H, W, C, h, w), 1;
     if (B > 0 && (!a || !b)) return set_error("%s: null pointer", fn), 1;
+    if ((long long)H * h >= 0x7fffffffLL || (long long)W * w >= 0x7fffffffLL)
+        return set_error("%s: extents too large", fn), 1;
     return 0;
 }
 
@@ -56,7 +58,7 @@ using namespace pdw;
 
 extern "C" {
 
-int pdw_version(void) { return 2; }
+int pdw_version(void) { return 3; }
 
 const char* pdw_last_error(void) { return g_err; }
 
@@ -190,6 +192,68 @@ int pdw_add_rowbias(void* y, const float* v, int B, int P, int C, int dtype, voi
     if (B == 0 || P == 0) return 0;
     if (!y || !v) return set_error("pdw_add_rowbias: null pointer"), 1;
     return add_rowbias_launch(y, v, B, P, C, dtype, (hipStream_t)stream);
+}
+
+size_t pdw_pool_branch_workspace_bytes(int B, int P, int D) {
+    if (B < 1 || P < 1 || D < 1) return 0;
+    return pool_branch_workspace(B, P, D);
+}
+
+int pdw_pool_branch_fwd(const void* x, const void* w_pool, const void* b_pool, const void* b_out, void* m,
+                        float* rowbias, void* workspace, size_t workspace_bytes, int B, int P, int D, int dtype,
+                        void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_pool_branch_fwd: unknown dtype %d", dtype), 1;
+    if (B < 0 || P < 1 || D < 1) return set_error("pdw_pool_branch_fwd: bad extents B=%d P=%d D=%d", B, P, D), 1;
+    if (B == 0) return 0;
+    if (!x || !w_pool || !m || !rowbias) return set_error("pdw_pool_branch_fwd: null pointer"), 1;
+    if (!workspace || workspace_bytes < pool_branch_workspace(B, P, D))
+        return set_error("pdw_pool_branch_fwd: workspace too small"), 1;
+    return pool_branch_fwd_launch(x, w_pool, b_pool, b_out, m, rowbias, (float*)workspace, B, P, D, dtype,
+                                  (hipStream_t)stream);
+}
+
+int pdw_pool_branch_bwd(const void* gy, const void* m, const void* w_pool, void* gbias, void* gw_pool, float* dmean,
+                        void* workspace, size_t workspace_bytes, int B, int P, int D, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_pool_branch_bwd: unknown dtype %d", dtype), 1;
+    if (B < 1 || P < 1 || D < 1) return set_error("pdw_pool_branch_bwd: bad extents B=%d P=%d D=%d", B, P, D), 1;
+    if (!gy || !m || !w_pool || !gbias || !gw_pool || !dmean) return set_error("pdw_pool_branch_bwd: null pointer"), 1;
+    if (!workspace || workspace_bytes < pool_branch_workspace(B, P, D))
+        return set_error("pdw_pool_branch_bwd: workspace too small"), 1;
+    return pool_branch_bwd_launch(gy, m, w_pool, gbias, gw_pool, dmean, (float*)workspace, B, P, D, dtype,
+                                  (hipStream_t)stream);
+}
+
+int pdw_dense_supported(int K, int NO, int dtype) {
+    return (dense_rows_supported(K, NO, dtype) && dense_wgrad_supported(K, NO, dtype)) ? 1 : 0;
+}
+
+int pdw_dense_fwd(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
+                  long long N, int K, int NO, int P, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd: unknown dtype %d", dtype), 1;
+    if (N < 0 || K < 1 || NO < 1) return set_error("pdw_dense_fwd: bad extents N=%lld K=%d NO=%d", N, K, NO), 1;
+    if (N > 0 && (!x || !w || !y)) return set_error("pdw_dense_fwd: null pointer"), 1;
+    if (rowbias && P < 1) return set_error("pdw_dense_fwd: rowbias needs P >= 1"), 1;
+    const int r = dense_rows_launch(x, w, w_kmajor ? 1 : 0, bias, rowbias, y, N, K, NO, P, dtype, (hipStream_t)stream);
+    if (r == -1) return set_error("pdw_dense_fwd: K=%d NO=%d dtype=%d not supported (see pdw_dense_supported)", K, NO, dtype), 3;
+    return r;
+}
+
+size_t pdw_dense_wgrad_workspace_bytes(long long N, int M, int NO) {
+    if (N < 0 || M < 1 || NO < 1) return 0;
+    return dense_wgrad_workspace(N, M, NO);
+}
+
+int pdw_dense_wgrad(const void* a, const void* b, void* dw, void* workspace, size_t workspace_bytes, long long N, int M,
+                    int NO, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_dense_wgrad: unknown dtype %d", dtype), 1;
+    if (N < 0 || M < 1 || NO < 1) return set_error("pdw_dense_wgrad: bad extents N=%lld M=%d NO=%d", N, M, NO), 1;
+    if (!dw || (N > 0 && (!a || !b))) return set_error("pdw_dense_wgrad: null pointer"), 1;
+    const size_t need = dense_wgrad_workspace(N, M, NO);
+    if (!workspace || workspace_bytes < need)
+        return set_error("pdw_dense_wgrad: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
+    const int r = dense_wgrad_launch(a, b, dw, workspace, N, M, NO, dtype, (hipStream_t)stream);
+    if (r == -1) return set_error("pdw_dense_wgrad: M=%d NO=%d dtype=%d not supported", M, NO, dtype), 3;
+    return r;
 }
 
 }  // extern "C"

@@ -46,5 +46,19 @@ int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I,
 size_t spatial_sum_workspace(int B, int P, int C);
 int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C, int dtype, hipStream_t s);
 int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, hipStream_t s);
+size_t pool_branch_workspace(int B, int P, int D);
+int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const void* bo, void* m, float* rowbias,
+                           float* ws, int B, int P, int D, int dtype, hipStream_t s);
+int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gwp, float* dmean,
+                           float* ws, int B, int P, int D, int dtype, hipStream_t s);
+
+// dense.hip: thin dense layers on the matrix cores (16-bit types, inner dims <= 128); -1 = not covered
+int dense_rows_supported(int K, int NO, int dtype);
+int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
+                      long long N, int K, int NO, int P, int dtype, hipStream_t s);
+int dense_wgrad_supported(int M, int NO, int dtype);
+size_t dense_wgrad_workspace(long long N, int M, int NO);
+int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,
+                       hipStream_t s);
 
 }  // namespace pdw

@@ -10,9 +10,10 @@
 namespace pdw {
 
 // ---------------------------------------------------------------- adaptive average pool
-__device__ __forceinline__ int bin_start(int i, int in, int out) { return (int)(((long long)i * in) / out); }
+// Host side guarantees in * out < 2^31 (checked in the launchers), so 32-bit arithmetic is exact.
+__device__ __forceinline__ int bin_start(int i, int in, int out) { return (int)((unsigned)(i * in) / (unsigned)out); }
 __device__ __forceinline__ int bin_end(int i, int in, int out) {
-    return (int)(((long long)(i + 1) * in + out - 1) / out);
+    return (int)((unsigned)((i + 1) * in + out - 1) / (unsigned)out);
 }
 
 template <typename T, int VEC>
@@ -58,8 +59,8 @@ __global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T
     t /= W;
     const int ih = (int)(t % H);
     const long long b = t / H;
-    const int i0 = (int)(((long long)ih * h) / H), i1 = (int)((((long long)(ih + 1)) * h + H - 1) / H) - 1;
-    const int j0 = (int)(((long long)iw * w) / W), j1 = (int)((((long long)(iw + 1)) * w + W - 1) / W) - 1;
+    const int i0 = (int)((unsigned)(ih * h) / (unsigned)H), i1 = (int)((unsigned)((ih + 1) * h + H - 1) / (unsigned)H) - 1;
+    const int j0 = (int)((unsigned)(iw * w) / (unsigned)W), j1 = (int)((unsigned)((iw + 1) * w + W - 1) / (unsigned)W) - 1;
     float acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
@@ -163,17 +164,40 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
     const T* gb = gy + b * H * W * ldg + c;
-    for (int i = ilo; i <= ihi; ++i) {
-        const float wy = bl_weight(i, sy, h, m);
-        if (wy == 0.f) continue;
-        for (int j = jlo; j <= jhi; ++j) {
-            const float wx = bl_weight(j, sx, w, n);
-            if (wx == 0.f) continue;
-            float gv[VEC];
-            load_f32<T, VEC>(gb + ((long long)i * W + j) * ldg, gv);
-            const float ww = wy * wx;
+    constexpr int NC = 10;  // candidate destinations per axis kept in registers (enough for scale >= 1/3)
+    if (ihi - ilo < NC && jhi - jlo < NC) {
+        float wy[NC], wx[NC];
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, gv[v], acc[v]);
+        for (int q = 0; q < NC; ++q) {
+            wy[q] = ilo + q <= ihi ? bl_weight(ilo + q, sy, h, m) : 0.f;
+            wx[q] = jlo + q <= jhi ? bl_weight(jlo + q, sx, w, n) : 0.f;
+        }
+#pragma unroll
+        for (int p = 0; p < NC; ++p) {
+            if (wy[p] == 0.f) continue;
+#pragma unroll
+            for (int q = 0; q < NC; ++q) {
+                if (wx[q] == 0.f) continue;
+                float gv[VEC];
+                load_f32<T, VEC>(gb + ((long long)(ilo + p) * W + (jlo + q)) * ldg, gv);
+                const float ww = wy[p] * wx[q];
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, gv[v], acc[v]);
+            }
+        }
+    } else {
+        for (int i = ilo; i <= ihi; ++i) {
+            const float wy = bl_weight(i, sy, h, m);
+            if (wy == 0.f) continue;
+            for (int j = jlo; j <= jhi; ++j) {
+                const float wx = bl_weight(j, sx, w, n);
+                if (wx == 0.f) continue;
+                float gv[VEC];
+                load_f32<T, VEC>(gb + ((long long)i * W + j) * ldg, gv);
+                const float ww = wy * wx;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, gv[v], acc[v]);
+            }
         }
     }
     store_f32<T, VEC>(gx + ((b * h + m) * w + n) * C + c, acc);
@@ -254,12 +278,137 @@ __global__ __launch_bounds__(256) void spatial_sum_part_k(const T* __restrict__ 
 
 __global__ __launch_bounds__(256) void spatial_sum_final_k(const float* __restrict__ part, float* __restrict__ out,
                                                            int nchunks, int C, int total) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int c = idx % C, b = idx / C;
+    __shared__ float red[8][32];
+    const int el = threadIdx.x & 31, ql = threadIdx.x >> 5;
+    const int idx = blockIdx.x * 32 + el;
     float s = 0.f;
-    for (int q = 0; q < nchunks; ++q) s += part[((long long)b * nchunks + q) * C + c];
-    out[idx] = s;
+    if (idx < total) {
+        const int c = idx % C, b = idx / C;
+        for (int q = ql; q < nchunks; q += 8) s += part[((long long)b * nchunks + q) * C + c];
+    }
+    red[ql][el] = s;
+    __syncthreads();
+    if (ql == 0 && idx < total)
+        out[idx] = ((red[0][el] + red[1][el]) + (red[2][el] + red[3][el])) +
+                   ((red[4][el] + red[5][el]) + (red[6][el] + red[7][el]));
+}
+
+// ---------------------------------------------------------------- pooled branch (global mean -> dense layer)
+// Forward, one workgroup per image: m[b,:] = (sum of the chunk partials) / P rounded to T, then
+// rowbias[b,o] = sum_c m[b,c] * Wp[o,c] + bp[o] + bo[o]  (fp32).  The dot products are spread over
+// 8 lanes per output feature (strided over c, combined with wavefront shuffles).
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_fwd_k(const float* __restrict__ part, int nchunks, int D, float inv_p,
+                                                         const T* __restrict__ wp, const T* __restrict__ bp,
+                                                         const T* __restrict__ bo, T* __restrict__ m,
+                                                         float* __restrict__ rowbias) {
+    extern __shared__ float sm[];  // [D]
+    const int b = blockIdx.x;
+    for (int c = threadIdx.x; c < D; c += 256) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        const float* pp = part + (long long)b * nchunks * D + c;
+        int q = 0;
+        for (; q + 4 <= nchunks; q += 4) {
+            s0 += pp[(long long)q * D], s1 += pp[(long long)(q + 1) * D];
+            s2 += pp[(long long)(q + 2) * D], s3 += pp[(long long)(q + 3) * D];
+        }
+        for (; q < nchunks; ++q) s0 += pp[(long long)q * D];
+        const T mv = from_f32<T>(((s0 + s1) + (s2 + s3)) * inv_p);
+        m[(long long)b * D + c] = mv;
+        sm[c] = to_f32(mv);
+    }
+    __syncthreads();
+    const int sub = threadIdx.x & 7;
+    for (int o = threadIdx.x >> 3; o < D; o += 32) {
+        const T* wr = wp + (long long)o * D;
+        float acc = 0.f;
+#pragma unroll 4
+        for (int c = sub; c < D; c += 8) acc = fmaf(sm[c], to_f32(wr[c]), acc);
+        acc += __shfl_xor(acc, 1);
+        acc += __shfl_xor(acc, 2);
+        acc += __shfl_xor(acc, 4);
+        if (sub == 0) {
+            if (bp) acc += to_f32(bp[o]);
+            if (bo) acc += to_f32(bo[o]);
+            rowbias[(long long)b * D + o] = acc;
+        }
+    }
+}
+
+// Backward part A, one workgroup per image: gs[b,:] = sum of the chunk partials of gy's column sums and
+// dmean[b,c] = inv_p * sum_o gs[b,o] * Wp[o,c]   (the gradient that flows back through the mean).
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_bwd_a_k(const float* __restrict__ part, int nchunks, int D,
+                                                           float inv_p, const T* __restrict__ wp,
+                                                           float* __restrict__ gs, float* __restrict__ dmean) {
+    extern __shared__ float sm[];  // [D] column sums, then [OL][D] partial products
+    const int b = blockIdx.x;
+    for (int c = threadIdx.x; c < D; c += 256) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        const float* pp = part + (long long)b * nchunks * D + c;
+        int q = 0;
+        for (; q + 4 <= nchunks; q += 4) {
+            s0 += pp[(long long)q * D], s1 += pp[(long long)(q + 1) * D];
+            s2 += pp[(long long)(q + 2) * D], s3 += pp[(long long)(q + 3) * D];
+        }
+        for (; q < nchunks; ++q) s0 += pp[(long long)q * D];
+        const float s = (s0 + s1) + (s2 + s3);
+        gs[(long long)b * D + c] = s;
+        sm[c] = s;
+    }
+    __syncthreads();
+    // thread (ol, c): rows o = ol, ol+OL, ...  of Wp, coalesced over c; OL row lanes combined through LDS
+    const int OL = D <= 128 ? 256 / (D < 32 ? 32 : D) : 1;   // row lanes when D <= 128
+    float* prod = sm + D;
+    if (OL > 1) {
+        const int cw = 256 / OL;
+        const int c = threadIdx.x % cw, ol = threadIdx.x / cw;
+        float acc = 0.f;
+        if (c < D) {
+#pragma unroll 4
+            for (int o = ol; o < D; o += OL) acc = fmaf(sm[o], to_f32(wp[(long long)o * D + c]), acc);
+            prod[ol * D + c] = acc;
+        }
+        __syncthreads();
+        if (ol == 0 && c < D) {
+            float t = 0.f;
+            for (int q = 0; q < OL; ++q) t += prod[q * D + c];
+            dmean[(long long)b * D + c] = t * inv_p;
+        }
+    } else {
+        for (int c = threadIdx.x; c < D; c += 256) {
+            float acc = 0.f;
+#pragma unroll 4
+            for (int o = 0; o < D; ++o) acc = fmaf(sm[o], to_f32(wp[(long long)o * D + c]), acc);
+            dmean[(long long)b * D + c] = acc * inv_p;
+        }
+    }
+}
+
+// Backward part B, one workgroup per output feature o: gbias[o] = sum_b gs[b,o] and
+// gwp[o,c] = sum_b gs[b,o] * m[b,c].
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_bwd_b_k(const float* __restrict__ gs, const T* __restrict__ m, int B,
+                                                           int D, T* __restrict__ gbias, T* __restrict__ gwp) {
+    extern __shared__ float gcol[];  // [B] = gs[:, o]
+    const int o = blockIdx.x;
+    for (int b = threadIdx.x; b < B; b += 256) gcol[b] = gs[(long long)b * D + o];
+    __syncthreads();
+    for (int c = threadIdx.x; c < D; c += 256) {
+        float a0 = 0.f, a1 = 0.f;
+        int b = 0;
+        for (; b + 2 <= B; b += 2) {
+            a0 = fmaf(gcol[b], to_f32(m[(long long)b * D + c]), a0);
+            a1 = fmaf(gcol[b + 1], to_f32(m[(long long)(b + 1) * D + c]), a1);
+        }
+        if (b < B) a0 = fmaf(gcol[b], to_f32(m[(long long)b * D + c]), a0);
+        gwp[(long long)o * D + c] = from_f32<T>(a0 + a1);
+    }
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+        for (int b = 0; b < B; ++b) s += gcol[b];
+        gbias[o] = from_f32<T>(s);
+    }
 }
 
 // y[b,p,c] += v[b,c]  (v in fp32, one rounding)
@@ -413,6 +562,23 @@ size_t spatial_sum_workspace(int B, int P, int C) {
     return (size_t)B * n * C * sizeof(float);
 }
 
+// Pass 1 only: ws[b][chunk][c]; returns the number of chunks through *nchunks.
+static int spatial_sum_parts(const void* x, float* ws, int B, int P, int C, int dtype, hipStream_t s, int* nchunks) {
+    int n, len;
+    spatial_sum_plan(B, P, &n, &len);
+    *nchunks = n;
+    const void* ptrs[1] = {x};
+    int vec = pick_vec(C, esize(dtype), ptrs, 1);
+    if (C / vec > 256) return set_error("spatial sum: more than %d channels not supported", 256 * vec), 1;
+    const int pl = 256 / (C / vec);
+    const size_t lds = (size_t)pl * C * sizeof(float);
+    if (lds > 64 * 1024) return set_error("spatial sum: channel count %d too large", C), 1;
+#define CALL(T, V) hipLaunchKernelGGL((spatial_sum_part_k<T, V>), dim3(n, B), dim3(256), lds, s, (const T*)x, ws, P, C, len);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("spatial_sum_part");
+}
+
 int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C, int dtype, hipStream_t s) {
     int n, len;
     spatial_sum_plan(B, P, &n, &len);
@@ -427,7 +593,7 @@ int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C
 #undef CALL
     if (int e = check_launch("spatial_sum_part")) return e;
     const int total = B * C;
-    hipLaunchKernelGGL(spatial_sum_final_k, dim3(cdiv(total, 256)), dim3(256), 0, s, ws, out, n, C, total);
+    hipLaunchKernelGGL(spatial_sum_final_k, dim3(cdiv(total, 32)), dim3(256), 0, s, ws, out, n, C, total);
     return check_launch("spatial_sum_final");
 }
 
@@ -442,6 +608,53 @@ int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, 
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("add_rowbias");
+}
+
+size_t pool_branch_workspace(int B, int P, int D) { return spatial_sum_workspace(B, P, D) + (size_t)B * D * sizeof(float); }
+
+int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const void* bo, void* m, float* rowbias,
+                           float* ws, int B, int P, int D, int dtype, hipStream_t s) {
+    int n;
+    if (int e = spatial_sum_parts(x, ws, B, P, D, dtype, s, &n)) return e;
+    const float inv_p = 1.f / (float)P;
+    const size_t lds = (size_t)D * sizeof(float);
+    switch (dtype) {
+        case kF32:
+            hipLaunchKernelGGL((pool_branch_fwd_k<float>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const float*)wp,
+                               (const float*)bp, (const float*)bo, (float*)m, rowbias);
+            break;
+        case kF16:
+            hipLaunchKernelGGL((pool_branch_fwd_k<f16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const f16_t*)wp,
+                               (const f16_t*)bp, (const f16_t*)bo, (f16_t*)m, rowbias);
+            break;
+        default:
+            hipLaunchKernelGGL((pool_branch_fwd_k<bf16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p,
+                               (const bf16_t*)wp, (const bf16_t*)bp, (const bf16_t*)bo, (bf16_t*)m, rowbias);
+    }
+    return check_launch("pool_branch_fwd");
+}
+
+int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gwp, float* dmean,
+                           float* ws, int B, int P, int D, int dtype, hipStream_t s) {
+    int n;
+    if (int e = spatial_sum_parts(gy, ws, B, P, D, dtype, s, &n)) return e;
+    float* gs = ws + spatial_sum_workspace(B, P, D) / sizeof(float);
+    const float inv_p = 1.f / (float)P;
+    const size_t lds = (size_t)D * 9 * sizeof(float);
+    const size_t ldsb = (size_t)B * sizeof(float);
+    if (lds > 64 * 1024 || ldsb > 64 * 1024) return set_error("pool branch: extents too large"), 1;
+#define PDW_PB(T)                                                                                                  \
+    hipLaunchKernelGGL((pool_branch_bwd_a_k<T>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const T*)wp, gs, dmean); \
+    if (int e = check_launch("pool_branch_bwd_a")) return e;                                                       \
+    hipLaunchKernelGGL((pool_branch_bwd_b_k<T>), dim3(D), dim3(256), ldsb, s, gs, (const T*)m, B, D, (T*)gbias,    \
+                       (T*)gwp);
+    switch (dtype) {
+        case kF32: PDW_PB(float) break;
+        case kF16: PDW_PB(f16_t) break;
+        default: PDW_PB(bf16_t) break;
+    }
+#undef PDW_PB
+    return check_launch("pool_branch_bwd_b");
 }
 
 }  // namespace pdw

@@ -127,3 +127,76 @@ def add_rowbias_(y, v):
     if y.numel():
         _launch("pdw_add_rowbias", dev, y.data_ptr(), v.data_ptr(), B, P, C, _lib.dtype_code(y.dtype))
     return y
+
+
+def dense_supported(K, NO, dtype):
+    """True when the matrix-core dense kernels cover an inner size K, output size NO layer of this dtype."""
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    return bool(_lib.lib().pdw_dense_supported(int(K), int(NO), _lib.dtype_code(dtype)))
+
+
+def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=1):
+    """y[..., o] = sum_k x[..., k] * W(o, k) + bias[o] + rowbias[image][o].
+
+    w is [NO, K] (nn.Linear layout) or, with w_kmajor, [K, NO].  rowbias is fp32 [B, NO], one row per
+    `rows_per_image` consecutive rows of x."""
+    dev = _lib.require_device(x, w)
+    K = x.shape[-1]
+    NO = w.shape[1] if w_kmajor else w.shape[0]
+    assert (w.shape[0] if w_kmajor else w.shape[1]) == K and x.is_contiguous() and w.is_contiguous()
+    N = x.numel() // K
+    y = torch.empty(x.shape[:-1] + (NO,), device=dev, dtype=x.dtype)
+    if N:
+        _launch("pdw_dense_fwd", dev, x.data_ptr(), w.data_ptr(), 1 if w_kmajor else 0,
+                bias.data_ptr() if bias is not None else None, rowbias.data_ptr() if rowbias is not None else None,
+                y.data_ptr(), N, K, NO, int(rows_per_image), _lib.dtype_code(x.dtype))
+    return y
+
+
+def dense_wgrad(a, b):
+    """dw[m, o] = sum_n a[n, m] * b[n, o] over all leading dimensions; returns [M, NO] in a's dtype."""
+    dev = _lib.require_device(a, b)
+    M, NO = a.shape[-1], b.shape[-1]
+    N = a.numel() // M
+    assert b.numel() // NO == N and a.is_contiguous() and b.is_contiguous()
+    dw = torch.empty((M, NO), device=dev, dtype=a.dtype)
+    nbytes = _lib.lib().pdw_dense_wgrad_workspace_bytes(N, M, NO)
+    ws = torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
+    _launch("pdw_dense_wgrad", dev, a.data_ptr(), b.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel() * 4, N, M, NO,
+            _lib.dtype_code(a.dtype))
+    return dw
+
+
+def _pool_ws(B, P, D, dev):
+    nbytes = _lib.lib().pdw_pool_branch_workspace_bytes(B, P, D)
+    return torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
+
+
+def pool_branch_forward(x, w_pool, b_pool=None, b_out=None):
+    """x [B, ..., D] -> (m [B, D] in x's dtype: the per-image mean; rowbias fp32 [B, D] = m @ w_pool^T + b_pool + b_out)."""
+    dev = _lib.require_device(x, w_pool)
+    B, D = x.shape[0], x.shape[-1]
+    P = x.numel() // max(B * D, 1)
+    m = torch.empty((B, D), device=dev, dtype=x.dtype)
+    rowbias = torch.empty((B, D), device=dev, dtype=torch.float32)
+    if B and P:
+        ws = _pool_ws(B, P, D, dev)
+        _launch("pdw_pool_branch_fwd", dev, x.data_ptr(), w_pool.data_ptr(),
+                b_pool.data_ptr() if b_pool is not None else None, b_out.data_ptr() if b_out is not None else None,
+                m.data_ptr(), rowbias.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, P, D, _lib.dtype_code(x.dtype))
+    return m, rowbias
+
+
+def pool_branch_backward(gy, m, w_pool):
+    """-> (gbias [D], gw_pool [D, D] in gy's dtype, dmean fp32 [B, D])."""
+    dev = _lib.require_device(gy, m, w_pool)
+    B, D = gy.shape[0], gy.shape[-1]
+    P = gy.numel() // max(B * D, 1)
+    gbias = torch.empty((D,), device=dev, dtype=gy.dtype)
+    gwp = torch.empty((D, D), device=dev, dtype=gy.dtype)
+    dmean = torch.empty((B, D), device=dev, dtype=torch.float32)
+    ws = _pool_ws(B, P, D, dev)
+    _launch("pdw_pool_branch_bwd", dev, gy.data_ptr(), m.data_ptr(), w_pool.data_ptr(), gbias.data_ptr(), gwp.data_ptr(),
+            dmean.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, P, D, _lib.dtype_code(gy.dtype))
+    return gbias, gwp, dmean

@@ -125,3 +125,52 @@ def test_spatial_sum_and_rowbias(dtype, shape):
     y = x.cuda().clone()
     ops.add_rowbias_(y, v.cuda())
     assert_close(y, x.double().numpy() + v.double().numpy()[:, None, None, :], dtype, "rowbias")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("K,NO", [(128, 64), (64, 128), (96, 48), (48, 96), (64, 32), (32, 64), (8, 8), (120, 104), (16, 24)])
+@pytest.mark.parametrize("N,P", [(3 * 35, 35), (1, 1), (4 * 3136, 3136)])
+def test_dense_layers(dtype, K, NO, N, P):
+    """Matrix-core dense kernels against float64: forward in both weight layouts with bias and per-image
+    row bias, and the weight gradient."""
+    from pyramidconvblock_amd import ops
+
+    if not (ops.dense_supported(K, NO, dtype) and ops.dense_supported(NO, K, dtype)):
+        pytest.skip("shape not covered by the dense kernels in both directions")
+    gen = torch.Generator().manual_seed(K * 1000 + NO + N)
+    x = randn(gen, N, K).to(dtype)
+    w = (randn(gen, NO, K) / K ** 0.5).to(dtype)
+    b = randn(gen, NO).to(dtype)
+    rb = randn(gen, N // P, NO)
+    ref = x.double() @ w.double().t() + b.double() + rb.double().repeat_interleave(P, 0)
+    y = ops.dense_forward(x.cuda(), w.cuda(), bias=b.cuda(), rowbias=rb.cuda(), rows_per_image=P)
+    assert_close(y, ref.numpy(), dtype, "dense fwd")
+    g = randn(gen, N, NO).to(dtype)
+    dx = ops.dense_forward(g.cuda(), w.cuda(), w_kmajor=True)         # g @ w : [N,NO] x [NO,K]
+    assert_close(dx, (g.double() @ w.double()).numpy(), dtype, "dense dgrad")
+    dw = ops.dense_wgrad(g.cuda(), x.cuda())                           # g^T @ x : [NO, K]
+    assert_close(dw, (g.double().t() @ x.double()).numpy(), dtype, "dense wgrad")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 9, 7, 24), (32, 56, 56, 128), (3, 57, 61, 200)])
+def test_pool_branch(dtype, shape):
+    """Global-mean branch (conv_block.py:46-47) forward and backward against float64."""
+    from pyramidconvblock_amd import ops
+
+    B, H, W, D = shape
+    gen = torch.Generator().manual_seed(D)
+    x = randn(gen, *shape).to(dtype)
+    wp = (randn(gen, D, D) / D ** 0.5).to(dtype)
+    bp, bo = randn(gen, D).to(dtype), randn(gen, D).to(dtype)
+    m, rb = ops.pool_branch_forward(x.cuda(), wp.cuda(), bp.cuda(), bo.cuda())
+    m_ref = x.double().mean(dim=(1, 2))
+    assert_close(m, m_ref.numpy(), dtype, "mean")
+    rb_ref = m.double().cpu() @ wp.double().t() + bp.double() + bo.double()   # from the rounded mean, as computed
+    assert_close(rb, rb_ref.numpy(), torch.float32, "rowbias", scale=2.0)
+    gy = randn(gen, *shape).to(dtype)
+    gbias, gwp, dmean = ops.pool_branch_backward(gy.cuda(), m, wp.cuda())
+    gs = gy.double().sum(dim=(1, 2))
+    assert_close(gbias, gs.sum(0).numpy(), dtype, "bias grad")
+    assert_close(gwp, (gs.t() @ m.double().cpu()).numpy(), dtype, "w_pool grad")
+    assert_close(dmean, ((gs @ wp.double()) / (H * W)).numpy(), torch.float32, "dmean", scale=8.0)
