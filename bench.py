@@ -28,6 +28,15 @@ VALU_PEAK = 157.3e12  # fp32 vector FLOP/s, MI355X published
 
 WORKLOAD = dict(B=32, H=56, W=56, D=128, k=13, dtype="bf16")
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --kernel ...`, each
+# scaled by what the same counter reads for a plain copy of known size (`bench.py --kernel copy`); the
+# runs and the scale factors are recorded under profiles/.  None = not measured.
+MEASURED_TRAFFIC = {
+    "dwconv_fwd[32x56x56x64,k=13]": (14115 + 12544) * 1024,   # fetch 14.45 MB + write 12.85 MB
+    "dwconv_dgrad[32x56x56x64,k=13]": (14115 + 12544) * 1024,  # same kernel, same shape
+    "dwconv_wgrad[32x56x56x64,k=13]": (27247 + 5408 + 5419 + 21) * 1024,
+}
+
 
 def block_alg_bytes(B, H, W, D, k, esize, scales=(1.0, 0.5)):
     """Compulsory HBM traffic of the unfused op graph (each op reads each input once and writes
@@ -70,25 +79,36 @@ def time_gpu(fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def time_kernel_events(launch, nbuf, iters=30, warmup=5):
-    """Average duration of one launch measured with HIP events recorded on the stream the kernel is
-    enqueued on (torch's current stream); `launch(i)` uses buffer set i % nbuf so consecutive
-    launches do not hit in the 256 MB Infinity Cache."""
-    for i in range(warmup):
-        launch(i % nbuf)
+def time_kernel_events(launch, nbuf, iters=24, reps=4):
+    """Average duration of one launch.  `iters` launches (launch(i) uses buffer set i % nbuf, so that
+    consecutive launches do not hit in the 256 MB Infinity Cache) are captured into a HIP graph, and the
+    replays are bracketed by HIP events recorded on the stream the graph runs on, so the figure is GPU
+    time per launch, free of the host's per-call overhead."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(min(nbuf, 3)):
+            launch(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(iters):
+            launch(i % nbuf)
+    graph.replay()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     start.record()
-    for i in range(iters):
-        launch(i % nbuf)
+    for _ in range(reps):
+        graph.replay()
     stop.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) * 1e-3 / iters
+    return start.elapsed_time(stop) * 1e-3 / (iters * reps)
 
 
 def kernel_rooflines(B, H, W, D, k, dtype):
     """Times each hot kernel of the block alone at its real shapes; returns a list of dicts."""
-    from pyramidconvblock_amd import avgpool, dwconv, up
+    from pyramidconvblock_amd import avgpool, dwconv, ops, up
 
     I, G = D // 2, D // 4
     es = torch.empty((), dtype=dtype).element_size()
@@ -125,6 +145,22 @@ def kernel_rooflines(B, H, W, D, k, dtype):
     ):
         t = time_kernel_events(fn, nbuf)
         out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=0.0))
+    # gate and the dense conv_up layer ([N,D] <-> [N,I])
+    c = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    xin = [torch.randn(B, H, W, D, device="cuda").to(dtype) for _ in range(4)]
+    wup = (torch.randn(I, D, device="cuda") / D ** 0.5).to(dtype)
+    N = B * H * W
+    for name, fn, nb_, nbytes, fl in (
+        ("gate_fwd", lambda i: ops.gate_forward(c[i]), nbuf, es * 1.5 * N * I, 0.0),
+        ("gate_bwd", lambda i: ops.gate_backward(c[i], gbig[i]), nbuf, es * 2.5 * N * I, 0.0),
+        ("dense_fwd", lambda i: ops.dense_forward(xin[i], wup), 4, es * (N * D + N * I + D * I), 2.0 * N * D * I),
+        ("dense_dgrad", lambda i: ops.dense_forward(a[i], wup, w_kmajor=True), 4, es * (N * D + N * I + D * I),
+         2.0 * N * D * I),
+        ("dense_wgrad", lambda i: ops.dense_wgrad(a[i % 4], xin[i % 4]), 4, es * (N * D + N * I + D * I),
+         2.0 * N * D * I),
+    ):
+        t = time_kernel_events(fn, nb_)
+        out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=fl))
     return out
 
 
@@ -138,7 +174,11 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     h, w = H // 2, W // 2
     geo = ((1, 1), (k // 2, k // 2), (1, 1))
     op, _, res = name.partition("_")
-    if op in ("fwd", "dgrad", "wgrad"):
+    if name == "copy":  # a plain copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.randn(B, H, W, I, device="cuda").to(dtype)
+        dst = torch.empty_like(src)
+        fn = lambda: dst.copy_(src)
+    elif op in ("fwd", "dgrad", "wgrad"):
         hh, ww = (H, W) if res == "full" else (h, w)
         x = torch.randn(B, hh, ww, I, device="cuda").to(dtype)
         g = torch.randn(B, hh, ww, I, device="cuda").to(dtype)
@@ -208,7 +248,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep and forward-only timings")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel event timings")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
-                    "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, dense_{fwd,dgrad,wgrad}")
+                    "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, dense_{fwd,dgrad,wgrad}, copy")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -295,11 +335,16 @@ def main():
 
     if not args.no_kernels:
         ks = kernel_rooflines(B, H, W, D, k, dtype)
-        dom = max(ks, key=lambda r: r["seconds"])
+        # Dominant kernel = largest share of the step.  Forward and input gradient are the same kernel
+        # function (dwconv_tiled_k) at the same shape, so their launches count together.
+        def share(r):
+            return r["seconds"] * (2 if r["kernel"].startswith(("dwconv_fwd", "dwconv_dgrad")) else 1)
+
+        dom = max(ks, key=share)
         result["roofline"] = {
             "kernel": dom["kernel"], "bound": "hbm", "achieved": dom["alg_bytes"] / dom["seconds"] / 1e9,
             "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom["alg_bytes"] / dom["seconds"] / HBM_PEAK,
-            "traffic": None, "avg_us": dom["seconds"] * 1e6,
+            "traffic": MEASURED_TRAFFIC.get(dom["kernel"]), "avg_us": dom["seconds"] * 1e6,
             "valu_frac": dom["flops"] / dom["seconds"] / VALU_PEAK,
         }
         result["kernels"] = [{"kernel": r["kernel"], "us": round(r["seconds"] * 1e6, 2),

@@ -549,7 +549,7 @@ int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I,
 }
 
 static void spatial_sum_plan(int B, int P, int* nchunks, int* chunk_len) {
-    int n = cdiv(1024, B > 0 ? B : 1);  // about four workgroups per CU over the batch
+    int n = cdiv(512, B > 0 ? B : 1);  // about two workgroups per CU over the batch
     if (n > cdiv(P, 64)) n = cdiv(P, 64);
     if (n < 1) n = 1;
     *chunk_len = cdiv(P, n);
