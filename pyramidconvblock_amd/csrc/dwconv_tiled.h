@@ -339,12 +339,14 @@ struct TiledPlan {
 };
 
 template <typename T, int KW, int R, int Q, int CS>
-static TiledPlan plan_tiled(int OH, int OW, int KH) {
+static TiledPlan plan_tiled(int OH, int OW, int KH, int B, int C) {
     constexpr int PK = PackOf<T>::PK;
     constexpr int NP = (KW + PK - 1) / PK;
-    // Estimated wave-instructions per workgroup (compute rounds + staging) times the number of
-    // workgroups; ragged edges show up as extra workgroups, halo re-reads as staging.
+    // Estimated wave-instructions per tile (compute rounds + staging) times the makespan, in tiles, of
+    // spreading the tiles over the chip (pick_chunks); ragged edges show up as extra tiles, halo re-reads
+    // as staging, too few tiles as idle CUs.
     const int slots = 4 * (64 / CS);
+    const int slices = cdiv(C, CS);
     TiledPlan best;
     for (int nrg = 1; nrg <= 32; ++nrg)
         for (int nst = 1; nst <= 16; ++nst) {
@@ -355,12 +357,17 @@ static TiledPlan plan_tiled(int OH, int OW, int KH) {
             const int rows_in = th + KH - 1, cpn = (tw + KW - 1 + PK - 1) / PK;
             const long long lds = ((long long)rows_in * cpn + (long long)KH * NP) * CS * 4;
             if (lds > 72 * 1024) continue;
-            const double nt = (double)cdiv(OH, th) * cdiv(OW, tw);
+            const long long nt = (long long)B * cdiv(OH, th) * cdiv(OW, tw);
+            int occ = (int)((160 * 1024) / (lds + 512));
+            occ = occ < 1 ? 1 : (occ > 3 ? 3 : occ);
+            double span;
+            pick_chunks(nt, slices, occ, &span);
             const int rounds = cdiv(np, slots);
             const double compute =
                 4.0 * rounds * (KH * (Q * R * NP + NP) * (PK == 2 ? 1.06 : 1.0) + 6.0 * Q * R + 60);
             const double stage = rows_in * cpn * (CS / 8) / 64.0 * 40.0 + KH * NP * CS / 64.0 * 14.0 + 150;
-            const double cost = nt * (compute + stage);
+            // Plenty of tiles: minimise total work.  Fewer workgroups than CUs: minimise the makespan.
+            const double cost = (nt * slices >= 512 ? (double)nt * slices / 512.0 : span) * (compute + stage);
             if (best.cost < 0 || cost < best.cost) best.cost = cost, best.nrg = nrg, best.nst = nst;
         }
     return best;
@@ -385,7 +392,7 @@ static int launch_tiled(const TiledPlan& plan, const void* x, const void* w, voi
     if (ntiles > 0x7fffffffLL || (long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL)
         return -1;
     g.ntiles = (int)ntiles;
-    // Persistent workgroups: as many as fit on the chip at once (LDS-limited, at most 3 per CU), then
+    // Persistent workgroups: as many as fit on the chip at once (LDS allows `occ` per CU, at most 3), then
     // trimmed so the tiles divide as evenly as possible among them.
     int occ = (int)((160 * 1024) / (lds + 512));
     const int occ_max = getenv("PDW_OCC") ? atoi(getenv("PDW_OCC")) : 3;
@@ -432,9 +439,9 @@ template <typename T, int KW>
 static int launch_best(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
                        bool flip, hipStream_t s) {
     const int OH = H + 2 * PH - KH + 1, OW = W + 2 * PW - KW + 1;
-    const TiledPlan p0 = plan_tiled<T, KW, 8, 2, 32>(OH, OW, KH);
-    const TiledPlan p1 = plan_tiled<T, KW, 14, 1, 32>(OH, OW, KH);
-    const TiledPlan p2 = plan_tiled<T, KW, 14, 2, 32>(OH, OW, KH);
+    const TiledPlan p0 = plan_tiled<T, KW, 8, 2, 32>(OH, OW, KH, B, C);
+    const TiledPlan p1 = plan_tiled<T, KW, 14, 1, 32>(OH, OW, KH, B, C);
+    const TiledPlan p2 = plan_tiled<T, KW, 14, 2, 32>(OH, OW, KH, B, C);
     int pick = -1;
     double best = -1;
     const TiledPlan* ps[3] = {&p0, &p1, &p2};

@@ -172,6 +172,7 @@ static WgradPlan plan_wgrad(int B, int H, int W, int C, int PH, int PW) {
     g.slices = cdiv(C, CS);
     const int red_bytes = 4 * K * CS * 4;
     double best = -1;
+    int best_nch = 1;
     for (int th = 1; th <= 32; ++th)
         for (int nsp = 1; nsp <= 4; ++nsp) {
             const int tw = 2 * nsp * R;
@@ -180,13 +181,17 @@ static WgradPlan plan_wgrad(int B, int H, int W, int C, int PH, int PW) {
             const long long lds = ((long long)(th + K - 1) * cpx + (long long)th * cpg) * CS * 4;
             if (lds > 78 * 1024) continue;
             const int t_h = cdiv(g.OH, th), t_w = cdiv(g.OW, tw);
-            const double ntiles = (double)B * t_h * t_w;
+            const long long ntiles = (long long)B * t_h * t_w;
+            if (ntiles > 0x7fffffffLL) continue;
             // wave-instructions per tile: compute rounds over rows (4 waves) + staging
             const double compute = cdiv(th + K - 1, 4) * nsp * (K * K * (R / PK) * th / (double)(th + K - 1) + 60.0);
             const double stage = ((th + K - 1) * cpx + th * cpg) * (CS / 8) / 64.0 * 40.0 + 100;
-            const double cost = ntiles * (4 * compute + stage);
+            double span;
+            const int nch = pick_chunks(ntiles, g.slices, 2, &span);
+            // makespan in tile units times the tile cost, plus the partial-sum traffic of the chunks
+            const double cost = span * (4 * compute + stage) + 0.02 * nch * K * K;
             if (best < 0 || cost < best) {
-                best = cost;
+                best = cost, best_nch = nch;
                 g.TH = th, g.NSP = nsp, g.tiles_h = t_h, g.tiles_w = t_w, g.CPX = cpx, g.CPG = cpg;
                 p.lds = (size_t)(lds > red_bytes ? lds : red_bytes);
             }
@@ -199,21 +204,12 @@ static WgradPlan plan_wgrad(int B, int H, int W, int C, int PH, int PW) {
         g.CPX = (tw + K - 1 + PK - 1) / PK, g.CPG = tw / PK;
         const long long lds = ((long long)(g.TH + K - 1) * g.CPX + (long long)g.TH * g.CPG) * CS * 4;
         p.lds = (size_t)(lds > red_bytes ? lds : red_bytes);
+        best_nch = pick_chunks((long long)B * g.tiles_h * g.tiles_w, g.slices, 2, nullptr);
     }
     const long long ntiles = (long long)B * g.tiles_h * g.tiles_w;
     if (ntiles > 0x7fffffffLL) return p;
     g.ntiles = (int)ntiles;
-    // Position chunks: aim for two workgroups per CU over all slices, with tiles dividing evenly.
-    const int target = 512 / g.slices > 1 ? 512 / g.slices : 1;
-    int nch = (int)(ntiles < target ? ntiles : target);
-    double beste = -1;
-    for (int cand = (target + 1) / 2; cand <= 2 * target && cand <= ntiles; ++cand) {
-        const double rounds = (double)cdiv(ntiles, cand);
-        const long long blocks = (long long)cand * g.slices;
-        const double eff = ntiles / (rounds * cand) * blocks / (double)(cdiv(blocks, 256) * 256) -
-                           1e-4 * cand / target;  // mild preference for fewer partials
-        if (eff > beste) beste = eff, nch = cand;
-    }
+    int nch = best_nch;
     if (getenv("PDW_WG_NCH")) nch = atoi(getenv("PDW_WG_NCH"));
     g.nchunks = nch < 1 ? 1 : nch;
     p.nblocks = g.nchunks * g.slices;

@@ -102,6 +102,25 @@ __device__ __forceinline__ void stage_tile(uint32_t* __restrict__ xl, const T* _
     }
 }
 
+// Number of persistent workgroups per channel slice for `ntiles` equal tiles, all resident at once
+// (at most `max_resident` per CU over 256 CUs): minimises the estimated makespan
+// rounds * (1 + 0.15 * (workgroups sharing a CU - 1)), preferring more workgroups on ties.  Returns the
+// makespan in units of one tile's stand-alone time through *cost.
+inline int pick_chunks(long long ntiles, int slices, int max_resident, double* cost) {
+    int best_n = 1;
+    double best = -1;
+    long long hi = (256LL * max_resident) / slices;
+    if (hi < 1) hi = 1;
+    if (hi > ntiles) hi = ntiles;
+    for (long long cand = 1; cand <= hi; ++cand) {
+        const long long per_cu = (cand * slices + 255) / 256;
+        const double t = (double)((ntiles + cand - 1) / cand) * (1.0 + 0.15 * (per_cu - 1));
+        if (best < 0 || t <= best + 1e-9) best = t, best_n = (int)cand;
+    }
+    if (cost) *cost = best;
+    return best_n;
+}
+
 // log2 of the staging threads laid along a row of CPn units (see stage_tile).
 inline int stage_ulog(int CPn, int CS, int V) {
     const int ut = 256 / (CS / V);
