@@ -1,17 +1,19 @@
 // Thin dense layers of the block (inner dimensions <= 128, millions of rows) on the matrix
-// cores.  These products are HBM-bound: the kernels stream the row matrix once with 16-byte
-// vector loads straight into MFMA operand registers (no LDS), keep the small weight matrix in
-// registers for the whole kernel, and fuse the bias / per-image broadcast add into the store.
+// cores.  These products are HBM-bound: the row matrix is streamed once with 16-byte vector loads
+// straight into MFMA operand registers, the small weight matrix is staged to LDS once per
+// workgroup, and the bias / per-image broadcast add is fused into the store.
 //
 //   rows:  Y[n,o] = sum_k X[n,k] * W(o,k) + bias[o] + rowbias[n / P][o]
 //          computed as D = Wtile (32 features x 16 k) * Xtile^T (16 k x 32 rows) with
-//          v_mfma_f32_32x32x16_{bf16,f16}; a lane then owns one row and 4 consecutive
-//          features per accumulator group, so the store is an 8-byte vector.
+//          v_mfma_f32_32x32x16_{bf16,f16}; a lane then owns one row and 4 consecutive features per
+//          accumulator group; the tile is transposed through a per-wave LDS buffer so the global
+//          stores are whole 128-byte lines.
 //   wgrad: dW[m,o] = sum_n A[n,m] * B[n,o]   (reduction over the rows)
-//          both operands are gathered with the row index as the MFMA k dimension; every
-//          wavefront accumulates all (m,o) tiles over its row range in registers, the
-//          wavefronts of a workgroup are summed through LDS and the per-workgroup fp32
-//          partials are reduced in a fixed order by wgrad_reduce_parts (no atomics).
+//          64-row stages of A and B are copied to LDS with coalesced loads (requested one stage
+//          ahead); the MFMA k dimension is the row index, so fragments are read from LDS column-wise.
+//          Every wavefront accumulates all (m,o) tiles in registers, the wavefronts of a workgroup
+//          are summed through LDS and the per-workgroup fp32 partials are reduced in a fixed order by
+//          wgrad_reduce_parts (no atomics).
 #include <stdlib.h>
 
 #include "common.h"
