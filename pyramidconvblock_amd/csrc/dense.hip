@@ -44,17 +44,57 @@ constexpr int kNT = 4;  // feature tiles of 32 (<= 128 features)
 __device__ __forceinline__ uint32_t ld16(const bf16_t* p) { return (uint32_t) * reinterpret_cast<const unsigned short*>(p); }
 __device__ __forceinline__ uint32_t ld16(const f16_t* p) { return (uint32_t) * reinterpret_cast<const unsigned short*>(p); }
 
-// 8 values p[0], p[stride], ..., p[7*stride] (zeros where !ok) packed as a fragment.
+// 8 values p[0], p[stride], ..., p[7*stride] packed as a fragment (zeros where !ok; p must be readable
+// either way, so the 8 reads are issued back to back without a branch).
 template <typename T>
 __device__ __forceinline__ Frag gather8(const T* p, long long stride, bool ok) {
+    uint32_t e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = ld16(p + j * stride);
     Frag f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t lo = ok ? ld16(p + (2 * j) * stride) : 0u;
-        const uint32_t hi = ok ? ld16(p + (2 * j + 1) * stride) : 0u;
-        f.v[j] = lo | (hi << 16);
-    }
+    for (int j = 0; j < 4; ++j) f.v[j] = ok ? (e[2 * j] | (e[2 * j + 1] << 16)) : 0u;
     return f;
+}
+
+// Offsets out[i] = (c / per_row) * pitch + (c % per_row) * unit for c = first + i * step, i < L (-1 once
+// c / per_row >= max_rows), with one integer division instead of 2 L: a runtime division costs ~40 instructions.
+template <int L>
+__device__ __forceinline__ void strided_offsets(int first, int step, int per_row, int pitch, int unit, int max_rows,
+                                                int (&out)[L]) {
+    int r = first / per_row, c = first - r * per_row;
+    const int qr = step / per_row, qc = step - qr * per_row;  // uniform: scalar ALU
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+        out[i] = r < max_rows ? r * pitch + c * unit : -1;
+        r += qr, c += qc;
+        if (c >= per_row) c -= per_row, ++r;
+    }
+}
+
+// W[k][o] (K x NO, o fastest) -> wl[o][k] (pitch ldw): each thread moves IT groups of 4 consecutive o, consecutive
+// threads take consecutive k so the 16-bit LDS writes of a wavefront fall into consecutive banks.  All of a
+// thread's global loads are issued before the first LDS write waits for one.
+template <typename T, int IT>
+__device__ __forceinline__ void stage_w_transposed(const T* __restrict__ W, T* wl, int K, int NO, int ldw, int tid) {
+    const int nv = NO / 4;
+    int src[IT], dst[IT];  // item idx = tid + it*256: k = idx % K, o group = idx / K
+    strided_offsets<IT>(tid, 256, K, 4, NO, nv, src);        // W offset  k * NO + 4 * group
+    strided_offsets<IT>(tid, 256, K, 4 * ldw, 1, nv, dst);   // wl offset 4 * group * ldw + k
+    uint2 wv[IT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) wv[it] = *reinterpret_cast<const uint2*>(W + (src[it] >= 0 ? src[it] : 0));
+    unsigned short* wls = reinterpret_cast<unsigned short*>(wl);
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        if (dst[it] >= 0) {
+            unsigned short* q = wls + dst[it];
+            q[0] = (unsigned short)(wv[it].x & 0xffffu);
+            q[ldw] = (unsigned short)(wv[it].x >> 16);
+            q[2 * ldw] = (unsigned short)(wv[it].y & 0xffffu);
+            q[3 * ldw] = (unsigned short)(wv[it].y >> 16);
+        }
+    }
 }
 
 // Weights live in LDS as wl[NO][K + 8] (the pad keeps 16-byte fragment reads of 32 consecutive rows off
@@ -64,7 +104,7 @@ __device__ __forceinline__ Frag gather8(const T* p, long long stride, bool ok) {
 // from global memory run ~2.5x slower on this part.  The same buffer transposes the result tile so the
 // global stores are whole 128-byte lines as well.
 template <typename T>
-__global__ __launch_bounds__(256) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W, int w_kmajor,
+__global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W, int w_kmajor,
                                                     const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                     T* __restrict__ Y, long long N, int K, int NO, int P, int nkt,
                                                     int nnt) {
@@ -92,30 +132,33 @@ __global__ __launch_bounds__(256) void dense_rows_k(const T* __restrict__ X, con
         }
     };
     if (gw < ntiles) load_tile(gw);                     // requested before the weights are staged
-    if (!w_kmajor) {  // W[o][k]: 16-byte copies
+    // weight staging: all global loads of a thread are issued before the first LDS write waits for one
+    if (!w_kmajor) {  // W[o][k]: 16-byte copies (at most kKT*kNT*64/256 per thread)
         const int kv = K / 8;
-        for (int idx = tid; idx < NO * kv; idx += 256) {
-            const int n = idx / kv, k8 = (idx % kv) * 8;
-            *reinterpret_cast<Frag*>(wl + n * ldw + k8) = *reinterpret_cast<const Frag*>(W + (long long)n * K + k8);
-        }
-    } else {  // W[k][o]: read along o, write transposed
-        const int nv = NO / 4;
-        for (int idx = tid; idx < K * nv; idx += 256) {
-            const int k = idx / nv, n4 = (idx % nv) * 4;
-            const ChanVec<T, 4> v = *reinterpret_cast<const ChanVec<T, 4>*>(W + (long long)k * NO + n4);
+        constexpr int IT = kKT * kNT * 64 / 256;
+        int src[IT], dst[IT];
+        strided_offsets<IT>(tid, 256, kv, K, 8, NO, src);
+        strided_offsets<IT>(tid, 256, kv, ldw, 8, NO, dst);
+        Frag wv[IT];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) wl[(n4 + i) * ldw + k] = v.v[i];
-        }
+        for (int it = 0; it < IT; ++it) wv[it] = *reinterpret_cast<const Frag*>(W + (src[it] >= 0 ? src[it] : 0));
+#pragma unroll
+        for (int it = 0; it < IT; ++it)
+            if (dst[it] >= 0) *reinterpret_cast<Frag*>(wl + dst[it]) = wv[it];
+    } else {
+        stage_w_transposed<T, kKT * kNT * 128 / 256>(W, wl, K, NO, ldw, tid);
     }
-    __syncthreads();
     const int cpr = NO / 8;  // 16-byte chunks per output row (NO % 8 == 0 on this path)
+    constexpr int LO = 2 * kNT;  // 16-byte chunks per lane of a 32 x NO tile (NO <= 32 * kNT)
+    int oin[LP], oout[LO];   // LDS offsets of this lane's input / output chunks (the same for every tile)
+    strided_offsets<LP>(lane, 64, cpk, ldt, 8, 32, oin);
+    strided_offsets<LO>(lane, 64, cpr, ldt, 8, 32, oout);
+    __syncthreads();
     for (long long tile = gw; tile < ntiles; tile += nw) {
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
 #pragma unroll
-        for (int i = 0; i < LP; ++i) {
-            const int cidx = i * 64 + lane;
-            if (cidx < nin) *reinterpret_cast<Frag*>(tl + (cidx / cpk) * ldt + (cidx % cpk) * 8) = raw[i];
-        }
+        for (int i = 0; i < LP; ++i)
+            if (oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes have landed
         Frag xf[kKT];
 #pragma unroll
@@ -133,6 +176,12 @@ __global__ __launch_bounds__(256) void dense_rows_k(const T* __restrict__ X, con
             f32x16 acc;
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+            float4 r4[4];  // this lane's per-image terms, requested before the MFMA chain
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int n0 = nt * 32 + g4 * 8 + half * 4;
+                r4[g4] = (rb && n0 < NO) ? *reinterpret_cast<const float4*>(rb + n0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
             const int n = nt * 32 + l32;
             const T* wr = wl + (n < NO ? n : 0) * ldw + 8 * half;
 #pragma unroll
@@ -154,27 +203,31 @@ __global__ __launch_bounds__(256) void dense_rows_k(const T* __restrict__ X, con
 #pragma unroll
                         for (int i = 0; i < 4; ++i) o[i] += to_f32(bias[n0 + i]);
                     }
-                    if (rb) {
-                        const float4 r4 = *reinterpret_cast<const float4*>(rb + n0);
-                        o[0] += r4.x, o[1] += r4.y, o[2] += r4.z, o[3] += r4.w;
-                    }
+                    o[0] += r4[g4].x, o[1] += r4[g4].y, o[2] += r4[g4].z, o[3] += r4[g4].w;
                     store_f32<T, 4>(tl + l32 * ldt + n0, o);
                 }
             }
         }
         // coalesced copy-out of the 32 x NO tile (same wavefront wrote it: no workgroup barrier needed)
         __builtin_amdgcn_s_waitcnt(0xc07f);
-        const int nchunk = 32 * cpr;
-        for (int cidx = lane; cidx < nchunk; cidx += 64) {
-            const int r = cidx / cpr, cc = (cidx % cpr) * 8;
-            const long long row = tile * 32 + r;
-            if (row < N) *reinterpret_cast<Frag*>(Y + row * NO + cc) = *reinterpret_cast<const Frag*>(tl + r * ldt + cc);
+        {
+            const long long rows_left = N - tile * 32;
+            const int valid = (rows_left >= 32 ? 32 : (int)rows_left) * cpr;
+            T* yb = Y + tile * 32 * NO;
+            Frag ov[LO];
+#pragma unroll
+            for (int i = 0; i < LO; ++i) ov[i] = *reinterpret_cast<const Frag*>(tl + (oout[i] >= 0 ? oout[i] : 0));
+#pragma unroll
+            for (int i = 0; i < LO; ++i) {
+                const int cidx = i * 64 + lane;
+                if (cidx < valid) *reinterpret_cast<Frag*>(yb + (long long)cidx * 8) = ov[i];
+            }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // copy-out reads done before the next tile overwrites the buffer
     }
 }
 
-// dW partials.  A workgroup of 4 wavefronts walks its contiguous range of 64-row stages: the stage's rows
+// dW partials.  A workgroup of 4 wavefronts walks 64-row stages b, b + gridDim.x, ...: the stage's rows
 // of A and B are copied to LDS with coalesced 16-byte loads (requested one stage ahead and held in
 // registers while the current stage is multiplied), then wavefront w multiplies rows 16w..16w+15, reading
 // the k-major MFMA fragments (8 consecutive rows of one feature) from LDS with 16-bit reads.
@@ -205,9 +258,10 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A,
     constexpr int PB = (kWgRows * 16 * NT / 8 * 2 + 255) / 256;
     Frag pa[PA], pb[PB];
     const long long nstages = (N + kWgRows - 1) / kWgRows;
-    const long long st0 = (long long)blockIdx.x * stages_per_block;
-    long long st1 = st0 + stages_per_block;
-    if (st1 > nstages) st1 = nstages;
+    // workgroup b takes stages b, b + gridDim.x, ...: at any moment the chip reads one contiguous window
+    const long long st0 = blockIdx.x, sstep = gridDim.x;
+    const long long st1 = nstages;
+    (void)stages_per_block;
 
     auto fetch = [&](long long st) {
         const long long r0 = st * kWgRows;
@@ -246,9 +300,9 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A,
         commit(0);
     }
     __syncthreads();
-    for (long long st = st0; st < st1; ++st) {
-        const int buf = (int)((st - st0) & 1);
-        if (st + 1 < st1) fetch(st + 1);  // in flight while this stage is multiplied
+    int buf = 0;
+    for (long long st = st0; st < st1; st += sstep, buf ^= 1) {
+        if (st + sstep < st1) fetch(st + sstep);  // in flight while this stage is multiplied
         const T* la = lds + buf * buf_elems + (wave * 16 + 8 * half) * lda;
         const T* lb = lds + buf * buf_elems + kWgRows * lda + (wave * 16 + 8 * half) * ldb;
         Frag af[MT], bf[NT];
@@ -276,7 +330,7 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A,
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = mfma32(af[mt], bf[nt], acc[mt][nt], T());
-        if (st + 1 < st1) commit(buf ^ 1);
+        if (st + sstep < st1) commit(buf ^ 1);
         __syncthreads();
     }
     // sum the 4 waves through LDS, tile by tile; D lane map: column n = l32, row m = 8*(i/4) + 4*half + i%4
@@ -290,11 +344,16 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A,
 #pragma unroll
             for (int i = 0; i < 16; ++i) red[(wave * 16 + i) * 64 + lane] = acc[mt][nt][i];
             __syncthreads();
-            for (int idx = threadIdx.x; idx < 16 * 64; idx += 256) {
+            {   // thread -> 4 consecutive lanes' values = 4 consecutive n of one dW row
+                const int idx = threadIdx.x * 4;
                 const int i = idx >> 6, l = idx & 63;
-                const float sum = (red[idx] + red[1024 + idx]) + (red[2048 + idx] + red[3072 + idx]);
+                const float4 a = *reinterpret_cast<const float4*>(red + idx), b = *reinterpret_cast<const float4*>(red + 1024 + idx);
+                const float4 c = *reinterpret_cast<const float4*>(red + 2048 + idx), d = *reinterpret_cast<const float4*>(red + 3072 + idx);
                 const int m = mt * 32 + 8 * (i / 4) + 4 * (l >> 5) + (i % 4), n = nt * 32 + (l & 31);
-                if (m < M && n < NO) pout[(long long)m * NO + n] = sum;
+                if (m < M && n < NO)  // NO % 8 == 0: the four values are in range together
+                    *reinterpret_cast<float4*>(pout + (long long)m * NO + n) =
+                        make_float4((a.x + b.x) + (c.x + d.x), (a.y + b.y) + (c.y + d.y), (a.z + b.z) + (c.z + d.z),
+                                    (a.w + b.w) + (c.w + d.w));
             }
         }
 }
@@ -315,7 +374,7 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
         return -1;
     const int nkt = cdiv(K, 16), nnt = cdiv(NO, 32);
     const long long ntiles = (N + 31) / 32;
-    long long blocks = (ntiles + 7) / 8;  // about two row tiles per wavefront
+    long long blocks = (ntiles + 3) / 4;  // one row tile per wavefront until the cap
     const int cap = getenv("PDW_DENSE_BLOCKS") ? atoi(getenv("PDW_DENSE_BLOCKS")) : 512;
     if (blocks > cap) blocks = cap;  // persistent workgroups: the weights are staged to LDS once each
     if (blocks < 1) blocks = 1;
