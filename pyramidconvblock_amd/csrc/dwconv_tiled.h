@@ -150,12 +150,11 @@ __global__ __launch_bounds__(256) void dwconv_tiled_k(const T* __restrict__ x, c
         const bool ok0 = rok && iw0 >= 0 && iw0 < g.W;
         const bool ok1 = rok && iw0 + 1 >= 0 && iw0 + 1 < g.W;
         uint32_t out[V];
+        if constexpr (PK == 2) {
+            pack_pairs<T, V>(ld[0], ld[NL - 1], (ok0 ? 0xffffu : 0u) | (ok1 ? 0xffff0000u : 0u), out);
+        } else {
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-            if constexpr (PK == 2)
-                out[i] = (ok0 ? bits16(ld[0].v[i]) : 0u) | ((ok1 ? bits16(ld[NL - 1].v[i]) : 0u) << 16);
-            else
-                out[i] = ok0 ? __builtin_bit_cast(uint32_t, ld[0].v[i]) : 0u;
+            for (int i = 0; i < V; ++i) out[i] = ok0 ? __builtin_bit_cast(uint32_t, ld[0].v[i]) : 0u;
         }
         uint32_t* dst = xl + (r * g.CPn + u) * CS + scv * V;
         if constexpr (V % 4 == 0) {

@@ -33,7 +33,6 @@ struct WgradGeom {
     int tiles_h, tiles_w, ntiles;  // ntiles = B * tiles_h * tiles_w
     int nchunks, slices;
     int CPX, CPG;   // LDS units per staged row of x / gy
-    int ulogx, ulogg;
 };
 
 constexpr int kWgCS = 32;  // channels per workgroup slice (two strip groups per wavefront)
@@ -47,6 +46,8 @@ __global__ __launch_bounds__(256, 2) void dwconv_wgrad_tiled_k(const T* __restri
     constexpr int RU = R / PK;                     // gy units per strip
     constexpr int XU = (R + K - 1) / PK;           // x units per strip window
     constexpr int NWR = 4 / USPLIT;                // wavefronts sharing a class (split the rows)
+    constexpr int NPX = NU * K > 100 ? 3 : (NU * K > 84 ? 5 : 6);  // staging passes of the x / gy windows held in registers
+    constexpr int NPG = NU * K > 100 ? 1 : 2;      // for the next tile (fewer when the accumulators are many)
     static_assert(R % 2 == 0 && K % 2 == 1 && 4 % USPLIT == 0, "bad wgrad parameters");
     extern __shared__ uint32_t smem[];
     const int xrows = g.TH + K - 1;
@@ -68,15 +69,32 @@ __global__ __launch_bounds__(256, 2) void dwconv_wgrad_tiled_k(const T* __restri
         for (int v = 0; v < K; ++v) acc[a][v] = 0.f;
 
     const int tiles_per_img = g.tiles_h * g.tiles_w;
+    // The next tile's windows are requested while the current one is multiplied (register prefetch).
+    TileStager<T, CS, V, NPX> sx;
+    TileStager<T, CS, V, NPG> sg;
+    sx.init(tid, c0, g.C, xrows, g.CPX);
+    sg.init(tid, c0, g.C, g.TH, g.CPG);
+    auto origin = [&](int tile, int& b, int& row0, int& col0) {
+        b = tile / tiles_per_img;
+        const int rem = tile - b * tiles_per_img;
+        const int th_i = rem / g.tiles_w;
+        row0 = th_i * g.TH, col0 = (rem - th_i * g.tiles_w) * (2 * g.NSP * R);
+    };
+    auto request = [&](int tile) {
+        int b, row0, col0;
+        origin(tile, b, row0, col0);
+        sx.issue(x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
+        sg.issue(gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0);
+    };
+    if (chunk < g.ntiles) request(chunk);
     for (int tile = chunk; tile < g.ntiles; tile += g.nchunks) {
-        const int b = tile / tiles_per_img, rem = tile % tiles_per_img;
-        const int row0 = (rem / g.tiles_w) * g.TH, col0 = (rem % g.tiles_w) * (2 * g.NSP * R);
+        int b, row0, col0;
+        origin(tile, b, row0, col0);
         __syncthreads();  // previous tile fully consumed
-        stage_tile<T, CS, V, 2>(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW, xrows,
-                             g.CPX, g.ulogx, c0, tid);
-        stage_tile<T, CS, V, 2>(gl, gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0, g.TH, g.CPG,
-                             g.ulogg, c0, tid);
+        sx.commit(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
+        sg.commit(gl, gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0);
         __syncthreads();
+        if (tile + g.nchunks < g.ntiles) request(tile + g.nchunks);
         for (int r = wr; r < xrows; r += NWR) {
             for (int sp = 0; sp < g.NSP; ++sp) {
                 const int st = 2 * sp + grp;
@@ -121,23 +139,41 @@ __global__ __launch_bounds__(256, 2) void dwconv_wgrad_tiled_k(const T* __restri
     for (int a = 0; a < NU; ++a)
 #pragma unroll
         for (int v = 0; v < K; ++v) acc[a][v] += __shfl_xor(acc[a][v], 32);
-    float* red = reinterpret_cast<float*>(smem);  // [4 waves][K][CS]
+    float* red = reinterpret_cast<float*>(smem);  // [4 waves][NU][K][CS]
     float* pout = part + (long long)chunk * K * K * g.C;
+    constexpr int WSZ = NU * K * CS;  // floats per wavefront
+    __syncthreads();                  // every wavefront is done with the tile buffers
+    if (grp == 0) {
 #pragma unroll
-    for (int a = 0; a < NU; ++a) {
-        __syncthreads();
-        if (grp == 0) {
+        for (int a = 0; a < NU; ++a)
 #pragma unroll
-            for (int v = 0; v < K; ++v) red[(wv * K + v) * CS + c] = acc[a][v];
+            for (int v = 0; v < K; ++v) red[wv * WSZ + (a * K + v) * CS + c] = acc[a][v];
+    }
+    __syncthreads();
+    // element e = ((cls * NU + a) * K + v) * CS + cc, four channels per thread and pass
+    const bool vec4 = (g.C & 3) == 0;
+#pragma unroll 4
+    for (int e = tid * 4; e < USPLIT * WSZ; e += 1024) {
+        const int cls = e / WSZ, o = e - cls * WSZ;
+        const int cc = o % CS, av = o / CS;
+        const int a = av / K, v = av - a * K;
+        const int u = cls * NU + a;
+        float4 s = *reinterpret_cast<const float4*>(red + cls * WSZ + o);
+#pragma unroll
+        for (int q = 1; q < NWR; ++q) {
+            const float4 t = *reinterpret_cast<const float4*>(red + (q * USPLIT + cls) * WSZ + o);
+            s.x += t.x, s.y += t.y, s.z += t.z, s.w += t.w;
         }
-        __syncthreads();
-        for (int idx = tid; idx < USPLIT * K * CS; idx += 256) {
-            const int cc = idx % CS, v = (idx / CS) % K, cls = idx / (CS * K);
-            const int u = cls * NU + a;
-            float s = 0.f;
+        if (u < K) {
+            float* dst = pout + (u * K + v) * g.C + c0 + cc;
+            if (vec4 && c0 + cc + 3 < g.C) {
+                *reinterpret_cast<float4*>(dst) = s;
+            } else {
+                const float sv[4] = {s.x, s.y, s.z, s.w};
 #pragma unroll
-            for (int q = 0; q < NWR; ++q) s += red[((q * USPLIT + cls) * K + v) * CS + cc];
-            if (u < K && c0 + cc < g.C) pout[(u * K + v) * g.C + c0 + cc] = s;
+                for (int j = 0; j < 4; ++j)
+                    if (c0 + cc + j < g.C) dst[j] = sv[j];
+            }
         }
     }
 }
@@ -170,7 +206,8 @@ static WgradPlan plan_wgrad(int B, int H, int W, int C, int PH, int PW) {
     if (g.OH < 1 || g.OW < 1) return p;
     if ((long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL) return p;
     g.slices = cdiv(C, CS);
-    const int red_bytes = 4 * K * CS * 4;
+    constexpr int USPLIT_ = WgradCfg<T, K>::USPLIT;
+    const int red_bytes = 4 * ((K + USPLIT_ - 1) / USPLIT_) * K * CS * 4;  // the final cross-wavefront sum
     double best = -1;
     int best_nch = 1;
     for (int th = 1; th <= 32; ++th)
@@ -236,7 +273,6 @@ static int wgrad_tiled_launch_t(const void* x, const void* gy, void* dw, void* w
 #define PDW_GO(V)                                                                                                 \
     {                                                                                                             \
         auto kern = dwconv_wgrad_tiled_k<T, K, R, USPLIT, V>;                                                     \
-        g.ulogx = stage_ulog(g.CPX, kWgCS, V), g.ulogg = stage_ulog(g.CPG, kWgCS, V);                             \
         static bool attr_done = false;                                                                            \
         if (!attr_done) {                                                                                         \
             (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \

@@ -26,6 +26,26 @@ __device__ __forceinline__ float dot2acc(uint32_t a, uint32_t b, float c, f16_t)
 __device__ __forceinline__ uint32_t bits16(bf16_t v) { return (uint32_t)__builtin_bit_cast(unsigned short, v); }
 __device__ __forceinline__ uint32_t bits16(f16_t v) { return (uint32_t)__builtin_bit_cast(unsigned short, v); }
 
+// Interleaves two pixels (adjacent columns a, b; V channels each) into V dwords (low half = a's channel,
+// high half = b's), then clears the halves whose pixel lies outside the image: `mask` has 0xffff in the low
+// half if a is inside and 0xffff0000 if b is.  Two byte-permutes per channel pair instead of shifts and selects.
+template <typename T, int V>
+__device__ __forceinline__ void pack_pairs(const ChanVec<T, V>& a, const ChanVec<T, V>& b, uint32_t mask, uint32_t* out) {
+    static_assert(sizeof(T) == 2, "16-bit element types only");
+    if constexpr (V % 2 == 0) {
+        const uint32_t* aw = reinterpret_cast<const uint32_t*>(&a);
+        const uint32_t* bw = reinterpret_cast<const uint32_t*>(&b);
+#pragma unroll
+        for (int j = 0; j < V / 2; ++j) {
+            out[2 * j] = __builtin_amdgcn_perm(bw[j], aw[j], 0x05040100u) & mask;
+            out[2 * j + 1] = __builtin_amdgcn_perm(bw[j], aw[j], 0x07060302u) & mask;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) out[i] = (bits16(a.v[i]) | (bits16(b.v[i]) << 16)) & mask;
+    }
+}
+
 // XCD-aware work order: consecutive workgroup ids go to the 8 XCDs round-robin, so give each
 // XCD a contiguous range of work items (neighbouring tiles of one image share an L2).
 __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
@@ -79,12 +99,12 @@ __device__ __forceinline__ void stage_tile(uint32_t* __restrict__ xl, const T* _
                     const int ih = row0 + r;
                     const bool rok = ih >= 0 && ih < H;
                     uint32_t out[V];
+                    if constexpr (PK == 2) {
+                        const uint32_t mask = ((rok && cok[0]) ? 0xffffu : 0u) | ((rok && cok[NL - 1]) ? 0xffff0000u : 0u);
+                        pack_pairs<T, V>(ld[s][0], ld[s][NL - 1], mask, out);
+                    } else {
 #pragma unroll
-                    for (int i = 0; i < V; ++i) {
-                        if constexpr (PK == 2)
-                            out[i] = ((rok && cok[0]) ? bits16(ld[s][0].v[i]) : 0u) |
-                                     (((rok && cok[NL - 1]) ? bits16(ld[s][NL - 1].v[i]) : 0u) << 16);
-                        else
+                        for (int i = 0; i < V; ++i)
                             out[i] = (rok && cok[0]) ? __builtin_bit_cast(uint32_t, ld[s][0].v[i]) : 0u;
                     }
                     uint32_t* dst = xl + (r * CPn + u) * CS + cv * V;
@@ -101,6 +121,100 @@ __device__ __forceinline__ void stage_tile(uint32_t* __restrict__ xl, const T* _
         }
     }
 }
+
+// Software-pipelined form of stage_tile for persistent workgroups: issue() requests the first NPRE staging
+// passes of a window (clamped, always valid addresses) and keeps them in registers while the previous tile is
+// being computed; commit() packs them into LDS (zeros outside the image / channel range) and stages whatever
+// the window has beyond NPRE passes directly.  Thread t owns channel vector t % CV of unit t / CV in pass 0 and
+// advances by 256 / CV units per pass, units numbered row-major over the (rows x CPn) window.
+template <typename T, int CS, int V, int NPRE>
+struct TileStager {
+    static constexpr int PK = PackOf<T>::PK;
+    static constexpr int NL = PK;          // pixels loaded per LDS unit
+    static constexpr int CV = CS / V;      // channel vectors per unit
+    static constexpr int UPP = 256 / CV;   // units per pass of the workgroup
+    int scv, sr0, su0, step_r, step_u, CPn, rows, chc;
+    bool chok;
+    ChanVec<T, V> pre[NPRE][NL];
+
+    __device__ __forceinline__ void init(int tid, int c0, int C, int rows_, int CPn_) {
+        scv = tid % CV;
+        const int tu = tid / CV;
+        CPn = CPn_, rows = rows_;
+        sr0 = tu / CPn, su0 = tu - sr0 * CPn;
+        step_r = UPP / CPn, step_u = UPP - step_r * CPn;
+        const int ch = c0 + scv * V;
+        chok = ch < C;
+        chc = chok ? ch : 0;
+    }
+
+    __device__ __forceinline__ void issue(const T* __restrict__ img, int H, int W, int C, int row0, int col0) {
+        const T* xb = img + chc;
+        int r = sr0, u = su0;
+#pragma unroll
+        for (int it = 0; it < NPRE; ++it) {
+            const int ih = min(max(row0 + min(r, rows - 1), 0), H - 1);
+#pragma unroll
+            for (int l = 0; l < NL; ++l) {
+                const int iw = min(max(col0 + NL * u + l, 0), W - 1);
+                pre[it][l] = *reinterpret_cast<const ChanVec<T, V>*>(xb + (ih * W + iw) * C);
+            }
+            r += step_r, u += step_u;
+            if (u >= CPn) u -= CPn, ++r;
+        }
+    }
+
+    __device__ __forceinline__ void put(uint32_t* __restrict__ xl, const ChanVec<T, V>* ld, int r, int u, int H, int W,
+                                        int row0, int col0) const {
+        const int ih = row0 + r;
+        const bool rok = chok && ih >= 0 && ih < H;
+        const int iw0 = col0 + NL * u;
+        const bool ok0 = rok && iw0 >= 0 && iw0 < W;
+        const bool ok1 = rok && iw0 + 1 >= 0 && iw0 + 1 < W;
+        uint32_t out[V];
+        if constexpr (PK == 2) {
+            pack_pairs<T, V>(ld[0], ld[NL - 1], (ok0 ? 0xffffu : 0u) | (ok1 ? 0xffff0000u : 0u), out);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) out[i] = ok0 ? __builtin_bit_cast(uint32_t, ld[0].v[i]) : 0u;
+        }
+        uint32_t* dst = xl + (r * CPn + u) * CS + scv * V;
+        if constexpr (V % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < V; i += 4)
+                *reinterpret_cast<uint4*>(dst + i) = make_uint4(out[i], out[i + 1], out[i + 2], out[i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) dst[i] = out[i];
+        }
+    }
+
+    __device__ __forceinline__ void commit(uint32_t* __restrict__ xl, const T* __restrict__ img, int H, int W, int C,
+                                           int row0, int col0) {
+        int r = sr0, u = su0;
+#pragma unroll
+        for (int it = 0; it < NPRE; ++it) {
+            if (r < rows) put(xl, pre[it], r, u, H, W, row0, col0);
+            r += step_r, u += step_u;
+            if (u >= CPn) u -= CPn, ++r;
+        }
+        if (NPRE * UPP < rows * CPn) {  // window larger than the prefetch depth (uniform branch)
+            const T* xb = img + chc;
+            while (r < rows) {
+                ChanVec<T, V> ld[NL];
+                const int ih = min(max(row0 + r, 0), H - 1);
+#pragma unroll
+                for (int l = 0; l < NL; ++l) {
+                    const int iw = min(max(col0 + NL * u + l, 0), W - 1);
+                    ld[l] = *reinterpret_cast<const ChanVec<T, V>*>(xb + (ih * W + iw) * C);
+                }
+                put(xl, ld, r, u, H, W, row0, col0);
+                r += step_r, u += step_u;
+                if (u >= CPn) u -= CPn, ++r;
+            }
+        }
+    }
+};
 
 // Number of persistent workgroups per channel slice for `ntiles` equal tiles, all resident at once
 // (at most `max_resident` per CU over 256 CUs): minimises the estimated makespan
