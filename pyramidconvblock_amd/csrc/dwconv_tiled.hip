@@ -1,6 +1,8 @@
 // Dispatch of the LDS-tiled depthwise convolution (stride 1, dilation 1) by filter width.
 // The kernel template and its description live in dwconv_tiled.h; each width is instantiated
 // in its own translation unit (dwconv_tiled_kw*.hip).
+#include <stdlib.h>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -23,12 +25,31 @@ int dwconv_tiled_kw15(const void* x, const void* w, void* y, int B, int H, int W
 int dwconv_tiled_kw17(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
                       bool flip, int dtype, hipStream_t s);
 
+int dwconv_mfma_k13(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+
+// Matrix-core kernel for square filters and 16-bit types; -1 when it does not cover the case.
+static int dwconv_mfma_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
+                              int PW, bool flip, int dtype, hipStream_t s) {
+    if (KH != KW || dtype == kF32) return -1;
+    const char* e = getenv("PDW_MFMA");
+    if (e && atoi(e) == 0) return -1;
+    switch (KW) {
+        case 13: return dwconv_mfma_k13(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        default: return -1;
+    }
+}
+
 // Returns -1 when the tiled kernel does not cover the case (the caller then uses the direct
 // kernel), otherwise the launch status.  With flip the 180-degree rotated filter is used: the
 // caller passes gy as x with padding k-1-p, which yields the input gradient.
 int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
                         int PW, bool flip, int dtype, hipStream_t s) {
     if (KH > 31 || H + 2 * PH - KH + 1 < 1 || W + 2 * PW - KW + 1 < 1) return -1;
+    {
+        const int r = dwconv_mfma_launch(x, w, y, B, H, W, C, KH, KW, PH, PW, flip, dtype, s);
+        if (r != -1) return r;
+    }
     switch (KW) {
         case 3: return dwconv_tiled_kw3(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
         case 5: return dwconv_tiled_kw5(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);

@@ -127,20 +127,22 @@ __device__ __forceinline__ void stage_tile(uint32_t* __restrict__ xl, const T* _
 // being computed; commit() packs them into LDS (zeros outside the image / channel range) and stages whatever
 // the window has beyond NPRE passes directly.  Thread t owns channel vector t % CV of unit t / CV in pass 0 and
 // advances by 256 / CV units per pass, units numbered row-major over the (rows x CPn) window.
-template <typename T, int CS, int V, int NPRE>
+// LDS layout: xl[row][unit][CS] (channel fastest), or with CHMAJOR xl[row][channel][pitch] (unit fastest,
+// `pitch` >= CPn dwords per channel row), the operand order of the matrix-core kernels.
+template <typename T, int CS, int V, int NPRE, bool CHMAJOR = false>
 struct TileStager {
     static constexpr int PK = PackOf<T>::PK;
     static constexpr int NL = PK;          // pixels loaded per LDS unit
     static constexpr int CV = CS / V;      // channel vectors per unit
     static constexpr int UPP = 256 / CV;   // units per pass of the workgroup
-    int scv, sr0, su0, step_r, step_u, CPn, rows, chc;
+    int scv, sr0, su0, step_r, step_u, CPn, rows, chc, pitch;
     bool chok;
     ChanVec<T, V> pre[NPRE][NL];
 
-    __device__ __forceinline__ void init(int tid, int c0, int C, int rows_, int CPn_) {
+    __device__ __forceinline__ void init(int tid, int c0, int C, int rows_, int CPn_, int pitch_ = 0) {
         scv = tid % CV;
         const int tu = tid / CV;
-        CPn = CPn_, rows = rows_;
+        CPn = CPn_, rows = rows_, pitch = pitch_;
         sr0 = tu / CPn, su0 = tu - sr0 * CPn;
         step_r = UPP / CPn, step_u = UPP - step_r * CPn;
         const int ch = c0 + scv * V;
@@ -178,14 +180,20 @@ struct TileStager {
 #pragma unroll
             for (int i = 0; i < V; ++i) out[i] = ok0 ? __builtin_bit_cast(uint32_t, ld[0].v[i]) : 0u;
         }
-        uint32_t* dst = xl + (r * CPn + u) * CS + scv * V;
-        if constexpr (V % 4 == 0) {
+        if constexpr (CHMAJOR) {
+            uint32_t* dst = xl + (r * CS + scv * V) * pitch + u;
 #pragma unroll
-            for (int i = 0; i < V; i += 4)
-                *reinterpret_cast<uint4*>(dst + i) = make_uint4(out[i], out[i + 1], out[i + 2], out[i + 3]);
+            for (int i = 0; i < V; ++i) dst[i * pitch] = out[i];
         } else {
+            uint32_t* dst = xl + (r * CPn + u) * CS + scv * V;
+            if constexpr (V % 4 == 0) {
 #pragma unroll
-            for (int i = 0; i < V; ++i) dst[i] = out[i];
+                for (int i = 0; i < V; i += 4)
+                    *reinterpret_cast<uint4*>(dst + i) = make_uint4(out[i], out[i + 1], out[i + 2], out[i + 3]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) dst[i] = out[i];
+            }
         }
     }
 
