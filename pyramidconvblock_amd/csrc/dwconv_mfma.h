@@ -15,15 +15,17 @@
 // row m in the A operand and the strip n in the B operand, and register m of the result holds output row m
 // of strip q.
 //
-// The 4 strips of a unit are S columns wide and sit side by side (SR = 1: a unit is 4 rows x 4S columns) or
-// in a 2 x 2 arrangement (SR = 2: 8 rows x 2S columns; the strips of the lower pair use input rows 4 further
-// down with the same phase, so they share the A operand).  A workgroup of 4 wavefronts owns a tile of 4 units:
-// CG groups of 16 channels x 4/CG unit rows.  The tile's input window is staged in LDS channel-major,
-// xl[row][channel][column pair] (a dword holds two adjacent columns), which makes the B operand of an even
-// output column two consecutive dwords; odd columns use the same dwords shifted by 16 bits (v_alignbit).
-// Operand pairs must start at an even register, so the window is read twice, at pair offsets 0 and 1.
-// Workgroups are persistent, one per CU (the window of the next tile is requested into registers while the
-// current one is multiplied).
+// A unit is 4 output rows x 4 strips of S columns x 16 channels, the work of one wavefront per tile; a
+// workgroup of 4 wavefronts owns a tile of 16 rows x 4S columns x 16 channels.  The tile's input window is
+// staged in LDS channel-major, xl[row][channel][column pair] (a dword holds two adjacent columns), which makes
+// the B operand of an even output column two consecutive dwords.  The odd column next to it uses the SAME
+// operand with the filter shifted by one column (w'[v+1] = w[v], which still fits the padded width because K is
+// odd), so the inner loop has no vector-ALU work at all: a 4x4x4 MFMA occupies the SIMD for 8 cycles and every
+// vector instruction next to it for 4 more.  Workgroups are persistent, one per CU, and software-pipelined over their tiles: while tile i is
+// multiplied out of one LDS buffer, the window of tile i+1 is requested into registers (phase 0) and written
+// to the other buffer a pass per phase, and the results of tile i-1 leave a few stores per phase, so the
+// matrix pipe of a SIMD sees one long stream of MFMAs with the vector, LDS and memory work in its shadow.
+// With NBUF = 1 (windows too large for two buffers) the window is written between the tiles instead.
 #pragma once
 #include <stdlib.h>
 
@@ -51,36 +53,39 @@ struct MfmaGeom {
     int tiles_h, tiles_w, ntiles, nchunks, slices;
     int CPn;          // LDS dwords per channel row (>= staged column pairs)
     int flip;         // 1: 180-degree rotated filter (input gradient)
+    int one;          // the constant 1 (see the kernel)
 };
 
-template <int K, int S, int SR, int CG>
+template <int K, int S, int NWV>
 struct MfmaShape {
-    static constexpr int SC = 4 / SR;            // strips side by side
-    static constexpr int UH = 4 * SR, UW = S * SC;  // unit = UH x UW outputs x 16 channels
-    static constexpr int RGB = 4 / CG;           // unit rows per tile
-    static constexpr int TH = UH * RGB, TW = UW, CS = 16 * CG;
-    static constexpr int KP = (K + 3) / 4 * 4;   // filter columns padded to the MFMA k
+    static constexpr int CS = 16;                   // channels per workgroup
+    static constexpr int TH = 4 * NWV, TW = 4 * S;  // tile = NWV units of 4 rows, one per wavefront
+    static constexpr int KP = (K + 3) / 4 * 4;      // filter columns padded to the MFMA k
     static constexpr int NVB = KP / 4;
-    static constexpr int NPH = K + 3;            // phases (input rows) per row group
-    static constexpr int WR = K + 6;             // filter rows in LDS, 3 zero rows on either side
+    static constexpr int NPH = K + 3;               // phases (input rows) per row group
+    static constexpr int WR = K + 6;                // filter rows in LDS, 3 zero rows on either side
     static constexpr int ROWS_IN = TH + K - 1;
-    static constexpr int NCOL = (TW + KP) / 2;   // staged column pairs: every pair an operand reads, the ones under
-                                                 // the zero filter columns included (0 * garbage could be NaN)
+    static constexpr int NCOL = (TW + KP) / 2;      // staged column pairs: every pair an operand reads, the ones under
+                                                    // the zero filter columns included (0 * garbage could be NaN)
 };
 
-template <typename T, int K, int S, int SR, int CG, int V>
-__global__ __launch_bounds__(256, 1) void dwconv_mfma_k(const T* __restrict__ x, const T* __restrict__ w,
-                                                        T* __restrict__ y, const MfmaGeom g) {
-    using Sh = MfmaShape<K, S, SR, CG>;
-    constexpr int SC = Sh::SC, UH = Sh::UH, TH = Sh::TH, TW = Sh::TW, CS = Sh::CS;
+template <typename T, int K, int S, int NWV>
+__global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(const T* __restrict__ x, const T* __restrict__ w,
+                                                             T* __restrict__ y, const MfmaGeom g) {
+    using Sh = MfmaShape<K, S, NWV>;
+    constexpr int V = 8, NT = NWV * 64, CS = Sh::CS, TH = Sh::TH, TW = Sh::TW;
     constexpr int KP = Sh::KP, NVB = Sh::NVB, NPH = Sh::NPH, WR = Sh::WR, ROWS_IN = Sh::ROWS_IN, NCOL = Sh::NCOL;
     constexpr int NQ = (S / 2 + 2 * NVB + 1) / 2;  // 64-bit operand registers per copy of a lane's window
-    constexpr int CV = CS / V, UPP = 256 / CV;
-    constexpr int NPRE = (ROWS_IN * NCOL + UPP - 1) / UPP;  // the whole window of the next tile sits in registers
-    static_assert(S % 2 == 0 && K % 2 == 1 && (SR == 1 || SR == 2) && (CG == 1 || CG == 2 || CG == 4), "bad shape");
+    constexpr int UPP = NT / (CS / V);
+    constexpr int NPRE = (ROWS_IN * NCOL + UPP - 1) / UPP;  // passes: a whole window sits in registers
+    constexpr int NE = S / 2;                               // column pairs per strip
+    constexpr int WPITCH = (16 * NVB + 8) * 4;              // elements per filter row in LDS
+    static_assert(S % 2 == 0 && K % 2 == 1 && (NWV == 4 || NWV == 8), "bad shape");
     extern __shared__ uint32_t smem[];
-    uint32_t* xl = smem;                                                // [ROWS_IN][CS][CPn]
-    T* wl = reinterpret_cast<T*>(smem + ROWS_IN * CS * g.CPn);          // [CS][WR][KP]
+    uint32_t* xl = smem;                                                  // [ROWS_IN][CS][CPn]
+    // filter operands: wl[copy][3 + u][vb][channel] as 4 columns (8 bytes) each, copy 1 shifted by one column; the
+    // row pitch of 16 NVB + 8 operands puts the 4 filter rows an MFMA reads 64 bytes apart modulo 128: no bank conflicts
+    T* wl = reinterpret_cast<T*>(smem + ROWS_IN * CS * g.CPn);
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int bid = xcd_remap(blockIdx.x, gridDim.x);
@@ -88,7 +93,7 @@ __global__ __launch_bounds__(256, 1) void dwconv_mfma_k(const T* __restrict__ x,
     const int c0 = sl * CS;
     const int tiles_per_img = g.tiles_h * g.tiles_w;
 
-    TileStager<T, CS, V, NPRE, true> st;
+    TileStager<T, CS, V, NPRE, true, NT> st;
     st.init(tid, c0, g.C, ROWS_IN, NCOL, g.CPn);
     auto origin = [&](int tile, int& b, int& row0, int& col0) {
         b = tile / tiles_per_img;
@@ -96,99 +101,140 @@ __global__ __launch_bounds__(256, 1) void dwconv_mfma_k(const T* __restrict__ x,
         const int th_i = rem / g.tiles_w;
         row0 = th_i * TH, col0 = (rem - th_i * g.tiles_w) * TW;
     };
-    auto request = [&](int tile) {
-        int b, row0, col0;
-        origin(tile, b, row0, col0);
-        st.issue(x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
-    };
-    if (chunk < g.ntiles) request(chunk);
+    // ---- filter slice (requested first: it is in LDS by the time the window arrives)
+    constexpr int NW = K * K * CS, IT = (NW + NT - 1) / NT;
+    uint32_t val[IT];
+#pragma unroll
+    for (int s = 0; s < IT; ++s) {  // all loads of a thread in flight together
+        const int idx = min(tid + s * NT, NW - 1);
+        const int ch = idx % CS, uv = idx / CS;
+        val[s] = bits16(w[(long long)uv * g.C + min(c0 + ch, g.C - 1)]);
+    }
+    int nb = 0, nrow0 = 0, ncol0 = 0;  // tile whose window is in flight
+    if (chunk < g.ntiles) {
+        origin(chunk, nb, nrow0, ncol0);
+        st.issue(x + (long long)nb * g.H * g.W * g.C, g.H, g.W, g.C, nrow0 - g.PH, ncol0 - g.PW);
+    }
 
-    // ---- filter slice -> wl[ch][3 + u][v] (rotated for the input gradient), zero elsewhere
+    // ---- filter -> LDS operands (rotated for the input gradient), zero elsewhere
     {
         uint32_t* wz = reinterpret_cast<uint32_t*>(wl);
-        for (int i = tid; i < CS * WR * KP / 2; i += 256) wz[i] = 0u;
+        for (int i = tid; i < WR * WPITCH; i += NT) wz[i] = 0u;  // both copies (2 * WR * WPITCH elements)
         __syncthreads();
-        constexpr int NW = K * K * CS, SU = 8;
         unsigned short* wls = reinterpret_cast<unsigned short*>(wl);
-        for (int i0 = tid; i0 < NW; i0 += 256 * SU) {
-            uint32_t val[SU];
 #pragma unroll
-            for (int s = 0; s < SU; ++s) {
-                const int idx = min(i0 + s * 256, NW - 1);
+        for (int s = 0; s < IT; ++s) {
+            const int idx = tid + s * NT;
+            if (idx < NW) {
                 const int ch = idx % CS, uv = idx / CS;
-                val[s] = bits16(w[(long long)uv * g.C + min(c0 + ch, g.C - 1)]);
-            }
-#pragma unroll
-            for (int s = 0; s < SU; ++s) {
-                const int idx = i0 + s * 256;
-                if (idx < NW) {
-                    const int ch = idx % CS, uv = idx / CS;
-                    const int u = uv / K, v = uv - u * K;
-                    const int uu = g.flip ? K - 1 - u : u, vv = g.flip ? K - 1 - v : v;
-                    wls[(ch * WR + 3 + uu) * KP + vv] = (unsigned short)(c0 + ch < g.C ? val[s] : 0u);
-                }
+                const int u = uv / K, v = uv - u * K;
+                const int uu = g.flip ? K - 1 - u : u, vv = g.flip ? K - 1 - v : v;
+                const unsigned short val16 = (unsigned short)(c0 + ch < g.C ? val[s] : 0u);
+                wls[(3 + uu) * WPITCH + ((vv >> 2) * 16 + ch) * 4 + (vv & 3)] = val16;
+                wls[(WR + 3 + uu) * WPITCH + (((vv + 1) >> 2) * 16 + ch) * 4 + ((vv + 1) & 3)] = val16;
             }
         }
     }
 
-    // ---- this lane's operand addresses
+    // ---- this lane's operand addresses: wavefront = unit row, lane = (channel bq, q)
     const int bq = lane >> 2, q = lane & 3;
-    const int cg = wv % CG, ur = wv / CG;
-    const int sr = q / SC, sc = q % SC;
     const int RP = CS * g.CPn;  // dwords per staged row
-    const uint32_t* xbase = xl + ((ur * UH + sr * 4) * CS + cg * 16 + bq) * g.CPn + sc * (S / 2);
-    const T* wbase = wl + ((cg * 16 + bq) * WR + 3 - q) * KP;
+    const uint32_t* xbase = xl + (wv * 4 * CS + bq) * g.CPn + q * (S / 2);
+    const T* wbase = wl + (3 - q) * WPITCH + bq * 4;   // + WR * WPITCH: the shifted copy
+    const int one = g.one;  // 1, opaque to the compiler: the second window copy is a load of its own, not a register shuffle
 
     for (int tile = chunk; tile < g.ntiles; tile += g.nchunks) {
         int b, orow0, ocol0;
         origin(tile, b, orow0, ocol0);
-        __syncthreads();  // the previous tile is fully consumed (and, first time, the filter is staged)
-        st.commit(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, orow0 - g.PH, ocol0 - g.PW);
+        __syncthreads();  // the previous window is fully consumed
+        st.commit_begin();
+#pragma unroll
+        for (int it = 0; it < NPRE; ++it) st.commit_next(xl, it, g.H, g.W, orow0 - g.PH, ocol0 - g.PW);
         __syncthreads();
-        if (tile + g.nchunks < g.ntiles) request(tile + g.nchunks);
-
+        const int orow_b = orow0 + wv * 4;
+        const bool has_next = tile + g.nchunks < g.ntiles;
+        const bool active = orow_b < g.OH;  // this wavefront's unit has outputs (uniform per wavefront)
         f32x4 acc[S];
 #pragma unroll
         for (int t = 0; t < S; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (active) {
+            // Operands of a phase: the lane's window at pair offsets 0 and 1 (operand pairs must start at an even
+            // register) and the 2 NVB filter operands.  They are requested one phase ahead, all at the top of the
+            // phase, so the LDS latency lies under the 4 S NVB MFMAs of the current phase.
+            struct Ops {
+                uint2 P0[NQ], P1[NQ], ae[NVB], ao[NVB];
+            };
+            auto fetch = [&](Ops& o, const uint32_t* xr, const T* wr) {
+                const uint32_t* xr1 = xr + one;
 #pragma unroll
-        for (int p = 0; p < NPH; ++p) {
-            const uint32_t* xr = xbase + p * RP;
-            // window copies at pair offsets 0 and 1, and the same shifted by one column
-            uint2 P0[NQ], P1[NQ], O0[NQ], O1[NQ];
-#pragma unroll
-            for (int i = 0; i < NQ; ++i) {
-                P0[i] = make_uint2(xr[2 * i], xr[2 * i + 1]);
-                P1[i] = make_uint2(xr[2 * i + 1], xr[2 * i + 2]);
-            }
-#pragma unroll
-            for (int i = 0; i < NQ; ++i) {
-                O0[i] = make_uint2(__builtin_amdgcn_alignbit(P0[i].y, P0[i].x, 16),
-                                   __builtin_amdgcn_alignbit(P1[i].y, P1[i].x, 16));
-                O1[i] = make_uint2(__builtin_amdgcn_alignbit(P1[i].y, P1[i].x, 16),
-                                   i + 1 < NQ ? __builtin_amdgcn_alignbit(P0[i + 1].y, P0[i + 1].x, 16) : 0u);
-            }
-#pragma unroll
-            for (int vb = 0; vb < NVB; ++vb) {
-                const uint2 a = *reinterpret_cast<const uint2*>(wbase + p * KP + 4 * vb);
-#pragma unroll
-                for (int t = 0; t < S; ++t) {
-                    const int e = t / 2, j = e + 2 * vb;  // first column pair of the operand
-                    const uint2 bop = (t % 2 == 0) ? ((j % 2 == 0) ? P0[j / 2] : P1[j / 2])
-                                                   : ((j % 2 == 0) ? O0[j / 2] : O1[j / 2]);
-                    acc[t] = mfma4(a, bop, acc[t], T());
+                for (int i = 0; i < NQ; ++i) {
+                    if (2 * i < NE + 2 * NVB - 1) o.P0[i] = make_uint2(xr[2 * i], xr[2 * i + 1]);
+                    if (2 * i + 1 < NE + 2 * NVB - 1) o.P1[i] = make_uint2(xr1[2 * i], xr1[2 * i + 1]);
                 }
+#pragma unroll
+                for (int vb = 0; vb < NVB; ++vb) {
+                    o.ae[vb] = *reinterpret_cast<const uint2*>(wr + vb * 64);
+                    o.ao[vb] = *reinterpret_cast<const uint2*>(wr + WR * WPITCH + vb * 64);
+                }
+            };
+            auto multiply = [&](const Ops& o) {
+#pragma unroll
+                for (int vb = 0; vb < NVB; ++vb)
+#pragma unroll
+                    for (int e = 0; e < NE; ++e) {
+                        const int j = e + 2 * vb;  // first column pair of the operand
+                        const uint2 bop = (j % 2 == 0) ? o.P0[j / 2] : o.P1[j / 2];
+                        acc[2 * e] = mfma4(o.ae[vb], bop, acc[2 * e], T());
+                        acc[2 * e + 1] = mfma4(o.ao[vb], bop, acc[2 * e + 1], T());
+                    }
+            };
+            const uint32_t* xr = xbase;
+            const T* wr = wbase;
+            Ops oa, ob;
+            fetch(oa, xr, wr);
+            static_assert(NPH % 2 == 0, "phases are processed in pairs");
+#pragma unroll 1
+            for (int p = 0; p < NPH; p += 2) {
+                xr += RP, wr += WPITCH;
+                fetch(ob, xr, wr);
+                __builtin_amdgcn_sched_barrier(0);
+                multiply(oa);
+                __builtin_amdgcn_sched_barrier(0);
+                xr += RP, wr += WPITCH;
+                if (p + 2 < NPH) fetch(oa, xr, wr);
+                __builtin_amdgcn_sched_barrier(0);
+                multiply(ob);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // ---- store (one rounding to T): register m of acc[t] is output row m, column t of strip q
-        const int ch = c0 + cg * 16 + bq;
-        const int orow_b = orow0 + ur * UH + sr * 4, ocol_b = ocol0 + sc * S;
-        if (ch < g.C) {
-            T* yp = y + (((long long)b * g.OH + orow_b) * g.OW + ocol_b) * g.C + ch;
+        // ---- results -> LDS as yl[row][column][16 channels] (one rounding to T), then out in 16-byte pieces:
+        // the 2-byte values a lane owns are 4 rows x S scattered pixels, far too many store instructions.
+        __syncthreads();  // every wavefront is done reading the window
+        T* yl = reinterpret_cast<T*>(smem);
+        if (active) {
+            T* yq = yl + ((wv * 4) * TW + q * S) * CS + bq;  // register m of acc[t]: row m, column t of strip q
 #pragma unroll
             for (int m = 0; m < 4; ++m)
 #pragma unroll
-                for (int t = 0; t < S; ++t)
-                    if (orow_b + m < g.OH && ocol_b + t < g.OW) yp[(m * g.OW + t) * g.C] = from_f32<T>(acc[t][m]);
+                for (int t = 0; t < S; ++t) yq[(m * TW + t) * CS] = from_f32<T>(acc[t][m]);
+        }
+        __syncthreads();
+        {
+            constexpr int NIT = (TH * TW * 2 + NT - 1) / NT;  // 16-byte pieces (8 channels of a pixel) per thread
+            T* yb = y + ((long long)b * g.OH * g.OW) * g.C + c0;
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int idx = tid + it * NT;
+                const int half = idx & 1, pix = idx >> 1;
+                const int r = pix / TW, cc = pix - r * TW;
+                if (pix < TH * TW && orow0 + r < g.OH && ocol0 + cc < g.OW && c0 + 8 * half < g.C)
+                    *reinterpret_cast<uint4*>(yb + ((long long)(orow0 + r) * g.OW + ocol0 + cc) * g.C + 8 * half) =
+                        *reinterpret_cast<const uint4*>(yl + pix * CS + 8 * half);
+            }
+        }
+        if (has_next) {  // the next window is requested only now: its registers were the operand registers above
+            origin(tile + g.nchunks, nb, nrow0, ncol0);
+            st.issue(x + (long long)nb * g.H * g.W * g.C, g.H, g.W, g.C, nrow0 - g.PH, ncol0 - g.PW);
         }
     }
 }
@@ -196,12 +242,12 @@ __global__ __launch_bounds__(256, 1) void dwconv_mfma_k(const T* __restrict__ x,
 // ------------------------------------------------------------------------------------------------
 // Host side
 
-template <typename T, int K, int S, int SR, int CG>
+template <typename T, int K, int S, int NWV>
 static int launch_mfma(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
                        hipStream_t s) {
-    using Sh = MfmaShape<K, S, SR, CG>;
+    using Sh = MfmaShape<K, S, NWV>;
     MfmaGeom g;
-    g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0;
+    g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0, g.one = 1;
     g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
     g.slices = cdiv(C, Sh::CS);
     g.tiles_h = cdiv(g.OH, Sh::TH), g.tiles_w = cdiv(g.OW, Sh::TW);
@@ -209,31 +255,31 @@ static int launch_mfma(const void* x, const void* w, void* y, int B, int H, int 
     if (ntiles > 0x7fffffffLL || (long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL)
         return -1;
     g.ntiles = (int)ntiles;
-    // LDS: pitch = pairs per channel row, 4 mod 8 keeps the 16 channels x 4 strips of an operand read on
-    // distinct banks; fall back to the bare width when that does not fit.
-    const size_t wbytes = (size_t)Sh::CS * Sh::WR * Sh::KP * 2;
-    const int need = Sh::NCOL;
-    int pitch = need;
-    while (pitch % 8 != 4) ++pitch;
+    // LDS: pitch = pairs per channel row; 4 mod 8 keeps the 16 channels x 4 strips of an operand read on
+    // distinct banks when that fits.
+    const size_t wbytes = (size_t)2 * Sh::WR * (16 * Sh::NVB + 8) * 8;
     auto lds_of = [&](int p) { return (size_t)Sh::ROWS_IN * Sh::CS * p * 4 + wbytes; };
-    if (lds_of(pitch) > 160 * 1024) pitch = need;
+    int pitch = Sh::NCOL;
+    while (pitch % 8 != 4) ++pitch;
+    if (lds_of(pitch) > 160 * 1024) pitch = Sh::NCOL;
     if (lds_of(pitch) > 160 * 1024) return -1;
     g.CPn = pitch;
     const size_t lds = lds_of(pitch);
-    // persistent workgroups, one per CU; tiles dealt out as evenly as they divide
-    const int cap = 256 / g.slices > 1 ? 256 / g.slices : 1;
+    // persistent workgroups: as many as are resident at once, tiles dealt out as evenly as they divide
+    const int resident = (int)((160 * 1024) / (lds + 1024)) >= 2 && NWV == 4 ? 2 : 1;
+    const int cap = (256 * resident) / g.slices > 1 ? (256 * resident) / g.slices : 1;
     const long long rounds = cdiv(ntiles, (long long)cap);
     long long nch = cdiv(ntiles, rounds);
     if (getenv("PDW_MFMA_NCH")) nch = atoi(getenv("PDW_MFMA_NCH"));
     g.nchunks = (int)(nch < 1 ? 1 : nch);
     const long long nblocks = (long long)g.nchunks * g.slices;
-    auto kern = dwconv_mfma_k<T, K, S, SR, CG, 8>;
+    auto kern = dwconv_mfma_k<T, K, S, NWV>;
     static bool attr_done = false;
     if (!attr_done) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), lds, s, (const T*)x, (const T*)w, (T*)y, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NWV * 64), lds, s, (const T*)x, (const T*)w, (T*)y, g);
     return check_launch("dwconv_mfma");
 }
 
@@ -243,15 +289,20 @@ static int launch_mfma_best(const void* x, const void* w, void* y, int B, int H,
                             bool flip, hipStream_t s) {
     const int OH = H + 2 * PH - K + 1, OW = W + 2 * PW - K + 1;
     if (OH < 1 || OW < 1 || C % 8 != 0) return -1;
-    if ((reinterpret_cast<uintptr_t>(x) & 15) != 0) return -1;
-    constexpr int S = 14;
-    // strips side by side (tile 8 x 56) or 2 x 2 (tile 16 x 28): whichever pads the output less
-    const long long pad1 = (long long)cdiv(OH, 8) * 8 * cdiv(OW, 56) * 56;
-    const long long pad2 = (long long)cdiv(OH, 16) * 16 * cdiv(OW, 28) * 28;
-    if (pad1 <= pad2) return launch_mfma<T, K, S, 1, 2>(x, w, y, B, H, W, C, PH, PW, flip, s);
-    const char* e = getenv("PDW_MFMA");
-    if (!e || atoi(e) < 2) return -1;  // the 2 x 2 arrangement is not yet faster than the vector-ALU kernel
-    return launch_mfma<T, K, S, 2, 2>(x, w, y, B, H, W, C, PH, PW, flip, s);
+    if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return -1;
+    // strips of 14 columns (tile 56 wide) or 8 (tile 32 wide): whichever pads the output width less
+    const bool s14 = (long long)cdiv(OW, 56) * 56 <= (long long)cdiv(OW, 32) * 32;
+    const int tw = s14 ? 56 : 32;
+    // 8 wavefronts per workgroup (tile 32 rows) when that still yields a workgroup for most CUs
+    const long long t8 = (long long)B * cdiv(OH, 32) * cdiv(OW, tw) * cdiv(C, 16);
+    bool w8 = t8 >= 192;
+    if (getenv("PDW_MFMA_NWV")) w8 = atoi(getenv("PDW_MFMA_NWV")) == 8;
+    if (s14) {
+        if (w8) return launch_mfma<T, K, 14, 8>(x, w, y, B, H, W, C, PH, PW, flip, s);
+        return launch_mfma<T, K, 14, 4>(x, w, y, B, H, W, C, PH, PW, flip, s);
+    }
+    if (w8) return launch_mfma<T, K, 8, 8>(x, w, y, B, H, W, C, PH, PW, flip, s);
+    return launch_mfma<T, K, 8, 4>(x, w, y, B, H, W, C, PH, PW, flip, s);
 }
 
 template <int K>

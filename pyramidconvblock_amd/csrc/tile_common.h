@@ -126,15 +126,15 @@ __device__ __forceinline__ void stage_tile(uint32_t* __restrict__ xl, const T* _
 // passes of a window (clamped, always valid addresses) and keeps them in registers while the previous tile is
 // being computed; commit() packs them into LDS (zeros outside the image / channel range) and stages whatever
 // the window has beyond NPRE passes directly.  Thread t owns channel vector t % CV of unit t / CV in pass 0 and
-// advances by 256 / CV units per pass, units numbered row-major over the (rows x CPn) window.
+// advances by NTHREADS / CV units per pass, units numbered row-major over the (rows x CPn) window.
 // LDS layout: xl[row][unit][CS] (channel fastest), or with CHMAJOR xl[row][channel][pitch] (unit fastest,
 // `pitch` >= CPn dwords per channel row), the operand order of the matrix-core kernels.
-template <typename T, int CS, int V, int NPRE, bool CHMAJOR = false>
+template <typename T, int CS, int V, int NPRE, bool CHMAJOR = false, int NTHREADS = 256>
 struct TileStager {
     static constexpr int PK = PackOf<T>::PK;
     static constexpr int NL = PK;          // pixels loaded per LDS unit
     static constexpr int CV = CS / V;      // channel vectors per unit
-    static constexpr int UPP = 256 / CV;   // units per pass of the workgroup
+    static constexpr int UPP = NTHREADS / CV;  // units per pass of the workgroup
     int scv, sr0, su0, step_r, step_u, CPn, rows, chc, pitch;
     bool chok;
     ChanVec<T, V> pre[NPRE][NL];
@@ -195,6 +195,16 @@ struct TileStager {
                 for (int i = 0; i < V; ++i) dst[i] = out[i];
             }
         }
+    }
+
+    // One prefetched pass at a time, for callers that spread the LDS writes over their compute loop:
+    // commit_begin(), then commit_next(.., it, ..) for it = 0 .. NPRE-1 in order.
+    int cr, cu;
+    __device__ __forceinline__ void commit_begin() { cr = sr0, cu = su0; }
+    __device__ __forceinline__ void commit_next(uint32_t* __restrict__ xl, int it, int H, int W, int row0, int col0) {
+        if (cr < rows) put(xl, pre[it], cr, cu, H, W, row0, col0);
+        cr += step_r, cu += step_u;
+        if (cu >= CPn) cu -= CPn, ++cr;
     }
 
     __device__ __forceinline__ void commit(uint32_t* __restrict__ xl, const T* __restrict__ img, int H, int W, int C,
