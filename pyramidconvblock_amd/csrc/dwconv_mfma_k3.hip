@@ -1,0 +1,13 @@
+// Matrix-core depthwise convolution (forward / input gradient), 3x3 filter: the instantiations of
+// the kernel template in dwconv_mfma.h for this size, one translation unit per size so the build
+// compiles them in parallel.
+#include "dwconv_mfma.h"
+
+namespace pdw {
+
+int dwconv_mfma_k3(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s) {
+    return launch_mfma_dtype<3>(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+}
+
+}  // namespace pdw

@@ -25,7 +25,21 @@ int dwconv_tiled_kw15(const void* x, const void* w, void* y, int B, int H, int W
 int dwconv_tiled_kw17(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
                       bool flip, int dtype, hipStream_t s);
 
+int dwconv_mfma_k3(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+int dwconv_mfma_k5(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+int dwconv_mfma_k7(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+int dwconv_mfma_k9(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+int dwconv_mfma_k11(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
 int dwconv_mfma_k13(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+int dwconv_mfma_k15(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
+                    int dtype, hipStream_t s);
+int dwconv_mfma_k17(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
                     int dtype, hipStream_t s);
 
 // Matrix-core kernel for square filters and 16-bit types; -1 when it does not cover the case.
@@ -35,7 +49,14 @@ static int dwconv_mfma_launch(const void* x, const void* w, void* y, int B, int 
     const char* e = getenv("PDW_MFMA");
     if (e && atoi(e) == 0) return -1;
     switch (KW) {
+        case 3: return dwconv_mfma_k3(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 5: return dwconv_mfma_k5(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 7: return dwconv_mfma_k7(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 9: return dwconv_mfma_k9(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 11: return dwconv_mfma_k11(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
         case 13: return dwconv_mfma_k13(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 15: return dwconv_mfma_k15(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 17: return dwconv_mfma_k17(x, w, y, B, H, W, C, PH, PW, flip, dtype, s);
         default: return -1;
     }
 }
