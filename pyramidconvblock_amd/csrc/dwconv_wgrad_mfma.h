@@ -1,0 +1,275 @@
+// Depthwise-convolution weight gradient on the matrix cores (16-bit types, stride 1, dilation 1, odd square
+// filters):      dw[u,v,c] = sum_{b,i,j} gy[b,i,j,c] * x[b, i+u-PH, j+v-PW, c].
+//
+// v_mfma_f32_4x4x4_16b_{bf16,f16} multiplies 16 independent 4x4x4 blocks per instruction; a block is one
+// channel.  For the staged input row rr (window coordinates: rr = i + u) and a block of 4 output columns j0..j0+3
+//     D[m][n] += sum_k A[m][k] * B[k][n]
+//     A[m][k] = gy[rr - 4 ub - m][j0 + k]            filter row u = 4 ub + m   (zero outside the tile's rows)
+//     B[k][n] = x[rr][j0 + k + v],  v = 8 vg + 2 n + par
+// accumulates dw[4 ub + m][8 vg + 2 n + par] for the 16 channels of the workgroup: 1024 multiply-adds per
+// instruction, 66 % of them on real taps at K = 13.  Even v read the input row as aligned column pairs, odd v
+// the same pairs shifted by 16 bits (two v_alignbit per operand).  A lane is (channel b = lane / 4, q = lane % 4),
+// q being m in the A operand and n in the B operand.
+//
+// Operand reuse.  With rr = 4 rho + s the A operand of filter-row block ub is G_s[rho - ub], where G_s[c] holds
+// gy row 4 c + s - m in lane m: one new operand per input row serves ceil(K/4) consecutive rows, so a wavefront
+// that keeps (j0, s) fixed and walks rho reads one gy operand and ceil((K+1)/8) input-row operands from LDS per
+// 2 ceil(K/4) ceil((K+1)/8) MFMAs.  The (j0, s) combinations of a tile are dealt out to the wavefronts; every
+// wavefront accumulates all taps of its 16 channels in registers, the wavefronts are summed through LDS at the
+// end and the workgroup writes one fp32 partial, reduced over the workgroups in a fixed order by
+// wgrad_reduce_parts (no atomics: bit-reproducible).
+//
+// Both windows are staged in LDS channel-major, [row][channel][column pair], as in dwconv_mfma.h.
+#pragma once
+#include <stdlib.h>
+
+#include "common.h"
+#include "dwconv_mfma.h"
+#include "kernels.h"
+#include "tile_common.h"
+
+namespace pdw {
+
+struct WgradMfmaGeom {
+    int H, W, C;      // x extents
+    int OH, OW;       // gy extents
+    int PH, PW;
+    int TH, TW;       // tile of gy positions (TW a multiple of 4)
+    int tiles_h, tiles_w, ntiles, nchunks, slices;
+    int XP, GP;       // LDS dwords per channel row of the x / gy window
+    int red_tiles;    // accumulator tiles summed per round of the final cross-wavefront reduction
+};
+
+template <int K>
+struct WgradMfmaShape {
+    static constexpr int CS = 16;
+    static constexpr int NUB = (K + 3) / 4;        // filter-row blocks
+    static constexpr int NVG = ((K + 1) / 2 + 3) / 4;  // groups of 4 even (or odd) filter columns
+    static constexpr int NTILE = NUB * NVG * 2;    // accumulator tiles (4 registers each) per lane
+};
+
+template <typename T, int K, int NWV>
+__global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __restrict__ x, const T* __restrict__ gy,
+                                                                   float* __restrict__ part, const WgradMfmaGeom g) {
+    using Sh = WgradMfmaShape<K>;
+    constexpr int V = 8, NT = NWV * 64, CS = Sh::CS, NUB = Sh::NUB, NVG = Sh::NVG, NTILE = Sh::NTILE;
+    constexpr int NPX = 6, NPG = 4;  // staging passes of the x / gy windows requested at once (more: staged directly)
+    extern __shared__ uint32_t smem[];
+    const int XR = g.TH + K - 1;                    // x window rows
+    const int NCX = g.TW / 2 + 4 * NVG;             // x window pairs: every pair an operand reads
+    uint32_t* xl = smem;                            // [XR][CS][XP]
+    uint32_t* gl = smem + XR * CS * g.XP;           // [TH][CS][GP]
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int sl = bid % g.slices, chunk = bid / g.slices;
+    const int c0 = sl * CS;
+    const int tiles_per_img = g.tiles_h * g.tiles_w;
+    const int bq = lane >> 2, q = lane & 3;
+
+    TileStager<T, CS, V, NPX, true, NT> sx;
+    TileStager<T, CS, V, NPG, true, NT> sg;
+    sx.init(tid, c0, g.C, XR, NCX, g.XP);
+    sg.init(tid, c0, g.C, g.TH, g.TW / 2, g.GP);
+    auto origin = [&](int tile, int& b, int& row0, int& col0) {
+        b = tile / tiles_per_img;
+        const int rem = tile - b * tiles_per_img;
+        const int th_i = rem / g.tiles_w;
+        row0 = th_i * g.TH, col0 = (rem - th_i * g.tiles_w) * g.TW;
+    };
+    auto request = [&](int tile) {
+        int b, row0, col0;
+        origin(tile, b, row0, col0);
+        sx.issue(x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
+        sg.issue(gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0);
+    };
+    if (chunk < g.ntiles) request(chunk);
+
+    f32x4 acc[NUB][NVG][2];
+#pragma unroll
+    for (int ub = 0; ub < NUB; ++ub)
+#pragma unroll
+        for (int vg = 0; vg < NVG; ++vg)
+#pragma unroll
+            for (int par = 0; par < 2; ++par) acc[ub][vg][par] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int RPX = CS * g.XP, RPG = CS * g.GP;  // dwords per staged row
+    const int ncombo = g.TW;                     // (column block, s) combinations: TW / 4 blocks x 4
+    for (int tile = chunk; tile < g.ntiles; tile += g.nchunks) {
+        int b, row0, col0;
+        origin(tile, b, row0, col0);
+        __syncthreads();  // the previous windows are fully consumed
+        sx.commit(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
+        sg.commit(gl, gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0);
+        __syncthreads();
+        for (int combo = wv; combo < ncombo; combo += NWV) {
+            const int jb = combo >> 2, s = combo & 3;
+            // lane addresses: x pairs start at 2 jb + n (+ 4 vg + 0..2), gy pairs at 2 jb (+0, 1)
+            const uint32_t* xq = xl + bq * g.XP + 2 * jb + q;
+            const uint32_t* gq = gl + bq * g.GP + 2 * jb;
+            uint2 ring[NUB];  // G_s[rho - ub] lives in ring[(rho - ub) mod NUB]
+#pragma unroll
+            for (int i = 0; i < NUB; ++i) ring[i] = make_uint2(0u, 0u);
+            // one x row (rr = 4 rho + s) per step; the steps are unrolled NUB at a time so the ring index is static
+            for (int rho0 = 0; 4 * rho0 + s < XR; rho0 += NUB) {
+#pragma unroll
+                for (int uu = 0; uu < NUB; ++uu) {
+                    const int rho = rho0 + uu;
+                    const int rr = 4 * rho + s;
+                    // new gy operand: row 4 rho + s - m of this lane (zero outside the tile)
+                    const int gr = rr - q;
+                    const bool gok = gr >= 0 && gr < g.TH;
+                    const uint32_t* gp = gq + (gok ? gr : 0) * RPG;
+                    uint2 gnew = make_uint2(gp[0], gp[1]);
+                    if (!gok) gnew = make_uint2(0u, 0u);
+                    ring[uu] = gnew;
+                    if (rr < XR) {
+                        const uint32_t* xr = xq + rr * RPX;
+                        uint2 be[NVG], bo[NVG];
+#pragma unroll
+                        for (int vg = 0; vg < NVG; ++vg) {
+                            const uint32_t p0 = xr[4 * vg], p1 = xr[4 * vg + 1], p2 = xr[4 * vg + 2];
+                            be[vg] = make_uint2(p0, p1);
+                            bo[vg] = make_uint2(__builtin_amdgcn_alignbit(p1, p0, 16), __builtin_amdgcn_alignbit(p2, p1, 16));
+                        }
+#pragma unroll
+                        for (int ub = 0; ub < NUB; ++ub) {
+                            // gy rows 4 (rho - ub) + s - m: all outside the tile for rho < ub or past its end
+                            const int c = rho - ub;
+                            if (c >= 0 && 4 * c + s - 3 < g.TH) {
+                                const uint2 a = ring[(uu - ub + NUB) % NUB];
+#pragma unroll
+                                for (int vg = 0; vg < NVG; ++vg) {
+                                    acc[ub][vg][0] = mfma4(a, be[vg], acc[ub][vg][0], T());
+                                    acc[ub][vg][1] = mfma4(a, bo[vg], acc[ub][vg][1], T());
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        if (tile + g.nchunks < g.ntiles) request(tile + g.nchunks);
+    }
+
+    // ---- sum the wavefronts through LDS, red_tiles accumulator tiles per round; register m of tile (ub, vg, par):
+    // filter row 4 ub + m, lane (b, n): filter column 8 vg + 2 n + par of channel b
+    float* red = reinterpret_cast<float*>(smem);  // [NWV][RT][4][64]
+    float* pout = part + (long long)chunk * K * K * g.C;
+    const int RT = g.red_tiles;
+    for (int t0 = 0; t0 < NTILE; t0 += RT) {
+        __syncthreads();
+#pragma unroll
+        for (int ub = 0; ub < NUB; ++ub)
+#pragma unroll
+            for (int vg = 0; vg < NVG; ++vg)
+#pragma unroll
+                for (int par = 0; par < 2; ++par) {
+                    const int ti = (ub * NVG + vg) * 2 + par;
+                    if (ti >= t0 && ti < t0 + RT) {
+#pragma unroll
+                        for (int m = 0; m < 4; ++m)
+                            red[((wv * RT + ti - t0) * 4 + m) * 64 + lane] = acc[ub][vg][par][m];
+                    }
+                }
+        __syncthreads();
+        const int nout = (NTILE - t0 < RT ? NTILE - t0 : RT) * 256;
+        for (int o = tid; o < nout; o += NT) {
+            const int ch = o & 15, n = (o >> 4) & 3, m = (o >> 6) & 3, ti = t0 + (o >> 8);
+            float s = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < NWV; ++w2) s += red[((w2 * RT + ti - t0) * 4 + m) * 64 + 4 * ch + n];
+            const int par = ti & 1, vg = (ti >> 1) % NVG, ub = (ti >> 1) / NVG;
+            const int u = 4 * ub + m, v = 8 * vg + 2 * n + par;
+            if (u < K && v < K && c0 + ch < g.C) pout[(u * K + v) * g.C + c0 + ch] = s;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Host side
+
+struct WgradMfmaPlan {
+    bool ok = false;
+    WgradMfmaGeom g;
+    size_t lds = 0;
+    int nblocks = 0;
+};
+
+template <typename T, int K, int NWV>
+static WgradMfmaPlan plan_wgrad_mfma(int B, int H, int W, int C, int PH, int PW) {
+    using Sh = WgradMfmaShape<K>;
+    WgradMfmaPlan p;
+    WgradMfmaGeom& g = p.g;
+    g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW;
+    g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
+    if (g.OH < 1 || g.OW < 1 || C % 8 != 0) return p;
+    if ((long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL) return p;
+    g.slices = cdiv(C, Sh::CS);
+    // tile width: the whole row up to 56 columns, a multiple of 4
+    const int ow4 = cdiv(g.OW, 4) * 4;
+    g.tiles_w = cdiv(ow4, 56);
+    g.TW = cdiv(cdiv(ow4, g.tiles_w), 4) * 4;
+    auto pad = [](int n) {  // 4 mod 8 keeps the 16 channels x 4 lanes of an operand read on distinct banks
+        while (n % 8 != 4) ++n;
+        return n;
+    };
+    g.XP = pad(g.TW / 2 + 4 * Sh::NVG), g.GP = pad(g.TW / 2);
+    auto lds_of = [&](int th) { return ((size_t)(th + K - 1) * Sh::CS * g.XP + (size_t)th * Sh::CS * g.GP) * 4; };
+    // tile height: about one tile per CU, within LDS and the staging registers
+    long long want_h = ((long long)B * g.slices * g.tiles_w + 255) / 256;  // images*slices per CU column
+    int tiles_h = (int)(256 / ((long long)B * g.slices * g.tiles_w > 0 ? (long long)B * g.slices * g.tiles_w : 1));
+    (void)want_h;
+    if (tiles_h < 1) tiles_h = 1;
+    if (tiles_h > g.OH) tiles_h = g.OH;
+    int th = cdiv(g.OH, tiles_h);
+    if (th < 4) th = g.OH < 4 ? g.OH : 4;
+    while (th > 1 && lds_of(th) > 150 * 1024) --th;
+    if (lds_of(th) > 150 * 1024) return p;
+    g.TH = th;
+    g.tiles_h = cdiv(g.OH, th);
+    const long long ntiles = (long long)B * g.tiles_h * g.tiles_w;
+    if (ntiles > 0x7fffffffLL) return p;
+    g.ntiles = (int)ntiles;
+    const int cap = 256 / g.slices > 1 ? 256 / g.slices : 1;
+    const long long rounds = cdiv(ntiles, (long long)cap);
+    g.nchunks = (int)cdiv(ntiles, rounds);
+    p.nblocks = g.nchunks * g.slices;
+    size_t lds = lds_of(th);
+    // final reduction: NWV wavefronts x red_tiles x 1 KB
+    int rt = Sh::NTILE;
+    while ((size_t)NWV * rt * 1024 > 150 * 1024) rt = (rt + 1) / 2;
+    g.red_tiles = rt;
+    if (lds < (size_t)NWV * rt * 1024) lds = (size_t)NWV * rt * 1024;
+    p.lds = lds;
+    p.ok = true;
+    return p;
+}
+
+template <typename T, int K>
+static size_t wgrad_mfma_workspace_t(int B, int H, int W, int C, int PH, int PW) {
+    const WgradMfmaPlan p = plan_wgrad_mfma<T, K, 8>(B, H, W, C, PH, PW);
+    return p.ok ? (size_t)p.g.nchunks * K * K * C * sizeof(float) : 0;
+}
+
+// -1: not covered (the caller uses the vector-ALU tiled kernel).
+template <typename T, int K>
+static int wgrad_mfma_launch_t(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                               int PW, hipStream_t s) {
+    constexpr int NWV = 8;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(gy) & 15)) return -1;
+    const WgradMfmaPlan p = plan_wgrad_mfma<T, K, NWV>(B, H, W, C, PH, PW);
+    if (!p.ok) return -1;
+    auto kern = dwconv_wgrad_mfma_k<T, K, NWV>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.nblocks), dim3(NWV * 64), p.lds, s, (const T*)x, (const T*)gy, (float*)ws,
+                       p.g);
+    if (int e = check_launch("dwconv_wgrad_mfma")) return e;
+    return wgrad_reduce_launch<T>((const float*)ws, dw, p.g.nchunks, K * K * C, s);
+}
+
+}  // namespace pdw

@@ -1,6 +1,8 @@
 // Dispatch of the LDS-tiled depthwise-convolution weight gradient (stride 1, dilation 1, odd
 // square filters up to 17x17) by filter size.  The kernel template and its description live in
 // dwconv_wgrad_tiled.h; each size is instantiated in its own translation unit.
+#include <stdlib.h>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -31,26 +33,95 @@ size_t dwconv_wgrad_tiled_ws_k17(int B, int H, int W, int C, int PH, int PW, int
 int dwconv_wgrad_tiled_k17(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
                            int PW, int dtype, hipStream_t s);
 
-// Bytes of fp32 workspace the tiled weight gradient needs; 0 when it does not cover the case.
-size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype) {
-    if (KH != KW) return 0;
-    switch (KH) {
-        case 3: return dwconv_wgrad_tiled_ws_k3(B, H, W, C, PH, PW, dtype);
-        case 5: return dwconv_wgrad_tiled_ws_k5(B, H, W, C, PH, PW, dtype);
-        case 7: return dwconv_wgrad_tiled_ws_k7(B, H, W, C, PH, PW, dtype);
-        case 9: return dwconv_wgrad_tiled_ws_k9(B, H, W, C, PH, PW, dtype);
-        case 11: return dwconv_wgrad_tiled_ws_k11(B, H, W, C, PH, PW, dtype);
-        case 13: return dwconv_wgrad_tiled_ws_k13(B, H, W, C, PH, PW, dtype);
-        case 15: return dwconv_wgrad_tiled_ws_k15(B, H, W, C, PH, PW, dtype);
-        case 17: return dwconv_wgrad_tiled_ws_k17(B, H, W, C, PH, PW, dtype);
+size_t dwconv_wgrad_mfma_ws_k3(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k3(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k5(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k5(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k7(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k7(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k9(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k9(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k11(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k11(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k13(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k13(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k15(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k15(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+size_t dwconv_wgrad_mfma_ws_k17(int B, int H, int W, int C, int PH, int PW, int dtype);
+int dwconv_wgrad_mfma_k17(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
+                            int PW, int dtype, hipStream_t s);
+
+// Matrix-core variant (16-bit types): workspace bytes (0 = not covered) and launch (-1 = not covered).
+static bool wgrad_mfma_enabled(int dtype) {
+    if (dtype == kF32) return false;
+    const char* e = getenv("PDW_MFMA");
+    return !(e && atoi(e) == 0);
+}
+static size_t wgrad_mfma_workspace(int B, int H, int W, int C, int K, int PH, int PW, int dtype) {
+    if (!wgrad_mfma_enabled(dtype)) return 0;
+    switch (K) {
+        case 3: return dwconv_wgrad_mfma_ws_k3(B, H, W, C, PH, PW, dtype);
+        case 5: return dwconv_wgrad_mfma_ws_k5(B, H, W, C, PH, PW, dtype);
+        case 7: return dwconv_wgrad_mfma_ws_k7(B, H, W, C, PH, PW, dtype);
+        case 9: return dwconv_wgrad_mfma_ws_k9(B, H, W, C, PH, PW, dtype);
+        case 11: return dwconv_wgrad_mfma_ws_k11(B, H, W, C, PH, PW, dtype);
+        case 13: return dwconv_wgrad_mfma_ws_k13(B, H, W, C, PH, PW, dtype);
+        case 15: return dwconv_wgrad_mfma_ws_k15(B, H, W, C, PH, PW, dtype);
+        case 17: return dwconv_wgrad_mfma_ws_k17(B, H, W, C, PH, PW, dtype);
         default: return 0;
     }
+}
+static int wgrad_mfma_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int K, int PH,
+                             int PW, int dtype, hipStream_t s) {
+    if (!wgrad_mfma_enabled(dtype)) return -1;
+    switch (K) {
+        case 3: return dwconv_wgrad_mfma_k3(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 5: return dwconv_wgrad_mfma_k5(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 7: return dwconv_wgrad_mfma_k7(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 9: return dwconv_wgrad_mfma_k9(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 11: return dwconv_wgrad_mfma_k11(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 13: return dwconv_wgrad_mfma_k13(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 15: return dwconv_wgrad_mfma_k15(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        case 17: return dwconv_wgrad_mfma_k17(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        default: return -1;
+    }
+}
+
+// Bytes of fp32 workspace the tiled weight gradient needs (the larger of its two variants); 0 when it does not
+// cover the case.
+size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype) {
+    if (KH != KW) return 0;
+    const size_t wm = wgrad_mfma_workspace(B, H, W, C, KH, PH, PW, dtype);
+    size_t wt = 0;
+    switch (KH) {
+        case 3: wt = dwconv_wgrad_tiled_ws_k3(B, H, W, C, PH, PW, dtype); break;
+        case 5: wt = dwconv_wgrad_tiled_ws_k5(B, H, W, C, PH, PW, dtype); break;
+        case 7: wt = dwconv_wgrad_tiled_ws_k7(B, H, W, C, PH, PW, dtype); break;
+        case 9: wt = dwconv_wgrad_tiled_ws_k9(B, H, W, C, PH, PW, dtype); break;
+        case 11: wt = dwconv_wgrad_tiled_ws_k11(B, H, W, C, PH, PW, dtype); break;
+        case 13: wt = dwconv_wgrad_tiled_ws_k13(B, H, W, C, PH, PW, dtype); break;
+        case 15: wt = dwconv_wgrad_tiled_ws_k15(B, H, W, C, PH, PW, dtype); break;
+        case 17: wt = dwconv_wgrad_tiled_ws_k17(B, H, W, C, PH, PW, dtype); break;
+        default: return 0;
+    }
+    return wt > wm ? wt : wm;
 }
 
 // Returns -1 when the case is not covered (the caller then uses the direct kernel).
 int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int KH,
                               int KW, int PH, int PW, int dtype, hipStream_t s) {
     if (KH != KW) return -1;
+    {
+        const int r = wgrad_mfma_launch(x, gy, dw, ws, B, H, W, C, KH, PH, PW, dtype, s);
+        if (r != -1) return r;
+    }
     switch (KH) {
         case 3: return dwconv_wgrad_tiled_k3(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
         case 5: return dwconv_wgrad_tiled_k5(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
