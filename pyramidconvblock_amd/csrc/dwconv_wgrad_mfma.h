@@ -60,7 +60,8 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
     uint32_t* xl = smem;                            // [XR][CS][XP]
     uint32_t* gl = smem + XR * CS * g.XP;           // [TH][CS][GP]
 
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it branches uniformly
     const int bid = xcd_remap(blockIdx.x, gridDim.x);
     const int sl = bid % g.slices, chunk = bid / g.slices;
     const int c0 = sl * CS;
@@ -94,7 +95,11 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
             for (int par = 0; par < 2; ++par) acc[ub][vg][par] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int RPX = CS * g.XP, RPG = CS * g.GP;  // dwords per staged row
-    const int ncombo = g.TW;                     // (column block, s) combinations: TW / 4 blocks x 4
+    // Work items of a tile: (group of JB column blocks, s, row range); NWV of them, one per wavefront.
+    constexpr int JB = 7;
+    const int nblk = g.TW / 4;                       // column blocks (<= 14)
+    const int ngrp = (nblk + JB - 1) / JB;           // 1 or 2
+    const int nrs = NWV / (4 * ngrp);                // row ranges (NWV = 8: 2 or 1)
     for (int tile = chunk; tile < g.ntiles; tile += g.nchunks) {
         int b, row0, col0;
         origin(tile, b, row0, col0);
@@ -102,46 +107,65 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
         sx.commit(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
         sg.commit(gl, gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0);
         __syncthreads();
-        for (int combo = wv; combo < ncombo; combo += NWV) {
-            const int jb = combo >> 2, s = combo & 3;
+        {
+            const int s = wv & 3, grp = (wv >> 2) % ngrp, rs = (wv >> 2) / ngrp;
+            const int jb0 = grp * JB;
+            // x rows of this item: 4 rho + s for rho in [rho_lo, rho_hi)
+            const int nrho = (XR - s + 3) / 4;
+            const int rho_lo = rs * ((nrho + nrs - 1) / nrs);
+            const int rho_hi = min(nrho, (rs + 1) * ((nrho + nrs - 1) / nrs));
             // lane addresses: x pairs start at 2 jb + n (+ 4 vg + 0..2), gy pairs at 2 jb (+0, 1)
-            const uint32_t* xq = xl + bq * g.XP + 2 * jb + q;
-            const uint32_t* gq = gl + bq * g.GP + 2 * jb;
-            uint2 ring[NUB];  // G_s[rho - ub] lives in ring[(rho - ub) mod NUB]
+            const uint32_t* xq = xl + bq * g.XP + 2 * jb0 + q;
+            const uint32_t* gq = gl + bq * g.GP + 2 * jb0;
+            uint2 ring[JB][NUB];  // G_s[rho - ub] of column block j lives in ring[j][(rho - ub) mod NUB]
 #pragma unroll
-            for (int i = 0; i < NUB; ++i) ring[i] = make_uint2(0u, 0u);
-            // one x row (rr = 4 rho + s) per step; the steps are unrolled NUB at a time so the ring index is static
-            for (int rho0 = 0; 4 * rho0 + s < XR; rho0 += NUB) {
+            for (int j = 0; j < JB; ++j)
+#pragma unroll
+                for (int i = 0; i < NUB; ++i) ring[j][i] = make_uint2(0u, 0u);
+            // The walk starts NUB - 1 steps early to fill the ring (no MFMAs there); the steps are unrolled NUB at
+            // a time so the ring index is static.
+            const int rho_start = rho_lo - (NUB - 1) > 0 ? ((rho_lo - (NUB - 1)) / NUB) * NUB : 0;
+            for (int rho0 = rho_start; rho0 < rho_hi; rho0 += NUB) {
 #pragma unroll
                 for (int uu = 0; uu < NUB; ++uu) {
                     const int rho = rho0 + uu;
                     const int rr = 4 * rho + s;
-                    // new gy operand: row 4 rho + s - m of this lane (zero outside the tile)
+                    // new gy operands: row rr - m of this lane (zero outside the tile)
                     const int gr = rr - q;
                     const bool gok = gr >= 0 && gr < g.TH;
                     const uint32_t* gp = gq + (gok ? gr : 0) * RPG;
-                    uint2 gnew = make_uint2(gp[0], gp[1]);
-                    if (!gok) gnew = make_uint2(0u, 0u);
-                    ring[uu] = gnew;
-                    if (rr < XR) {
+#pragma unroll
+                    for (int j = 0; j < JB; ++j) {
+                        const int jc = jb0 + j < nblk ? j : 0;  // past the tile: reread block 0, unused
+                        const uint32_t g0 = gp[2 * jc], g1 = gp[2 * jc + 1];  // always a valid address
+                        ring[j][uu] = make_uint2(gok ? g0 : 0u, gok ? g1 : 0u);
+                    }
+                    if (rho >= rho_lo && rho < rho_hi) {
                         const uint32_t* xr = xq + rr * RPX;
-                        uint2 be[NVG], bo[NVG];
 #pragma unroll
-                        for (int vg = 0; vg < NVG; ++vg) {
-                            const uint32_t p0 = xr[4 * vg], p1 = xr[4 * vg + 1], p2 = xr[4 * vg + 2];
-                            be[vg] = make_uint2(p0, p1);
-                            bo[vg] = make_uint2(__builtin_amdgcn_alignbit(p1, p0, 16), __builtin_amdgcn_alignbit(p2, p1, 16));
-                        }
-#pragma unroll
-                        for (int ub = 0; ub < NUB; ++ub) {
-                            // gy rows 4 (rho - ub) + s - m: all outside the tile for rho < ub or past its end
-                            const int c = rho - ub;
-                            if (c >= 0 && 4 * c + s - 3 < g.TH) {
-                                const uint2 a = ring[(uu - ub + NUB) % NUB];
+                        for (int j = 0; j < JB; ++j) {
+                            if (jb0 + j < nblk) {
+                                uint2 be[NVG], bo[NVG];
 #pragma unroll
                                 for (int vg = 0; vg < NVG; ++vg) {
-                                    acc[ub][vg][0] = mfma4(a, be[vg], acc[ub][vg][0], T());
-                                    acc[ub][vg][1] = mfma4(a, bo[vg], acc[ub][vg][1], T());
+                                    const uint32_t p0 = xr[2 * j + 4 * vg], p1 = xr[2 * j + 4 * vg + 1],
+                                                   p2 = xr[2 * j + 4 * vg + 2];
+                                    be[vg] = make_uint2(p0, p1);
+                                    bo[vg] = make_uint2(__builtin_amdgcn_alignbit(p1, p0, 16),
+                                                        __builtin_amdgcn_alignbit(p2, p1, 16));
+                                }
+#pragma unroll
+                                for (int ub = 0; ub < NUB; ++ub) {
+                                    // gy rows 4 (rho - ub) + s - m: all outside the tile for rho < ub or past its end
+                                    const int c = rho - ub;
+                                    if (c >= 0 && 4 * c + s - 3 < g.TH) {
+                                        const uint2 a = ring[j][(uu - ub + NUB) % NUB];
+#pragma unroll
+                                        for (int vg = 0; vg < NVG; ++vg) {
+                                            acc[ub][vg][0] = mfma4(a, be[vg], acc[ub][vg][0], T());
+                                            acc[ub][vg][1] = mfma4(a, bo[vg], acc[ub][vg][1], T());
+                                        }
+                                    }
                                 }
                             }
                         }
@@ -154,9 +178,10 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
 
     // ---- sum the wavefronts through LDS, red_tiles accumulator tiles per round; register m of tile (ub, vg, par):
     // filter row 4 ub + m, lane (b, n): filter column 8 vg + 2 n + par of channel b
-    float* red = reinterpret_cast<float*>(smem);  // [NWV][RT][4][64]
+    float* red = reinterpret_cast<float*>(smem);  // [NWV][RT][m][n][16 channels]
     float* pout = part + (long long)chunk * K * K * g.C;
     const int RT = g.red_tiles;
+    const int slot = q * 16 + bq;  // lane (b, n) -> channel-fastest
     for (int t0 = 0; t0 < NTILE; t0 += RT) {
         __syncthreads();
 #pragma unroll
@@ -169,19 +194,23 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
                     if (ti >= t0 && ti < t0 + RT) {
 #pragma unroll
                         for (int m = 0; m < 4; ++m)
-                            red[((wv * RT + ti - t0) * 4 + m) * 64 + lane] = acc[ub][vg][par][m];
+                            red[((wv * RT + ti - t0) * 4 + m) * 64 + slot] = acc[ub][vg][par][m];
                     }
                 }
         __syncthreads();
-        const int nout = (NTILE - t0 < RT ? NTILE - t0 : RT) * 256;
+        const int nout = (NTILE - t0 < RT ? NTILE - t0 : RT) * 64;  // float4 outputs: 4 channels each
         for (int o = tid; o < nout; o += NT) {
-            const int ch = o & 15, n = (o >> 4) & 3, m = (o >> 6) & 3, ti = t0 + (o >> 8);
-            float s = 0.f;
+            const int c4 = (o & 3) * 4, n = (o >> 2) & 3, m = (o >> 4) & 3, ti = t0 + (o >> 6);
+            float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-            for (int w2 = 0; w2 < NWV; ++w2) s += red[((w2 * RT + ti - t0) * 4 + m) * 64 + 4 * ch + n];
+            for (int w2 = 0; w2 < NWV; ++w2) {
+                const float4 t = *reinterpret_cast<const float4*>(red + ((w2 * RT + ti - t0) * 4 + m) * 64 + n * 16 + c4);
+                s.x += t.x, s.y += t.y, s.z += t.z, s.w += t.w;
+            }
             const int par = ti & 1, vg = (ti >> 1) % NVG, ub = (ti >> 1) / NVG;
             const int u = 4 * ub + m, v = 8 * vg + 2 * n + par;
-            if (u < K && v < K && c0 + ch < g.C) pout[(u * K + v) * g.C + c0 + ch] = s;
+            if (u < K && v < K && c0 + c4 < g.C)  // C % 8 == 0: the 4 channels are in range together
+                *reinterpret_cast<float4*>(pout + (u * K + v) * g.C + c0 + c4) = s;
         }
     }
 }
