@@ -190,21 +190,33 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
             };
             const uint32_t* xr = xbase;
             const T* wr = wbase;
-            Ops oa, ob;
-            fetch(oa, xr, wr);
-            static_assert(NPH % 2 == 0, "phases are processed in pairs");
+            // two operand sets when the registers allow it (2 wavefronts per SIMD: 256 registers each)
+            constexpr bool kAhead = 2 * (4 * NQ + 4 * NVB) + 4 * S <= 176;
+            if constexpr (kAhead) {
+                Ops oa, ob;
+                fetch(oa, xr, wr);
+                static_assert(NPH % 2 == 0, "phases are processed in pairs");
 #pragma unroll 1
-            for (int p = 0; p < NPH; p += 2) {
-                xr += RP, wr += WPITCH;
-                fetch(ob, xr, wr);
-                __builtin_amdgcn_sched_barrier(0);
-                multiply(oa);
-                __builtin_amdgcn_sched_barrier(0);
-                xr += RP, wr += WPITCH;
-                if (p + 2 < NPH) fetch(oa, xr, wr);
-                __builtin_amdgcn_sched_barrier(0);
-                multiply(ob);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int p = 0; p < NPH; p += 2) {
+                    xr += RP, wr += WPITCH;
+                    fetch(ob, xr, wr);
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(oa);
+                    __builtin_amdgcn_sched_barrier(0);
+                    xr += RP, wr += WPITCH;
+                    if (p + 2 < NPH) fetch(oa, xr, wr);
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(ob);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll 1
+                for (int p = 0; p < NPH; ++p) {
+                    Ops oa;
+                    fetch(oa, xr, wr);
+                    multiply(oa);
+                    xr += RP, wr += WPITCH;
+                }
             }
         }
         // ---- results -> LDS as yl[row][column][16 channels] (one rounding to T), then out in 16-byte pieces:

@@ -58,7 +58,8 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
     const int XR = g.TH + K - 1;                    // x window rows
     const int NCX = g.TW / 2 + 4 * NVG;             // x window pairs: every pair an operand reads
     uint32_t* xl = smem;                            // [XR][CS][XP]
-    uint32_t* gl = smem + XR * CS * g.XP;           // [TH][CS][GP]
+    uint32_t* gl = smem + XR * CS * g.XP;           // [TH][CS][GP], rows one dword further apart: the 4 gy rows an
+                                                    // operand read touches then fall on different banks
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it branches uniformly
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
     TileStager<T, CS, V, NPX, true, NT> sx;
     TileStager<T, CS, V, NPG, true, NT> sg;
     sx.init(tid, c0, g.C, XR, NCX, g.XP);
-    sg.init(tid, c0, g.C, g.TH, g.TW / 2, g.GP);
+    sg.init(tid, c0, g.C, g.TH, g.TW / 2, g.GP, CS * g.GP + 1);
     auto origin = [&](int tile, int& b, int& row0, int& col0) {
         b = tile / tiles_per_img;
         const int rem = tile - b * tiles_per_img;
@@ -94,12 +95,14 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
 #pragma unroll
             for (int par = 0; par < 2; ++par) acc[ub][vg][par] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int RPX = CS * g.XP, RPG = CS * g.GP;  // dwords per staged row
-    // Work items of a tile: (group of JB column blocks, s, row range); NWV of them, one per wavefront.
-    constexpr int JB = 7;
+    const int RPX = CS * g.XP, RPG = CS * g.GP + 1;  // dwords per staged row
+    // Work items of a tile: (group of JB column blocks, s, row range), dealt out to the wavefronts.  JB = 7 fits the
+    // 14 blocks of a 56-column row in two groups; large filters keep fewer blocks in flight (registers).
+    constexpr int JB = NTILE <= 16 ? 7 : 4;
     const int nblk = g.TW / 4;                       // column blocks (<= 14)
-    const int ngrp = (nblk + JB - 1) / JB;           // 1 or 2
-    const int nrs = NWV / (4 * ngrp);                // row ranges (NWV = 8: 2 or 1)
+    const int ngrp = (nblk + JB - 1) / JB;
+    const int nrs = NWV / (4 * ngrp) > 1 ? NWV / (4 * ngrp) : 1;  // row ranges: enough items for every wavefront
+    const int nitems = 4 * ngrp * nrs;
     for (int tile = chunk; tile < g.ntiles; tile += g.nchunks) {
         int b, row0, col0;
         origin(tile, b, row0, col0);
@@ -107,8 +110,8 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
         sx.commit(xl, x + (long long)b * g.H * g.W * g.C, g.H, g.W, g.C, row0 - g.PH, col0 - g.PW);
         sg.commit(gl, gy + (long long)b * g.OH * g.OW * g.C, g.OH, g.OW, g.C, row0, col0);
         __syncthreads();
-        {
-            const int s = wv & 3, grp = (wv >> 2) % ngrp, rs = (wv >> 2) / ngrp;
+        for (int item = wv; item < nitems; item += NWV) {
+            const int s = item & 3, grp = (item >> 2) % ngrp, rs = (item >> 2) / ngrp;
             const int jb0 = grp * JB;
             // x rows of this item: 4 rho + s for rho in [rho_lo, rho_hi)
             const int nrho = (XR - s + 3) / 4;
@@ -244,7 +247,7 @@ static WgradMfmaPlan plan_wgrad_mfma(int B, int H, int W, int C, int PH, int PW)
         return n;
     };
     g.XP = pad(g.TW / 2 + 4 * Sh::NVG), g.GP = pad(g.TW / 2);
-    auto lds_of = [&](int th) { return ((size_t)(th + K - 1) * Sh::CS * g.XP + (size_t)th * Sh::CS * g.GP) * 4; };
+    auto lds_of = [&](int th) { return ((size_t)(th + K - 1) * Sh::CS * g.XP + (size_t)th * (Sh::CS * g.GP + 1)) * 4; };
     // tile height: about one tile per CU, within LDS and the staging registers
     long long want_h = ((long long)B * g.slices * g.tiles_w + 255) / 256;  // images*slices per CU column
     int tiles_h = (int)(256 / ((long long)B * g.slices * g.tiles_w > 0 ? (long long)B * g.slices * g.tiles_w : 1));

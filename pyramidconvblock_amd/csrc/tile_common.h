@@ -135,14 +135,15 @@ struct TileStager {
     static constexpr int NL = PK;          // pixels loaded per LDS unit
     static constexpr int CV = CS / V;      // channel vectors per unit
     static constexpr int UPP = NTHREADS / CV;  // units per pass of the workgroup
-    int scv, sr0, su0, step_r, step_u, CPn, rows, chc, pitch;
+    int scv, sr0, su0, step_r, step_u, CPn, rows, chc, pitch, rpitch;
     bool chok;
     ChanVec<T, V> pre[NPRE][NL];
 
-    __device__ __forceinline__ void init(int tid, int c0, int C, int rows_, int CPn_, int pitch_ = 0) {
+    // pitch_: dwords per channel row, rpitch_: dwords per staged row (default CS * pitch_), CHMAJOR only
+    __device__ __forceinline__ void init(int tid, int c0, int C, int rows_, int CPn_, int pitch_ = 0, int rpitch_ = 0) {
         scv = tid % CV;
         const int tu = tid / CV;
-        CPn = CPn_, rows = rows_, pitch = pitch_;
+        CPn = CPn_, rows = rows_, pitch = pitch_, rpitch = rpitch_ > 0 ? rpitch_ : CS * pitch_;
         sr0 = tu / CPn, su0 = tu - sr0 * CPn;
         step_r = UPP / CPn, step_u = UPP - step_r * CPn;
         const int ch = c0 + scv * V;
@@ -181,7 +182,7 @@ struct TileStager {
             for (int i = 0; i < V; ++i) out[i] = ok0 ? __builtin_bit_cast(uint32_t, ld[0].v[i]) : 0u;
         }
         if constexpr (CHMAJOR) {
-            uint32_t* dst = xl + (r * CS + scv * V) * pitch + u;
+            uint32_t* dst = xl + r * rpitch + scv * V * pitch + u;
 #pragma unroll
             for (int i = 0; i < V; ++i) dst[i * pitch] = out[i];
         } else {
