@@ -25,6 +25,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK = 8.0e12  # B/s, MI355X published
 VALU_PEAK = 157.3e12  # fp32 vector FLOP/s, MI355X published
+MFMA_PEAK = 2.5e15    # dense bf16/fp16 matrix FLOP/s, MI355X published
 
 WORKLOAD = dict(B=32, H=56, W=56, D=128, k=13, dtype="bf16")
 
@@ -32,9 +33,9 @@ WORKLOAD = dict(B=32, H=56, W=56, D=128, k=13, dtype="bf16")
 # scaled by what the same counter reads for a plain copy of known size (`bench.py --kernel copy`); the
 # runs and the scale factors are recorded under profiles/.  None = not measured.
 MEASURED_TRAFFIC = {
-    "dwconv_fwd[32x56x56x64,k=13]": (14115 + 12544) * 1024,   # fetch 14.45 MB + write 12.85 MB
-    "dwconv_dgrad[32x56x56x64,k=13]": (14115 + 12544) * 1024,  # same kernel, same shape
-    "dwconv_wgrad[32x56x56x64,k=13]": (27247 + 5408 + 5419 + 21) * 1024,
+    "dwconv_fwd[32x56x56x64,k=13]": (13144 + 14080) * 1024,   # fetch 13.46 MB + write 14.42 MB
+    "dwconv_dgrad[32x56x56x64,k=13]": (13144 + 14080) * 1024,  # same kernel, same shape
+    "dwconv_wgrad[32x56x56x64,k=13]": (25392 + 2704 + 2721 + 21) * 1024,  # main kernel + partial reduction
 }
 
 
@@ -336,7 +337,7 @@ def main():
     if not args.no_kernels:
         ks = kernel_rooflines(B, H, W, D, k, dtype)
         # Dominant kernel = largest share of the step.  Forward and input gradient are the same kernel
-        # function (dwconv_tiled_k) at the same shape, so their launches count together.
+        # function (dwconv_mfma_k) at the same shape, so their launches count together.
         def share(r):
             return r["seconds"] * (2 if r["kernel"].startswith(("dwconv_fwd", "dwconv_dgrad")) else 1)
 
@@ -346,10 +347,12 @@ def main():
             "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom["alg_bytes"] / dom["seconds"] / HBM_PEAK,
             "traffic": MEASURED_TRAFFIC.get(dom["kernel"]), "avg_us": dom["seconds"] * 1e6,
             "valu_frac": dom["flops"] / dom["seconds"] / VALU_PEAK,
+            "mfma_frac": dom["flops"] / dom["seconds"] / MFMA_PEAK,
         }
         result["kernels"] = [{"kernel": r["kernel"], "us": round(r["seconds"] * 1e6, 2),
                               "hbm_frac": round(r["alg_bytes"] / r["seconds"] / HBM_PEAK, 4),
-                              "valu_frac": round(r["flops"] / r["seconds"] / VALU_PEAK, 4)} for r in ks]
+                              "valu_frac": round(r["flops"] / r["seconds"] / VALU_PEAK, 4),
+                              "mfma_frac": round(r["flops"] / r["seconds"] / MFMA_PEAK, 4)} for r in ks]
 
     if not args.no_cpu:
         threads = min(os.cpu_count() or 1, 16)
