@@ -144,6 +144,56 @@ __device__ __forceinline__ void bl_dst_range(int m, float scale, int out, int& l
     if (hi > out - 1) hi = out - 1;
 }
 
+// Exactly doubled extents (H = 2h, W = 2w, the block's half-resolution gate): source m is read by the 4
+// destinations 2m-1 .. 2m+2 and no others, so the taps are fixed and all 16 loads go out together.  The weights
+// come from the same bl_weight as the general kernel (bit-identical results, borders included).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_bwd_x2_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w,
+                                                         int C, int ldg, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int H = 2 * h, W = 2 * w;
+    const int CV = C / VEC;
+    const int c = (int)(idx % CV) * VEC;
+    long long t = idx / CV;
+    const int n = (int)(t % w);
+    t /= w;
+    const int m = (int)(t % h);
+    const long long b = t / h;
+    float wy[4], wx[4];
+    int iy[4], ix[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int di = 2 * m - 1 + k, dj = 2 * n - 1 + k;
+        const bool oky = di >= 0 && di < H, okx = dj >= 0 && dj < W;
+        iy[k] = oky ? di : 0, ix[k] = okx ? dj : 0;
+        wy[k] = oky ? bl_weight(iy[k], 0.5f, h, m) : 0.f;
+        wx[k] = okx ? bl_weight(ix[k], 0.5f, w, n) : 0.f;
+    }
+    const T* gb = gy + b * H * W * ldg + c;
+    ChanVec<T, VEC> gv[4][4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            gv[p][q] = *reinterpret_cast<const ChanVec<T, VEC>*>(gb + ((long long)iy[p] * W + ix[q]) * ldg);
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    // same order of accumulation as the general kernel: destinations ascending, rows outer
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float ww = wy[p] * wx[q];
+            if (ww != 0.f) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, to_f32(gv[p][q].v[v]), acc[v]);
+            }
+        }
+    store_f32<T, VEC>(gx + ((b * h + m) * w + n) * C + c, acc);
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w,
                                                       int C, int H, int W, int ldg, float sy, float sx,
@@ -514,6 +564,12 @@ int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, in
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
     const float sy = (float)h / (float)H, sx = (float)w / (float)W;
+    if (H == 2 * h && W == 2 * w && h >= 2 && w >= 2) {
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_bwd_x2_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, h, w, C, ldg, total);
+        PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+        return check_launch("bilinear_bwd");
+    }
 #define CALL(T, V) hipLaunchKernelGGL((bilinear_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, h, w, C, H, W, ldg, sy, sx, total);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
