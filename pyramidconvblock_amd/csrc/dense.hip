@@ -72,30 +72,45 @@ __device__ __forceinline__ void strided_offsets(int first, int step, int per_row
     }
 }
 
-// W[k][o] (K x NO, o fastest) -> wl[o][k] (pitch ldw): each thread moves IT groups of 4 consecutive o, consecutive
-// threads take consecutive k so the 16-bit LDS writes of a wavefront fall into consecutive banks.  All of a
-// thread's global loads are issued before the first LDS write waits for one.
+// W[k][o] (K x NO, o fastest) -> wl[o][k] (pitch ldw) in 4 x 4 sub-blocks: a thread loads 4 consecutive o of 4
+// consecutive k (four 8-byte loads), transposes them with 8 byte-permutes and writes 4 consecutive k of each o
+// as one 8-byte LDS store; consecutive threads take consecutive k groups, so the stores fall on consecutive banks.
+// Split in two so that the caller can put other global loads between the request and the LDS writes.
 template <typename T, int IT>
-__device__ __forceinline__ void stage_w_transposed(const T* __restrict__ W, T* wl, int K, int NO, int ldw, int tid) {
-    const int nv = NO / 4;
-    int src[IT], dst[IT];  // item idx = tid + it*256: k = idx % K, o group = idx / K
-    strided_offsets<IT>(tid, 256, K, 4, NO, nv, src);        // W offset  k * NO + 4 * group
-    strided_offsets<IT>(tid, 256, K, 4 * ldw, 1, nv, dst);   // wl offset 4 * group * ldw + k
-    uint2 wv[IT];
+struct WTransposer {
+    uint2 row[IT][4];
+    int dst[IT];
+    __device__ __forceinline__ void load(const T* __restrict__ W, int K, int NO, int ldw, int tid) {
+        const int kq = K / 4, nitem = kq * (NO / 4);
+        int src[IT];
+        strided_offsets<IT>(tid, 256, kq, 4, 4 * NO, NO / 4, src);       // W offset   4 kq * NO + 4 oq
+        strided_offsets<IT>(tid, 256, kq, 4 * ldw, 4, NO / 4, dst);      // wl offset  4 oq * ldw + 4 kq
+        (void)nitem;
 #pragma unroll
-    for (int it = 0; it < IT; ++it) wv[it] = *reinterpret_cast<const uint2*>(W + (src[it] >= 0 ? src[it] : 0));
-    unsigned short* wls = reinterpret_cast<unsigned short*>(wl);
+        for (int it = 0; it < IT; ++it)
 #pragma unroll
-    for (int it = 0; it < IT; ++it) {
-        if (dst[it] >= 0) {
-            unsigned short* q = wls + dst[it];
-            q[0] = (unsigned short)(wv[it].x & 0xffffu);
-            q[ldw] = (unsigned short)(wv[it].x >> 16);
-            q[2 * ldw] = (unsigned short)(wv[it].y & 0xffffu);
-            q[3 * ldw] = (unsigned short)(wv[it].y >> 16);
+            for (int r = 0; r < 4; ++r)
+                row[it][r] = *reinterpret_cast<const uint2*>(W + (src[it] >= 0 ? src[it] : 0) + r * NO);
+    }
+    __device__ __forceinline__ void store(T* wl, int ldw) const {
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            if (dst[it] >= 0) {
+                T* q = wl + dst[it];
+                const uint2* r = row[it];
+                // o = 0: low halves of .x, o = 1: high halves of .x, o = 2 / 3: the same of .y
+                *reinterpret_cast<uint2*>(q) = make_uint2(__builtin_amdgcn_perm(r[1].x, r[0].x, 0x05040100u),
+                                                          __builtin_amdgcn_perm(r[3].x, r[2].x, 0x05040100u));
+                *reinterpret_cast<uint2*>(q + ldw) = make_uint2(__builtin_amdgcn_perm(r[1].x, r[0].x, 0x07060302u),
+                                                                __builtin_amdgcn_perm(r[3].x, r[2].x, 0x07060302u));
+                *reinterpret_cast<uint2*>(q + 2 * ldw) = make_uint2(__builtin_amdgcn_perm(r[1].y, r[0].y, 0x05040100u),
+                                                                    __builtin_amdgcn_perm(r[3].y, r[2].y, 0x05040100u));
+                *reinterpret_cast<uint2*>(q + 3 * ldw) = make_uint2(__builtin_amdgcn_perm(r[1].y, r[0].y, 0x07060302u),
+                                                                    __builtin_amdgcn_perm(r[3].y, r[2].y, 0x07060302u));
+            }
         }
     }
-}
+};
 
 // Weights live in LDS as wl[NO][K + 8] (the pad keeps 16-byte fragment reads of 32 consecutive rows off
 // the same banks); every MFMA reads its weight fragment from there.  Row tiles (32 rows x K) are loaded
@@ -103,8 +118,8 @@ __device__ __forceinline__ void stage_w_transposed(const T* __restrict__ W, T* w
 // and re-shaped into MFMA fragments through a per-wave LDS buffer: row-strided fragment loads straight
 // from global memory run ~2.5x slower on this part.  The same buffer transposes the result tile so the
 // global stores are whole 128-byte lines as well.
-template <typename T>
-__global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W, int w_kmajor,
+template <typename T, bool KMAJOR>
+__global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
                                                     const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                     T* __restrict__ Y, long long N, int K, int NO, int P, int nkt,
                                                     int nnt) {
@@ -131,22 +146,26 @@ __global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, 
             raw[i] = cidx < valid ? *reinterpret_cast<const Frag*>(base + (long long)cidx * 8) : Frag{{0u, 0u, 0u, 0u}};
         }
     };
-    if (gw < ntiles) load_tile(gw);                     // requested before the weights are staged
-    // weight staging: all global loads of a thread are issued before the first LDS write waits for one
-    if (!w_kmajor) {  // W[o][k]: 16-byte copies (at most kKT*kNT*64/256 per thread)
+    // The weights are requested first and written to LDS after the first tile's loads have been issued: loads
+    // return in order, so the other way round the weights would wait for the whole tile.
+    constexpr int ITW = kKT * kNT * 64 / 256;   // 16-byte copies (W[o][k]) or 4 x 4 sub-blocks (W[k][o]) per thread
+    if constexpr (!KMAJOR) {
         const int kv = K / 8;
-        constexpr int IT = kKT * kNT * 64 / 256;
-        int src[IT], dst[IT];
-        strided_offsets<IT>(tid, 256, kv, K, 8, NO, src);
-        strided_offsets<IT>(tid, 256, kv, ldw, 8, NO, dst);
-        Frag wv[IT];
+        Frag wv[ITW];
+        int src[ITW], wdst[ITW];
+        strided_offsets<ITW>(tid, 256, kv, K, 8, NO, src);
+        strided_offsets<ITW>(tid, 256, kv, ldw, 8, NO, wdst);
 #pragma unroll
-        for (int it = 0; it < IT; ++it) wv[it] = *reinterpret_cast<const Frag*>(W + (src[it] >= 0 ? src[it] : 0));
+        for (int it = 0; it < ITW; ++it) wv[it] = *reinterpret_cast<const Frag*>(W + (src[it] >= 0 ? src[it] : 0));
+        if (gw < ntiles) load_tile(gw);
 #pragma unroll
-        for (int it = 0; it < IT; ++it)
-            if (dst[it] >= 0) *reinterpret_cast<Frag*>(wl + dst[it]) = wv[it];
+        for (int it = 0; it < ITW; ++it)
+            if (wdst[it] >= 0) *reinterpret_cast<Frag*>(wl + wdst[it]) = wv[it];
     } else {
-        stage_w_transposed<T, kKT * kNT * 128 / 256>(W, wl, K, NO, ldw, tid);
+        WTransposer<T, ITW> wt;
+        wt.load(W, K, NO, ldw, tid);
+        if (gw < ntiles) load_tile(gw);
+        wt.store(wl, ldw);
     }
     const int cpr = NO / 8;  // 16-byte chunks per output row (NO % 8 == 0 on this path)
     constexpr int LO = 2 * kNT;  // 16-byte chunks per lane of a 32 x NO tile (NO <= 32 * kNT)
@@ -379,14 +398,15 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     if (blocks > cap) blocks = cap;  // persistent workgroups: the weights are staged to LDS once each
     if (blocks < 1) blocks = 1;
     const size_t lds = ((size_t)NO * (K + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2;
-    if (dtype == kF16)
-        hipLaunchKernelGGL((dense_rows_k<f16_t>), dim3((unsigned)blocks), dim3(256), lds, s, (const f16_t*)x,
-                           (const f16_t*)w, w_kmajor, (const f16_t*)bias, rowbias, (f16_t*)y, N, K, NO, P > 0 ? P : 1,
-                           nkt, nnt);
-    else
-        hipLaunchKernelGGL((dense_rows_k<bf16_t>), dim3((unsigned)blocks), dim3(256), lds, s, (const bf16_t*)x,
-                           (const bf16_t*)w, w_kmajor, (const bf16_t*)bias, rowbias, (bf16_t*)y, N, K, NO,
-                           P > 0 ? P : 1, nkt, nnt);
+#define PDW_GO(T, KM)                                                                                          \
+    hipLaunchKernelGGL((dense_rows_k<T, KM>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x, (const T*)w, \
+                       (const T*)bias, rowbias, (T*)y, N, K, NO, P > 0 ? P : 1, nkt, nnt)
+    if (dtype == kF16) {
+        if (w_kmajor) PDW_GO(f16_t, true); else PDW_GO(f16_t, false);
+    } else {
+        if (w_kmajor) PDW_GO(bf16_t, true); else PDW_GO(bf16_t, false);
+    }
+#undef PDW_GO
     return check_launch("dense_rows");
 }
 
