@@ -159,15 +159,13 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
                                 }
 #pragma unroll
                                 for (int ub = 0; ub < NUB; ++ub) {
-                                    // gy rows 4 (rho - ub) + s - m: all outside the tile for rho < ub or past its end
-                                    const int c = rho - ub;
-                                    if (c >= 0 && 4 * c + s - 3 < g.TH) {
-                                        const uint2 a = ring[j][(uu - ub + NUB) % NUB];
+                                    // gy rows 4 (rho - ub) + s - m; outside the tile the ring holds zeros.  Skipping
+                                    // those products would cost a branch per 2 NVG MFMAs, more than they do.
+                                    const uint2 a = ring[j][(uu - ub + NUB) % NUB];
 #pragma unroll
-                                        for (int vg = 0; vg < NVG; ++vg) {
-                                            acc[ub][vg][0] = mfma4(a, be[vg], acc[ub][vg][0], T());
-                                            acc[ub][vg][1] = mfma4(a, bo[vg], acc[ub][vg][1], T());
-                                        }
+                                    for (int vg = 0; vg < NVG; ++vg) {
+                                        acc[ub][vg][0] = mfma4(a, be[vg], acc[ub][vg][0], T());
+                                        acc[ub][vg][1] = mfma4(a, bo[vg], acc[ub][vg][1], T());
                                     }
                                 }
                             }
