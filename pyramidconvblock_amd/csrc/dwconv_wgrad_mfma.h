@@ -139,20 +139,22 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
                     const uint32_t* gp = gq + (gok ? gr : 0) * RPG;
 #pragma unroll
                     for (int j = 0; j < JB; ++j) {
-                        const int jc = jb0 + j < nblk ? j : 0;  // past the tile: reread block 0, unused
+                        const bool jok = jb0 + j < nblk;  // past the tile: reread block 0 and zero the operand
+                        const int jc = jok ? j : 0;
                         const uint32_t g0 = gp[2 * jc], g1 = gp[2 * jc + 1];  // always a valid address
-                        ring[j][uu] = make_uint2(gok ? g0 : 0u, gok ? g1 : 0u);
+                        ring[j][uu] = make_uint2(gok && jok ? g0 : 0u, gok && jok ? g1 : 0u);
                     }
                     if (rho >= rho_lo && rho < rho_hi) {
                         const uint32_t* xr = xq + rr * RPX;
 #pragma unroll
                         for (int j = 0; j < JB; ++j) {
-                            if (jb0 + j < nblk) {
+                            {
+                                const int jc = jb0 + j < nblk ? j : 0;
                                 uint2 be[NVG], bo[NVG];
 #pragma unroll
                                 for (int vg = 0; vg < NVG; ++vg) {
-                                    const uint32_t p0 = xr[2 * j + 4 * vg], p1 = xr[2 * j + 4 * vg + 1],
-                                                   p2 = xr[2 * j + 4 * vg + 2];
+                                    const uint32_t p0 = xr[2 * jc + 4 * vg], p1 = xr[2 * jc + 4 * vg + 1],
+                                                   p2 = xr[2 * jc + 4 * vg + 2];
                                     be[vg] = make_uint2(p0, p1);
                                     bo[vg] = make_uint2(__builtin_amdgcn_alignbit(p1, p0, 16),
                                                         __builtin_amdgcn_alignbit(p2, p1, 16));
