@@ -309,7 +309,17 @@ __global__ __launch_bounds__(256) void spatial_sum_part_k(const T* __restrict__ 
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
     if (pl < PL) {
         const T* xb = x + ((long long)b * P) * C + cv * VEC;
-        for (int p = p0 + pl; p < p1; p += PL) {
+        int p = p0 + pl;
+        for (; p + 3 * PL < p1; p += 4 * PL) {  // four loads in flight per thread
+            ChanVec<T, VEC> xv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) xv[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + (long long)(p + u * PL) * C);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] += to_f32(xv[u].v[v]);
+        }
+        for (; p < p1; p += PL) {
             float xv[VEC];
             load_f32<T, VEC>(xb + (long long)p * C, xv);
 #pragma unroll
@@ -458,6 +468,162 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_b_k(const float* __restri
         float s = 0.f;
         for (int b = 0; b < B; ++b) s += gcol[b];
         gbias[o] = from_f32<T>(s);
+    }
+}
+
+// ---- the same three kernels for 16-bit types with D % 8 == 0 and D <= 128 (the block's widths): 16-byte weight
+// loads, every global load of a thread issued before the first use (these kernels are pure latency), partial
+// products combined through LDS.
+template <typename T>
+__device__ __forceinline__ float colsum_parts(const float* __restrict__ pp, int nchunks, int D) {
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int q = 0;
+#pragma unroll 4
+    for (; q + 4 <= nchunks; q += 4) {
+        s0 += pp[(long long)q * D], s1 += pp[(long long)(q + 1) * D];
+        s2 += pp[(long long)(q + 2) * D], s3 += pp[(long long)(q + 3) * D];
+    }
+    for (; q < nchunks; ++q) s0 += pp[(long long)q * D];
+    return (s0 + s1) + (s2 + s3);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restrict__ part, int nchunks, int D,
+                                                            float inv_p, const T* __restrict__ wp,
+                                                            const T* __restrict__ bp, const T* __restrict__ bo,
+                                                            T* __restrict__ m, float* __restrict__ rowbias) {
+    extern __shared__ float sm[];  // [D]
+    const int b = blockIdx.x, tid = threadIdx.x;
+    // weight rows of this thread: outputs o = tid/8 + 32*pass, channel vectors sub + 8*i  (requested first)
+    const int sub = tid & 7, ol = tid >> 3;
+    ChanVec<T, 8> wv[4][2];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int o = ol + 32 * pass, v = sub + 8 * i;
+            const bool ok = o < D && v * 8 < D;
+            wv[pass][i] = *reinterpret_cast<const ChanVec<T, 8>*>(wp + (ok ? (long long)o * D + v * 8 : 0));
+        }
+    if (tid < D) {
+        const T mv = from_f32<T>(colsum_parts<T>(part + (long long)b * nchunks * D + tid, nchunks, D) * inv_p);
+        m[(long long)b * D + tid] = mv;
+        sm[tid] = to_f32(mv);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int o = ol + 32 * pass;
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int v = sub + 8 * i;
+            if (o < D && v * 8 < D) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc = fmaf(sm[v * 8 + j], to_f32(wv[pass][i].v[j]), acc);
+            }
+        }
+        acc += __shfl_xor(acc, 1);
+        acc += __shfl_xor(acc, 2);
+        acc += __shfl_xor(acc, 4);
+        if (sub == 0 && o < D) {
+            if (bp) acc += to_f32(bp[o]);
+            if (bo) acc += to_f32(bo[o]);
+            rowbias[(long long)b * D + o] = acc;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_bwd_a_v8_k(const float* __restrict__ part, int nchunks, int D,
+                                                              float inv_p, const T* __restrict__ wp,
+                                                              float* __restrict__ gs, float* __restrict__ dmean) {
+    extern __shared__ float sm[];  // [D] column sums, then [16][D] partial products
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int cv = tid & 15, ol = tid >> 4;  // channel vector, row lane: rows o = ol + 16*it
+    ChanVec<T, 8> wv[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int o = ol + 16 * it;
+        const bool ok = o < D && cv * 8 < D;
+        wv[it] = *reinterpret_cast<const ChanVec<T, 8>*>(wp + (ok ? (long long)o * D + cv * 8 : 0));
+    }
+    if (tid < D) {
+        const float sv = colsum_parts<T>(part + (long long)b * nchunks * D + tid, nchunks, D);
+        gs[(long long)b * D + tid] = sv;
+        sm[tid] = sv;
+    }
+    __syncthreads();
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int o = ol + 16 * it;
+        if (o < D && cv * 8 < D) {
+            const float gsv = sm[o];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = fmaf(gsv, to_f32(wv[it].v[j]), acc[j]);
+        }
+    }
+    float* prod = sm + D;
+    if (cv * 8 < D) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) prod[ol * D + cv * 8 + j] = acc[j];
+    }
+    __syncthreads();
+    if (tid < D) {
+        float t = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) t += prod[q * D + tid];
+        dmean[(long long)b * D + tid] = t * inv_p;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_bwd_b_v8_k(const float* __restrict__ gs, const T* __restrict__ m,
+                                                              int B, int D, T* __restrict__ gbias,
+                                                              T* __restrict__ gwp) {
+    extern __shared__ float sm[];  // [B] = gs[:, o], then [16][D] partial products
+    const int o = blockIdx.x, tid = threadIdx.x;
+    const int cv = tid & 15, bl = tid >> 4;  // channel vector, batch lane: images b = bl + 16*it
+    for (int b = tid; b < B; b += 256) sm[b] = gs[(long long)b * D + o];
+    __syncthreads();
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    if (cv * 8 < D) {
+        int b = bl;
+        for (; b + 16 < B; b += 32) {  // two loads in flight
+            const ChanVec<T, 8> m0 = *reinterpret_cast<const ChanVec<T, 8>*>(m + (long long)b * D + cv * 8);
+            const ChanVec<T, 8> m1 = *reinterpret_cast<const ChanVec<T, 8>*>(m + (long long)(b + 16) * D + cv * 8);
+            const float g0 = sm[b], g1 = sm[b + 16];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = fmaf(g1, to_f32(m1.v[j]), fmaf(g0, to_f32(m0.v[j]), acc[j]));
+        }
+        for (; b < B; b += 16) {
+            const ChanVec<T, 8> m0 = *reinterpret_cast<const ChanVec<T, 8>*>(m + (long long)b * D + cv * 8);
+            const float g0 = sm[b];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = fmaf(g0, to_f32(m0.v[j]), acc[j]);
+        }
+    }
+    float* prod = sm + B;
+    if (cv * 8 < D) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) prod[bl * D + cv * 8 + j] = acc[j];
+    }
+    __syncthreads();
+    if (tid < D) {
+        float t = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) t += prod[q * D + tid];
+        gwp[(long long)o * D + tid] = from_f32<T>(t);
+    }
+    if (tid == 0) {
+        float sv = 0.f;
+        for (int b = 0; b < B; ++b) sv += sm[b];
+        gbias[o] = from_f32<T>(sv);
     }
 }
 
@@ -674,6 +840,16 @@ int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const 
     if (int e = spatial_sum_parts(x, ws, B, P, D, dtype, s, &n)) return e;
     const float inv_p = 1.f / (float)P;
     const size_t lds = (size_t)D * sizeof(float);
+    const bool v8 = dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0;
+    if (v8) {
+        if (dtype == kF16)
+            hipLaunchKernelGGL((pool_branch_fwd_v8_k<f16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p,
+                               (const f16_t*)wp, (const f16_t*)bp, (const f16_t*)bo, (f16_t*)m, rowbias);
+        else
+            hipLaunchKernelGGL((pool_branch_fwd_v8_k<bf16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p,
+                               (const bf16_t*)wp, (const bf16_t*)bp, (const bf16_t*)bo, (bf16_t*)m, rowbias);
+        return check_launch("pool_branch_fwd");
+    }
     switch (dtype) {
         case kF32:
             hipLaunchKernelGGL((pool_branch_fwd_k<float>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const float*)wp,
@@ -699,6 +875,22 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
     const size_t lds = (size_t)D * 9 * sizeof(float);
     const size_t ldsb = (size_t)B * sizeof(float);
     if (lds > 64 * 1024 || ldsb > 64 * 1024) return set_error("pool branch: extents too large"), 1;
+    const bool v8 = dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(m) & 15) == 0 && (size_t)(B + 16 * D) * sizeof(float) <= 64 * 1024;
+    if (v8) {
+        const size_t la = (size_t)17 * D * sizeof(float), lb = (size_t)(B + 16 * D) * sizeof(float);
+#define PDW_PB8(T)                                                                                                     \
+    hipLaunchKernelGGL((pool_branch_bwd_a_v8_k<T>), dim3(B), dim3(256), la, s, ws, n, D, inv_p, (const T*)wp, gs, dmean); \
+    if (int e = check_launch("pool_branch_bwd_a")) return e;                                                          \
+    hipLaunchKernelGGL((pool_branch_bwd_b_v8_k<T>), dim3(D), dim3(256), lb, s, gs, (const T*)m, B, D, (T*)gbias, (T*)gwp);
+        if (dtype == kF16) {
+            PDW_PB8(f16_t)
+        } else {
+            PDW_PB8(bf16_t)
+        }
+#undef PDW_PB8
+        return check_launch("pool_branch_bwd_b");
+    }
 #define PDW_PB(T)                                                                                                  \
     hipLaunchKernelGGL((pool_branch_bwd_a_k<T>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const T*)wp, gs, dmean); \
     if (int e = check_launch("pool_branch_bwd_a")) return e;                                                       \
