@@ -131,6 +131,13 @@ __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restric
     float s0 = 0.f, s1 = 0.f;
     if (e < n) {
         int p = q;
+        for (; p + 56 < nparts; p += 64) {  // eight loads in flight per lane: the pass is pure latency
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(long long)(p + 8 * u) * n + e];
+            s0 += (v[0] + v[2]) + (v[4] + v[6]);
+            s1 += (v[1] + v[3]) + (v[5] + v[7]);
+        }
         for (; p + 8 < nparts; p += 16) {
             s0 += part[(long long)p * n + e];
             s1 += part[(long long)(p + 8) * n + e];
