@@ -96,6 +96,18 @@ int pdw_gate_fwd(const void *x, void *y, long long M, int I, int ldy, int dtype,
 /* gx[m,c] = gy*x[m,G+c]*sqrt(G);  gx[m,G+c] = gy*x[m,c]*sqrt(G); gy rows ldgy elements apart (0 = dense). */
 int pdw_gate_bwd(const void *x, const void *gy, void *gx, long long M, int I, int ldgy, int dtype, void *stream);
 
+/* Gate followed by the bilinear resize, in one pass: x[B,h,w,I] -> y[B,H,W,I/2], pixels of y ldy elements apart
+ * (0 = dense).  Each gate value is rounded to the storage type before it is interpolated, as when pdw_gate_fwd
+ * and pdw_bilinear_fwd run one after the other; the gated tensor itself is never written.
+ * Replaces conv_block.py:18-21 for a branch with scale_factor != 1. */
+int pdw_gate_bilinear_fwd(const void *x, void *y, int B, int h, int w, int I, int H, int W, int ldy, int dtype,
+                          void *stream);
+/* Gradient of the pair for exactly doubled extents (H = 2h, W = 2w, h,w >= 2; anything else is an error and the
+ * caller runs pdw_bilinear_bwd then pdw_gate_bwd): gy[B,H,W,I/2] (pixels ldgy apart) and the gate's input
+ * x[B,h,w,I] -> gx[B,h,w,I].  What autograd derives for conv_block.py:18-21. */
+int pdw_bilinear_gate_bwd(const void *gy, const void *x, void *gx, int B, int h, int w, int I, int H, int W,
+                          int ldgy, int dtype, void *stream);
+
 /* Per-image sum over positions: x[B,P,C] -> out[B,C] (fp32), two deterministic passes through `workspace`.
  * Replaces x.mean(dim=(1,2)) at conv_block.py:46 (divide by P on the host side) and, in the backward, the
  * reduction of the broadcast add at conv_block.py:49. */

@@ -34,6 +34,8 @@ _SIGS = {
     "pdw_bilinear_bwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
     "pdw_gate_fwd": (c_int, [c_void_p] * 2 + [c_longlong, c_int, c_int, c_int, c_void_p]),
     "pdw_gate_bwd": (c_int, [c_void_p] * 3 + [c_longlong, c_int, c_int, c_int, c_void_p]),
+    "pdw_gate_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
+    "pdw_bilinear_gate_bwd": (c_int, [c_void_p] * 3 + [c_int] * 8 + [c_void_p]),
     "pdw_spatial_sum_workspace_bytes": (c_size_t, [c_int] * 3),
     "pdw_spatial_sum": (c_int, [c_void_p] * 3 + [c_size_t] + [c_int] * 4 + [c_void_p]),
     "pdw_add_rowbias": (c_int, [c_void_p] * 2 + [c_int] * 4 + [c_void_p]),

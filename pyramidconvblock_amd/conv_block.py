@@ -110,7 +110,7 @@ class ConvBlockFunction(torch.autograd.Function):
             if s != 1.:
                 p = ops.avgpool_forward(a, (int(H * s), int(W * s)))
                 c = dwconv_forward(p, w, *geo)
-                ops.bilinear_forward(ops.gate_forward(c), (H, W), out=dst)
+                ops.gate_bilinear_forward(c, (H, W), out=dst)
             else:
                 p = None
                 c = dwconv_forward(a, w, *geo)
@@ -185,7 +185,7 @@ class ConvBlockFunction(torch.autograd.Function):
             dslice = dcat[..., i * G:(i + 1) * G]
             c = convs[i]
             if s != 1.:
-                gc = ops.gate_backward(c, ops.bilinear_backward(dslice, (c.shape[1], c.shape[2])))
+                gc = ops.bilinear_gate_backward(c, dslice)
                 src = pooled[i]
             else:
                 gc = ops.gate_backward(c, dslice)

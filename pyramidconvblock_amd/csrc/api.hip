@@ -169,6 +169,28 @@ int pdw_gate_bwd(const void* x, const void* gy, void* gx, long long M, int I, in
     return gate_bwd_launch(x, gy, gx, M, I, ldgy, dtype, (hipStream_t)stream);
 }
 
+int pdw_gate_bilinear_fwd(const void* x, void* y, int B, int h, int w, int I, int H, int W, int ldy, int dtype,
+                          void* stream) {
+    if (int e = check_resample("pdw_gate_bilinear_fwd", x, y, B, H, W, I, h, w, dtype)) return e;
+    if (I < 2 || (I & 1)) return set_error("pdw_gate_bilinear_fwd: need even I >= 2 (I=%d)", I), 1;
+    if (ldy == 0) ldy = I / 2;
+    if (ldy < I / 2) return set_error("pdw_gate_bilinear_fwd: ldy=%d smaller than I/2=%d", ldy, I / 2), 1;
+    return gate_bilinear_fwd_launch(x, y, B, h, w, I, H, W, ldy, dtype, (hipStream_t)stream);
+}
+
+int pdw_bilinear_gate_bwd(const void* gy, const void* x, void* gx, int B, int h, int w, int I, int H, int W, int ldgy,
+                          int dtype, void* stream) {
+    if (int e = check_resample("pdw_bilinear_gate_bwd", gy, gx, B, H, W, I, h, w, dtype)) return e;
+    if (I < 2 || (I & 1)) return set_error("pdw_bilinear_gate_bwd: need even I >= 2 (I=%d)", I), 1;
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2)
+        return set_error("pdw_bilinear_gate_bwd: needs H = 2h, W = 2w, h,w >= 2 (h=%d w=%d H=%d W=%d); use "
+                         "pdw_bilinear_bwd + pdw_gate_bwd", h, w, H, W), 1;
+    if ((long long)B * h * w > 0 && !x) return set_error("pdw_bilinear_gate_bwd: null pointer"), 1;
+    if (ldgy == 0) ldgy = I / 2;
+    if (ldgy < I / 2) return set_error("pdw_bilinear_gate_bwd: ldgy=%d smaller than I/2=%d", ldgy, I / 2), 1;
+    return bilinear_gate_bwd_launch(gy, x, gx, B, h, w, I, H, W, ldgy, dtype, (hipStream_t)stream);
+}
+
 size_t pdw_spatial_sum_workspace_bytes(int B, int P, int C) {
     if (B < 1 || P < 1 || C < 1) return 0;
     return spatial_sum_workspace(B, P, C);

@@ -42,6 +42,10 @@ int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int 
 int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int ldg, int dtype,
                         hipStream_t s);
 int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s);
+int gate_bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int I, int H, int W, int ldy, int dtype,
+                             hipStream_t s);
+int bilinear_gate_bwd_launch(const void* gy, const void* x, void* gx, int B, int h, int w, int I, int H, int W, int ldg,
+                             int dtype, hipStream_t s);
 int gate_bwd_launch(const void* x, const void* gy, void* gx, long long M, int I, int ldg, int dtype, hipStream_t s);
 size_t spatial_sum_workspace(int B, int P, int C);
 int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C, int dtype, hipStream_t s);

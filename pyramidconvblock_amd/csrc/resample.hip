@@ -292,6 +292,108 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
 }
 
 
+// ---------------------------------------------------------------- gate fused with the resampling next to it
+// Gate then bilinear resize in one pass: y[b,i,j,c] = interp of gate(x)[b,:,:,c], x[B,h,w,I] -> y[B,H,W,G] (G = I/2).
+// The gate value of each of the 4 source pixels is rounded to T first, exactly what the two separate kernels
+// produce, so the gated tensor never exists in memory.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
+                                                           int I, int H, int W, int ldy, float sy, float sx, float s,
+                                                           long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int G = I / 2, GV = G / VEC;
+    const int c = (int)(idx % GV) * VEC;
+    long long t = idx / GV;
+    const int j = (int)(t % W);
+    t /= W;
+    const int i = (int)(t % H);
+    const long long b = t / H;
+    int y0, y1, x0, x1;
+    float ly, lx;
+    bl_src(i, sy, h, y0, y1, ly);
+    bl_src(j, sx, w, x0, x1, lx);
+    const T* xb = x + b * h * w * I + c;
+    const long long o00 = ((long long)y0 * w + x0) * I, o01 = ((long long)y0 * w + x1) * I;
+    const long long o10 = ((long long)y1 * w + x0) * I, o11 = ((long long)y1 * w + x1) * I;
+    ChanVec<T, VEC> pa[4], pb[4];  // all eight loads in flight
+    pa[0] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o00), pb[0] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o00 + G);
+    pa[1] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o01), pb[1] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o01 + G);
+    pa[2] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o10), pb[2] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o10 + G);
+    pa[3] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o11), pb[3] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o11 + G);
+    const float hy = 1.f - ly, hx = 1.f - lx;
+    float o[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        float gv[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) gv[k] = to_f32(from_f32<T>(to_f32(pa[k].v[v]) * to_f32(pb[k].v[v]) * s));
+        o[v] = hy * (hx * gv[0] + lx * gv[1]) + ly * (hx * gv[2] + lx * gv[3]);
+    }
+    store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
+}
+
+// Backward of the pair for exactly doubled extents: the bilinear gather of bilinear_bwd_x2_k (rounded to T),
+// then the gate's gradient, written as gx[B,h,w,I].
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_gate_bwd_x2_k(const T* __restrict__ gy, const T* __restrict__ x,
+                                                              T* __restrict__ gx, int h, int w, int I, int ldg, float s,
+                                                              long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int H = 2 * h, W = 2 * w;
+    const int G = I / 2, GV = G / VEC;
+    const int c = (int)(idx % GV) * VEC;
+    long long t = idx / GV;
+    const int n = (int)(t % w);
+    t /= w;
+    const int m = (int)(t % h);
+    const long long b = t / h;
+    float wy[4], wx[4];
+    int iy[4], ix[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int di = 2 * m - 1 + k, dj = 2 * n - 1 + k;
+        const bool oky = di >= 0 && di < H, okx = dj >= 0 && dj < W;
+        iy[k] = oky ? di : 0, ix[k] = okx ? dj : 0;
+        wy[k] = oky ? bl_weight(iy[k], 0.5f, h, m) : 0.f;
+        wx[k] = okx ? bl_weight(ix[k], 0.5f, w, n) : 0.f;
+    }
+    const T* gb = gy + b * H * W * ldg + c;
+    const T* xp = x + ((b * h + m) * w + n) * I + c;
+    const ChanVec<T, VEC> xa = *reinterpret_cast<const ChanVec<T, VEC>*>(xp);
+    const ChanVec<T, VEC> xb = *reinterpret_cast<const ChanVec<T, VEC>*>(xp + G);
+    ChanVec<T, VEC> gv[4][4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            gv[p][q] = *reinterpret_cast<const ChanVec<T, VEC>*>(gb + ((long long)iy[p] * W + ix[q]) * ldg);
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float ww = wy[p] * wx[q];
+            if (ww != 0.f) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, to_f32(gv[p][q].v[v]), acc[v]);
+            }
+        }
+    float ga[VEC], gbv[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        const float g = to_f32(from_f32<T>(acc[v]));  // the resampled gradient as the separate kernel stores it
+        ga[v] = g * to_f32(xb.v[v]) * s;
+        gbv[v] = g * to_f32(xa.v[v]) * s;
+    }
+    T* op = gx + ((b * h + m) * w + n) * I + c;
+    store_f32<T, VEC>(op, ga);
+    store_f32<T, VEC>(op + G, gbv);
+}
+
 // ---------------------------------------------------------------- per-image column sums and broadcast add
 // Pass 1 of the spatial sum: block (chunk, b) adds its share of the P positions of image b for all C
 // channels; threads are (channel vector, position lane); position lanes are combined through LDS.
@@ -740,6 +842,38 @@ int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, in
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("bilinear_bwd");
+}
+
+int gate_bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int I, int H, int W, int ldy, int dtype,
+                             hipStream_t s) {
+    const void* ptrs[2] = {x, y};
+    const int vec = pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 2);
+    const long long total = (long long)B * H * W * (I / 2 / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+    const float sy = (float)h / (float)H, sx = (float)w / (float)W, sc = sqrtf((float)(I / 2));
+#define CALL(T, V) hipLaunchKernelGGL((gate_bilinear_fwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, h, w, I, H, W, ldy, sy, sx, sc, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("gate_bilinear_fwd");
+}
+
+// -1: extents are not exactly doubled (the caller runs the two separate kernels).
+int bilinear_gate_bwd_launch(const void* gy, const void* x, void* gx, int B, int h, int w, int I, int H, int W, int ldg,
+                             int dtype, hipStream_t s) {
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2) return -1;
+    const void* ptrs[3] = {gy, x, gx};
+    const int vec = pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 3);
+    const long long total = (long long)B * h * w * (I / 2 / vec);
+    unsigned blocks;
+    if (total == 0) return 0;
+    if (!grid_for(total, &blocks)) return 1;
+    const float sc = sqrtf((float)(I / 2));
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_gate_bwd_x2_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (const T*)x, (T*)gx, h, w, I, ldg, sc, total);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("bilinear_gate_bwd");
 }
 
 int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s) {

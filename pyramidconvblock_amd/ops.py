@@ -101,6 +101,36 @@ def gate_backward(x, gy):
     return gx
 
 
+def gate_bilinear_forward(x, out_hw, out=None):
+    """gate then bilinear resize to out_hw in one kernel; x [B,h,w,I] -> [B,H,W,I/2] (conv_block.py:18-21)."""
+    dev = _lib.require_device(x)
+    B, h, w, I = x.shape
+    if I % 2:
+        raise ValueError("gate needs an even channel count")
+    H, W = int(out_hw[0]), int(out_hw[1])
+    if out is None:
+        out = torch.empty((B, H, W, I // 2), device=dev, dtype=x.dtype)
+    if x.numel() and out.numel():
+        _launch("pdw_gate_bilinear_fwd", dev, x.data_ptr(), out.data_ptr(), B, h, w, I, H, W, _pixel_stride(out),
+                _lib.dtype_code(x.dtype))
+    return out
+
+
+def bilinear_gate_backward(x, gy):
+    """Gradient of gate_bilinear_forward w.r.t. x; gy [B,H,W,I/2] may be a channel slice of a wider tensor.
+    One kernel when the extents are exactly doubled, the two separate ones otherwise."""
+    dev = _lib.require_device(x, gy)
+    B, h, w, I = x.shape
+    H, W = gy.shape[1], gy.shape[2]
+    if H == 2 * h and W == 2 * w and h >= 2 and w >= 2:
+        gx = torch.empty_like(x)
+        if gx.numel():
+            _launch("pdw_bilinear_gate_bwd", dev, gy.data_ptr(), x.data_ptr(), gx.data_ptr(), B, h, w, I, H, W,
+                    _pixel_stride(gy), _lib.dtype_code(x.dtype))
+        return gx
+    return gate_backward(x, bilinear_backward(gy, (h, w)))
+
+
 def spatial_sum(x):
     """x [B, ..., C] -> fp32 [B, C]: sum over all middle dimensions."""
     dev = _lib.require_device(x)

@@ -111,6 +111,35 @@ def test_strided_outputs_and_accumulate(oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hw,out,I", [((5, 6), (10, 12), 24), ((28, 28), (56, 56), 64), ((4, 5), (9, 11), 6),
+                                      ((14, 14), (28, 28), 256), ((2, 2), (4, 4), 2), ((3, 7), (6, 14), 20)])
+def test_gate_bilinear_fused(oracle, dtype, hw, out, I):
+    """The one-kernel gate+resize pair (forward into a channel slice, backward out of one) against the
+    oracle's gate and bilinear applied in turn, and against the two separate kernels."""
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(I + hw[0])
+    B, G = 2, I // 2
+    x = randn(gen, B, *hw, I).to(dtype)
+    xd = x.cuda()
+    wide = torch.full((B, *out, 2 * G + 8), 3.0, dtype=dtype, device="cuda")
+    dst = wide[..., 8:8 + G]
+    ops.gate_bilinear_forward(xd, out, out=dst)
+    ref = oracle.bilinear_fwd(oracle.gate_fwd(x.double().numpy()), out)
+    assert_close(dst, ref, dtype, "gate+bilinear y")
+    assert torch.all(wide[..., :8] == 3) and torch.all(wide[..., 8 + G:] == 3)
+    two = ops.bilinear_forward(ops.gate_forward(xd), out)
+    assert_close(dst, two.double().cpu().numpy(), dtype, "gate+bilinear y vs separate kernels")
+    g = randn(gen, B, *out, 2 * G + 8).to(dtype)
+    gs = g.cuda()[..., 8:8 + G]
+    gx = ops.bilinear_gate_backward(xd, gs)
+    gref = oracle.gate_bwd(x.double().numpy(), oracle.bilinear_bwd(g[..., 8:8 + G].double().numpy(), hw))
+    assert_close(gx, gref, dtype, "gate+bilinear dx")
+    gtwo = ops.gate_backward(xd, ops.bilinear_backward(gs, hw))
+    assert_close(gx, gtwo.double().cpu().numpy(), dtype, "gate+bilinear dx vs separate kernels")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(3, 7, 9, 20), (32, 56, 56, 128), (2, 57, 61, 200), (1, 1, 1, 4), (5, 33, 2, 3)])
 def test_spatial_sum_and_rowbias(dtype, shape):
     from pyramidconvblock_amd import ops
