@@ -53,6 +53,16 @@ int pdw_dwconv_fwd(const void *x, const void *w, void *y, int B, int H, int W, i
 int pdw_dwconv_dgrad(const void *gy, const void *w, void *dx, int B, int H, int W, int C, int KH, int KW,
                      int SH, int SW, int PH, int PW, int DH, int DW, int dtype, void *stream);
 
+/* pdw_dwconv_dgrad plus the gradient of an adaptive average pool taken of the same tensor:
+ * dx[B,H,W,C] = dgrad(gy) + avgpool_bwd(gp[B,h,wp,C] -> (H,W)).  This is the sum autograd forms for the
+ * tensor that feeds both the full-resolution gate and, through conv_block.py:14, a pooled one
+ * (conv_block.py:41).  One kernel when the pool halves both extents exactly (stride 1, dilation 1, 16-bit
+ * types, C % 8 == 0), otherwise pdw_dwconv_dgrad followed by an accumulating pdw_avgpool_bwd; either way dx is
+ * rounded to the storage type after each of the two terms. */
+int pdw_dwconv_dgrad_addpool(const void *gy, const void *w, const void *gp, void *dx, int B, int H, int W, int C,
+                             int KH, int KW, int SH, int SW, int PH, int PW, int DH, int DW, int h, int wp,
+                             int dtype, void *stream);
+
 /* Bytes of device scratch pdw_dwconv_wgrad needs for these extents (fp32 partial sums). */
 size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW,
                                         int PH, int PW, int DH, int DW, int dtype);

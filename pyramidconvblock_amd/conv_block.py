@@ -176,7 +176,10 @@ class ConvBlockFunction(torch.autograd.Function):
 
         da = None
         grad_w_dw = [None] * ns
-        order = sorted(range(ns), key=lambda i: scales[i] != 1.)   # dense gates first: they initialise da
+        # pooled branches first: the gradient of one of them is added inside the input-gradient kernel of the
+        # first full-resolution branch, the others are accumulated into its result
+        order = sorted(range(ns), key=lambda i: scales[i] == 1.)
+        waiting = []                                               # pooled gradients not yet added to da
         for i in order:
             s = scales[i]
             w = w_dw[i].detach().to(dt).contiguous()
@@ -191,14 +194,17 @@ class ConvBlockFunction(torch.autograd.Function):
                 gc = ops.gate_backward(c, dslice)
                 src = a
             grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo).to(w_dw[i].dtype)
-            dp = dwconv_dgrad(gc, w, src.shape, *geo)
             if s != 1.:
-                if da is None:
-                    da = ops.avgpool_backward(dp, (H, W))
-                else:
-                    ops.avgpool_backward(dp, (H, W), out=da, accumulate=True)
+                waiting.append(dwconv_dgrad(gc, w, src.shape, *geo))
+            elif da is None:
+                da = dwconv_dgrad(gc, w, src.shape, *geo, pooled_grad=waiting.pop() if waiting else None)
             else:
-                da = dp if da is None else da.add_(dp)
+                da.add_(dwconv_dgrad(gc, w, src.shape, *geo))
+        for dp in waiting:
+            if da is None:
+                da = ops.avgpool_backward(dp, (H, W))
+            else:
+                ops.avgpool_backward(dp, (H, W), out=da, accumulate=True)
         a2d = da.view(N, I)
         grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
         dx = None

@@ -95,6 +95,25 @@ int pdw_dwconv_dgrad(const void* gy, const void* w, void* dx, int B, int H, int 
                                       (hipStream_t)stream);
 }
 
+int pdw_dwconv_dgrad_addpool(const void* gy, const void* w, const void* gp, void* dx, int B, int H, int W, int C, int KH,
+                             int KW, int SH, int SW, int PH, int PW, int DH, int DW, int h, int wp, int dtype,
+                             void* stream) {
+    if (int e = check_conv("pdw_dwconv_dgrad_addpool", gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype))
+        return e;
+    if (int e = check_resample("pdw_dwconv_dgrad_addpool", gp, dx, B, H, W, C, h, wp, dtype)) return e;
+    if (B == 0) return 0;
+    if (SH == 1 && SW == 1 && DH == 1 && DW == 1 && PH <= KH - 1 && PW <= KW - 1 && H == 2 * h && W == 2 * wp) {
+        const int OH = conv_out_size(H, KH, 1, PH, 1), OW = conv_out_size(W, KW, 1, PW, 1);
+        if (OH > 0 && OW > 0) {
+            const int r = dwconv_tiled_launch(gy, w, dx, B, OH, OW, C, KH, KW, KH - 1 - PH, KW - 1 - PW, true, dtype,
+                                              (hipStream_t)stream, gp);
+            if (r != -1) return r;
+        }
+    }
+    if (int e = pdw_dwconv_dgrad(gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype, stream)) return e;
+    return avgpool_bwd_launch(gp, dx, B, H, W, C, h, wp, 1, dtype, (hipStream_t)stream);
+}
+
 size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW,
                                         int DH, int DW, int dtype) {
     if (check_conv("pdw_dwconv_wgrad_workspace_bytes", "", "", "", B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype))

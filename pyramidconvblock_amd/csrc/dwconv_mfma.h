@@ -21,11 +21,10 @@
 // the B operand of an even output column two consecutive dwords.  The odd column next to it uses the SAME
 // operand with the filter shifted by one column (w'[v+1] = w[v], which still fits the padded width because K is
 // odd), so the inner loop has no vector-ALU work at all: a 4x4x4 MFMA occupies the SIMD for 8 cycles and every
-// vector instruction next to it for 4 more.  Workgroups are persistent, one per CU, and software-pipelined over their tiles: while tile i is
-// multiplied out of one LDS buffer, the window of tile i+1 is requested into registers (phase 0) and written
-// to the other buffer a pass per phase, and the results of tile i-1 leave a few stores per phase, so the
-// matrix pipe of a SIMD sees one long stream of MFMAs with the vector, LDS and memory work in its shadow.
-// With NBUF = 1 (windows too large for two buffers) the window is written between the tiles instead.
+// vector instruction next to it for 4 more.  Workgroups are persistent over their tiles: the filter operands are
+// built in LDS once, a tile's window is requested into registers as early as possible (the first before the
+// filter is staged, the next ones as soon as the operand registers are free) and written to LDS in passes,
+// and the results leave through LDS as 16-byte stores.
 #pragma once
 #include <stdlib.h>
 
@@ -46,6 +45,19 @@ __device__ __forceinline__ f32x4 mfma4(uint2 a, uint2 b, f32x4 c, f16_t) {
     return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
 }
 
+// 8 values of T: a + b / 4, rounded once more (what an accumulating pool gradient does to a stored tensor).
+template <typename T>
+__device__ __forceinline__ uint4 add_quarter(uint4 a, uint4 b) {
+    union U {
+        uint4 u;
+        T t[8];
+    } ua, ub, uo;
+    ua.u = a, ub.u = b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) uo.t[i] = from_f32<T>(to_f32(ua.t[i]) + 0.25f * to_f32(ub.t[i]));
+    return uo.u;
+}
+
 struct MfmaGeom {
     int H, W, C;      // input extents
     int OH, OW;       // output extents
@@ -53,6 +65,7 @@ struct MfmaGeom {
     int tiles_h, tiles_w, ntiles, nchunks, slices;
     int CPn;          // LDS dwords per channel row (>= staged column pairs)
     int flip;         // 1: 180-degree rotated filter (input gradient)
+    int AH, AW;       // extents of the half-resolution addend (OH = 2 AH, OW = 2 AW), 0 without one
     int one;          // the constant 1 (see the kernel)
 };
 
@@ -69,9 +82,10 @@ struct MfmaShape {
                                                     // the zero filter columns included (0 * garbage could be NaN)
 };
 
-template <typename T, int K, int S, int NWV>
+template <typename T, int K, int S, int NWV, bool ADD>
 __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(const T* __restrict__ x, const T* __restrict__ w,
-                                                             T* __restrict__ y, const MfmaGeom g) {
+                                                             const T* __restrict__ add, T* __restrict__ y,
+                                                             const MfmaGeom g) {
     using Sh = MfmaShape<K, S, NWV>;
     constexpr int V = 8, NT = NWV * 64, CS = Sh::CS, TH = Sh::TH, TW = Sh::TW;
     constexpr int KP = Sh::KP, NVB = Sh::NVB, NPH = Sh::NPH, WR = Sh::WR, ROWS_IN = Sh::ROWS_IN, NCOL = Sh::NCOL;
@@ -221,6 +235,7 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         }
         // ---- results -> LDS as yl[row][column][16 channels] (one rounding to T), then out in 16-byte pieces:
         // the 2-byte values a lane owns are 4 rows x S scattered pixels, far too many store instructions.
+        constexpr int NIT = (TH * TW * 2 + NT - 1) / NT;  // 16-byte pieces (8 channels of a pixel) per thread
         __syncthreads();  // every wavefront is done reading the window
         T* yl = reinterpret_cast<T*>(smem);
         if (active) {
@@ -230,18 +245,35 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
 #pragma unroll
                 for (int t = 0; t < S; ++t) yq[(m * TW + t) * CS] = from_f32<T>(acc[t][m]);
         }
+        // The addend (gradient of a 2x2 average pool taken of the same tensor: a quarter of the pooled gradient at
+        // every pixel of its window) is requested once the accumulators are free.
+        uint4 av[NIT];
+        if constexpr (ADD) {
+            __builtin_amdgcn_sched_barrier(0);
+            const T* ab = add + ((long long)b * g.AH * g.AW) * g.C + c0;
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int idx = tid + it * NT;
+                const int half = idx & 1, pix = idx >> 1;
+                const int r = pix / TW, cc = pix - r * TW;
+                const int ar = min((orow0 + r) >> 1, g.AH - 1), ac = min((ocol0 + cc) >> 1, g.AW - 1);
+                const int ach = min(8 * half, g.C - c0 - 8);  // C % 8 == 0: always a whole piece inside the tensor
+                av[it] = *reinterpret_cast<const uint4*>(ab + ((long long)ar * g.AW + ac) * g.C + ach);
+            }
+        }
         __syncthreads();
         {
-            constexpr int NIT = (TH * TW * 2 + NT - 1) / NT;  // 16-byte pieces (8 channels of a pixel) per thread
             T* yb = y + ((long long)b * g.OH * g.OW) * g.C + c0;
 #pragma unroll
             for (int it = 0; it < NIT; ++it) {
                 const int idx = tid + it * NT;
                 const int half = idx & 1, pix = idx >> 1;
                 const int r = pix / TW, cc = pix - r * TW;
-                if (pix < TH * TW && orow0 + r < g.OH && ocol0 + cc < g.OW && c0 + 8 * half < g.C)
-                    *reinterpret_cast<uint4*>(yb + ((long long)(orow0 + r) * g.OW + ocol0 + cc) * g.C + 8 * half) =
-                        *reinterpret_cast<const uint4*>(yl + pix * CS + 8 * half);
+                if (pix < TH * TW && orow0 + r < g.OH && ocol0 + cc < g.OW && c0 + 8 * half < g.C) {
+                    uint4 o = *reinterpret_cast<const uint4*>(yl + pix * CS + 8 * half);
+                    if constexpr (ADD) o = add_quarter<T>(o, av[it]);
+                    *reinterpret_cast<uint4*>(yb + ((long long)(orow0 + r) * g.OW + ocol0 + cc) * g.C + 8 * half) = o;
+                }
             }
         }
         if (has_next) {  // the next window is requested only now: its registers were the operand registers above
@@ -255,12 +287,13 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
 // Host side
 
 template <typename T, int K, int S, int NWV>
-static int launch_mfma(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW, bool flip,
-                       hipStream_t s) {
+static int launch_mfma(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH,
+                       int PW, bool flip, hipStream_t s) {
     using Sh = MfmaShape<K, S, NWV>;
     MfmaGeom g;
     g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0, g.one = 1;
     g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
+    g.AH = add ? g.OH / 2 : 0, g.AW = add ? g.OW / 2 : 0;
     g.slices = cdiv(C, Sh::CS);
     g.tiles_h = cdiv(g.OH, Sh::TH), g.tiles_w = cdiv(g.OW, Sh::TW);
     const long long ntiles = (long long)B * g.tiles_h * g.tiles_w;
@@ -285,23 +318,25 @@ static int launch_mfma(const void* x, const void* w, void* y, int B, int H, int 
     if (getenv("PDW_MFMA_NCH")) nch = atoi(getenv("PDW_MFMA_NCH"));
     g.nchunks = (int)(nch < 1 ? 1 : nch);
     const long long nblocks = (long long)g.nchunks * g.slices;
-    auto kern = dwconv_mfma_k<T, K, S, NWV>;
-    static bool attr_done = false;
-    if (!attr_done) {
+    auto kern = add ? dwconv_mfma_k<T, K, S, NWV, true> : dwconv_mfma_k<T, K, S, NWV, false>;
+    static bool attr_done[2] = {false, false};
+    if (!attr_done[add ? 1 : 0]) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_done = true;
+        attr_done[add ? 1 : 0] = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NWV * 64), lds, s, (const T*)x, (const T*)w, (T*)y, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NWV * 64), lds, s, (const T*)x, (const T*)w, (const T*)add,
+                       (T*)y, g);
     return check_launch("dwconv_mfma");
 }
 
 // -1: not covered (the caller falls back to the vector-ALU tiled kernel).
 template <typename T, int K>
-static int launch_mfma_best(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW,
-                            bool flip, hipStream_t s) {
+static int launch_mfma_best(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH,
+                            int PW, bool flip, hipStream_t s) {
     const int OH = H + 2 * PH - K + 1, OW = W + 2 * PW - K + 1;
     if (OH < 1 || OW < 1 || C % 8 != 0) return -1;
     if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return -1;
+    if (add && ((OH | OW) & 1 || (reinterpret_cast<uintptr_t>(add) & 15) != 0)) return -1;
     // strips of 14 columns (tile 56 wide) or 8 (tile 32 wide): whichever pads the output width less
     const bool s14 = (long long)cdiv(OW, 56) * 56 <= (long long)cdiv(OW, 32) * 32;
     const int tw = s14 ? 56 : 32;
@@ -310,19 +345,19 @@ static int launch_mfma_best(const void* x, const void* w, void* y, int B, int H,
     bool w8 = t8 >= 192;
     if (getenv("PDW_MFMA_NWV")) w8 = atoi(getenv("PDW_MFMA_NWV")) == 8;
     if (s14) {
-        if (w8) return launch_mfma<T, K, 14, 8>(x, w, y, B, H, W, C, PH, PW, flip, s);
-        return launch_mfma<T, K, 14, 4>(x, w, y, B, H, W, C, PH, PW, flip, s);
+        if (w8) return launch_mfma<T, K, 14, 8>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
+        return launch_mfma<T, K, 14, 4>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
     }
-    if (w8) return launch_mfma<T, K, 8, 8>(x, w, y, B, H, W, C, PH, PW, flip, s);
-    return launch_mfma<T, K, 8, 4>(x, w, y, B, H, W, C, PH, PW, flip, s);
+    if (w8) return launch_mfma<T, K, 8, 8>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
+    return launch_mfma<T, K, 8, 4>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
 }
 
 template <int K>
-static int launch_mfma_dtype(const void* x, const void* w, void* y, int B, int H, int W, int C, int PH, int PW,
-                             bool flip, int dtype, hipStream_t s) {
+static int launch_mfma_dtype(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH,
+                             int PW, bool flip, int dtype, hipStream_t s) {
     switch (dtype) {
-        case kF16: return launch_mfma_best<f16_t, K>(x, w, y, B, H, W, C, PH, PW, flip, s);
-        case kBF16: return launch_mfma_best<bf16_t, K>(x, w, y, B, H, W, C, PH, PW, flip, s);
+        case kF16: return launch_mfma_best<f16_t, K>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
+        case kBF16: return launch_mfma_best<bf16_t, K>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
         default: return -1;
     }
 }

@@ -40,17 +40,29 @@ def dwconv_forward(x, weight, stride, padding, dilation):
     return y
 
 
-def dwconv_dgrad(gy, weight, in_shape, stride, padding, dilation):
+def dwconv_dgrad(gy, weight, in_shape, stride, padding, dilation, pooled_grad=None):
+    """dx[in_shape]; with pooled_grad [B,h,w,C] the gradient of an adaptive average pool of the same
+    tensor to (h, w) is added to it."""
     dev = _lib.require_device(gy, weight)
     L = _lib.lib()
     dx = torch.empty(in_shape, device=dev, dtype=gy.dtype)
     if dx.numel():
         if gy.numel() == 0:
-            return dx.zero_()
+            dx.zero_()
+            if pooled_grad is not None and pooled_grad.numel():
+                from . import ops
+                ops.avgpool_backward(pooled_grad, (in_shape[1], in_shape[2]), out=dx, accumulate=True)
+            return dx
         args = _conv_args(in_shape, weight.shape, stride, padding, dilation)
         with _lib.on_device(dev):
-            _lib.check(L.pdw_dwconv_dgrad(gy.data_ptr(), weight.data_ptr(), dx.data_ptr(), *args,
-                                          _lib.dtype_code(gy.dtype), _lib.stream_ptr(dev)), "pdw_dwconv_dgrad")
+            if pooled_grad is None:
+                _lib.check(L.pdw_dwconv_dgrad(gy.data_ptr(), weight.data_ptr(), dx.data_ptr(), *args,
+                                              _lib.dtype_code(gy.dtype), _lib.stream_ptr(dev)), "pdw_dwconv_dgrad")
+            else:
+                gp = pooled_grad.contiguous()
+                _lib.check(L.pdw_dwconv_dgrad_addpool(gy.data_ptr(), weight.data_ptr(), gp.data_ptr(), dx.data_ptr(),
+                                                      *args, gp.shape[1], gp.shape[2], _lib.dtype_code(gy.dtype),
+                                                      _lib.stream_ptr(dev)), "pdw_dwconv_dgrad_addpool")
     return dx
 
 

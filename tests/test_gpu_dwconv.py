@@ -133,3 +133,23 @@ def test_full_size_properties(dtype):
     tol = 5e-3 if dtype != torch.float32 else 1e-4
     assert abs(float((dx.double() * x.double()).sum()) - lhs) <= tol * abs(lhs)
     assert abs(float((dw.double() * w.double()).sum()) - lhs) <= tol * abs(lhs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 16, 24, 32, 13, (8, 12)), (1, 56, 56, 24, 9, (28, 28)), (2, 12, 10, 8, 3, (6, 5)),
+                                   (2, 14, 18, 16, 5, (5, 7)), (1, 40, 36, 12, 7, (20, 18)), (3, 9, 9, 8, 5, (4, 4))])
+def test_dgrad_with_pooled_gradient(oracle, dtype, shape):
+    """Input gradient plus the gradient of an average pool of the same tensor: the fused kernel (exact
+    halving, 16-bit, C % 8 == 0) and the two-kernel path behind the same entry point."""
+    from pyramidconvblock_amd.dwconv import dwconv_dgrad
+
+    B, H, W, C, k, hw = shape
+    gen = torch.Generator().manual_seed(H * W + k)
+    g = randn(gen, B, H, W, C).to(dtype)
+    w = (randn(gen, k, k, C) / k).to(dtype)
+    gp = randn(gen, B, *hw, C).to(dtype)
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    dx = dwconv_dgrad(g.cuda(), w.cuda(), (B, H, W, C), *geo, pooled_grad=gp.cuda())
+    ref = (oracle.dwconv_dgrad(g.double().numpy(), w.double().numpy(), (H, W), 1, k // 2, 1)
+           + oracle.avgpool_bwd(gp.double().numpy(), (H, W)))
+    assert_close(dx, ref, dtype, "dgrad + pooled gradient")
