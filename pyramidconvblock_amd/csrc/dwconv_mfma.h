@@ -300,13 +300,14 @@ static int launch_mfma(const void* x, const void* w, const void* add, void* y, i
     if (ntiles > 0x7fffffffLL || (long long)H * W * C > 0x7fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL)
         return -1;
     g.ntiles = (int)ntiles;
-    // LDS: pitch = pairs per channel row; 4 mod 8 keeps the 16 channels x 4 strips of an operand read on
-    // distinct banks when that fits.
+    // LDS: pitch = pairs per channel row.  A lane's operand reads start at pitch * channel + S/2 * strip: measured
+    // on the part, a pitch of 4 mod 8 is free of bank conflicts for strips of 14 columns, an odd one for strips of 8.
     const size_t wbytes = (size_t)2 * Sh::WR * (16 * Sh::NVB + 8) * 8;
     auto lds_of = [&](int p) { return (size_t)Sh::ROWS_IN * Sh::CS * p * 4 + wbytes; };
     int pitch = Sh::NCOL;
-    while (pitch % 8 != 4) ++pitch;
+    while (S == 14 ? pitch % 8 != 4 : pitch % 2 != 1) ++pitch;
     if (lds_of(pitch) > 160 * 1024) pitch = Sh::NCOL;
+    if (getenv("PDW_MFMA_PITCH") && atoi(getenv("PDW_MFMA_PITCH")) >= Sh::NCOL) pitch = atoi(getenv("PDW_MFMA_PITCH"));
     if (lds_of(pitch) > 160 * 1024) return -1;
     g.CPn = pitch;
     const size_t lds = lds_of(pitch);

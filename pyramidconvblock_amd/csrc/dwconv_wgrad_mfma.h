@@ -247,6 +247,8 @@ static WgradMfmaPlan plan_wgrad_mfma(int B, int H, int W, int C, int PH, int PW)
         return n;
     };
     g.XP = pad(g.TW / 2 + 4 * Sh::NVG), g.GP = pad(g.TW / 2);
+    if (getenv("PDW_WG_XP") && atoi(getenv("PDW_WG_XP")) >= g.TW / 2 + 4 * Sh::NVG) g.XP = atoi(getenv("PDW_WG_XP"));
+    if (getenv("PDW_WG_GP") && atoi(getenv("PDW_WG_GP")) >= g.TW / 2) g.GP = atoi(getenv("PDW_WG_GP"));
     auto lds_of = [&](int th) { return ((size_t)(th + K - 1) * Sh::CS * g.XP + (size_t)th * (Sh::CS * g.GP + 1)) * 4; };
     // tile height: about one tile per CU, within LDS and the staging registers
     long long want_h = ((long long)B * g.slices * g.tiles_w + 255) / 256;  // images*slices per CU column
