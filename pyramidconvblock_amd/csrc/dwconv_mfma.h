@@ -210,17 +210,27 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
                 Ops oa, ob;
                 fetch(oa, xr, wr);
                 static_assert(NPH % 2 == 0, "phases are processed in pairs");
+                // LDS reads of the next phase interleaved with the MFMAs of this one, one read per MPR MFMAs: issued
+                // in a block they would leave the matrix pipe idle, a wavefront issues in order
+                constexpr int NLD = NE + 2 * NVB + NVB, MPR = (2 * NE * NVB) / NLD > 1 ? (2 * NE * NVB) / NLD : 1;
+                auto interleave = [&]() {
+#pragma unroll
+                    for (int i = 0; i < NLD; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+                    }
+                };
 #pragma unroll 1
                 for (int p = 0; p < NPH; p += 2) {
                     xr += RP, wr += WPITCH;
                     fetch(ob, xr, wr);
-                    __builtin_amdgcn_sched_barrier(0);
                     multiply(oa);
+                    interleave();
                     __builtin_amdgcn_sched_barrier(0);
                     xr += RP, wr += WPITCH;
-                    if (p + 2 < NPH) fetch(oa, xr, wr);
-                    __builtin_amdgcn_sched_barrier(0);
+                    fetch(oa, xr, wr);  // after the last phase: one row past the window and the filter, unused
                     multiply(ob);
+                    interleave();
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
@@ -302,7 +312,7 @@ static int launch_mfma(const void* x, const void* w, const void* add, void* y, i
     g.ntiles = (int)ntiles;
     // LDS: pitch = pairs per channel row.  A lane's operand reads start at pitch * channel + S/2 * strip: measured
     // on the part, a pitch of 4 mod 8 is free of bank conflicts for strips of 14 columns, an odd one for strips of 8.
-    const size_t wbytes = (size_t)2 * Sh::WR * (16 * Sh::NVB + 8) * 8;
+    const size_t wbytes = (size_t)(2 * Sh::WR + 1) * (16 * Sh::NVB + 8) * 8;  // + the row the last prefetch reads
     auto lds_of = [&](int p) { return (size_t)Sh::ROWS_IN * Sh::CS * p * 4 + wbytes; };
     int pitch = Sh::NCOL;
     while (S == 14 ? pitch % 8 != 4 : pitch % 2 != 1) ++pitch;
@@ -310,7 +320,8 @@ static int launch_mfma(const void* x, const void* w, const void* add, void* y, i
     if (getenv("PDW_MFMA_PITCH") && atoi(getenv("PDW_MFMA_PITCH")) >= Sh::NCOL) pitch = atoi(getenv("PDW_MFMA_PITCH"));
     if (lds_of(pitch) > 160 * 1024) return -1;
     g.CPn = pitch;
-    const size_t lds = lds_of(pitch);
+    size_t lds = lds_of(pitch);
+    if (getenv("PDW_MFMA_LDSMIN") && lds < (size_t)atoi(getenv("PDW_MFMA_LDSMIN"))) lds = atoi(getenv("PDW_MFMA_LDSMIN"));
     // persistent workgroups: as many as are resident at once, tiles dealt out as evenly as they divide
     const int resident = (int)((160 * 1024) / (lds + 1024)) >= 2 && NWV == 4 ? 2 : 1;
     const int cap = (256 * resident) / g.slices > 1 ? (256 * resident) / g.slices : 1;
