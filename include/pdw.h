@@ -63,6 +63,16 @@ int pdw_dwconv_dgrad_addpool(const void *gy, const void *w, const void *gp, void
                              int KH, int KW, int SH, int SW, int PH, int PW, int DH, int DW, int h, int wp,
                              int dtype, void *stream);
 
+/* The weight-gradient entry points (pdw_dwconv_wgrad, pdw_dense_wgrad) end with a small kernel that sums their
+ * fp32 partial results.  Between pdw_reduce_defer_begin() and pdw_reduce_defer_flush(stream), on the calling host
+ * thread, that last step is only recorded (up to 8 of them, further ones run at once as usual), and the flush
+ * runs all recorded ones in a single launch on `stream`: the outputs are not valid, and the workspaces must not
+ * be reused or freed, until then.  No counterpart in the reference (its backward launches every kernel
+ * separately, dwconv_triton.py:358-385); the ConvBlock backward (conv_block.py:36-49 under autograd) uses it
+ * for its four weight gradients. */
+int pdw_reduce_defer_begin(void);
+int pdw_reduce_defer_flush(void *stream);
+
 /* Bytes of device scratch pdw_dwconv_wgrad needs for these extents (fp32 partial sums). */
 size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW,
                                         int PH, int PW, int DH, int DW, int dtype);

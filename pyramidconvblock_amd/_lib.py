@@ -6,6 +6,7 @@ tensor is not on a HIP device, the operators raise.
 from __future__ import annotations
 
 import ctypes
+import threading
 import os
 from ctypes import c_char_p, c_int, c_longlong, c_size_t, c_void_p
 
@@ -26,6 +27,8 @@ _SIGS = {
     "pdw_conv_out_size": (c_int, [c_int] * 5),
     "pdw_dwconv_fwd": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
     "pdw_dwconv_dgrad": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
+    "pdw_reduce_defer_begin": (c_int, []),
+    "pdw_reduce_defer_flush": (c_int, [c_void_p]),
     "pdw_dwconv_dgrad_addpool": (c_int, [c_void_p] * 4 + _CONV + [c_int, c_int, c_int, c_void_p]),
     "pdw_dwconv_wgrad_workspace_bytes": (c_size_t, _CONV + [c_int]),
     "pdw_dwconv_wgrad": (c_int, [c_void_p] * 4 + [c_size_t] + _CONV + [c_int, c_void_p]),
@@ -113,3 +116,34 @@ class on_device:
         if self.prev is not None:
             torch.cuda.set_device(self.prev)
         return False
+
+
+_defer = threading.local()
+
+
+class deferred_reductions:
+    """Within the block the final summation kernels of the weight-gradient calls are recorded and then run in one
+    launch on `dev`'s current stream at exit; their results must not be read (or converted) before that."""
+
+    def __init__(self, dev: torch.device):
+        self.dev = dev
+
+    def __enter__(self):
+        check(lib().pdw_reduce_defer_begin(), "pdw_reduce_defer_begin")
+        _defer.keep = []
+        return self
+
+    def __exit__(self, *exc):
+        try:
+            with on_device(self.dev):
+                check(lib().pdw_reduce_defer_flush(stream_ptr(self.dev)), "pdw_reduce_defer_flush")
+        finally:
+            _defer.keep = None
+        return False
+
+
+def keep_until_flush(t: torch.Tensor) -> None:
+    """A workspace whose contents a deferred reduction still has to read stays referenced until the flush."""
+    keep = getattr(_defer, "keep", None)
+    if keep is not None:
+        keep.append(t)

@@ -167,56 +167,61 @@ class ConvBlockFunction(torch.autograd.Function):
         grad_b_pool = gbias.to(w_pool.dtype) if ctx.has_bias[2] else None
 
         fast_up, fast_out = ctx.fast
-        if fast_out:
-            dcat = ops.dense_forward(gy, w_out.detach().contiguous(), w_kmajor=True)
-            grad_w_out = ops.dense_wgrad(gy, cat).to(w_out.dtype)
-        else:
-            dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
-            grad_w_out = _weight_grad(g2d, cat.view(N, G * ns)).to(w_out.dtype)
+        # the four weight gradients end in a small summation kernel each: they are run as one launch at the end
+        with _lib.deferred_reductions(gy.device):
+            if fast_out:
+                dcat = ops.dense_forward(gy, w_out.detach().contiguous(), w_kmajor=True)
+                grad_w_out = ops.dense_wgrad(gy, cat)
+            else:
+                dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
+                grad_w_out = _weight_grad(g2d, cat.view(N, G * ns))
 
-        da = None
-        grad_w_dw = [None] * ns
-        # pooled branches first: the gradient of one of them is added inside the input-gradient kernel of the
-        # first full-resolution branch, the others are accumulated into its result
-        order = sorted(range(ns), key=lambda i: scales[i] == 1.)
-        waiting = []                                               # pooled gradients not yet added to da
-        for i in order:
-            s = scales[i]
-            w = w_dw[i].detach().to(dt).contiguous()
-            k1, k2 = w.shape[0], w.shape[1]
-            geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
-            dslice = dcat[..., i * G:(i + 1) * G]
-            c = convs[i]
-            if s != 1.:
-                gc = ops.bilinear_gate_backward(c, dslice)
-                src = pooled[i]
+            da = None
+            grad_w_dw = [None] * ns
+            # pooled branches first: the gradient of one of them is added inside the input-gradient kernel of the
+            # first full-resolution branch, the others are accumulated into its result
+            order = sorted(range(ns), key=lambda i: scales[i] == 1.)
+            waiting = []                                               # pooled gradients not yet added to da
+            for i in order:
+                s = scales[i]
+                w = w_dw[i].detach().to(dt).contiguous()
+                k1, k2 = w.shape[0], w.shape[1]
+                geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
+                dslice = dcat[..., i * G:(i + 1) * G]
+                c = convs[i]
+                if s != 1.:
+                    gc = ops.bilinear_gate_backward(c, dslice)
+                    src = pooled[i]
+                else:
+                    gc = ops.gate_backward(c, dslice)
+                    src = a
+                grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo)
+                if s != 1.:
+                    waiting.append(dwconv_dgrad(gc, w, src.shape, *geo))
+                elif da is None:
+                    da = dwconv_dgrad(gc, w, src.shape, *geo, pooled_grad=waiting.pop() if waiting else None)
+                else:
+                    da.add_(dwconv_dgrad(gc, w, src.shape, *geo))
+            for dp in waiting:
+                if da is None:
+                    da = ops.avgpool_backward(dp, (H, W))
+                else:
+                    ops.avgpool_backward(dp, (H, W), out=da, accumulate=True)
+            a2d = da.view(N, I)
+            grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
+            dx = None
+            if fast_up:
+                grad_w_up = ops.dense_wgrad(da, x)
+                if ctx.needs_input_grad[0]:
+                    dx = ops.dense_forward(da, w_up.detach().contiguous(), w_kmajor=True, rowbias=dmean,
+                                           rows_per_image=H * W)
             else:
-                gc = ops.gate_backward(c, dslice)
-                src = a
-            grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo).to(w_dw[i].dtype)
-            if s != 1.:
-                waiting.append(dwconv_dgrad(gc, w, src.shape, *geo))
-            elif da is None:
-                da = dwconv_dgrad(gc, w, src.shape, *geo, pooled_grad=waiting.pop() if waiting else None)
-            else:
-                da.add_(dwconv_dgrad(gc, w, src.shape, *geo))
-        for dp in waiting:
-            if da is None:
-                da = ops.avgpool_backward(dp, (H, W))
-            else:
-                ops.avgpool_backward(dp, (H, W), out=da, accumulate=True)
-        a2d = da.view(N, I)
-        grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
-        dx = None
-        if fast_up:
-            grad_w_up = ops.dense_wgrad(da, x).to(w_up.dtype)
-            if ctx.needs_input_grad[0]:
-                dx = ops.dense_forward(da, w_up.detach().contiguous(), w_kmajor=True, rowbias=dmean,
-                                       rows_per_image=H * W)
-        else:
-            grad_w_up = _weight_grad(a2d, x.view(N, D)).to(w_up.dtype)
-            if ctx.needs_input_grad[0]:
-                dx = ops.add_rowbias_(torch.matmul(a2d, w_up).view(B, H, W, D), dmean)
+                grad_w_up = _weight_grad(a2d, x.view(N, D))
+                if ctx.needs_input_grad[0]:
+                    dx = ops.add_rowbias_(torch.matmul(a2d, w_up).view(B, H, W, D), dmean)
+        grad_w_out = grad_w_out.to(w_out.dtype)
+        grad_w_up = grad_w_up.to(w_up.dtype)
+        grad_w_dw = [g.to(w_dw[i].dtype) for i, g in enumerate(grad_w_dw)]
         return (dx, None, grad_w_up, grad_b_up, grad_w_out, grad_b_out, grad_w_pool, grad_b_pool, *grad_w_dw)
 
 

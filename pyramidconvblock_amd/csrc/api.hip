@@ -114,6 +114,10 @@ int pdw_dwconv_dgrad_addpool(const void* gy, const void* w, const void* gp, void
     return avgpool_bwd_launch(gp, dx, B, H, W, C, h, wp, 1, dtype, (hipStream_t)stream);
 }
 
+int pdw_reduce_defer_begin(void) { return reduce_defer_begin(); }
+
+int pdw_reduce_defer_flush(void* stream) { return reduce_defer_flush((hipStream_t)stream); }
+
 size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW,
                                         int DH, int DW, int dtype) {
     if (check_conv("pdw_dwconv_wgrad_workspace_bytes", "", "", "", B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype))

@@ -123,11 +123,10 @@ __global__ __launch_bounds__(256) void dwconv_wgrad_direct(const T* __restrict__
 // Block = 32 outputs x 8 part lanes; lane q adds parts q, q+8, ... and the 8 lanes are combined
 // through LDS, so the reads of one part are contiguous and many parts are in flight.
 template <typename T>
-__global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restrict__ part, T* __restrict__ dw,
-                                                          int nparts, int n) {
-    __shared__ float red[8][32];
+__device__ __forceinline__ void reduce_parts_block(const float* __restrict__ part, T* __restrict__ dw, int nparts, int n,
+                                                   int blk, float (*red)[32]) {
     const int el = threadIdx.x & 31, q = threadIdx.x >> 5;
-    const int e = blockIdx.x * 32 + el;
+    const int e = blk * 32 + el;
     float s0 = 0.f, s1 = 0.f;
     if (e < n) {
         int p = q;
@@ -151,6 +150,63 @@ __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restric
                         ((red[4][el] + red[5][el]) + (red[6][el] + red[7][el]));
         dw[e] = from_f32<T>(s);
     }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restrict__ part, T* __restrict__ dw,
+                                                          int nparts, int n) {
+    __shared__ float red[8][32];
+    reduce_parts_block<T>(part, dw, nparts, n, blockIdx.x, red);
+}
+
+// Several such reductions in one launch: the weight gradients of a backward pass are each a few microseconds of
+// latency, and nothing reads them before the pass is over.
+constexpr int kMaxReduceJobs = 8;
+struct ReduceJobs {
+    const float* part[kMaxReduceJobs];
+    void* out[kMaxReduceJobs];
+    int nparts[kMaxReduceJobs], n[kMaxReduceJobs], dtype[kMaxReduceJobs];
+    int first_block[kMaxReduceJobs + 1];
+    int njobs;
+};
+
+__global__ __launch_bounds__(256) void wgrad_reduce_many(const ReduceJobs jobs) {
+    __shared__ float red[8][32];
+    int j = 0;
+    while (j + 1 < jobs.njobs && (int)blockIdx.x >= jobs.first_block[j + 1]) ++j;  // uniform: scalar ALU
+    const int blk = blockIdx.x - jobs.first_block[j];
+    switch (jobs.dtype[j]) {
+        case kF32: reduce_parts_block<float>(jobs.part[j], (float*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
+        case kF16: reduce_parts_block<f16_t>(jobs.part[j], (f16_t*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
+        default: reduce_parts_block<bf16_t>(jobs.part[j], (bf16_t*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
+    }
+}
+
+// Deferred mode (per host thread): between reduce_defer_begin and reduce_defer_flush the reductions are only
+// recorded; the flush runs them all in one launch.
+static thread_local bool t_defer = false;
+static thread_local ReduceJobs t_jobs;
+
+int reduce_defer_begin() {
+    if (t_defer) return set_error("pdw_reduce_defer_begin: already deferring on this thread"), 1;
+    t_defer = true;
+    t_jobs.njobs = 0;
+    t_jobs.first_block[0] = 0;
+    return 0;
+}
+
+int reduce_defer_flush(hipStream_t s) {
+    if (!t_defer) return set_error("pdw_reduce_defer_flush: pdw_reduce_defer_begin was not called"), 1;
+    t_defer = false;
+    if (t_jobs.njobs == 0) return 0;
+    hipLaunchKernelGGL(wgrad_reduce_many, dim3(t_jobs.first_block[t_jobs.njobs]), dim3(256), 0, s, t_jobs);
+    t_jobs.njobs = 0;
+    return check_launch("wgrad_reduce_many");
+}
+
+template <typename T>
+static constexpr int dtype_of() {
+    return sizeof(T) == 4 ? kF32 : (__is_same(T, f16_t) ? kF16 : kBF16);
 }
 
 static ConvGeom make_geom(int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW, int DH,
@@ -223,6 +279,13 @@ size_t dwconv_wgrad_direct_workspace(int B, int H, int W, int C, int KH, int KW,
 
 template <typename T>
 int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s) {
+    if (t_defer && t_jobs.njobs < kMaxReduceJobs) {
+        const int j = t_jobs.njobs++;
+        t_jobs.part[j] = part, t_jobs.out[j] = dw, t_jobs.nparts[j] = nparts, t_jobs.n[j] = n;
+        t_jobs.dtype[j] = dtype_of<T>();
+        t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv(n, 32);
+        return 0;
+    }
     hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, 32)), dim3(256), 0, s, part, (T*)dw, nparts, n);
     return check_launch("wgrad_reduce_parts");
 }

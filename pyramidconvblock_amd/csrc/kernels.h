@@ -22,6 +22,8 @@ int dwconv_wgrad_direct_launch(const void* x, const void* gy, void* dw, void* ws
                                hipStream_t s);
 template <typename T>
 int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s);
+int reduce_defer_begin();
+int reduce_defer_flush(hipStream_t s);
 
 // dwconv_tiled.hip: LDS-tiled forward / input gradient for stride 1, dilation 1, odd KW <= 17.
 // Returns -1 if the case is not covered (the caller then uses the direct kernel).

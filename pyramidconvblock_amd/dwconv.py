@@ -79,6 +79,7 @@ def dwconv_wgrad(x, gy, w_shape, stride, padding, dilation):
     with _lib.on_device(dev):
         _lib.check(L.pdw_dwconv_wgrad(x.data_ptr(), gy.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel() * 4,
                                       *args, code, _lib.stream_ptr(dev)), "pdw_dwconv_wgrad")
+    _lib.keep_until_flush(ws)
     return dw
 
 

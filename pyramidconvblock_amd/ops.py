@@ -195,6 +195,7 @@ def dense_wgrad(a, b):
     ws = torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
     _launch("pdw_dense_wgrad", dev, a.data_ptr(), b.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel() * 4, N, M, NO,
             _lib.dtype_code(a.dtype))
+    _lib.keep_until_flush(ws)
     return dw
 
 

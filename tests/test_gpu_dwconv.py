@@ -153,3 +153,31 @@ def test_dgrad_with_pooled_gradient(oracle, dtype, shape):
     ref = (oracle.dwconv_dgrad(g.double().numpy(), w.double().numpy(), (H, W), 1, k // 2, 1)
            + oracle.avgpool_bwd(gp.double().numpy(), (H, W)))
     assert_close(dx, ref, dtype, "dgrad + pooled gradient")
+
+
+def test_deferred_reductions_match_immediate_ones():
+    """Weight gradients whose summation kernels are recorded and run as one launch are bit-identical to the
+    ones computed call by call (more jobs than the table holds included)."""
+    from pyramidconvblock_amd import _lib, ops
+    from pyramidconvblock_amd.dwconv import dwconv_wgrad
+
+    gen = torch.Generator().manual_seed(11)
+    cases = []
+    for (B, H, W, C, k, dt) in [(2, 20, 24, 32, 13, torch.bfloat16), (1, 9, 11, 5, 3, torch.float32),
+                                (2, 16, 16, 16, 9, torch.float16), (1, 30, 30, 8, 5, torch.bfloat16)]:
+        x = randn(gen, B, H, W, C).to(dt).cuda()
+        g = randn(gen, B, H, W, C).to(dt).cuda()
+        cases.append((x, g, (k, k, C), ((1, 1), (k // 2, k // 2), (1, 1))))
+    a = randn(gen, 4096, 64).to(torch.bfloat16).cuda()
+    b = randn(gen, 4096, 128).to(torch.bfloat16).cuda()
+    ref = [dwconv_wgrad(x, g, ws, *geo) for (x, g, ws, geo) in cases] + [ops.dense_wgrad(a, b)]
+    for reps in (1, 3):   # 5 jobs, then 15: beyond the 8 the table holds
+        with _lib.deferred_reductions(a.device):
+            got = []
+            for _ in range(reps):
+                got += [dwconv_wgrad(x, g, ws, *geo) for (x, g, ws, geo) in cases] + [ops.dense_wgrad(a, b)]
+        torch.cuda.synchronize()
+        for i, t in enumerate(got):
+            assert torch.equal(t, ref[i % len(ref)]), i
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.lib().pdw_reduce_defer_flush(None), "flush without begin")
