@@ -128,6 +128,16 @@ int pdw_gate_bilinear_fwd(const void *x, void *y, int B, int h, int w, int I, in
 int pdw_bilinear_gate_bwd(const void *gy, const void *x, void *gx, int B, int h, int w, int I, int H, int W,
                           int ldgy, int dtype, void *stream);
 
+/* The two gates of a block with scales (1, s) in one launch: y[..., 0:G] = gate(xf[B,H,W,I]) and
+ * y[..., G:2G] = bilinear(gate(xh[B,h,w,I])) -> (H,W), G = I/2, pixels of y ldy elements apart (0 = 2G): the
+ * torch.cat of conv_block.py:43 written directly (conv_block.py:18-21 for both entries of self.gates). */
+int pdw_gate_pair_fwd(const void *xf, const void *xh, void *y, int B, int H, int W, int h, int w, int I, int ldy,
+                      int dtype, void *stream);
+/* Its gradient for exactly doubled extents (anything else is an error; the caller then uses the single-branch
+ * entry points): gy[B,H,W,2G] (pixels ldgy apart) -> gxf[B,H,W,I], gxh[B,h,w,I]. */
+int pdw_gate_pair_bwd(const void *gy, const void *xf, const void *xh, void *gxf, void *gxh, int B, int H, int W,
+                      int h, int w, int I, int ldgy, int dtype, void *stream);
+
 /* Per-image sum over positions: x[B,P,C] -> out[B,C] (fp32), two deterministic passes through `workspace`.
  * Replaces x.mean(dim=(1,2)) at conv_block.py:46 (divide by P on the host side) and, in the backward, the
  * reduction of the broadcast add at conv_block.py:49. */
@@ -147,12 +157,14 @@ size_t pdw_pool_branch_workspace_bytes(int B, int P, int D);
 int pdw_pool_branch_fwd(const void *x, const void *w_pool, const void *b_pool, const void *b_out, void *m,
                         float *rowbias, void *workspace, size_t workspace_bytes, int B, int P, int D, int dtype,
                         void *stream);
-/* Its backward from gy[B,P,D]: gbias[o] = sum over all positions of gy (the gradient of both biases),
+/* Its backward from gy[B,P,D]: gbias[o] = sum over all positions of gy (the gradient of both biases; gbias2,
+ * if not null, receives a second copy so that each bias owns its gradient tensor),
  * gw_pool[o,c] = sum_b gs[b,o] * m[b,c] with gs the per-image column sums of gy, and
  * dmean[b,c] = (1/P) * sum_o gs[b,o] * w_pool[o,c] (fp32), the per-image term that the mean's gradient
  * adds to every position of dx. */
-int pdw_pool_branch_bwd(const void *gy, const void *m, const void *w_pool, void *gbias, void *gw_pool, float *dmean,
-                        void *workspace, size_t workspace_bytes, int B, int P, int D, int dtype, void *stream);
+int pdw_pool_branch_bwd(const void *gy, const void *m, const void *w_pool, void *gbias, void *gbias2, void *gw_pool,
+                        float *dmean, void *workspace, size_t workspace_bytes, int B, int P, int D, int dtype,
+                        void *stream);
 
 /* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 4 == 0;
  * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).

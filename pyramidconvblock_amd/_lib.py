@@ -38,6 +38,8 @@ _SIGS = {
     "pdw_bilinear_bwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
     "pdw_gate_fwd": (c_int, [c_void_p] * 2 + [c_longlong, c_int, c_int, c_int, c_void_p]),
     "pdw_gate_bwd": (c_int, [c_void_p] * 3 + [c_longlong, c_int, c_int, c_int, c_void_p]),
+    "pdw_gate_pair_fwd": (c_int, [c_void_p] * 3 + [c_int] * 8 + [c_void_p]),
+    "pdw_gate_pair_bwd": (c_int, [c_void_p] * 5 + [c_int] * 8 + [c_void_p]),
     "pdw_gate_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
     "pdw_bilinear_gate_bwd": (c_int, [c_void_p] * 3 + [c_int] * 8 + [c_void_p]),
     "pdw_spatial_sum_workspace_bytes": (c_size_t, [c_int] * 3),
@@ -45,7 +47,7 @@ _SIGS = {
     "pdw_add_rowbias": (c_int, [c_void_p] * 2 + [c_int] * 4 + [c_void_p]),
     "pdw_pool_branch_workspace_bytes": (c_size_t, [c_int] * 3),
     "pdw_pool_branch_fwd": (c_int, [c_void_p] * 7 + [c_size_t] + [c_int] * 4 + [c_void_p]),
-    "pdw_pool_branch_bwd": (c_int, [c_void_p] * 7 + [c_size_t] + [c_int] * 4 + [c_void_p]),
+    "pdw_pool_branch_bwd": (c_int, [c_void_p] * 8 + [c_size_t] + [c_int] * 4 + [c_void_p]),
     "pdw_dense_supported": (c_int, [c_int] * 3),
     "pdw_dense_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong] + [c_int] * 4
                       + [c_void_p]),

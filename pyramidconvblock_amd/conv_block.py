@@ -83,6 +83,10 @@ def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
     return torch.bmm(a, b).float().sum(0)
 
 
+def _is_pair(scales) -> bool:
+    return len(scales) == 2 and scales[0] == 1. and scales[1] != 1.
+
+
 class ConvBlockFunction(torch.autograd.Function):
     """The whole block of conv_block.py:36-49 as one differentiable op.
 
@@ -102,6 +106,7 @@ class ConvBlockFunction(torch.autograd.Function):
         ns = len(scales)
         cat = torch.empty((B, H, W, G * ns), device=dev, dtype=dt)
         convs, pooled = [], []
+        pair = _is_pair(scales)           # scales (1, s): both gates go into cat in one launch
         for i, s in enumerate(scales):
             w = w_dw[i].detach().to(dt).contiguous()
             k1, k2 = w.shape[0], w.shape[1]
@@ -110,13 +115,17 @@ class ConvBlockFunction(torch.autograd.Function):
             if s != 1.:
                 p = ops.avgpool_forward(a, (int(H * s), int(W * s)))
                 c = dwconv_forward(p, w, *geo)
-                ops.gate_bilinear_forward(c, (H, W), out=dst)
+                if not pair:
+                    ops.gate_bilinear_forward(c, (H, W), out=dst)
             else:
                 p = None
                 c = dwconv_forward(a, w, *geo)
-                ops.gate_forward(c, out=dst)
+                if not pair:
+                    ops.gate_forward(c, out=dst)
             convs.append(c)
             pooled.append(p)
+        if pair:
+            ops.gate_pair_forward(convs[0], convs[1], cat)
         same_dt = w_pool.dtype == dt and all(b is None or b.dtype == dt for b in (b_pool, b_out))
         if same_dt and B > 0:
             # mean over positions -> conv_pool, plus conv_out's bias: one fp32 row per image
@@ -160,11 +169,11 @@ class ConvBlockFunction(torch.autograd.Function):
             gbias, grad_w_pool, dmean = ops.pool_branch_backward(gy, m, w_pool.detach().contiguous())
         else:
             gs = ops.spatial_sum(gy)                             # [B, D] fp32: column sums per image
-            gbias = gs.sum(0)
+            gbias = gs.sum(0).unsqueeze(0).repeat(2, 1)
             grad_w_pool = (gs.t() @ m.float()).to(w_pool.dtype)
             dmean = ((gs @ w_pool.float()) / float(H * W)).contiguous()   # gradient of the per-image mean
-        grad_b_out = gbias.to(w_out.dtype) if ctx.has_bias[1] else None
-        grad_b_pool = gbias.to(w_pool.dtype) if ctx.has_bias[2] else None
+        grad_b_out = gbias[0].to(w_out.dtype) if ctx.has_bias[1] else None      # a tensor of its own for each bias:
+        grad_b_pool = gbias[1].to(w_pool.dtype) if ctx.has_bias[2] else None    # autograd copies a shared one
 
         fast_up, fast_out = ctx.fast
         # the four weight gradients end in a small summation kernel each: they are run as one launch at the end
@@ -182,6 +191,7 @@ class ConvBlockFunction(torch.autograd.Function):
             # first full-resolution branch, the others are accumulated into its result
             order = sorted(range(ns), key=lambda i: scales[i] == 1.)
             waiting = []                                               # pooled gradients not yet added to da
+            gcs = ops.gate_pair_backward(convs[0], convs[1], dcat) if _is_pair(scales) else None
             for i in order:
                 s = scales[i]
                 w = w_dw[i].detach().to(dt).contiguous()
@@ -189,12 +199,13 @@ class ConvBlockFunction(torch.autograd.Function):
                 geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
                 dslice = dcat[..., i * G:(i + 1) * G]
                 c = convs[i]
-                if s != 1.:
+                src = pooled[i] if s != 1. else a
+                if gcs is not None:
+                    gc = gcs[i]
+                elif s != 1.:
                     gc = ops.bilinear_gate_backward(c, dslice)
-                    src = pooled[i]
                 else:
                     gc = ops.gate_backward(c, dslice)
-                    src = a
                 grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo)
                 if s != 1.:
                     waiting.append(dwconv_dgrad(gc, w, src.shape, *geo))

@@ -58,7 +58,7 @@ using namespace pdw;
 
 extern "C" {
 
-int pdw_version(void) { return 3; }
+int pdw_version(void) { return 4; }
 
 const char* pdw_last_error(void) { return g_err; }
 
@@ -214,6 +214,29 @@ int pdw_bilinear_gate_bwd(const void* gy, const void* x, void* gx, int B, int h,
     return bilinear_gate_bwd_launch(gy, x, gx, B, h, w, I, H, W, ldgy, dtype, (hipStream_t)stream);
 }
 
+int pdw_gate_pair_fwd(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
+                      int dtype, void* stream) {
+    if (int e = check_resample("pdw_gate_pair_fwd", xh, y, B, H, W, I, h, w, dtype)) return e;
+    if (I < 2 || (I & 1)) return set_error("pdw_gate_pair_fwd: need even I >= 2 (I=%d)", I), 1;
+    if (B > 0 && !xf) return set_error("pdw_gate_pair_fwd: null pointer"), 1;
+    if (ldy == 0) ldy = I;
+    if (ldy < I) return set_error("pdw_gate_pair_fwd: ldy=%d smaller than I=%d", ldy, I), 1;
+    return gate_pair_fwd_launch(xf, xh, y, B, H, W, h, w, I, ldy, dtype, (hipStream_t)stream);
+}
+
+int pdw_gate_pair_bwd(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
+                      int w, int I, int ldgy, int dtype, void* stream) {
+    if (int e = check_resample("pdw_gate_pair_bwd", gy, gxh, B, H, W, I, h, w, dtype)) return e;
+    if (I < 2 || (I & 1)) return set_error("pdw_gate_pair_bwd: need even I >= 2 (I=%d)", I), 1;
+    if (B > 0 && (!xf || !xh || !gxf)) return set_error("pdw_gate_pair_bwd: null pointer"), 1;
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2)
+        return set_error("pdw_gate_pair_bwd: needs H = 2h, W = 2w, h,w >= 2 (h=%d w=%d H=%d W=%d); use "
+                         "pdw_gate_bwd and pdw_bilinear_bwd + pdw_gate_bwd", h, w, H, W), 1;
+    if (ldgy == 0) ldgy = I;
+    if (ldgy < I) return set_error("pdw_gate_pair_bwd: ldgy=%d smaller than I=%d", ldgy, I), 1;
+    return gate_pair_bwd_launch(gy, xf, xh, gxf, gxh, B, H, W, h, w, I, ldgy, dtype, (hipStream_t)stream);
+}
+
 size_t pdw_spatial_sum_workspace_bytes(int B, int P, int C) {
     if (B < 1 || P < 1 || C < 1) return 0;
     return spatial_sum_workspace(B, P, C);
@@ -257,14 +280,15 @@ int pdw_pool_branch_fwd(const void* x, const void* w_pool, const void* b_pool, c
                                   (hipStream_t)stream);
 }
 
-int pdw_pool_branch_bwd(const void* gy, const void* m, const void* w_pool, void* gbias, void* gw_pool, float* dmean,
-                        void* workspace, size_t workspace_bytes, int B, int P, int D, int dtype, void* stream) {
+int pdw_pool_branch_bwd(const void* gy, const void* m, const void* w_pool, void* gbias, void* gbias2, void* gw_pool,
+                        float* dmean, void* workspace, size_t workspace_bytes, int B, int P, int D, int dtype,
+                        void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_pool_branch_bwd: unknown dtype %d", dtype), 1;
     if (B < 1 || P < 1 || D < 1) return set_error("pdw_pool_branch_bwd: bad extents B=%d P=%d D=%d", B, P, D), 1;
     if (!gy || !m || !w_pool || !gbias || !gw_pool || !dmean) return set_error("pdw_pool_branch_bwd: null pointer"), 1;
     if (!workspace || workspace_bytes < pool_branch_workspace(B, P, D))
         return set_error("pdw_pool_branch_bwd: workspace too small"), 1;
-    return pool_branch_bwd_launch(gy, m, w_pool, gbias, gw_pool, dmean, (float*)workspace, B, P, D, dtype,
+    return pool_branch_bwd_launch(gy, m, w_pool, gbias, gbias2, gw_pool, dmean, (float*)workspace, B, P, D, dtype,
                                   (hipStream_t)stream);
 }
 

@@ -45,6 +45,10 @@ int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int 
 int bilinear_bwd_launch(const void* gy, void* gx, int B, int h, int w, int C, int H, int W, int ldg, int dtype,
                         hipStream_t s);
 int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s);
+int gate_pair_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
+                         int dtype, hipStream_t s);
+int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
+                         int w, int I, int ldg, int dtype, hipStream_t s);
 int gate_bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int I, int H, int W, int ldy, int dtype,
                              hipStream_t s);
 int bilinear_gate_bwd_launch(const void* gy, const void* x, void* gx, int B, int h, int w, int I, int H, int W, int ldg,
@@ -56,8 +60,8 @@ int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, 
 size_t pool_branch_workspace(int B, int P, int D);
 int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const void* bo, void* m, float* rowbias,
                            float* ws, int B, int P, int D, int dtype, hipStream_t s);
-int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gwp, float* dmean,
-                           float* ws, int B, int P, int D, int dtype, hipStream_t s);
+int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gbias2, void* gwp,
+                           float* dmean, float* ws, int B, int P, int D, int dtype, hipStream_t s);
 
 // dense.hip: thin dense layers on the matrix cores (16-bit types, inner dims <= 128); -1 = not covered
 int dense_rows_supported(int K, int NO, int dtype);

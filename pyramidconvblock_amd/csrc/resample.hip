@@ -255,10 +255,8 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
 
 // ---------------------------------------------------------------- gate
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
-                                                  long long total) {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
+__device__ __forceinline__ void gate_fwd_item(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
+                                              long long idx) {
     const int G = I / 2, GV = G / VEC;
     const int c = (int)(idx % GV) * VEC;
     const long long m = idx / GV;
@@ -271,10 +269,15 @@ __global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __
 }
 
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const T* __restrict__ gy,
-                                                  T* __restrict__ gx, int I, int ldg, float s, long long total) {
+__global__ __launch_bounds__(256) void gate_fwd_k(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
+                                                  long long total) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
+    if (idx < total) gate_fwd_item<T, VEC>(x, y, I, ldy, s, idx);
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void gate_bwd_item(const T* __restrict__ x, const T* __restrict__ gy, T* __restrict__ gx,
+                                              int I, int ldg, float s, long long idx) {
     const int G = I / 2, GV = G / VEC;
     const int c = (int)(idx % GV) * VEC;
     const long long m = idx / GV;
@@ -291,17 +294,22 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
     store_f32<T, VEC>(gx + m * I + G + c, gb);
 }
 
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const T* __restrict__ gy,
+                                                  T* __restrict__ gx, int I, int ldg, float s, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) gate_bwd_item<T, VEC>(x, gy, gx, I, ldg, s, idx);
+}
+
 
 // ---------------------------------------------------------------- gate fused with the resampling next to it
 // Gate then bilinear resize in one pass: y[b,i,j,c] = interp of gate(x)[b,:,:,c], x[B,h,w,I] -> y[B,H,W,G] (G = I/2).
 // The gate value of each of the 4 source pixels is rounded to T first, exactly what the two separate kernels
 // produce, so the gated tensor never exists in memory.
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void gate_bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
-                                                           int I, int H, int W, int ldy, float sy, float sx, float s,
-                                                           long long total) {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
+__device__ __forceinline__ void gate_bilinear_fwd_item(const T* __restrict__ x, T* __restrict__ y, int h, int w, int I,
+                                                       int H, int W, int ldy, float sy, float sx, float s,
+                                                       long long idx) {
     const int G = I / 2, GV = G / VEC;
     const int c = (int)(idx % GV) * VEC;
     long long t = idx / GV;
@@ -333,14 +341,36 @@ __global__ __launch_bounds__(256) void gate_bilinear_fwd_k(const T* __restrict__
     store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
 }
 
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
+                                                           int I, int H, int W, int ldy, float sy, float sx, float s,
+                                                           long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) gate_bilinear_fwd_item<T, VEC>(x, y, h, w, I, H, W, ldy, sy, sx, s, idx);
+}
+
+// Both branches of a two-scale block in one launch: workgroups below nblk_full gate the full-resolution tensor into
+// channels [0, G) of y, the others gate and resize the pooled one into channels [G, 2G).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_pair_fwd_k(const T* __restrict__ xf, const T* __restrict__ xh,
+                                                       T* __restrict__ y, int h, int w, int I, int H, int W, int ldy,
+                                                       float sy, float sx, float s, unsigned nblk_full,
+                                                       long long total_full, long long total_half) {
+    if (blockIdx.x < nblk_full) {
+        const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+        if (idx < total_full) gate_fwd_item<T, VEC>(xf, y, I, ldy, s, idx);
+    } else {
+        const long long idx = (long long)(blockIdx.x - nblk_full) * blockDim.x + threadIdx.x;
+        if (idx < total_half) gate_bilinear_fwd_item<T, VEC>(xh, y + I / 2, h, w, I, H, W, ldy, sy, sx, s, idx);
+    }
+}
+
 // Backward of the pair for exactly doubled extents: the bilinear gather of bilinear_bwd_x2_k (rounded to T),
 // then the gate's gradient, written as gx[B,h,w,I].
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void bilinear_gate_bwd_x2_k(const T* __restrict__ gy, const T* __restrict__ x,
-                                                              T* __restrict__ gx, int h, int w, int I, int ldg, float s,
-                                                              long long total) {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
+__device__ __forceinline__ void bilinear_gate_bwd_x2_item(const T* __restrict__ gy, const T* __restrict__ x,
+                                                          T* __restrict__ gx, int h, int w, int I, int ldg, float s,
+                                                          long long idx) {
     const int H = 2 * h, W = 2 * w;
     const int G = I / 2, GV = G / VEC;
     const int c = (int)(idx % GV) * VEC;
@@ -392,6 +422,30 @@ __global__ __launch_bounds__(256) void bilinear_gate_bwd_x2_k(const T* __restric
     T* op = gx + ((b * h + m) * w + n) * I + c;
     store_f32<T, VEC>(op, ga);
     store_f32<T, VEC>(op + G, gbv);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_gate_bwd_x2_k(const T* __restrict__ gy, const T* __restrict__ x,
+                                                              T* __restrict__ gx, int h, int w, int I, int ldg, float s,
+                                                              long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) bilinear_gate_bwd_x2_item<T, VEC>(gy, x, gx, h, w, I, ldg, s, idx);
+}
+
+// Gradient of gate_pair_fwd_k for exactly doubled extents, the two branches again in one launch.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_pair_bwd_k(const T* __restrict__ gy, const T* __restrict__ xf,
+                                                       const T* __restrict__ xh, T* __restrict__ gxf,
+                                                       T* __restrict__ gxh, int h, int w, int I, int ldg, float s,
+                                                       unsigned nblk_full, long long total_full,
+                                                       long long total_half) {
+    if (blockIdx.x < nblk_full) {
+        const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+        if (idx < total_full) gate_bwd_item<T, VEC>(xf, gy, gxf, I, ldg, s, idx);
+    } else {
+        const long long idx = (long long)(blockIdx.x - nblk_full) * blockDim.x + threadIdx.x;
+        if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
+    }
 }
 
 // ---------------------------------------------------------------- per-image column sums and broadcast add
@@ -551,7 +605,8 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_a_k(const float* __restri
 // gwp[o,c] = sum_b gs[b,o] * m[b,c].
 template <typename T>
 __global__ __launch_bounds__(256) void pool_branch_bwd_b_k(const float* __restrict__ gs, const T* __restrict__ m, int B,
-                                                           int D, T* __restrict__ gbias, T* __restrict__ gwp) {
+                                                           int D, T* __restrict__ gbias, T* __restrict__ gbias2,
+                                                           T* __restrict__ gwp) {
     extern __shared__ float gcol[];  // [B] = gs[:, o]
     const int o = blockIdx.x;
     for (int b = threadIdx.x; b < B; b += 256) gcol[b] = gs[(long long)b * D + o];
@@ -570,6 +625,7 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_b_k(const float* __restri
         float s = 0.f;
         for (int b = 0; b < B; ++b) s += gcol[b];
         gbias[o] = from_f32<T>(s);
+        if (gbias2) gbias2[o] = from_f32<T>(s);
     }
 }
 
@@ -637,11 +693,11 @@ __global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restr
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void pool_branch_bwd_a_v8_k(const float* __restrict__ part, int nchunks, int D,
-                                                              float inv_p, const T* __restrict__ wp,
-                                                              float* __restrict__ gs, float* __restrict__ dmean) {
-    extern __shared__ float sm[];  // [D] column sums, then [16][D] partial products
-    const int b = blockIdx.x, tid = threadIdx.x;
+__device__ __forceinline__ void pool_branch_bwd_a_v8_body(const float* __restrict__ part, int nchunks, int D,
+                                                          float inv_p, const T* __restrict__ wp,
+                                                          float* __restrict__ gs, float* __restrict__ dmean, int b,
+                                                          float* sm) {  // sm: [D] column sums, then [16][D] products
+    const int tid = threadIdx.x;
     const int cv = tid & 15, ol = tid >> 4;  // channel vector, row lane: rows o = ol + 16*it
     ChanVec<T, 8> wv[8];
 #pragma unroll
@@ -682,15 +738,13 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_a_v8_k(const float* __res
     }
 }
 
+// sm: [B] = column sums gs[:, o] (filled by the caller, barrier included), then [16][D] partial products
 template <typename T>
-__global__ __launch_bounds__(256) void pool_branch_bwd_b_v8_k(const float* __restrict__ gs, const T* __restrict__ m,
-                                                              int B, int D, T* __restrict__ gbias,
-                                                              T* __restrict__ gwp) {
-    extern __shared__ float sm[];  // [B] = gs[:, o], then [16][D] partial products
-    const int o = blockIdx.x, tid = threadIdx.x;
+__device__ __forceinline__ void pool_branch_bwd_b_v8_body(const T* __restrict__ m, int B, int D, T* __restrict__ gbias,
+                                                          T* __restrict__ gbias2, T* __restrict__ gwp, int o,
+                                                          float* sm) {
+    const int tid = threadIdx.x;
     const int cv = tid & 15, bl = tid >> 4;  // channel vector, batch lane: images b = bl + 16*it
-    for (int b = tid; b < B; b += 256) sm[b] = gs[(long long)b * D + o];
-    __syncthreads();
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
@@ -726,7 +780,35 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_b_v8_k(const float* __res
         float sv = 0.f;
         for (int b = 0; b < B; ++b) sv += sm[b];
         gbias[o] = from_f32<T>(sv);
+        if (gbias2) gbias2[o] = from_f32<T>(sv);
     }
+}
+
+// Both parts in one launch: workgroups [0, B) are part A for image b, workgroups [B, B + D) part B for feature o.
+// Part B sums its column of the per-chunk sums itself (8 lanes per image), so it does not wait for part A.
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_bwd_v8_k(const float* __restrict__ part, int nchunks, int B, int D,
+                                                            float inv_p, const T* __restrict__ wp,
+                                                            const T* __restrict__ m, float* __restrict__ gs,
+                                                            float* __restrict__ dmean, T* __restrict__ gbias,
+                                                            T* __restrict__ gbias2, T* __restrict__ gwp) {
+    extern __shared__ float sm[];
+    if ((int)blockIdx.x < B) {
+        pool_branch_bwd_a_v8_body<T>(part, nchunks, D, inv_p, wp, gs, dmean, blockIdx.x, sm);
+        return;
+    }
+    const int o = blockIdx.x - B, tid = threadIdx.x, l8 = tid & 7;
+    for (int b = tid >> 3; b < B; b += 32) {
+        const float* pp = part + (long long)b * nchunks * D + o;
+        float sv = 0.f;
+        for (int q = l8; q < nchunks; q += 8) sv += pp[(long long)q * D];
+        sv += __shfl_xor(sv, 1);
+        sv += __shfl_xor(sv, 2);
+        sv += __shfl_xor(sv, 4);
+        if (l8 == 0) sm[b] = sv;
+    }
+    __syncthreads();
+    pool_branch_bwd_b_v8_body<T>(m, B, D, gbias, gbias2, gwp, o, sm);
 }
 
 // y[b,p,c] += v[b,c]  (v in fp32, one rounding)
@@ -876,6 +958,38 @@ int bilinear_gate_bwd_launch(const void* gy, const void* x, void* gx, int B, int
     return check_launch("bilinear_gate_bwd");
 }
 
+int gate_pair_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
+                         int dtype, hipStream_t s) {
+    const void* ptrs[3] = {xf, xh, y};
+    const int vec = pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 3);
+    const long long tf = (long long)B * H * W * (I / 2 / vec), th = tf;
+    unsigned bf, bh;
+    if (tf == 0) return 0;
+    if (!grid_for(tf, &bf) || !grid_for(th, &bh) || (unsigned long long)bf + bh > 0x7fffffffULL) return 1;
+    const float sy = (float)h / (float)H, sx = (float)w / (float)W, sc = sqrtf((float)(I / 2));
+#define CALL(T, V) hipLaunchKernelGGL((gate_pair_fwd_k<T, V>), dim3(bf + bh), dim3(256), 0, s, (const T*)xf, (const T*)xh, (T*)y, h, w, I, H, W, ldy, sy, sx, sc, bf, tf, th);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("gate_pair_fwd");
+}
+
+// -1: extents are not exactly doubled (the caller runs the separate kernels).
+int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
+                         int w, int I, int ldg, int dtype, hipStream_t s) {
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2) return -1;
+    const void* ptrs[5] = {gy, xf, xh, gxf, gxh};
+    const int vec = pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 5);
+    const long long tf = (long long)B * H * W * (I / 2 / vec), th = (long long)B * h * w * (I / 2 / vec);
+    unsigned bf, bh;
+    if (tf == 0) return 0;
+    if (!grid_for(tf, &bf) || !grid_for(th, &bh) || (unsigned long long)bf + bh > 0x7fffffffULL) return 1;
+    const float sc = sqrtf((float)(I / 2));
+#define CALL(T, V) hipLaunchKernelGGL((gate_pair_bwd_k<T, V>), dim3(bf + bh), dim3(256), 0, s, (const T*)gy, (const T*)xf, (const T*)xh, (T*)gxf, (T*)gxh, h, w, I, ldg, sc, bf, tf, th);
+    PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+    return check_launch("gate_pair_bwd");
+}
+
 int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s) {
     const void* ptrs[2] = {x, y};
     const int vec = pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 2);
@@ -1000,8 +1114,8 @@ int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const 
     return check_launch("pool_branch_fwd");
 }
 
-int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gwp, float* dmean,
-                           float* ws, int B, int P, int D, int dtype, hipStream_t s) {
+int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gbias2, void* gwp,
+                           float* dmean, float* ws, int B, int P, int D, int dtype, hipStream_t s) {
     int n;
     if (int e = spatial_sum_parts(gy, ws, B, P, D, dtype, s, &n)) return e;
     float* gs = ws + spatial_sum_workspace(B, P, D) / sizeof(float);
@@ -1013,23 +1127,21 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
                     (reinterpret_cast<uintptr_t>(m) & 15) == 0 && (size_t)(B + 16 * D) * sizeof(float) <= 64 * 1024;
     if (v8) {
         const size_t la = (size_t)17 * D * sizeof(float), lb = (size_t)(B + 16 * D) * sizeof(float);
-#define PDW_PB8(T)                                                                                                     \
-    hipLaunchKernelGGL((pool_branch_bwd_a_v8_k<T>), dim3(B), dim3(256), la, s, ws, n, D, inv_p, (const T*)wp, gs, dmean); \
-    if (int e = check_launch("pool_branch_bwd_a")) return e;                                                          \
-    hipLaunchKernelGGL((pool_branch_bwd_b_v8_k<T>), dim3(D), dim3(256), lb, s, gs, (const T*)m, B, D, (T*)gbias, (T*)gwp);
-        if (dtype == kF16) {
-            PDW_PB8(f16_t)
-        } else {
-            PDW_PB8(bf16_t)
-        }
-#undef PDW_PB8
-        return check_launch("pool_branch_bwd_b");
+        const size_t l = la > lb ? la : lb;
+        if (dtype == kF16)
+            hipLaunchKernelGGL((pool_branch_bwd_v8_k<f16_t>), dim3(B + D), dim3(256), l, s, ws, n, B, D, inv_p,
+                               (const f16_t*)wp, (const f16_t*)m, gs, dmean, (f16_t*)gbias, (f16_t*)gbias2, (f16_t*)gwp);
+        else
+            hipLaunchKernelGGL((pool_branch_bwd_v8_k<bf16_t>), dim3(B + D), dim3(256), l, s, ws, n, B, D, inv_p,
+                               (const bf16_t*)wp, (const bf16_t*)m, gs, dmean, (bf16_t*)gbias, (bf16_t*)gbias2,
+                               (bf16_t*)gwp);
+        return check_launch("pool_branch_bwd");
     }
 #define PDW_PB(T)                                                                                                  \
     hipLaunchKernelGGL((pool_branch_bwd_a_k<T>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const T*)wp, gs, dmean); \
     if (int e = check_launch("pool_branch_bwd_a")) return e;                                                       \
     hipLaunchKernelGGL((pool_branch_bwd_b_k<T>), dim3(D), dim3(256), ldsb, s, gs, (const T*)m, B, D, (T*)gbias,    \
-                       (T*)gwp);
+                       (T*)gbias2, (T*)gwp);
     switch (dtype) {
         case kF32: PDW_PB(float) break;
         case kF16: PDW_PB(f16_t) break;

@@ -131,6 +131,36 @@ def bilinear_gate_backward(x, gy):
     return gate_backward(x, bilinear_backward(gy, (h, w)))
 
 
+def gate_pair_forward(xf, xh, out):
+    """out[..., :G] = gate(xf), out[..., G:2G] = bilinear(gate(xh)) to xf's extents, one launch; out [B,H,W,>=2G]
+    may be a channel slice of a wider tensor."""
+    dev = _lib.require_device(xf, xh, out)
+    B, H, W, I = xf.shape
+    h, w = xh.shape[1], xh.shape[2]
+    if I % 2 or xh.shape[3] != I or out.shape[3] != I:
+        raise ValueError("gate pair: xf, xh need the same even channel count I and out I channels")
+    if xf.numel():
+        _launch("pdw_gate_pair_fwd", dev, xf.data_ptr(), xh.data_ptr(), out.data_ptr(), B, H, W, h, w, I,
+                _pixel_stride(out), _lib.dtype_code(xf.dtype))
+    return out
+
+
+def gate_pair_backward(xf, xh, gy):
+    """Gradients (gxf, gxh) of gate_pair_forward; gy [B,H,W,2G] may be a channel slice.  One launch when the
+    extents are exactly doubled, the single-branch kernels otherwise."""
+    dev = _lib.require_device(xf, xh, gy)
+    B, H, W, I = xf.shape
+    h, w = xh.shape[1], xh.shape[2]
+    G = I // 2
+    if H == 2 * h and W == 2 * w and h >= 2 and w >= 2:
+        gxf, gxh = torch.empty_like(xf), torch.empty_like(xh)
+        if xf.numel():
+            _launch("pdw_gate_pair_bwd", dev, gy.data_ptr(), xf.data_ptr(), xh.data_ptr(), gxf.data_ptr(),
+                    gxh.data_ptr(), B, H, W, h, w, I, _pixel_stride(gy), _lib.dtype_code(xf.dtype))
+        return gxf, gxh
+    return gate_backward(xf, gy[..., :G]), bilinear_gate_backward(xh, gy[..., G:2 * G])
+
+
 def spatial_sum(x):
     """x [B, ..., C] -> fp32 [B, C]: sum over all middle dimensions."""
     dev = _lib.require_device(x)
@@ -220,14 +250,16 @@ def pool_branch_forward(x, w_pool, b_pool=None, b_out=None):
 
 
 def pool_branch_backward(gy, m, w_pool):
-    """-> (gbias [D], gw_pool [D, D] in gy's dtype, dmean fp32 [B, D])."""
+    """-> (gbias [2, D]: the same sums twice, one tensor row for each bias; gw_pool [D, D] in gy's dtype;
+    dmean fp32 [B, D])."""
     dev = _lib.require_device(gy, m, w_pool)
     B, D = gy.shape[0], gy.shape[-1]
     P = gy.numel() // max(B * D, 1)
-    gbias = torch.empty((D,), device=dev, dtype=gy.dtype)
+    gbias = torch.empty((2, D), device=dev, dtype=gy.dtype)
     gwp = torch.empty((D, D), device=dev, dtype=gy.dtype)
     dmean = torch.empty((B, D), device=dev, dtype=torch.float32)
     ws = _pool_ws(B, P, D, dev)
-    _launch("pdw_pool_branch_bwd", dev, gy.data_ptr(), m.data_ptr(), w_pool.data_ptr(), gbias.data_ptr(), gwp.data_ptr(),
-            dmean.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, P, D, _lib.dtype_code(gy.dtype))
+    _launch("pdw_pool_branch_bwd", dev, gy.data_ptr(), m.data_ptr(), w_pool.data_ptr(), gbias[0].data_ptr(),
+            gbias[1].data_ptr(), gwp.data_ptr(), dmean.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, P, D,
+            _lib.dtype_code(gy.dtype))
     return gbias, gwp, dmean

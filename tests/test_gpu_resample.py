@@ -140,6 +140,33 @@ def test_gate_bilinear_fused(oracle, dtype, hw, out, I):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hw,out,I", [((5, 6), (10, 12), 24), ((28, 28), (56, 56), 64), ((4, 5), (9, 11), 6),
+                                      ((2, 2), (4, 4), 2), ((3, 7), (6, 14), 20)])
+def test_gate_pair(oracle, dtype, hw, out, I):
+    """Both gates of a two-scale block written into the concatenated tensor by one launch, and their gradients
+    taken from it by one launch, against the oracle's gate / bilinear applied branch by branch."""
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(I + out[0])
+    B, G = 2, I // 2
+    xf = randn(gen, B, *out, I).to(dtype)
+    xh = randn(gen, B, *hw, I).to(dtype)
+    wide = torch.full((B, *out, I + 8), 3.0, dtype=dtype, device="cuda")
+    cat = wide[..., 8:]
+    ops.gate_pair_forward(xf.cuda(), xh.cuda(), cat)
+    assert_close(cat[..., :G], oracle.gate_fwd(xf.double().numpy()), dtype, "pair: full-resolution gate")
+    assert_close(cat[..., G:], oracle.bilinear_fwd(oracle.gate_fwd(xh.double().numpy()), out), dtype,
+                 "pair: pooled gate")
+    assert torch.all(wide[..., :8] == 3)
+    g = randn(gen, B, *out, I + 8).to(dtype)
+    gs = g.cuda()[..., 8:]
+    gxf, gxh = ops.gate_pair_backward(xf.cuda(), xh.cuda(), gs)
+    assert_close(gxf, oracle.gate_bwd(xf.double().numpy(), g[..., 8:8 + G].double().numpy()), dtype, "pair: d full")
+    assert_close(gxh, oracle.gate_bwd(xh.double().numpy(), oracle.bilinear_bwd(g[..., 8 + G:].double().numpy(), hw)),
+                 dtype, "pair: d pooled")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(3, 7, 9, 20), (32, 56, 56, 128), (2, 57, 61, 200), (1, 1, 1, 4), (5, 33, 2, 3)])
 def test_spatial_sum_and_rowbias(dtype, shape):
     from pyramidconvblock_amd import ops
@@ -200,6 +227,7 @@ def test_pool_branch(dtype, shape):
     gy = randn(gen, *shape).to(dtype)
     gbias, gwp, dmean = ops.pool_branch_backward(gy.cuda(), m, wp.cuda())
     gs = gy.double().sum(dim=(1, 2))
-    assert_close(gbias, gs.sum(0).numpy(), dtype, "bias grad")
+    assert_close(gbias[0], gs.sum(0).numpy(), dtype, "bias grad")
+    assert torch.equal(gbias[0], gbias[1])
     assert_close(gwp, (gs.t() @ m.double().cpu()).numpy(), dtype, "w_pool grad")
     assert_close(dmean, ((gs @ wp.double()) / (H * W)).numpy(), torch.float32, "dmean", scale=8.0)
