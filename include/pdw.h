@@ -166,6 +166,16 @@ int pdw_pool_branch_bwd(const void *gy, const void *m, const void *w_pool, void 
                         float *dmean, void *workspace, size_t workspace_bytes, int B, int P, int D, int dtype,
                         void *stream);
 
+/* The same two steps from per-chunk column sums the caller already has (parts[B][nparts][D], fp32, chunks of
+ * equal or unequal length covering the P positions of an image), e.g. from pdw_dense_fwd_colsum: x / gy is not
+ * read again.  pdw_pool_branch_bwd_parts still takes the workspace of pdw_pool_branch_workspace_bytes. */
+int pdw_pool_branch_fwd_parts(const float *parts, int nparts, const void *w_pool, const void *b_pool,
+                              const void *b_out, void *m, float *rowbias, int B, int P, int D, int dtype,
+                              void *stream);
+int pdw_pool_branch_bwd_parts(const float *parts, int nparts, const void *m, const void *w_pool, void *gbias,
+                              void *gbias2, void *gw_pool, float *dmean, void *workspace, size_t workspace_bytes,
+                              int B, int P, int D, int dtype, void *stream);
+
 /* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 4 == 0;
  * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).
  *   y[n,o] = sum_k x[n,k] * W(o,k) + bias[o] + rowbias[n / P][o]        x[N,K] -> y[N,NO]
@@ -176,6 +186,15 @@ int pdw_pool_branch_bwd(const void *gy, const void *m, const void *w_pool, void 
 int pdw_dense_supported(int K, int NO, int dtype);
 int pdw_dense_fwd(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
                   long long N, int K, int NO, int P, int dtype, void *stream);
+
+/* pdw_dense_fwd that also writes colsum[t][k] = sum of x[n,k] over the rows n of the t-th group of 32 rows (fp32,
+ * ceil(N/32) x K): with 32 | P these are per-chunk sums of each image, which pdw_pool_branch_fwd_parts /
+ * _bwd_parts take in place of a second pass over x (the x.mean of conv_block.py:46 and its gradient ride on
+ * conv_up, conv_block.py:37, and on the input gradient of conv_out, conv_block.py:44).  K = 64 or 128 only:
+ * pdw_dense_colsum_supported. */
+int pdw_dense_colsum_supported(int K, int NO, int dtype);
+int pdw_dense_fwd_colsum(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
+                         float *colsum, long long N, int K, int NO, int P, int dtype, void *stream);
 
 /* Weight gradient of such a layer: dw[m,o] = sum_n a[n,m] * b[n,o]  (a[N,M], b[N,NO] -> dw[M,NO]), fp32
  * accumulation, two deterministic passes through `workspace` (no atomics). */

@@ -101,7 +101,13 @@ class ConvBlockFunction(torch.autograd.Function):
         I = w_up.shape[0]
         fast_up = (ops.dense_supported(D, I, dt) and ops.dense_supported(I, D, dt) and w_up.dtype == dt
                    and (b_up is None or b_up.dtype == dt))
-        a = ops.dense_forward(x, w_up.detach().contiguous(), bias=b_up) if fast_up else F.linear(x, w_up, b_up)
+        same_dt = w_pool.dtype == dt and all(b is None or b.dtype == dt for b in (b_pool, b_out))
+        # the per-image sums of x that the mean branch needs are taken by conv_up's kernel while it reads x
+        xparts = None
+        if fast_up and same_dt and B > 0 and ops.dense_colsum_supported(D, I, dt, H * W):
+            a, xparts = ops.dense_forward(x, w_up.detach().contiguous(), bias=b_up, colsum=True)
+        else:
+            a = ops.dense_forward(x, w_up.detach().contiguous(), bias=b_up) if fast_up else F.linear(x, w_up, b_up)
         G = I // 2
         ns = len(scales)
         cat = torch.empty((B, H, W, G * ns), device=dev, dtype=dt)
@@ -126,10 +132,9 @@ class ConvBlockFunction(torch.autograd.Function):
             pooled.append(p)
         if pair:
             ops.gate_pair_forward(convs[0], convs[1], cat)
-        same_dt = w_pool.dtype == dt and all(b is None or b.dtype == dt for b in (b_pool, b_out))
         if same_dt and B > 0:
             # mean over positions -> conv_pool, plus conv_out's bias: one fp32 row per image
-            m, yp = ops.pool_branch_forward(x, w_pool.detach().contiguous(), b_pool, b_out)
+            m, yp = ops.pool_branch_forward(x, w_pool.detach().contiguous(), b_pool, b_out, parts=xparts)
         else:
             m = (ops.spatial_sum(x) / float(H * W)).to(dt)
             yp = F.linear(m, w_pool, b_pool).float()
@@ -165,25 +170,31 @@ class ConvBlockFunction(torch.autograd.Function):
         gy = gy.to(dt).contiguous()
         g2d = gy.view(N, D)
 
-        if w_pool.dtype == dt and B > 0:
-            gbias, grad_w_pool, dmean = ops.pool_branch_backward(gy, m, w_pool.detach().contiguous())
-        else:
-            gs = ops.spatial_sum(gy)                             # [B, D] fp32: column sums per image
-            gbias = gs.sum(0).unsqueeze(0).repeat(2, 1)
-            grad_w_pool = (gs.t() @ m.float()).to(w_pool.dtype)
-            dmean = ((gs @ w_pool.float()) / float(H * W)).contiguous()   # gradient of the per-image mean
-        grad_b_out = gbias[0].to(w_out.dtype) if ctx.has_bias[1] else None      # a tensor of its own for each bias:
-        grad_b_pool = gbias[1].to(w_pool.dtype) if ctx.has_bias[2] else None    # autograd copies a shared one
-
         fast_up, fast_out = ctx.fast
+        pool_fast = w_pool.dtype == dt and B > 0
         # the four weight gradients end in a small summation kernel each: they are run as one launch at the end
         with _lib.deferred_reductions(gy.device):
+            gparts = None
             if fast_out:
-                dcat = ops.dense_forward(gy, w_out.detach().contiguous(), w_kmajor=True)
+                if pool_fast and ops.dense_colsum_supported(D, G * ns, dt, H * W):
+                    # the per-image sums of gy for the mean branch come out of the kernel that reads gy anyway
+                    dcat, gparts = ops.dense_forward(gy, w_out.detach().contiguous(), w_kmajor=True, colsum=True)
+                else:
+                    dcat = ops.dense_forward(gy, w_out.detach().contiguous(), w_kmajor=True)
                 grad_w_out = ops.dense_wgrad(gy, cat)
             else:
                 dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
                 grad_w_out = _weight_grad(g2d, cat.view(N, G * ns))
+
+            if pool_fast:
+                gbias, grad_w_pool, dmean = ops.pool_branch_backward(gy, m, w_pool.detach().contiguous(), parts=gparts)
+            else:
+                gs = ops.spatial_sum(gy)                             # [B, D] fp32: column sums per image
+                gbias = gs.sum(0).unsqueeze(0).repeat(2, 1)
+                grad_w_pool = (gs.t() @ m.float()).to(w_pool.dtype)
+                dmean = ((gs @ w_pool.float()) / float(H * W)).contiguous()   # gradient of the per-image mean
+            grad_b_out = gbias[0].to(w_out.dtype) if ctx.has_bias[1] else None    # a tensor of its own for each
+            grad_b_pool = gbias[1].to(w_pool.dtype) if ctx.has_bias[2] else None  # bias: autograd copies a shared one
 
             da = None
             grad_w_dw = [None] * ns

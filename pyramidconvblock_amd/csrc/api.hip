@@ -292,6 +292,48 @@ int pdw_pool_branch_bwd(const void* gy, const void* m, const void* w_pool, void*
                                   (hipStream_t)stream);
 }
 
+int pdw_pool_branch_fwd_parts(const float* parts, int nparts, const void* w_pool, const void* b_pool, const void* b_out,
+                              void* m, float* rowbias, int B, int P, int D, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_pool_branch_fwd_parts: unknown dtype %d", dtype), 1;
+    if (B < 1 || P < 1 || D < 1 || nparts < 1)
+        return set_error("pdw_pool_branch_fwd_parts: bad extents B=%d P=%d D=%d nparts=%d", B, P, D, nparts), 1;
+    if (!parts || !w_pool || !m || !rowbias) return set_error("pdw_pool_branch_fwd_parts: null pointer"), 1;
+    return pool_branch_fwd_launch(nullptr, w_pool, b_pool, b_out, m, rowbias, nullptr, B, P, D, dtype,
+                                  (hipStream_t)stream, parts, nparts);
+}
+
+int pdw_pool_branch_bwd_parts(const float* parts, int nparts, const void* m, const void* w_pool, void* gbias,
+                              void* gbias2, void* gw_pool, float* dmean, void* workspace, size_t workspace_bytes, int B,
+                              int P, int D, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_pool_branch_bwd_parts: unknown dtype %d", dtype), 1;
+    if (B < 1 || P < 1 || D < 1 || nparts < 1)
+        return set_error("pdw_pool_branch_bwd_parts: bad extents B=%d P=%d D=%d nparts=%d", B, P, D, nparts), 1;
+    if (!parts || !m || !w_pool || !gbias || !gw_pool || !dmean)
+        return set_error("pdw_pool_branch_bwd_parts: null pointer"), 1;
+    if (!workspace || workspace_bytes < pool_branch_workspace(B, P, D))
+        return set_error("pdw_pool_branch_bwd_parts: workspace too small"), 1;
+    return pool_branch_bwd_launch(nullptr, m, w_pool, gbias, gbias2, gw_pool, dmean, (float*)workspace, B, P, D, dtype,
+                                  (hipStream_t)stream, parts, nparts);
+}
+
+int pdw_dense_colsum_supported(int K, int NO, int dtype) {
+    return (dense_colsum_supported(K, NO, dtype) && dense_wgrad_supported(K, NO, dtype)) ? 1 : 0;
+}
+
+int pdw_dense_fwd_colsum(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
+                         float* colsum, long long N, int K, int NO, int P, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd_colsum: unknown dtype %d", dtype), 1;
+    if (N < 0 || K < 1 || NO < 1) return set_error("pdw_dense_fwd_colsum: bad extents N=%lld K=%d NO=%d", N, K, NO), 1;
+    if (N > 0 && (!x || !w || !y || !colsum)) return set_error("pdw_dense_fwd_colsum: null pointer"), 1;
+    if (rowbias && P < 1) return set_error("pdw_dense_fwd_colsum: rowbias needs P >= 1"), 1;
+    const int r = dense_rows_launch(x, w, w_kmajor ? 1 : 0, bias, rowbias, y, N, K, NO, P, dtype, (hipStream_t)stream,
+                                    colsum);
+    if (r == -1)
+        return set_error("pdw_dense_fwd_colsum: K=%d NO=%d dtype=%d not supported (see pdw_dense_colsum_supported)", K,
+                         NO, dtype), 3;
+    return r;
+}
+
 int pdw_dense_supported(int K, int NO, int dtype) {
     return (dense_rows_supported(K, NO, dtype) && dense_wgrad_supported(K, NO, dtype)) ? 1 : 0;
 }

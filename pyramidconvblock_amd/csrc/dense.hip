@@ -44,6 +44,16 @@ constexpr int kNT = 4;  // feature tiles of 32 (<= 128 features)
 __device__ __forceinline__ uint32_t ld16(const bf16_t* p) { return (uint32_t) * reinterpret_cast<const unsigned short*>(p); }
 __device__ __forceinline__ uint32_t ld16(const f16_t* p) { return (uint32_t) * reinterpret_cast<const unsigned short*>(p); }
 
+// The 16-bit pattern `h` (in the low half of a register) as a float.
+template <typename T>
+__device__ __forceinline__ float half_to_f32(uint32_t h) {
+    if constexpr (sizeof(T) == 2 && __is_same(T, bf16_t)) {
+        return __builtin_bit_cast(float, h << 16);
+    } else {
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
+    }
+}
+
 // 8 values p[0], p[stride], ..., p[7*stride] packed as a fragment (zeros where !ok; p must be readable
 // either way, so the 8 reads are issued back to back without a branch).
 template <typename T>
@@ -118,11 +128,16 @@ struct WTransposer {
 // and re-shaped into MFMA fragments through a per-wave LDS buffer: row-strided fragment loads straight
 // from global memory run ~2.5x slower on this part.  The same buffer transposes the result tile so the
 // global stores are whole 128-byte lines as well.
-template <typename T, bool KMAJOR>
+//
+// COLSUM: the kernel also writes colsum[tile][k] = sum over the tile's 32 rows of X[., k] (fp32), for callers that
+// need per-image sums of X over the positions and would otherwise read X a second time.  Chunk i*64+lane of a tile
+// is 8 columns of one row, and with 64 % (K/8) == 0 a lane keeps the same 8 columns for every chunk: 8 running
+// sums per lane, combined over the 512/K lanes that share them through the tile buffer once the fragments are out.
+template <typename T, bool KMAJOR, bool COLSUM>
 __global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
                                                     const T* __restrict__ bias, const float* __restrict__ rowbias,
-                                                    T* __restrict__ Y, long long N, int K, int NO, int P, int nkt,
-                                                    int nnt) {
+                                                    T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
+                                                    int NO, int P, int nkt, int nnt) {
     extern __shared__ uint32_t dsm[];
     T* wl = reinterpret_cast<T*>(dsm);
     const int ldw = K + 8;
@@ -178,6 +193,18 @@ __global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, 
 #pragma unroll
         for (int i = 0; i < LP; ++i)
             if (oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
+        float cs[8];
+        if constexpr (COLSUM) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cs[j] = 0.f;
+#pragma unroll
+            for (int i = 0; i < LP; ++i)   // chunks past the tile or the tensor are zero
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    cs[2 * j] += half_to_f32<T>(raw[i].v[j] & 0xffffu);
+                    cs[2 * j + 1] += half_to_f32<T>(raw[i].v[j] >> 16);
+                }
+        }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes have landed
         Frag xf[kKT];
 #pragma unroll
@@ -189,6 +216,28 @@ __global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, 
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // fragments are in registers: the buffer may be overwritten
         if (tile + nw < ntiles) load_tile(tile + nw);  // next tile in flight during the MFMAs and the store
+        if constexpr (COLSUM) {
+            float* tf = reinterpret_cast<float*>(tl);  // [512 / K lane groups][K]
+            *reinterpret_cast<float4*>(tf + lane * 8) = make_float4(cs[0], cs[1], cs[2], cs[3]);
+            *reinterpret_cast<float4*>(tf + lane * 8 + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            float* dst = colsum + tile * K;
+            if (K == 128) {
+                float2 t = *reinterpret_cast<const float2*>(tf + 2 * lane);
+#pragma unroll
+                for (int gidx = 1; gidx < 4; ++gidx) {
+                    const float2 u = *reinterpret_cast<const float2*>(tf + gidx * 128 + 2 * lane);
+                    t.x += u.x, t.y += u.y;
+                }
+                *reinterpret_cast<float2*>(dst + 2 * lane) = t;
+            } else {  // K == 64
+                float t = tf[lane];
+#pragma unroll
+                for (int gidx = 1; gidx < 8; ++gidx) t += tf[gidx * 64 + lane];
+                dst[lane] = t;
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // read before the result tile is written to the same buffer
+        }
         const long long m = tile * 32 + l32;
         const float* rb = rowbias ? rowbias + (long long)((int)(m < N ? m : N - 1) / P) * NO : nullptr;
         for (int nt = 0; nt < nnt; ++nt) {
@@ -383,9 +432,14 @@ static bool dense_dims_ok(int K, int NO, int dtype) {
 
 int dense_rows_supported(int K, int NO, int dtype) { return dense_dims_ok(K, NO, dtype) ? 1 : 0; }
 
+int dense_colsum_supported(int K, int NO, int dtype) {
+    return (dense_dims_ok(K, NO, dtype) && (K == 64 || K == 128)) ? 1 : 0;
+}
+
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
-                      long long N, int K, int NO, int P, int dtype, hipStream_t s) {
+                      long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum) {
     if (!dense_dims_ok(K, NO, dtype)) return -1;
+    if (colsum && (!dense_colsum_supported(K, NO, dtype) || (reinterpret_cast<uintptr_t>(colsum) & 15))) return -1;
     if (N == 0) return 0;
     if (N > 0x7fffffffLL) return -1;
     if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 15) ||
@@ -398,14 +452,20 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     if (blocks > cap) blocks = cap;  // persistent workgroups: the weights are staged to LDS once each
     if (blocks < 1) blocks = 1;
     const size_t lds = ((size_t)NO * (K + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2;
-#define PDW_GO(T, KM)                                                                                          \
-    hipLaunchKernelGGL((dense_rows_k<T, KM>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x, (const T*)w, \
-                       (const T*)bias, rowbias, (T*)y, N, K, NO, P > 0 ? P : 1, nkt, nnt)
+#define PDW_GO(T, KM, CSUM)                                                                                    \
+    hipLaunchKernelGGL((dense_rows_k<T, KM, CSUM>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x,        \
+                       (const T*)w, (const T*)bias, rowbias, (T*)y, colsum, N, K, NO, P > 0 ? P : 1, nkt, nnt)
+#define PDW_GO2(T, KM)            \
+    if (colsum)                   \
+        PDW_GO(T, KM, true);      \
+    else                          \
+        PDW_GO(T, KM, false)
     if (dtype == kF16) {
-        if (w_kmajor) PDW_GO(f16_t, true); else PDW_GO(f16_t, false);
+        if (w_kmajor) { PDW_GO2(f16_t, true); } else { PDW_GO2(f16_t, false); }
     } else {
-        if (w_kmajor) PDW_GO(bf16_t, true); else PDW_GO(bf16_t, false);
+        if (w_kmajor) { PDW_GO2(bf16_t, true); } else { PDW_GO2(bf16_t, false); }
     }
+#undef PDW_GO2
 #undef PDW_GO
     return check_launch("dense_rows");
 }

@@ -58,15 +58,20 @@ size_t spatial_sum_workspace(int B, int P, int C);
 int spatial_sum_launch(const void* x, float* out, float* ws, int B, int P, int C, int dtype, hipStream_t s);
 int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, hipStream_t s);
 size_t pool_branch_workspace(int B, int P, int D);
+// parts (optional): per-chunk column sums [B][nparts][D] already computed by the caller (x / gy is then not read)
 int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const void* bo, void* m, float* rowbias,
-                           float* ws, int B, int P, int D, int dtype, hipStream_t s);
+                           float* ws, int B, int P, int D, int dtype, hipStream_t s, const float* parts = nullptr,
+                           int nparts = 0);
 int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gbias2, void* gwp,
-                           float* dmean, float* ws, int B, int P, int D, int dtype, hipStream_t s);
+                           float* dmean, float* ws, int B, int P, int D, int dtype, hipStream_t s,
+                           const float* parts = nullptr, int nparts = 0);
 
 // dense.hip: thin dense layers on the matrix cores (16-bit types, inner dims <= 128); -1 = not covered
 int dense_rows_supported(int K, int NO, int dtype);
+// colsum (optional, fp32 [ceil(N/32)][K], K = 64 or 128): per-32-row sums of x, see dense_colsum_supported
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
-                      long long N, int K, int NO, int P, int dtype, hipStream_t s);
+                      long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum = nullptr);
+int dense_colsum_supported(int K, int NO, int dtype);
 int dense_wgrad_supported(int M, int NO, int dtype);
 size_t dense_wgrad_workspace(long long N, int M, int NO);
 int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,

@@ -645,12 +645,48 @@ __device__ __forceinline__ float colsum_parts(const float* __restrict__ pp, int 
     return (s0 + s1) + (s2 + s3);
 }
 
+// sm[c] = sum over q < nchunks of pp[q * D + c] for c < D, by the whole workgroup of 256: thread = (4-column vector
+// tid % 32, chunk lane tid / 32), up to 8 loads of a thread in flight, the 8 chunk lanes combined through
+// red[8][D].  D % 4 == 0, D <= 128.  Ends with a barrier; the order of the additions is fixed.
+__device__ __forceinline__ void colsum_coop(const float* __restrict__ pp, int nchunks, int D, float* sm, float* red) {
+    const int tid = threadIdx.x, cv = tid & 31, ql = tid >> 5;
+    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
+    if (cv * 4 < D) {
+        const float* p = pp + cv * 4;
+        int q = ql;
+        for (; q + 56 < nchunks; q += 64) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(p + (long long)(q + 8 * u) * D);
+#pragma unroll
+            for (int u = 0; u < 8; u += 2) {
+                a0.x += v[u].x, a0.y += v[u].y, a0.z += v[u].z, a0.w += v[u].w;
+                a1.x += v[u + 1].x, a1.y += v[u + 1].y, a1.z += v[u + 1].z, a1.w += v[u + 1].w;
+            }
+        }
+        for (; q < nchunks; q += 8) {
+            const float4 v = *reinterpret_cast<const float4*>(p + (long long)q * D);
+            a0.x += v.x, a0.y += v.y, a0.z += v.z, a0.w += v.w;
+        }
+        *reinterpret_cast<float4*>(red + ql * D + cv * 4) =
+            make_float4(a0.x + a1.x, a0.y + a1.y, a0.z + a1.z, a0.w + a1.w);
+    }
+    __syncthreads();
+    if (tid < D) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t += red[k * D + tid];
+        sm[tid] = t;
+    }
+    __syncthreads();
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restrict__ part, int nchunks, int D,
                                                             float inv_p, const T* __restrict__ wp,
                                                             const T* __restrict__ bp, const T* __restrict__ bo,
                                                             T* __restrict__ m, float* __restrict__ rowbias) {
-    extern __shared__ float sm[];  // [D]
+    extern __shared__ float sm[];  // [D] means, [8][D] partial column sums
     const int b = blockIdx.x, tid = threadIdx.x;
     // weight rows of this thread: outputs o = tid/8 + 32*pass, channel vectors sub + 8*i  (requested first)
     const int sub = tid & 7, ol = tid >> 3;
@@ -663,8 +699,9 @@ __global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restr
             const bool ok = o < D && v * 8 < D;
             wv[pass][i] = *reinterpret_cast<const ChanVec<T, 8>*>(wp + (ok ? (long long)o * D + v * 8 : 0));
         }
+    colsum_coop(part + (long long)b * nchunks * D, nchunks, D, sm, sm + D);
     if (tid < D) {
-        const T mv = from_f32<T>(colsum_parts<T>(part + (long long)b * nchunks * D + tid, nchunks, D) * inv_p);
+        const T mv = from_f32<T>(sm[tid] * inv_p);
         m[(long long)b * D + tid] = mv;
         sm[tid] = to_f32(mv);
     }
@@ -706,12 +743,8 @@ __device__ __forceinline__ void pool_branch_bwd_a_v8_body(const float* __restric
         const bool ok = o < D && cv * 8 < D;
         wv[it] = *reinterpret_cast<const ChanVec<T, 8>*>(wp + (ok ? (long long)o * D + cv * 8 : 0));
     }
-    if (tid < D) {
-        const float sv = colsum_parts<T>(part + (long long)b * nchunks * D + tid, nchunks, D);
-        gs[(long long)b * D + tid] = sv;
-        sm[tid] = sv;
-    }
-    __syncthreads();
+    colsum_coop(part + (long long)b * nchunks * D, nchunks, D, sm, sm + D);
+    if (tid < D) gs[(long long)b * D + tid] = sm[tid];
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
@@ -1083,18 +1116,24 @@ int add_rowbias_launch(void* y, const float* v, int B, int P, int C, int dtype, 
 size_t pool_branch_workspace(int B, int P, int D) { return spatial_sum_workspace(B, P, D) + (size_t)B * D * sizeof(float); }
 
 int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const void* bo, void* m, float* rowbias,
-                           float* ws, int B, int P, int D, int dtype, hipStream_t s) {
-    int n;
-    if (int e = spatial_sum_parts(x, ws, B, P, D, dtype, s, &n)) return e;
+                           float* ws, int B, int P, int D, int dtype, hipStream_t s, const float* parts, int nparts) {
+    int n = nparts;
+    if (!parts) {
+        if (int e = spatial_sum_parts(x, ws, B, P, D, dtype, s, &n)) return e;
+        parts = ws;
+    }
+    ws = const_cast<float*>(parts);
     const float inv_p = 1.f / (float)P;
     const size_t lds = (size_t)D * sizeof(float);
-    const bool v8 = dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0;
+    const bool v8 = dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(parts) & 15) == 0;
     if (v8) {
+        const size_t l8 = (size_t)9 * D * sizeof(float);
         if (dtype == kF16)
-            hipLaunchKernelGGL((pool_branch_fwd_v8_k<f16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p,
+            hipLaunchKernelGGL((pool_branch_fwd_v8_k<f16_t>), dim3(B), dim3(256), l8, s, ws, n, D, inv_p,
                                (const f16_t*)wp, (const f16_t*)bp, (const f16_t*)bo, (f16_t*)m, rowbias);
         else
-            hipLaunchKernelGGL((pool_branch_fwd_v8_k<bf16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p,
+            hipLaunchKernelGGL((pool_branch_fwd_v8_k<bf16_t>), dim3(B), dim3(256), l8, s, ws, n, D, inv_p,
                                (const bf16_t*)wp, (const bf16_t*)bp, (const bf16_t*)bo, (bf16_t*)m, rowbias);
         return check_launch("pool_branch_fwd");
     }
@@ -1115,16 +1154,22 @@ int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const 
 }
 
 int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* gbias, void* gbias2, void* gwp,
-                           float* dmean, float* ws, int B, int P, int D, int dtype, hipStream_t s) {
-    int n;
-    if (int e = spatial_sum_parts(gy, ws, B, P, D, dtype, s, &n)) return e;
-    float* gs = ws + spatial_sum_workspace(B, P, D) / sizeof(float);
+                           float* dmean, float* ws, int B, int P, int D, int dtype, hipStream_t s, const float* parts,
+                           int nparts) {
+    int n = nparts;
+    float* gs = ws + spatial_sum_workspace(B, P, D) / sizeof(float);  // the workspace always has both regions
+    if (!parts) {
+        if (int e = spatial_sum_parts(gy, ws, B, P, D, dtype, s, &n)) return e;
+        parts = ws;
+    }
+    ws = const_cast<float*>(parts);
     const float inv_p = 1.f / (float)P;
     const size_t lds = (size_t)D * 9 * sizeof(float);
     const size_t ldsb = (size_t)B * sizeof(float);
     if (lds > 64 * 1024 || ldsb > 64 * 1024) return set_error("pool branch: extents too large"), 1;
     const bool v8 = dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0 &&
-                    (reinterpret_cast<uintptr_t>(m) & 15) == 0 && (size_t)(B + 16 * D) * sizeof(float) <= 64 * 1024;
+                    (reinterpret_cast<uintptr_t>(m) & 15) == 0 && (size_t)(B + 16 * D) * sizeof(float) <= 64 * 1024 &&
+                    (reinterpret_cast<uintptr_t>(parts) & 15) == 0;
     if (v8) {
         const size_t la = (size_t)17 * D * sizeof(float), lb = (size_t)(B + 16 * D) * sizeof(float);
         const size_t l = la > lb ? la : lb;

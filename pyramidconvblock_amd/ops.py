@@ -196,17 +196,31 @@ def dense_supported(K, NO, dtype):
     return bool(_lib.lib().pdw_dense_supported(int(K), int(NO), _lib.dtype_code(dtype)))
 
 
-def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=1):
+def dense_colsum_supported(K, NO, dtype, rows_per_image) -> bool:
+    """Whether dense_forward(..., colsum=True) can deliver per-image chunk sums for this shape."""
+    return (dtype in _lib._DTYPES and rows_per_image % 32 == 0
+            and bool(_lib.lib().pdw_dense_colsum_supported(int(K), int(NO), _lib.dtype_code(dtype))))
+
+
+def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=1, colsum=False):
     """y[..., o] = sum_k x[..., k] * W(o, k) + bias[o] + rowbias[image][o].
 
     w is [NO, K] (nn.Linear layout) or, with w_kmajor, [K, NO].  rowbias is fp32 [B, NO], one row per
-    `rows_per_image` consecutive rows of x."""
+    `rows_per_image` consecutive rows of x.  With colsum (see dense_colsum_supported) the result is
+    (y, parts): parts fp32 [N / 32, K], the sums of x over each group of 32 consecutive rows."""
     dev = _lib.require_device(x, w)
     K = x.shape[-1]
     NO = w.shape[1] if w_kmajor else w.shape[0]
     assert (w.shape[0] if w_kmajor else w.shape[1]) == K and x.is_contiguous() and w.is_contiguous()
     N = x.numel() // K
     y = torch.empty(x.shape[:-1] + (NO,), device=dev, dtype=x.dtype)
+    if colsum:
+        parts = torch.empty(((N + 31) // 32, K), device=dev, dtype=torch.float32)
+        if N:
+            _launch("pdw_dense_fwd_colsum", dev, x.data_ptr(), w.data_ptr(), 1 if w_kmajor else 0,
+                    bias.data_ptr() if bias is not None else None, rowbias.data_ptr() if rowbias is not None else None,
+                    y.data_ptr(), parts.data_ptr(), N, K, NO, int(rows_per_image), _lib.dtype_code(x.dtype))
+        return y, parts
     if N:
         _launch("pdw_dense_fwd", dev, x.data_ptr(), w.data_ptr(), 1 if w_kmajor else 0,
                 bias.data_ptr() if bias is not None else None, rowbias.data_ptr() if rowbias is not None else None,
@@ -234,14 +248,20 @@ def _pool_ws(B, P, D, dev):
     return torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
 
 
-def pool_branch_forward(x, w_pool, b_pool=None, b_out=None):
-    """x [B, ..., D] -> (m [B, D] in x's dtype: the per-image mean; rowbias fp32 [B, D] = m @ w_pool^T + b_pool + b_out)."""
+def pool_branch_forward(x, w_pool, b_pool=None, b_out=None, parts=None):
+    """x [B, ..., D] -> (m [B, D] in x's dtype: the per-image mean; rowbias fp32 [B, D] = m @ w_pool^T + b_pool + b_out).
+    parts (fp32 [B * n, D], n equal-sized chunk sums per image, from dense_forward(colsum=True)) replaces the
+    pass over x."""
     dev = _lib.require_device(x, w_pool)
     B, D = x.shape[0], x.shape[-1]
     P = x.numel() // max(B * D, 1)
     m = torch.empty((B, D), device=dev, dtype=x.dtype)
     rowbias = torch.empty((B, D), device=dev, dtype=torch.float32)
-    if B and P:
+    if B and P and parts is not None:
+        _launch("pdw_pool_branch_fwd_parts", dev, parts.data_ptr(), parts.shape[0] // B, w_pool.data_ptr(),
+                b_pool.data_ptr() if b_pool is not None else None, b_out.data_ptr() if b_out is not None else None,
+                m.data_ptr(), rowbias.data_ptr(), B, P, D, _lib.dtype_code(x.dtype))
+    elif B and P:
         ws = _pool_ws(B, P, D, dev)
         _launch("pdw_pool_branch_fwd", dev, x.data_ptr(), w_pool.data_ptr(),
                 b_pool.data_ptr() if b_pool is not None else None, b_out.data_ptr() if b_out is not None else None,
@@ -249,9 +269,9 @@ def pool_branch_forward(x, w_pool, b_pool=None, b_out=None):
     return m, rowbias
 
 
-def pool_branch_backward(gy, m, w_pool):
+def pool_branch_backward(gy, m, w_pool, parts=None):
     """-> (gbias [2, D]: the same sums twice, one tensor row for each bias; gw_pool [D, D] in gy's dtype;
-    dmean fp32 [B, D])."""
+    dmean fp32 [B, D]).  parts: chunk sums of gy as in pool_branch_forward."""
     dev = _lib.require_device(gy, m, w_pool)
     B, D = gy.shape[0], gy.shape[-1]
     P = gy.numel() // max(B * D, 1)
@@ -259,6 +279,11 @@ def pool_branch_backward(gy, m, w_pool):
     gwp = torch.empty((D, D), device=dev, dtype=gy.dtype)
     dmean = torch.empty((B, D), device=dev, dtype=torch.float32)
     ws = _pool_ws(B, P, D, dev)
+    if parts is not None:
+        _launch("pdw_pool_branch_bwd_parts", dev, parts.data_ptr(), parts.shape[0] // B, m.data_ptr(), w_pool.data_ptr(),
+                gbias[0].data_ptr(), gbias[1].data_ptr(), gwp.data_ptr(), dmean.data_ptr(), ws.data_ptr(),
+                ws.numel() * 4, B, P, D, _lib.dtype_code(gy.dtype))
+        return gbias, gwp, dmean
     _launch("pdw_pool_branch_bwd", dev, gy.data_ptr(), m.data_ptr(), w_pool.data_ptr(), gbias[0].data_ptr(),
             gbias[1].data_ptr(), gwp.data_ptr(), dmean.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, P, D,
             _lib.dtype_code(gy.dtype))

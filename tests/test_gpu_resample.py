@@ -231,3 +231,31 @@ def test_pool_branch(dtype, shape):
     assert torch.equal(gbias[0], gbias[1])
     assert_close(gwp, (gs.t() @ m.double().cpu()).numpy(), dtype, "w_pool grad")
     assert_close(dmean, ((gs @ wp.double()) / (H * W)).numpy(), torch.float32, "dmean", scale=8.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,P,K,NO,kmajor", [(3, 64, 128, 64, False), (2, 96, 64, 128, True), (32, 3136, 128, 64, False),
+                                             (1, 32, 128, 8, True)])
+def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
+    """The dense kernel's by-product (sums of x over groups of 32 rows) against a float64 sum, and the mean branch
+    computed from it against the one that reads x itself."""
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(P + K)
+    x = randn(gen, B, P, K).to(dtype).cuda()
+    w = (randn(gen, K, NO) if kmajor else randn(gen, NO, K)).to(dtype).cuda() / 8
+    assert ops.dense_colsum_supported(K, NO, dtype, P)
+    y, parts = ops.dense_forward(x, w, w_kmajor=kmajor, colsum=True)
+    assert torch.equal(y, ops.dense_forward(x, w, w_kmajor=kmajor))
+    ref = x.double().view(B * P // 32, 32, K).sum(1)
+    assert (parts.double() - ref).abs().max().item() <= 1e-5 * max(1.0, ref.abs().max().item())
+    wp = (randn(gen, K, K) / 11).to(dtype).cuda()
+    bp = randn(gen, K).to(dtype).cuda()
+    m0, rb0 = ops.pool_branch_forward(x, wp, bp, None)
+    m1, rb1 = ops.pool_branch_forward(x, wp, bp, None, parts=parts)
+    assert_close(m1, m0.double().cpu().numpy(), dtype, "mean from parts")
+    assert (rb1 - rb0).abs().max().item() <= 2e-2 * max(1.0, rb0.abs().max().item())
+    g0 = ops.pool_branch_backward(x, m0, wp)
+    g1 = ops.pool_branch_backward(x, m0, wp, parts=parts)
+    for a, b, what in zip(g1, g0, ("bias grad", "pool weight grad", "mean grad")):
+        assert_close(a, b.double().cpu().numpy(), dtype, what + " from parts")
