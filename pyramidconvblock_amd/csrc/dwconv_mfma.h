@@ -130,11 +130,13 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         st.issue(x + (long long)nb * g.H * g.W * g.C, g.H, g.W, g.C, nrow0 - g.PH, ncol0 - g.PW);
     }
 
-    // ---- filter -> LDS operands (rotated for the input gradient), zero elsewhere
+    // ---- filter operands in LDS (rotated for the input gradient), zero elsewhere: cleared here, filled after the
+    // first window has been written (the window is what the workgroup waits for; the filter arrived long before)
     {
-        uint32_t* wz = reinterpret_cast<uint32_t*>(wl);
-        for (int i = tid; i < WR * WPITCH; i += NT) wz[i] = 0u;  // both copies (2 * WR * WPITCH elements)
-        __syncthreads();
+        uint4* wz = reinterpret_cast<uint4*>(wl);  // both copies: 2 * WR * WPITCH elements, a multiple of 8
+        for (int i = tid; i < WR * WPITCH / 4; i += NT) wz[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    auto fill_filter = [&]() {
         unsigned short* wls = reinterpret_cast<unsigned short*>(wl);
 #pragma unroll
         for (int s = 0; s < IT; ++s) {
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
                 wls[(WR + 3 + uu) * WPITCH + (((vv + 1) >> 2) * 16 + ch) * 4 + ((vv + 1) & 3)] = val16;
             }
         }
-    }
+    };
 
     // ---- this lane's operand addresses: wavefront = unit row, lane = (channel bq, q)
     const int bq = lane >> 2, q = lane & 3;
@@ -164,6 +166,7 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         st.commit_begin();
 #pragma unroll
         for (int it = 0; it < NPRE; ++it) st.commit_next(xl, it, g.H, g.W, orow0 - g.PH, ocol0 - g.PW);
+        if (tile == chunk) fill_filter();  // the barrier above lies between the clearing and these writes
         __syncthreads();
         const int orow_b = orow0 + wv * 4;
         const bool has_next = tile + g.nchunks < g.ntiles;
