@@ -33,8 +33,8 @@ WORKLOAD = dict(B=32, H=56, W=56, D=128, k=13, dtype="bf16")
 # scaled by what the same counter reads for a plain copy of known size (`bench.py --kernel copy`); the
 # runs and the scale factors are recorded under profiles/.  None = not measured.
 MEASURED_TRAFFIC = {
-    "dwconv_fwd[32x56x56x64,k=13]": (13144 + 14080) * 1024,   # fetch 13.46 MB + write 14.42 MB
-    "dwconv_dgrad[32x56x56x64,k=13]": (13144 + 14080) * 1024,  # same kernel, same shape
+    "dwconv_fwd[32x56x56x64,k=13]": (12872 + 12544) * 1024,   # fetch 13.18 MB + write 12.85 MB
+    "dwconv_dgrad[32x56x56x64,k=13]": (12872 + 12544) * 1024,  # same kernel, same shape
     "dwconv_wgrad[32x56x56x64,k=13]": (25392 + 2704 + 2721 + 21) * 1024,  # main kernel + partial reduction
 }
 
