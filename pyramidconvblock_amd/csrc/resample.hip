@@ -302,6 +302,65 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
 }
 
 
+// U items per thread, every load of a thread requested before the first use (a streaming kernel lives on the number
+// of loads in flight); items past the end read the last item's data and store nothing.
+constexpr int kGateItems = 4;  // full-resolution items per thread of the paired kernels
+
+template <typename T, int VEC, int U>
+__device__ __forceinline__ void gate_fwd_items(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
+                                               long long first, long long step, long long total) {
+    const int G = I / 2, GV = G / VEC;
+    ChanVec<T, VEC> a[U], b[U];
+    long long m[U];
+    int c[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const long long idx = min(first + u * step, total - 1);
+        c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
+        a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
+        b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float o[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) o[v] = to_f32(a[u].v[v]) * to_f32(b[u].v[v]) * s;
+        if (first + u * step < total) store_f32<T, VEC>(y + m[u] * ldy + c[u], o);
+    }
+}
+
+template <typename T, int VEC, int U>
+__device__ __forceinline__ void gate_bwd_items(const T* __restrict__ x, const T* __restrict__ gy, T* __restrict__ gx,
+                                               int I, int ldg, float s, long long first, long long step,
+                                               long long total) {
+    const int G = I / 2, GV = G / VEC;
+    ChanVec<T, VEC> a[U], b[U], g[U];
+    long long m[U];
+    int c[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const long long idx = min(first + u * step, total - 1);
+        c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
+        a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
+        b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
+        g[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(gy + m[u] * ldg + c[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float ga[VEC], gb[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            const float gv = to_f32(g[u].v[v]);
+            ga[v] = gv * to_f32(b[u].v[v]) * s;
+            gb[v] = gv * to_f32(a[u].v[v]) * s;
+        }
+        if (first + u * step < total) {
+            store_f32<T, VEC>(gx + m[u] * I + c[u], ga);
+            store_f32<T, VEC>(gx + m[u] * I + G + c[u], gb);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- gate fused with the resampling next to it
 // Gate then bilinear resize in one pass: y[b,i,j,c] = interp of gate(x)[b,:,:,c], x[B,h,w,I] -> y[B,H,W,G] (G = I/2).
 // The gate value of each of the 4 source pixels is rounded to T first, exactly what the two separate kernels
@@ -349,6 +408,66 @@ __global__ __launch_bounds__(256) void gate_bilinear_fwd_k(const T* __restrict__
     if (idx < total) gate_bilinear_fwd_item<T, VEC>(x, y, h, w, I, H, W, ldy, sy, sx, s, idx);
 }
 
+// The same for exactly doubled extents, a 2 x 2 block of outputs per thread: their 16 taps fall on a 3 x 3
+// neighbourhood of the source (rows m-1 .. m+1, columns n-1 .. n+1, clamped to the image), so 18 loads and 9 gate
+// values serve 4 outputs instead of 32 and 16.  Same weights (bl_src), same rounding.
+template <typename T, int VEC>
+__device__ __forceinline__ void gate_bilinear_fwd_x2_item(const T* __restrict__ x, T* __restrict__ y, int h, int w,
+                                                          int I, int ldy, float s, long long idx) {
+    const int H = 2 * h, W = 2 * w;
+    const int G = I / 2, GV = G / VEC;
+    const int c = (int)(idx % GV) * VEC;
+    long long t = idx / GV;
+    const int n = (int)(t % w);
+    t /= w;
+    const int m = (int)(t % h);
+    const long long b = t / h;
+    const T* xb = x + b * h * w * I + c;
+    ChanVec<T, VEC> pa[3][3], pb[3][3];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        const int rr = min(max(m - 1 + r, 0), h - 1);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int cc = min(max(n - 1 + k, 0), w - 1);
+            const T* p = xb + ((long long)rr * w + cc) * I;
+            pa[r][k] = *reinterpret_cast<const ChanVec<T, VEC>*>(p);
+            pb[r][k] = *reinterpret_cast<const ChanVec<T, VEC>*>(p + G);
+        }
+    }
+    float gv[3][3][VEC];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                gv[r][k][v] = to_f32(from_f32<T>(to_f32(pa[r][k].v[v]) * to_f32(pb[r][k].v[v]) * s));
+#pragma unroll
+    for (int di = 0; di < 2; ++di) {
+        // Output row 2m + di takes source rows m-1+di and m+di; at the image border bl_src moves the pair one
+        // row inwards, but the clamped neighbourhood then holds the same row twice, so the static entries
+        // (di, di+1) with bl_src's weights give the same sums.
+        int y0, y1;
+        float ly;
+        bl_src(2 * m + di, 0.5f, h, y0, y1, ly);
+        const float hy = 1.f - ly;
+#pragma unroll
+        for (int dj = 0; dj < 2; ++dj) {
+            int x0, x1;
+            float lx;
+            bl_src(2 * n + dj, 0.5f, w, x0, x1, lx);
+            const float hx = 1.f - lx;
+            float o[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                o[v] = hy * (hx * gv[di][dj][v] + lx * gv[di][dj + 1][v]) +
+                       ly * (hx * gv[di + 1][dj][v] + lx * gv[di + 1][dj + 1][v]);
+            store_f32<T, VEC>(y + ((b * H + 2 * m + di) * W + 2 * n + dj) * ldy + c, o);
+        }
+    }
+}
+
 // Both branches of a two-scale block in one launch: workgroups below nblk_full gate the full-resolution tensor into
 // channels [0, G) of y, the others gate and resize the pooled one into channels [G, 2G).
 template <typename T, int VEC>
@@ -357,11 +476,16 @@ __global__ __launch_bounds__(256) void gate_pair_fwd_k(const T* __restrict__ xf,
                                                        float sy, float sx, float s, unsigned nblk_full,
                                                        long long total_full, long long total_half) {
     if (blockIdx.x < nblk_full) {
-        const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-        if (idx < total_full) gate_fwd_item<T, VEC>(xf, y, I, ldy, s, idx);
+        const long long first = (long long)blockIdx.x * (kGateItems * 256) + threadIdx.x;
+        if (first < total_full) gate_fwd_items<T, VEC, kGateItems>(xf, y, I, ldy, s, first, 256, total_full);
     } else {
         const long long idx = (long long)(blockIdx.x - nblk_full) * blockDim.x + threadIdx.x;
-        if (idx < total_half) gate_bilinear_fwd_item<T, VEC>(xh, y + I / 2, h, w, I, H, W, ldy, sy, sx, s, idx);
+        if (idx < total_half) {
+            if (H == 2 * h && W == 2 * w)  // total_half then counts 2 x 2 output blocks
+                gate_bilinear_fwd_x2_item<T, VEC>(xh, y + I / 2, h, w, I, ldy, s, idx);
+            else
+                gate_bilinear_fwd_item<T, VEC>(xh, y + I / 2, h, w, I, H, W, ldy, sy, sx, s, idx);
+        }
     }
 }
 
@@ -440,8 +564,8 @@ __global__ __launch_bounds__(256) void gate_pair_bwd_k(const T* __restrict__ gy,
                                                        unsigned nblk_full, long long total_full,
                                                        long long total_half) {
     if (blockIdx.x < nblk_full) {
-        const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-        if (idx < total_full) gate_bwd_item<T, VEC>(xf, gy, gxf, I, ldg, s, idx);
+        const long long first = (long long)blockIdx.x * (kGateItems * 256) + threadIdx.x;
+        if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
     } else {
         const long long idx = (long long)(blockIdx.x - nblk_full) * blockDim.x + threadIdx.x;
         if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
@@ -995,10 +1119,13 @@ int gate_pair_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, 
                          int dtype, hipStream_t s) {
     const void* ptrs[3] = {xf, xh, y};
     const int vec = pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 3);
-    const long long tf = (long long)B * H * W * (I / 2 / vec), th = tf;
+    const long long tf = (long long)B * H * W * (I / 2 / vec);
+    const long long th = (H == 2 * h && W == 2 * w) ? (long long)B * h * w * (I / 2 / vec) : tf;
     unsigned bf, bh;
     if (tf == 0) return 0;
-    if (!grid_for(tf, &bf) || !grid_for(th, &bh) || (unsigned long long)bf + bh > 0x7fffffffULL) return 1;
+    if (!grid_for((tf + kGateItems - 1) / kGateItems, &bf) || !grid_for(th, &bh) ||
+        (unsigned long long)bf + bh > 0x7fffffffULL)
+        return 1;
     const float sy = (float)h / (float)H, sx = (float)w / (float)W, sc = sqrtf((float)(I / 2));
 #define CALL(T, V) hipLaunchKernelGGL((gate_pair_fwd_k<T, V>), dim3(bf + bh), dim3(256), 0, s, (const T*)xf, (const T*)xh, (T*)y, h, w, I, H, W, ldy, sy, sx, sc, bf, tf, th);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
@@ -1015,7 +1142,9 @@ int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* g
     const long long tf = (long long)B * H * W * (I / 2 / vec), th = (long long)B * h * w * (I / 2 / vec);
     unsigned bf, bh;
     if (tf == 0) return 0;
-    if (!grid_for(tf, &bf) || !grid_for(th, &bh) || (unsigned long long)bf + bh > 0x7fffffffULL) return 1;
+    if (!grid_for((tf + kGateItems - 1) / kGateItems, &bf) || !grid_for(th, &bh) ||
+        (unsigned long long)bf + bh > 0x7fffffffULL)
+        return 1;
     const float sc = sqrtf((float)(I / 2));
 #define CALL(T, V) hipLaunchKernelGGL((gate_pair_bwd_k<T, V>), dim3(bf + bh), dim3(256), 0, s, (const T*)gy, (const T*)xf, (const T*)xh, (T*)gxf, (T*)gxh, h, w, I, ldg, sc, bf, tf, th);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
