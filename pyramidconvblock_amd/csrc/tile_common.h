@@ -151,16 +151,27 @@ struct TileStager {
         chc = chok ? ch : 0;
     }
 
+    // Requests the first NPRE passes of a window.  For 16-bit types the address is the (uniform) image pointer plus
+    // an unsigned 32-bit byte offset, which the load takes as it is (no 64-bit arithmetic per load; the callers
+    // guard H * W * C < 2^31): the request phase is pure address arithmetic, and everything behind it waits for the
+    // data.
     __device__ __forceinline__ void issue(const T* __restrict__ img, int H, int W, int C, int row0, int col0) {
-        const T* xb = img + chc;
+        const char* base = reinterpret_cast<const char*>(img);
+        const int WC = W * C;
         int r = sr0, u = su0;
 #pragma unroll
         for (int it = 0; it < NPRE; ++it) {
             const int ih = min(max(row0 + min(r, rows - 1), 0), H - 1);
+            const int rowoff = ih * WC + chc;
 #pragma unroll
             for (int l = 0; l < NL; ++l) {
                 const int iw = min(max(col0 + NL * u + l, 0), W - 1);
-                pre[it][l] = *reinterpret_cast<const ChanVec<T, V>*>(xb + (ih * W + iw) * C);
+                if constexpr (sizeof(T) == 2) {  // < 2^31 elements: the byte offset fits 32 bits
+                    const unsigned off = (unsigned)(rowoff + iw * C) * 2u;
+                    pre[it][l] = *reinterpret_cast<const ChanVec<T, V>*>(base + off);
+                } else {
+                    pre[it][l] = *reinterpret_cast<const ChanVec<T, V>*>(img + (rowoff + iw * C));
+                }
             }
             r += step_r, u += step_u;
             if (u >= CPn) u -= CPn, ++r;
