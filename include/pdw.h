@@ -176,6 +176,19 @@ int pdw_pool_branch_bwd_parts(const float *parts, int nparts, const void *m, con
                               void *gbias2, void *gw_pool, float *dmean, void *workspace, size_t workspace_bytes,
                               int B, int P, int D, int dtype, void *stream);
 
+/* The middle of a two-scale block as one launch each way: pdw_gate_pair_fwd together with
+ * pdw_pool_branch_fwd_parts, and pdw_gate_pair_bwd together with pdw_pool_branch_bwd_parts (same arguments, same
+ * results; the mean branch is a handful of latency-bound workgroups that ride in the gate kernel's grid).  When
+ * the combination is not covered (fp32, D > 128, unaligned slices) the two kernels are launched one after the
+ * other.  P = positions per image of the tensor whose chunk sums `parts` holds (conv_block.py:40-49). */
+int pdw_block_mid_fwd(const void *xf, const void *xh, void *y, int B, int H, int W, int h, int w, int I, int ldy,
+                      const float *parts, int nparts, const void *w_pool, const void *b_pool, const void *b_out,
+                      void *m, float *rowbias, int P, int D, int dtype, void *stream);
+int pdw_block_mid_bwd(const void *gy, const void *xf, const void *xh, void *gxf, void *gxh, int B, int H, int W,
+                      int h, int w, int I, int ldgy, const float *parts, int nparts, const void *m,
+                      const void *w_pool, void *gbias, void *gbias2, void *gw_pool, float *dmean, void *workspace,
+                      size_t workspace_bytes, int P, int D, int dtype, void *stream);
+
 /* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 4 == 0;
  * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).
  *   y[n,o] = sum_k x[n,k] * W(o,k) + bias[o] + rowbias[n / P][o]        x[N,K] -> y[N,NO]

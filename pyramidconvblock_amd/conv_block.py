@@ -130,9 +130,16 @@ class ConvBlockFunction(torch.autograd.Function):
                     ops.gate_forward(c, out=dst)
             convs.append(c)
             pooled.append(p)
-        if pair:
+        if pair and xparts is not None:
+            # both gates and the mean branch (mean -> conv_pool, plus conv_out's bias: one fp32 row per image) in
+            # one launch
+            m, yp = ops.block_mid_forward(convs[0], convs[1], cat, xparts, H * W, w_pool.detach().contiguous(),
+                                          b_pool, b_out)
+        elif pair:
             ops.gate_pair_forward(convs[0], convs[1], cat)
-        if same_dt and B > 0:
+        if pair and xparts is not None:
+            pass
+        elif same_dt and B > 0:
             # mean over positions -> conv_pool, plus conv_out's bias: one fp32 row per image
             m, yp = ops.pool_branch_forward(x, w_pool.detach().contiguous(), b_pool, b_out, parts=xparts)
         else:
@@ -186,7 +193,14 @@ class ConvBlockFunction(torch.autograd.Function):
                 dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
                 grad_w_out = _weight_grad(g2d, cat.view(N, G * ns))
 
-            if pool_fast:
+            gcs = None
+            if (pool_fast and gparts is not None and _is_pair(scales) and H == 2 * convs[1].shape[1]
+                    and W == 2 * convs[1].shape[2] and convs[1].shape[1] >= 2 and convs[1].shape[2] >= 2):
+                # the gradients of both gates and the mean branch's backward in one launch
+                gcf, gch, gbias, grad_w_pool, dmean = ops.block_mid_backward(convs[0], convs[1], dcat, gparts, H * W, m,
+                                                                             w_pool.detach().contiguous())
+                gcs = (gcf, gch)
+            elif pool_fast:
                 gbias, grad_w_pool, dmean = ops.pool_branch_backward(gy, m, w_pool.detach().contiguous(), parts=gparts)
             else:
                 gs = ops.spatial_sum(gy)                             # [B, D] fp32: column sums per image
@@ -202,7 +216,8 @@ class ConvBlockFunction(torch.autograd.Function):
             # first full-resolution branch, the others are accumulated into its result
             order = sorted(range(ns), key=lambda i: scales[i] == 1.)
             waiting = []                                               # pooled gradients not yet added to da
-            gcs = ops.gate_pair_backward(convs[0], convs[1], dcat) if _is_pair(scales) else None
+            if gcs is None and _is_pair(scales):
+                gcs = ops.gate_pair_backward(convs[0], convs[1], dcat)
             for i in order:
                 s = scales[i]
                 w = w_dw[i].detach().to(dt).contiguous()

@@ -316,6 +316,48 @@ int pdw_pool_branch_bwd_parts(const float* parts, int nparts, const void* m, con
                                   (hipStream_t)stream, parts, nparts);
 }
 
+int pdw_block_mid_fwd(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
+                      const float* parts, int nparts, const void* w_pool, const void* b_pool, const void* b_out, void* m,
+                      float* rowbias, int P, int D, int dtype, void* stream) {
+    if (int e = check_resample("pdw_block_mid_fwd", xh, y, B, H, W, I, h, w, dtype)) return e;
+    if (I < 2 || (I & 1)) return set_error("pdw_block_mid_fwd: need even I >= 2 (I=%d)", I), 1;
+    if (B < 1 || P < 1 || D < 1 || nparts < 1)
+        return set_error("pdw_block_mid_fwd: bad extents B=%d P=%d D=%d nparts=%d", B, P, D, nparts), 1;
+    if (!xf || !parts || !w_pool || !m || !rowbias) return set_error("pdw_block_mid_fwd: null pointer"), 1;
+    if (ldy == 0) ldy = I;
+    if (ldy < I) return set_error("pdw_block_mid_fwd: ldy=%d smaller than I=%d", ldy, I), 1;
+    const int r = block_mid_fwd_launch(xf, xh, y, B, H, W, h, w, I, ldy, parts, nparts, w_pool, b_pool, b_out, m,
+                                       rowbias, P, D, dtype, (hipStream_t)stream);
+    if (r != -1) return r;
+    if (int e = gate_pair_fwd_launch(xf, xh, y, B, H, W, h, w, I, ldy, dtype, (hipStream_t)stream)) return e;
+    return pool_branch_fwd_launch(nullptr, w_pool, b_pool, b_out, m, rowbias, nullptr, B, P, D, dtype,
+                                  (hipStream_t)stream, parts, nparts);
+}
+
+int pdw_block_mid_bwd(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
+                      int w, int I, int ldgy, const float* parts, int nparts, const void* m, const void* w_pool,
+                      void* gbias, void* gbias2, void* gw_pool, float* dmean, void* workspace, size_t workspace_bytes,
+                      int P, int D, int dtype, void* stream) {
+    if (int e = check_resample("pdw_block_mid_bwd", gy, gxh, B, H, W, I, h, w, dtype)) return e;
+    if (I < 2 || (I & 1)) return set_error("pdw_block_mid_bwd: need even I >= 2 (I=%d)", I), 1;
+    if (B < 1 || P < 1 || D < 1 || nparts < 1)
+        return set_error("pdw_block_mid_bwd: bad extents B=%d P=%d D=%d nparts=%d", B, P, D, nparts), 1;
+    if (!xf || !xh || !gxf || !parts || !m || !w_pool || !gbias || !gw_pool || !dmean)
+        return set_error("pdw_block_mid_bwd: null pointer"), 1;
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2)
+        return set_error("pdw_block_mid_bwd: needs H = 2h, W = 2w, h,w >= 2 (h=%d w=%d H=%d W=%d)", h, w, H, W), 1;
+    if (!workspace || workspace_bytes < pool_branch_workspace(B, P, D))
+        return set_error("pdw_block_mid_bwd: workspace too small"), 1;
+    if (ldgy == 0) ldgy = I;
+    if (ldgy < I) return set_error("pdw_block_mid_bwd: ldgy=%d smaller than I=%d", ldgy, I), 1;
+    const int r = block_mid_bwd_launch(gy, xf, xh, gxf, gxh, B, H, W, h, w, I, ldgy, parts, nparts, m, w_pool, gbias,
+                                       gbias2, gw_pool, dmean, (float*)workspace, P, D, dtype, (hipStream_t)stream);
+    if (r != -1) return r;
+    if (int e = gate_pair_bwd_launch(gy, xf, xh, gxf, gxh, B, H, W, h, w, I, ldgy, dtype, (hipStream_t)stream)) return e;
+    return pool_branch_bwd_launch(nullptr, m, w_pool, gbias, gbias2, gw_pool, dmean, (float*)workspace, B, P, D, dtype,
+                                  (hipStream_t)stream, parts, nparts);
+}
+
 int pdw_dense_colsum_supported(int K, int NO, int dtype) {
     return (dense_colsum_supported(K, NO, dtype) && dense_wgrad_supported(K, NO, dtype)) ? 1 : 0;
 }

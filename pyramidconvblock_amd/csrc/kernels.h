@@ -49,6 +49,13 @@ int gate_pair_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, 
                          int dtype, hipStream_t s);
 int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
                          int w, int I, int ldg, int dtype, hipStream_t s);
+int block_mid_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
+                         const float* parts, int nparts, const void* wp, const void* bp, const void* bo, void* m,
+                         float* rowbias, int P, int D, int dtype, hipStream_t s);
+int block_mid_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
+                         int w, int I, int ldg, const float* parts, int nparts, const void* m, const void* wp,
+                         void* gbias, void* gbias2, void* gwp, float* dmean, float* ws, int P, int D, int dtype,
+                         hipStream_t s);
 int gate_bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int I, int H, int W, int ldy, int dtype,
                              hipStream_t s);
 int bilinear_gate_bwd_launch(const void* gy, const void* x, void* gx, int B, int h, int w, int I, int H, int W, int ldg,

@@ -806,12 +806,12 @@ __device__ __forceinline__ void colsum_coop(const float* __restrict__ pp, int nc
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restrict__ part, int nchunks, int D,
-                                                            float inv_p, const T* __restrict__ wp,
-                                                            const T* __restrict__ bp, const T* __restrict__ bo,
-                                                            T* __restrict__ m, float* __restrict__ rowbias) {
-    extern __shared__ float sm[];  // [D] means, [8][D] partial column sums
-    const int b = blockIdx.x, tid = threadIdx.x;
+__device__ __forceinline__ void pool_branch_fwd_v8_body(const float* __restrict__ part, int nchunks, int D,
+                                                        float inv_p, const T* __restrict__ wp,
+                                                        const T* __restrict__ bp, const T* __restrict__ bo,
+                                                        T* __restrict__ m, float* __restrict__ rowbias, int b,
+                                                        float* sm) {  // sm: [D] means, [8][D] partial column sums
+    const int tid = threadIdx.x;
     // weight rows of this thread: outputs o = tid/8 + 32*pass, channel vectors sub + 8*i  (requested first)
     const int sub = tid & 7, ol = tid >> 3;
     ChanVec<T, 8> wv[4][2];
@@ -851,6 +851,15 @@ __global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restr
             rowbias[(long long)b * D + o] = acc;
         }
     }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restrict__ part, int nchunks, int D,
+                                                            float inv_p, const T* __restrict__ wp,
+                                                            const T* __restrict__ bp, const T* __restrict__ bo,
+                                                            T* __restrict__ m, float* __restrict__ rowbias) {
+    extern __shared__ float sm[];
+    pool_branch_fwd_v8_body<T>(part, nchunks, D, inv_p, wp, bp, bo, m, rowbias, blockIdx.x, sm);
 }
 
 template <typename T>
@@ -944,17 +953,17 @@ __device__ __forceinline__ void pool_branch_bwd_b_v8_body(const T* __restrict__ 
 // Both parts in one launch: workgroups [0, B) are part A for image b, workgroups [B, B + D) part B for feature o.
 // Part B sums its column of the per-chunk sums itself (8 lanes per image), so it does not wait for part A.
 template <typename T>
-__global__ __launch_bounds__(256) void pool_branch_bwd_v8_k(const float* __restrict__ part, int nchunks, int B, int D,
-                                                            float inv_p, const T* __restrict__ wp,
-                                                            const T* __restrict__ m, float* __restrict__ gs,
-                                                            float* __restrict__ dmean, T* __restrict__ gbias,
-                                                            T* __restrict__ gbias2, T* __restrict__ gwp) {
-    extern __shared__ float sm[];
-    if ((int)blockIdx.x < B) {
-        pool_branch_bwd_a_v8_body<T>(part, nchunks, D, inv_p, wp, gs, dmean, blockIdx.x, sm);
+__device__ __forceinline__ void pool_branch_bwd_v8_block(const float* __restrict__ part, int nchunks, int B, int D,
+                                                         float inv_p, const T* __restrict__ wp,
+                                                         const T* __restrict__ m, float* __restrict__ gs,
+                                                         float* __restrict__ dmean, T* __restrict__ gbias,
+                                                         T* __restrict__ gbias2, T* __restrict__ gwp, int bid,
+                                                         float* sm) {
+    if (bid < B) {
+        pool_branch_bwd_a_v8_body<T>(part, nchunks, D, inv_p, wp, gs, dmean, bid, sm);
         return;
     }
-    const int o = blockIdx.x - B, tid = threadIdx.x, l8 = tid & 7;
+    const int o = bid - B, tid = threadIdx.x, l8 = tid & 7;
     for (int b = tid >> 3; b < B; b += 32) {
         const float* pp = part + (long long)b * nchunks * D + o;
         float sv = 0.f;
@@ -966,6 +975,88 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_v8_k(const float* __restr
     }
     __syncthreads();
     pool_branch_bwd_b_v8_body<T>(m, B, D, gbias, gbias2, gwp, o, sm);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void pool_branch_bwd_v8_k(const float* __restrict__ part, int nchunks, int B, int D,
+                                                            float inv_p, const T* __restrict__ wp,
+                                                            const T* __restrict__ m, float* __restrict__ gs,
+                                                            float* __restrict__ dmean, T* __restrict__ gbias,
+                                                            T* __restrict__ gbias2, T* __restrict__ gwp) {
+    extern __shared__ float sm[];
+    pool_branch_bwd_v8_block<T>(part, nchunks, B, D, inv_p, wp, m, gs, dmean, gbias, gbias2, gwp, blockIdx.x, sm);
+}
+
+// ---- the middle of a two-scale block in one launch each way: the (tiny, latency-bound) mean branch rides on the
+// gate kernels.  Its workgroups come first in the grid, the gate workgroups after them.
+struct PoolFwdJob {
+    const float* part;
+    int nchunks, B, D;
+    float inv_p;
+    const void *wp, *bp, *bo;
+    void* m;
+    float* rowbias;
+};
+struct PoolBwdJob {
+    const float* part;
+    int nchunks, B, D;
+    float inv_p;
+    const void *wp, *m;
+    float *gs, *dmean;
+    void *gbias, *gbias2, *gwp;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void block_mid_fwd_k(const T* __restrict__ xf, const T* __restrict__ xh,
+                                                       T* __restrict__ y, int h, int w, int I, int H, int W, int ldy,
+                                                       float sy, float sx, float s, unsigned nblk_full,
+                                                       long long total_full, long long total_half,
+                                                       const PoolFwdJob job) {
+    extern __shared__ float sm[];
+    constexpr int VEC = 8;
+    unsigned bid = blockIdx.x;
+    if (bid < (unsigned)job.B) {
+        pool_branch_fwd_v8_body<T>(job.part, job.nchunks, job.D, job.inv_p, (const T*)job.wp, (const T*)job.bp,
+                                   (const T*)job.bo, (T*)job.m, job.rowbias, bid, sm);
+        return;
+    }
+    bid -= job.B;
+    if (bid < nblk_full) {
+        const long long first = (long long)bid * (kGateItems * 256) + threadIdx.x;
+        if (first < total_full) gate_fwd_items<T, VEC, kGateItems>(xf, y, I, ldy, s, first, 256, total_full);
+    } else {
+        const long long idx = (long long)(bid - nblk_full) * blockDim.x + threadIdx.x;
+        if (idx < total_half) {
+            if (H == 2 * h && W == 2 * w)
+                gate_bilinear_fwd_x2_item<T, VEC>(xh, y + I / 2, h, w, I, ldy, s, idx);
+            else
+                gate_bilinear_fwd_item<T, VEC>(xh, y + I / 2, h, w, I, H, W, ldy, sy, sx, s, idx);
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy, const T* __restrict__ xf,
+                                                       const T* __restrict__ xh, T* __restrict__ gxf,
+                                                       T* __restrict__ gxh, int h, int w, int I, int ldg, float s,
+                                                       unsigned nblk_full, long long total_full,
+                                                       long long total_half, const PoolBwdJob job) {
+    extern __shared__ float sm[];
+    constexpr int VEC = 8;
+    unsigned bid = blockIdx.x;
+    if (bid < (unsigned)(job.B + job.D)) {
+        pool_branch_bwd_v8_block<T>(job.part, job.nchunks, job.B, job.D, job.inv_p, (const T*)job.wp, (const T*)job.m,
+                                    job.gs, job.dmean, (T*)job.gbias, (T*)job.gbias2, (T*)job.gwp, (int)bid, sm);
+        return;
+    }
+    bid -= job.B + job.D;
+    if (bid < nblk_full) {
+        const long long first = (long long)bid * (kGateItems * 256) + threadIdx.x;
+        if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
+    } else {
+        const long long idx = (long long)(bid - nblk_full) * blockDim.x + threadIdx.x;
+        if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
+    }
 }
 
 // y[b,p,c] += v[b,c]  (v in fp32, one rounding)
@@ -1150,6 +1241,68 @@ int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* g
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL
     return check_launch("gate_pair_bwd");
+}
+
+// The gate pair and the mean branch (from per-chunk sums `parts`) of a two-scale block in one launch; -1 when the
+// combination is not covered (the caller launches the two separately).
+static bool pool_v8_ok(const void* wp, const void* m_or_null, const float* parts, int B, int D, int dtype) {
+    return dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0 &&
+           (reinterpret_cast<uintptr_t>(m_or_null) & 15) == 0 && (reinterpret_cast<uintptr_t>(parts) & 15) == 0 &&
+           (size_t)(B + 16 * D) * sizeof(float) <= 64 * 1024;
+}
+
+int block_mid_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
+                         const float* parts, int nparts, const void* wp, const void* bp, const void* bo, void* m,
+                         float* rowbias, int P, int D, int dtype, hipStream_t s) {
+    const void* ptrs[3] = {xf, xh, y};
+    if (pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 3) != 8 || !pool_v8_ok(wp, nullptr, parts, B, D, dtype))
+        return -1;
+    const long long tf = (long long)B * H * W * (I / 2 / 8);
+    const long long th = (H == 2 * h && W == 2 * w) ? (long long)B * h * w * (I / 2 / 8) : tf;
+    unsigned bf, bh;
+    if (tf == 0) return -1;
+    if (!grid_for((tf + kGateItems - 1) / kGateItems, &bf) || !grid_for(th, &bh) ||
+        (unsigned long long)bf + bh + B > 0x7fffffffULL)
+        return 1;
+    const float sy = (float)h / (float)H, sx = (float)w / (float)W, sc = sqrtf((float)(I / 2));
+    const PoolFwdJob job{parts, nparts, B, D, 1.f / (float)P, wp, bp, bo, m, rowbias};
+    const size_t lds = (size_t)9 * D * sizeof(float);
+    if (dtype == kF16)
+        hipLaunchKernelGGL((block_mid_fwd_k<f16_t>), dim3(bf + bh + B), dim3(256), lds, s, (const f16_t*)xf,
+                           (const f16_t*)xh, (f16_t*)y, h, w, I, H, W, ldy, sy, sx, sc, bf, tf, th, job);
+    else
+        hipLaunchKernelGGL((block_mid_fwd_k<bf16_t>), dim3(bf + bh + B), dim3(256), lds, s, (const bf16_t*)xf,
+                           (const bf16_t*)xh, (bf16_t*)y, h, w, I, H, W, ldy, sy, sx, sc, bf, tf, th, job);
+    return check_launch("block_mid_fwd");
+}
+
+int block_mid_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
+                         int w, int I, int ldg, const float* parts, int nparts, const void* m, const void* wp,
+                         void* gbias, void* gbias2, void* gwp, float* dmean, float* ws, int P, int D, int dtype,
+                         hipStream_t s) {
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2) return -1;
+    const void* ptrs[5] = {gy, xf, xh, gxf, gxh};
+    if (pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 5) != 8 || !pool_v8_ok(wp, m, parts, B, D, dtype)) return -1;
+    const long long tf = (long long)B * H * W * (I / 2 / 8), th = (long long)B * h * w * (I / 2 / 8);
+    unsigned bf, bh;
+    if (tf == 0) return -1;
+    if (!grid_for((tf + kGateItems - 1) / kGateItems, &bf) || !grid_for(th, &bh) ||
+        (unsigned long long)bf + bh + B + D > 0x7fffffffULL)
+        return 1;
+    const float sc = sqrtf((float)(I / 2));
+    float* gs = ws + spatial_sum_workspace(B, P, D) / sizeof(float);
+    const PoolBwdJob job{parts, nparts, B, D, 1.f / (float)P, wp, m, gs, dmean, gbias, gbias2, gwp};
+    const size_t la = (size_t)17 * D * sizeof(float), lb = (size_t)(B + 16 * D) * sizeof(float);
+    const size_t lds = la > lb ? la : lb;
+    if (dtype == kF16)
+        hipLaunchKernelGGL((block_mid_bwd_k<f16_t>), dim3(bf + bh + B + D), dim3(256), lds, s, (const f16_t*)gy,
+                           (const f16_t*)xf, (const f16_t*)xh, (f16_t*)gxf, (f16_t*)gxh, h, w, I, ldg, sc, bf, tf, th,
+                           job);
+    else
+        hipLaunchKernelGGL((block_mid_bwd_k<bf16_t>), dim3(bf + bh + B + D), dim3(256), lds, s, (const bf16_t*)gy,
+                           (const bf16_t*)xf, (const bf16_t*)xh, (bf16_t*)gxf, (bf16_t*)gxh, h, w, I, ldg, sc, bf, tf,
+                           th, job);
+    return check_launch("block_mid_bwd");
 }
 
 int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s) {

@@ -161,6 +161,42 @@ def gate_pair_backward(xf, xh, gy):
     return gate_backward(xf, gy[..., :G]), bilinear_gate_backward(xh, gy[..., G:2 * G])
 
 
+def block_mid_forward(xf, xh, out, parts, P, w_pool, b_pool=None, b_out=None):
+    """gate_pair_forward(xf, xh, out) and pool_branch_forward(parts=...) as one launch -> (m, rowbias)."""
+    dev = _lib.require_device(xf, xh, out, w_pool)
+    B, H, W, I = xf.shape
+    h, w = xh.shape[1], xh.shape[2]
+    D = w_pool.shape[0]
+    if I % 2 or xh.shape[3] != I or out.shape[3] != I:
+        raise ValueError("gate pair: xf, xh need the same even channel count I and out I channels")
+    m = torch.empty((B, D), device=dev, dtype=xf.dtype)
+    rowbias = torch.empty((B, D), device=dev, dtype=torch.float32)
+    _launch("pdw_block_mid_fwd", dev, xf.data_ptr(), xh.data_ptr(), out.data_ptr(), B, H, W, h, w, I, _pixel_stride(out),
+            parts.data_ptr(), parts.shape[0] // B, w_pool.data_ptr(), b_pool.data_ptr() if b_pool is not None else None,
+            b_out.data_ptr() if b_out is not None else None, m.data_ptr(), rowbias.data_ptr(), int(P), D,
+            _lib.dtype_code(xf.dtype))
+    return m, rowbias
+
+
+def block_mid_backward(xf, xh, gy, parts, P, m, w_pool):
+    """gate_pair_backward and pool_branch_backward(parts=...) as one launch (exactly doubled extents only)
+    -> (gxf, gxh, gbias [2, D], gw_pool, dmean)."""
+    dev = _lib.require_device(xf, xh, gy, m, w_pool)
+    B, H, W, I = xf.shape
+    h, w = xh.shape[1], xh.shape[2]
+    D = w_pool.shape[0]
+    gxf, gxh = torch.empty_like(xf), torch.empty_like(xh)
+    gbias = torch.empty((2, D), device=dev, dtype=xf.dtype)
+    gwp = torch.empty((D, D), device=dev, dtype=xf.dtype)
+    dmean = torch.empty((B, D), device=dev, dtype=torch.float32)
+    ws = _pool_ws(B, int(P), D, dev)
+    _launch("pdw_block_mid_bwd", dev, gy.data_ptr(), xf.data_ptr(), xh.data_ptr(), gxf.data_ptr(), gxh.data_ptr(), B, H, W,
+            h, w, I, _pixel_stride(gy), parts.data_ptr(), parts.shape[0] // B, m.data_ptr(), w_pool.data_ptr(),
+            gbias[0].data_ptr(), gbias[1].data_ptr(), gwp.data_ptr(), dmean.data_ptr(), ws.data_ptr(), ws.numel() * 4,
+            int(P), D, _lib.dtype_code(xf.dtype))
+    return gxf, gxh, gbias, gwp, dmean
+
+
 def spatial_sum(x):
     """x [B, ..., C] -> fp32 [B, C]: sum over all middle dimensions."""
     dev = _lib.require_device(x)

@@ -259,3 +259,39 @@ def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
     g1 = ops.pool_branch_backward(x, m0, wp, parts=parts)
     for a, b, what in zip(g1, g0, ("bias grad", "pool weight grad", "mean grad")):
         assert_close(a, b.double().cpu().numpy(), dtype, what + " from parts")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,hw,I,D", [(2, (8, 12), 32, 64), (3, (28, 28), 64, 128), (1, (4, 8), 16, 128)])
+def test_block_mid_matches_separate_launches(dtype, B, hw, I, D):
+    """Gate pair + mean branch in one launch, forward and backward, against the separate entry points (which
+    have their own oracle tests)."""
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(B + I)
+    h, w = hw
+    H, W = 2 * h, 2 * w
+    P = H * W
+    xf = randn(gen, B, H, W, I).to(dtype).cuda()
+    xh = randn(gen, B, h, w, I).to(dtype).cuda()
+    x = randn(gen, B, P, D).to(dtype).cuda()
+    wd = (randn(gen, 64, D) / 8).to(dtype).cuda()
+    _, parts = ops.dense_forward(x, wd, colsum=True)
+    wp = (randn(gen, D, D) / 11).to(dtype).cuda()
+    bp, bo = randn(gen, D).to(dtype).cuda(), randn(gen, D).to(dtype).cuda()
+    cat0 = torch.zeros(B, H, W, I, dtype=dtype, device="cuda")
+    cat1 = torch.zeros_like(cat0)
+    ops.gate_pair_forward(xf, xh, cat0)
+    m0, rb0 = ops.pool_branch_forward(x, wp, bp, bo, parts=parts)
+    m1, rb1 = ops.block_mid_forward(xf, xh, cat1, parts, P, wp, bp, bo)
+    def same(t0, t1):   # two instantiations of the same arithmetic: at most a last-bit difference
+        d = (t0.double() - t1.double()).abs().max().item()
+        return d <= 2e-3 * max(1.0, t0.double().abs().max().item())
+
+    assert same(cat0, cat1) and torch.equal(m0, m1) and same(rb0, rb1)
+    g = randn(gen, B, H, W, I).to(dtype).cuda()
+    a0 = ops.gate_pair_backward(xf, xh, g)
+    b0 = ops.pool_branch_backward(x, m0, wp, parts=parts)
+    r1 = ops.block_mid_backward(xf, xh, g, parts, P, m0, wp)
+    for t0, t1 in zip(tuple(a0) + tuple(b0), r1):
+        assert same(t0, t1)
