@@ -72,6 +72,11 @@ int pdw_dwconv_dgrad_addpool(const void *gy, const void *w, const void *gp, void
  * for its four weight gradients. */
 int pdw_reduce_defer_begin(void);
 int pdw_reduce_defer_flush(void *stream);
+/* pdw_dense_fwd that also runs the reductions recorded so far (see above) in spare workgroups of its own launch;
+ * the later pdw_reduce_defer_flush then launches nothing.  For a dense layer that runs after the last kernel that
+ * produced the partial results: the input gradient of conv_up at the end of the block's backward. */
+int pdw_dense_fwd_flush(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
+                        long long N, int K, int NO, int P, int dtype, void *stream);
 
 /* Bytes of device scratch pdw_dwconv_wgrad needs for these extents (fp32 partial sums). */
 size_t pdw_dwconv_wgrad_workspace_bytes(int B, int H, int W, int C, int KH, int KW, int SH, int SW,

@@ -250,8 +250,9 @@ class ConvBlockFunction(torch.autograd.Function):
             if fast_up:
                 grad_w_up = ops.dense_wgrad(da, x)
                 if ctx.needs_input_grad[0]:
+                    # the last kernel of the pass: the recorded summations ride in its grid
                     dx = ops.dense_forward(da, w_up.detach().contiguous(), w_kmajor=True, rowbias=dmean,
-                                           rows_per_image=H * W)
+                                           rows_per_image=H * W, flush_reductions=True)
             else:
                 grad_w_up = _weight_grad(a2d, x.view(N, D))
                 if ctx.needs_input_grad[0]:

@@ -7,6 +7,7 @@
 #include "../../include/pdw.h"
 #include "common.h"
 #include "kernels.h"
+#include "reduce_parts.h"
 
 namespace pdw {
 
@@ -388,6 +389,23 @@ int pdw_dense_fwd(const void* x, const void* w, int w_kmajor, const void* bias, 
     if (rowbias && P < 1) return set_error("pdw_dense_fwd: rowbias needs P >= 1"), 1;
     const int r = dense_rows_launch(x, w, w_kmajor ? 1 : 0, bias, rowbias, y, N, K, NO, P, dtype, (hipStream_t)stream);
     if (r == -1) return set_error("pdw_dense_fwd: K=%d NO=%d dtype=%d not supported (see pdw_dense_supported)", K, NO, dtype), 3;
+    return r;
+}
+
+int pdw_dense_fwd_flush(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
+                        long long N, int K, int NO, int P, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd_flush: unknown dtype %d", dtype), 1;
+    if (N < 0 || K < 1 || NO < 1) return set_error("pdw_dense_fwd_flush: bad extents N=%lld K=%d NO=%d", N, K, NO), 1;
+    if (N > 0 && (!x || !w || !y)) return set_error("pdw_dense_fwd_flush: null pointer"), 1;
+    if (rowbias && P < 1) return set_error("pdw_dense_fwd_flush: rowbias needs P >= 1"), 1;
+    ReduceJobs jobs;
+    const bool ride = N > 0 && dense_rows_supported(K, NO, dtype) && reduce_defer_take(&jobs) > 0;
+    const int r = dense_rows_launch(x, w, w_kmajor ? 1 : 0, bias, rowbias, y, N, K, NO, P, dtype, (hipStream_t)stream,
+                                    nullptr, ride ? &jobs : nullptr);
+    if (r == -1) {
+        if (ride) (void)reduce_jobs_launch(jobs, (hipStream_t)stream);  // the reductions still run, on their own
+        return set_error("pdw_dense_fwd_flush: K=%d NO=%d dtype=%d not supported (see pdw_dense_supported)", K, NO, dtype), 3;
+    }
     return r;
 }
 

@@ -18,6 +18,7 @@
 
 #include "common.h"
 #include "kernels.h"
+#include "reduce_parts.h"
 
 namespace pdw {
 
@@ -139,11 +140,10 @@ struct WTransposer {
 // is 8 columns of one row, and with 64 % (K/8) == 0 a lane keeps the same 8 columns for every chunk: 8 running
 // sums per lane, combined over the 512/K lanes that share them through the tile buffer once the fragments are out.
 template <typename T, bool KMAJOR, bool COLSUM>
-__global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
-                                                    const T* __restrict__ bias, const float* __restrict__ rowbias,
-                                                    T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
-                                                    int NO, int P, int nkt, int nnt) {
-    extern __shared__ uint32_t dsm[];
+__device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T* __restrict__ W,
+                                                const T* __restrict__ bias, const float* __restrict__ rowbias,
+                                                T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
+                                                int NO, int P, int nkt, int nnt, int nblocks, uint32_t* dsm) {
     T* wl = reinterpret_cast<T*>(dsm);
     const int ldw = K + 8;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, 
     const int ldt = (K > NO ? K : NO) + 8;             // pitch of the per-wave tile buffer (elements)
     T* tl = wl + NO * ldw + wave * 32 * ldt;
     const long long ntiles = (N + 31) / 32;
-    const long long gw = (long long)blockIdx.x * 4 + wave, nw = (long long)gridDim.x * 4;
+    const long long gw = (long long)blockIdx.x * 4 + wave, nw = (long long)nblocks * 4;
     const int cpk = K / 8;                              // 16-byte chunks per input row
     const int nin = 32 * cpk;                           // chunks per input tile (<= 512)
     constexpr int LP = 8;                               // chunk loads per lane (K <= 128)
@@ -305,6 +305,32 @@ __global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, 
     }
 }
 
+template <typename T, bool KMAJOR, bool COLSUM>
+__global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
+                                                    const T* __restrict__ bias, const float* __restrict__ rowbias,
+                                                    T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
+                                                    int NO, int P, int nkt, int nnt) {
+    extern __shared__ uint32_t dsm[];
+    dense_rows_body<T, KMAJOR, COLSUM>(X, W, bias, rowbias, Y, colsum, N, K, NO, P, nkt, nnt, gridDim.x, dsm);
+}
+
+// The same with the deferred partial-sum reductions of a backward pass in the workgroups behind the first
+// `nblocks`: they are a few microseconds of latency that need no launch of their own when a dense layer runs
+// after the last of the kernels that produce the partials.
+template <typename T, bool KMAJOR>
+__global__ __launch_bounds__(256, 3) void dense_rows_rider_k(const T* __restrict__ X, const T* __restrict__ W,
+                                                          const T* __restrict__ bias,
+                                                          const float* __restrict__ rowbias, T* __restrict__ Y,
+                                                          long long N, int K, int NO, int P, int nkt, int nnt,
+                                                          int nblocks, const ReduceJobs jobs) {
+    extern __shared__ uint32_t dsm[];
+    if ((int)blockIdx.x >= nblocks) {
+        reduce_jobs_block(jobs, blockIdx.x - nblocks, reinterpret_cast<float(*)[32]>(dsm));
+        return;
+    }
+    dense_rows_body<T, KMAJOR, false>(X, W, bias, rowbias, Y, nullptr, N, K, NO, P, nkt, nnt, nblocks, dsm);
+}
+
 // dW partials.  A workgroup of 4 wavefronts walks 64-row stages b, b + gridDim.x, ...: the stage's rows
 // of A and B are copied to LDS with coalesced 16-byte loads (requested one stage ahead and held in
 // registers while the current stage is multiplied), then wavefront w multiplies rows 16w..16w+15, reading
@@ -447,8 +473,10 @@ int dense_colsum_supported(int K, int NO, int dtype) {
 }
 
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
-                      long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum) {
+                      long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum,
+                      const ReduceJobs* rider) {
     if (!dense_dims_ok(K, NO, dtype)) return -1;
+    if (rider && colsum) return -1;
     if (colsum && (!dense_colsum_supported(K, NO, dtype) || (reinterpret_cast<uintptr_t>(colsum) & 15))) return -1;
     if (N == 0) return 0;
     if (N > 0x7fffffffLL) return -1;
@@ -462,6 +490,19 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     if (blocks > cap) blocks = cap;  // persistent workgroups: the weights are staged to LDS once each
     if (blocks < 1) blocks = 1;
     const size_t lds = ((size_t)NO * (K + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2;
+    if (rider) {
+        const unsigned total = (unsigned)blocks + (unsigned)rider->first_block[rider->njobs];
+#define PDW_RIDE(T, KM)                                                                                           \
+    hipLaunchKernelGGL((dense_rows_rider_k<T, KM>), dim3(total), dim3(256), lds, s, (const T*)x, (const T*)w,     \
+                       (const T*)bias, rowbias, (T*)y, N, K, NO, P > 0 ? P : 1, nkt, nnt, (int)blocks, *rider)
+        if (dtype == kF16) {
+            if (w_kmajor) PDW_RIDE(f16_t, true); else PDW_RIDE(f16_t, false);
+        } else {
+            if (w_kmajor) PDW_RIDE(bf16_t, true); else PDW_RIDE(bf16_t, false);
+        }
+#undef PDW_RIDE
+        return check_launch("dense_rows_rider");
+    }
 #define PDW_GO(T, KM, CSUM)                                                                                    \
     hipLaunchKernelGGL((dense_rows_k<T, KM, CSUM>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x,        \
                        (const T*)w, (const T*)bias, rowbias, (T*)y, colsum, N, K, NO, P > 0 ? P : 1, nkt, nnt)

@@ -5,6 +5,7 @@
 // loads of one tap are one contiguous run of channels-last memory.
 #include "common.h"
 #include "kernels.h"
+#include "reduce_parts.h"
 
 namespace pdw {
 
@@ -119,39 +120,6 @@ __global__ __launch_bounds__(256) void dwconv_wgrad_direct(const T* __restrict__
     }
 }
 
-// Pass 2 of wgrad (shared with the tiled kernels): dw[e] = sum over parts in a fixed order.
-// Block = 32 outputs x 8 part lanes; lane q adds parts q, q+8, ... and the 8 lanes are combined
-// through LDS, so the reads of one part are contiguous and many parts are in flight.
-template <typename T>
-__device__ __forceinline__ void reduce_parts_block(const float* __restrict__ part, T* __restrict__ dw, int nparts, int n,
-                                                   int blk, float (*red)[32]) {
-    const int el = threadIdx.x & 31, q = threadIdx.x >> 5;
-    const int e = blk * 32 + el;
-    float s0 = 0.f, s1 = 0.f;
-    if (e < n) {
-        int p = q;
-        for (; p + 56 < nparts; p += 64) {  // eight loads in flight per lane: the pass is pure latency
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part[(long long)(p + 8 * u) * n + e];
-            s0 += (v[0] + v[2]) + (v[4] + v[6]);
-            s1 += (v[1] + v[3]) + (v[5] + v[7]);
-        }
-        for (; p + 8 < nparts; p += 16) {
-            s0 += part[(long long)p * n + e];
-            s1 += part[(long long)(p + 8) * n + e];
-        }
-        if (p < nparts) s0 += part[(long long)p * n + e];
-    }
-    red[q][el] = s0 + s1;
-    __syncthreads();
-    if (q == 0 && e < n) {
-        const float s = ((red[0][el] + red[1][el]) + (red[2][el] + red[3][el])) +
-                        ((red[4][el] + red[5][el]) + (red[6][el] + red[7][el]));
-        dw[e] = from_f32<T>(s);
-    }
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restrict__ part, T* __restrict__ dw,
                                                           int nparts, int n) {
@@ -159,33 +127,21 @@ __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restric
     reduce_parts_block<T>(part, dw, nparts, n, blockIdx.x, red);
 }
 
-// Several such reductions in one launch: the weight gradients of a backward pass are each a few microseconds of
-// latency, and nothing reads them before the pass is over.
-constexpr int kMaxReduceJobs = 8;
-struct ReduceJobs {
-    const float* part[kMaxReduceJobs];
-    void* out[kMaxReduceJobs];
-    int nparts[kMaxReduceJobs], n[kMaxReduceJobs], dtype[kMaxReduceJobs];
-    int first_block[kMaxReduceJobs + 1];
-    int njobs;
-};
-
 __global__ __launch_bounds__(256) void wgrad_reduce_many(const ReduceJobs jobs) {
     __shared__ float red[8][32];
-    int j = 0;
-    while (j + 1 < jobs.njobs && (int)blockIdx.x >= jobs.first_block[j + 1]) ++j;  // uniform: scalar ALU
-    const int blk = blockIdx.x - jobs.first_block[j];
-    switch (jobs.dtype[j]) {
-        case kF32: reduce_parts_block<float>(jobs.part[j], (float*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
-        case kF16: reduce_parts_block<f16_t>(jobs.part[j], (f16_t*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
-        default: reduce_parts_block<bf16_t>(jobs.part[j], (bf16_t*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
-    }
+    reduce_jobs_block(jobs, blockIdx.x, red);
 }
 
 // Deferred mode (per host thread): between reduce_defer_begin and reduce_defer_flush the reductions are only
 // recorded; the flush runs them all in one launch.
 static thread_local bool t_defer = false;
 static thread_local ReduceJobs t_jobs;
+
+int reduce_jobs_launch(const ReduceJobs& jobs, hipStream_t s) {
+    if (jobs.njobs == 0) return 0;
+    hipLaunchKernelGGL(wgrad_reduce_many, dim3(jobs.first_block[jobs.njobs]), dim3(256), 0, s, jobs);
+    return check_launch("wgrad_reduce_many");
+}
 
 int reduce_defer_begin() {
     if (t_defer) return set_error("pdw_reduce_defer_begin: already deferring on this thread"), 1;
@@ -199,9 +155,20 @@ int reduce_defer_flush(hipStream_t s) {
     if (!t_defer) return set_error("pdw_reduce_defer_flush: pdw_reduce_defer_begin was not called"), 1;
     t_defer = false;
     if (t_jobs.njobs == 0) return 0;
-    hipLaunchKernelGGL(wgrad_reduce_many, dim3(t_jobs.first_block[t_jobs.njobs]), dim3(256), 0, s, t_jobs);
+    const int r = reduce_jobs_launch(t_jobs, s);
     t_jobs.njobs = 0;
-    return check_launch("wgrad_reduce_many");
+    return r;
+}
+
+// Hands the recorded jobs to a caller that runs them inside another kernel's grid; the later flush then finds
+// nothing left to do.  Returns the number of jobs.
+int reduce_defer_take(ReduceJobs* out) {
+    if (!t_defer || t_jobs.njobs == 0) return 0;
+    *out = t_jobs;
+    const int n = t_jobs.njobs;
+    t_jobs.njobs = 0;
+    t_jobs.first_block[0] = 0;
+    return n;
 }
 
 template <typename T>

@@ -22,6 +22,9 @@ int dwconv_wgrad_direct_launch(const void* x, const void* gy, void* dw, void* ws
                                hipStream_t s);
 template <typename T>
 int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s);
+struct ReduceJobs;
+int reduce_defer_take(ReduceJobs* out);  // moves the recorded jobs out (0 = none); the flush then has nothing to do
+int reduce_jobs_launch(const ReduceJobs& jobs, hipStream_t s);
 int reduce_defer_begin();
 int reduce_defer_flush(hipStream_t s);
 
@@ -77,7 +80,8 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
 int dense_rows_supported(int K, int NO, int dtype);
 // colsum (optional, fp32 [ceil(N/32)][K], K = 64 or 128): per-32-row sums of x, see dense_colsum_supported
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
-                      long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum = nullptr);
+                      long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum = nullptr,
+                      const struct ReduceJobs* rider = nullptr);
 int dense_colsum_supported(int K, int NO, int dtype);
 int dense_wgrad_supported(int M, int NO, int dtype);
 size_t dense_wgrad_workspace(long long N, int M, int NO);

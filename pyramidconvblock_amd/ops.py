@@ -238,12 +238,14 @@ def dense_colsum_supported(K, NO, dtype, rows_per_image) -> bool:
             and bool(_lib.lib().pdw_dense_colsum_supported(int(K), int(NO), _lib.dtype_code(dtype))))
 
 
-def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=1, colsum=False):
+def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=1, colsum=False,
+                  flush_reductions=False):
     """y[..., o] = sum_k x[..., k] * W(o, k) + bias[o] + rowbias[image][o].
 
     w is [NO, K] (nn.Linear layout) or, with w_kmajor, [K, NO].  rowbias is fp32 [B, NO], one row per
     `rows_per_image` consecutive rows of x.  With colsum (see dense_colsum_supported) the result is
-    (y, parts): parts fp32 [N / 32, K], the sums of x over each group of 32 consecutive rows."""
+    (y, parts): parts fp32 [N / 32, K], the sums of x over each group of 32 consecutive rows.  With
+    flush_reductions, inside _lib.deferred_reductions, the summations recorded so far run in this launch."""
     dev = _lib.require_device(x, w)
     K = x.shape[-1]
     NO = w.shape[1] if w_kmajor else w.shape[0]
@@ -258,9 +260,10 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
                     y.data_ptr(), parts.data_ptr(), N, K, NO, int(rows_per_image), _lib.dtype_code(x.dtype))
         return y, parts
     if N:
-        _launch("pdw_dense_fwd", dev, x.data_ptr(), w.data_ptr(), 1 if w_kmajor else 0,
-                bias.data_ptr() if bias is not None else None, rowbias.data_ptr() if rowbias is not None else None,
-                y.data_ptr(), N, K, NO, int(rows_per_image), _lib.dtype_code(x.dtype))
+        _launch("pdw_dense_fwd_flush" if flush_reductions else "pdw_dense_fwd", dev, x.data_ptr(), w.data_ptr(),
+                1 if w_kmajor else 0, bias.data_ptr() if bias is not None else None,
+                rowbias.data_ptr() if rowbias is not None else None, y.data_ptr(), N, K, NO, int(rows_per_image),
+                _lib.dtype_code(x.dtype))
     return y
 
 

@@ -181,3 +181,29 @@ def test_deferred_reductions_match_immediate_ones():
             assert torch.equal(t, ref[i % len(ref)]), i
     with pytest.raises(RuntimeError):
         _lib.check(_lib.lib().pdw_reduce_defer_flush(None), "flush without begin")
+
+
+def test_deferred_reductions_ride_on_a_dense_layer():
+    """The recorded summations executed inside a dense layer's launch give the same weight gradients, and the
+    dense result is unchanged."""
+    from pyramidconvblock_amd import _lib, ops
+    from pyramidconvblock_amd.dwconv import dwconv_wgrad
+
+    gen = torch.Generator().manual_seed(12)
+    x = randn(gen, 2, 20, 24, 32).to(torch.bfloat16).cuda()
+    g = randn(gen, 2, 20, 24, 32).to(torch.bfloat16).cuda()
+    a = randn(gen, 960, 64).to(torch.bfloat16).cuda()
+    b = randn(gen, 960, 128).to(torch.bfloat16).cuda()
+    w = (randn(gen, 128, 64) / 8).to(torch.bfloat16).cuda()
+    geo = ((1, 1), (6, 6), (1, 1))
+    ref = (dwconv_wgrad(x, g, (13, 13, 32), *geo), ops.dense_wgrad(a, b), ops.dense_forward(a, w))
+    for kmajor in (False, True):
+        wk = w.t().contiguous() if kmajor else w
+        with _lib.deferred_reductions(a.device):
+            d0 = dwconv_wgrad(x, g, (13, 13, 32), *geo)
+            d1 = ops.dense_wgrad(a, b)
+            y = ops.dense_forward(a, wk, w_kmajor=kmajor, flush_reductions=True)
+        torch.cuda.synchronize()
+        assert torch.equal(d0, ref[0]) and torch.equal(d1, ref[1]) and torch.equal(y, ref[2])
+    y = ops.dense_forward(a, w, flush_reductions=True)   # nothing recorded: a plain dense layer
+    assert torch.equal(y, ref[2])
