@@ -187,10 +187,20 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         for (int it = 0; it < ITW; ++it)
             if (wdst[it] >= 0) *reinterpret_cast<Frag*>(wl + wdst[it]) = wv[it];
     } else {
-        WTransposer<T, ITW> wt;
-        wt.load(W, K, NO, ldw, tid);
-        if (gw < ntiles) load_tile(gw);
-        wt.store(wl, ldw);
+        // (K/4)(NO/4) sub-blocks over 256 threads: 2 per thread for 64 x 128, 4 at most (uniform switch, so that
+        // a small matrix does not pay for the largest one's address arithmetic and predicated passes)
+        const int nsub = (K / 4) * (NO / 4);
+        if (nsub <= 512) {
+            WTransposer<T, 2> wt;
+            wt.load(W, K, NO, ldw, tid);
+            if (gw < ntiles) load_tile(gw);
+            wt.store(wl, ldw);
+        } else {
+            WTransposer<T, 4> wt;
+            wt.load(W, K, NO, ldw, tid);
+            if (gw < ntiles) load_tile(gw);
+            wt.store(wl, ldw);
+        }
     }
     const int cpr = NO / 8;  // 16-byte chunks per output row (NO % 8 == 0 on this path)
     constexpr int LO = 2 * kNT;  // 16-byte chunks per lane of a 32 x NO tile (NO <= 32 * kNT)
