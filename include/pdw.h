@@ -45,6 +45,14 @@ int pdw_conv_out_size(int in, int k, int stride, int pad, int dil);
 int pdw_dwconv_fwd(const void *x, const void *w, void *y, int B, int H, int W, int C, int KH, int KW,
                    int SH, int SW, int PH, int PW, int DH, int DW, int dtype, void *stream);
 
+/* pdw_dwconv_fwd plus the adaptive average pool of the same input to (h, wp): y = conv(x), xp[B,h,wp,C] = pool(x).
+ * ConvBlock feeds one tensor to the full-resolution conv and, pooled, to the next scale (conv_block.py:14-16, 41);
+ * when the pool halves both extents exactly (and the conv keeps them: stride 1, 2*pad = k-1, pad even, 16-bit
+ * types, C % 8 == 0) the conv kernel writes the pooled tensor from its staged input window, otherwise
+ * pdw_dwconv_fwd and pdw_avgpool_fwd run one after the other. */
+int pdw_dwconv_fwd_pool(const void *x, const void *w, void *y, void *xp, int B, int H, int W, int C, int KH, int KW,
+                        int SH, int SW, int PH, int PW, int DH, int DW, int h, int wp, int dtype, void *stream);
+
 /* Input gradient (exact adjoint of pdw_dwconv_fwd in x): gy[B,OH,OW,C] -> dx[B,H,W,C]; H,W are
  * the forward INPUT extents.  Fully overwrites dx (no pre-zeroing needed).
  * Replaces the launch of _depthwise_conv_backward_input_kernel, dwconv_triton.py:358-366

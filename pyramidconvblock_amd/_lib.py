@@ -26,6 +26,7 @@ _SIGS = {
     "pdw_last_error": (c_char_p, []),
     "pdw_conv_out_size": (c_int, [c_int] * 5),
     "pdw_dwconv_fwd": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
+    "pdw_dwconv_fwd_pool": (c_int, [c_void_p] * 4 + _CONV + [c_int, c_int, c_int, c_void_p]),
     "pdw_dwconv_dgrad": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
     "pdw_reduce_defer_begin": (c_int, []),
     "pdw_reduce_defer_flush": (c_int, [c_void_p]),

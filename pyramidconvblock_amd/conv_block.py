@@ -113,19 +113,24 @@ class ConvBlockFunction(torch.autograd.Function):
         cat = torch.empty((B, H, W, G * ns), device=dev, dtype=dt)
         convs, pooled = [], []
         pair = _is_pair(scales)           # scales (1, s): both gates go into cat in one launch
+        ready = None                      # pooled input already produced by the full-resolution conv's kernel
         for i, s in enumerate(scales):
             w = w_dw[i].detach().to(dt).contiguous()
             k1, k2 = w.shape[0], w.shape[1]
             geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
             dst = cat[..., i * G:(i + 1) * G]
             if s != 1.:
-                p = ops.avgpool_forward(a, (int(H * s), int(W * s)))
+                hw = (int(H * s), int(W * s))
+                p = ready if ready is not None and tuple(ready.shape[1:3]) == hw else ops.avgpool_forward(a, hw)
                 c = dwconv_forward(p, w, *geo)
                 if not pair:
                     ops.gate_bilinear_forward(c, (H, W), out=dst)
             else:
                 p = None
-                c = dwconv_forward(a, w, *geo)
+                if pair and B > 0:   # the conv reads `a` anyway: it also writes the next scale's pooled input
+                    c, ready = dwconv_forward(a, w, *geo, pool_to=(int(H * scales[1]), int(W * scales[1])))
+                else:
+                    c = dwconv_forward(a, w, *geo)
                 if not pair:
                     ops.gate_forward(c, out=dst)
             convs.append(c)

@@ -79,6 +79,21 @@ int pdw_dwconv_fwd(const void* x, const void* w, void* y, int B, int H, int W, i
     return dwconv_fwd_direct_launch(x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype, (hipStream_t)stream);
 }
 
+int pdw_dwconv_fwd_pool(const void* x, const void* w, void* y, void* xp, int B, int H, int W, int C, int KH, int KW,
+                        int SH, int SW, int PH, int PW, int DH, int DW, int h, int wp, int dtype, void* stream) {
+    if (int e = check_conv("pdw_dwconv_fwd_pool", x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
+    if (int e = check_resample("pdw_dwconv_fwd_pool", x, xp, B, H, W, C, h, wp, dtype)) return e;
+    if (B == 0) return 0;
+    const int OH = conv_out_size(H, KH, SH, PH, DH), OW = conv_out_size(W, KW, SW, PW, DW);
+    if (OH > 0 && OW > 0 && SH == 1 && SW == 1 && DH == 1 && DW == 1 && H == 2 * h && W == 2 * wp) {
+        const int r = dwconv_tiled_launch(x, w, y, B, H, W, C, KH, KW, PH, PW, false, dtype, (hipStream_t)stream, nullptr,
+                                          xp);
+        if (r != -1) return r;
+    }
+    if (int e = pdw_dwconv_fwd(x, w, y, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype, stream)) return e;
+    return avgpool_fwd_launch(x, xp, B, H, W, C, h, wp, dtype, (hipStream_t)stream);
+}
+
 int pdw_dwconv_dgrad(const void* gy, const void* w, void* dx, int B, int H, int W, int C, int KH, int KW, int SH,
                      int SW, int PH, int PW, int DH, int DW, int dtype, void* stream) {
     if (int e = check_conv("pdw_dwconv_dgrad", gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;

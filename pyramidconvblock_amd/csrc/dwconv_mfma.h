@@ -45,6 +45,16 @@ __device__ __forceinline__ f32x4 mfma4(uint2 a, uint2 b, f32x4 c, f16_t) {
     return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
 }
 
+// The two 16-bit values of a window dword as floats.
+template <typename T>
+__device__ __forceinline__ float pair_lo(uint32_t d) {
+    return to_f32(__builtin_bit_cast(T, (unsigned short)(d & 0xffffu)));
+}
+template <typename T>
+__device__ __forceinline__ float pair_hi(uint32_t d) {
+    return to_f32(__builtin_bit_cast(T, (unsigned short)(d >> 16)));
+}
+
 // 8 values of T: a + b / 4, rounded once more (what an accumulating pool gradient does to a stored tensor).
 template <typename T>
 __device__ __forceinline__ uint4 add_quarter(uint4 a, uint4 b) {
@@ -82,10 +92,13 @@ struct MfmaShape {
                                                     // the zero filter columns included (0 * garbage could be NaN)
 };
 
-template <typename T, int K, int S, int NWV, bool ADD>
+// MODE 0: plain.  MODE 1 (input gradient of a tensor that was also average-pooled 2x2): y += add[i/2, j/2] / 4.
+// MODE 2 (forward): the 2x2 average pool of x itself is written to `pool` as a by-product, from the staged window.
+template <typename T, int K, int S, int NWV, int MODE>
 __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(const T* __restrict__ x, const T* __restrict__ w,
-                                                             const T* __restrict__ add, T* __restrict__ y,
-                                                             const MfmaGeom g) {
+                                                             const T* __restrict__ add, T* __restrict__ pool,
+                                                             T* __restrict__ y, const MfmaGeom g) {
+    constexpr bool ADD = MODE == 1;
     using Sh = MfmaShape<K, S, NWV>;
     constexpr int V = 8, NT = NWV * 64, CS = Sh::CS, TH = Sh::TH, TW = Sh::TW;
     constexpr int KP = Sh::KP, NVB = Sh::NVB, NPH = Sh::NPH, WR = Sh::WR, ROWS_IN = Sh::ROWS_IN, NCOL = Sh::NCOL;
@@ -168,6 +181,32 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         for (int it = 0; it < NPRE; ++it) st.commit_next(xl, it, g.H, g.W, orow0 - g.PH, ocol0 - g.PW);
         if (tile == chunk) fill_filter();  // the barrier above lies between the clearing and these writes
         __syncthreads();
+        if constexpr (MODE == 2) {
+            // 2x2 means of the tile's own input pixels (H = OH, W = OW, both even, PW even: a window dword is one of
+            // the pool's column pairs), 8 channels per item, summed in the order of the stand-alone pool kernel
+            constexpr int PWh = TW / 2, NITEM = (TH / 2) * PWh * 2;
+            const int AH = g.H >> 1, AW = g.W >> 1;
+            T* pb = pool + ((long long)b * AH * AW) * g.C + c0;
+            for (int it = tid; it < NITEM; it += NT) {
+                const int oct = it & 1, px = it >> 1;
+                const int pi = px / PWh, pj = px - pi * PWh;
+                const int gi = (orow0 >> 1) + pi, gj = (ocol0 >> 1) + pj;
+                if (gi < AH && gj < AW && c0 + 8 * oct < g.C) {
+                    const uint32_t* wp = xl + ((g.PH + 2 * pi) * CS + 8 * oct) * g.CPn + (g.PW >> 1) + pj;
+                    union {
+                        uint4 u;
+                        T t[8];
+                    } o;
+#pragma unroll
+                    for (int ch = 0; ch < 8; ++ch) {
+                        const uint32_t d0 = wp[ch * g.CPn], d1 = wp[CS * g.CPn + ch * g.CPn];
+                        const float s = ((pair_lo<T>(d0) + pair_hi<T>(d0)) + pair_lo<T>(d1)) + pair_hi<T>(d1);
+                        o.t[ch] = from_f32<T>(s * 0.25f);
+                    }
+                    *reinterpret_cast<uint4*>(pb + ((long long)gi * AW + gj) * g.C + 8 * oct) = o.u;
+                }
+            }
+        }
         const int orow_b = orow0 + wv * 4;
         const bool has_next = tile + g.nchunks < g.ntiles;
         const bool active = orow_b < g.OH;  // this wavefront's unit has outputs (uniform per wavefront)
@@ -300,8 +339,8 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
 // Host side
 
 template <typename T, int K, int S, int NWV>
-static int launch_mfma(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH,
-                       int PW, bool flip, hipStream_t s) {
+static int launch_mfma(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
+                       int PH, int PW, bool flip, hipStream_t s) {
     using Sh = MfmaShape<K, S, NWV>;
     MfmaGeom g;
     g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0, g.one = 1;
@@ -333,25 +372,28 @@ static int launch_mfma(const void* x, const void* w, const void* add, void* y, i
     if (getenv("PDW_MFMA_NCH")) nch = atoi(getenv("PDW_MFMA_NCH"));
     g.nchunks = (int)(nch < 1 ? 1 : nch);
     const long long nblocks = (long long)g.nchunks * g.slices;
-    auto kern = add ? dwconv_mfma_k<T, K, S, NWV, true> : dwconv_mfma_k<T, K, S, NWV, false>;
-    static bool attr_done[2] = {false, false};
-    if (!attr_done[add ? 1 : 0]) {
+    const int mode = add ? 1 : (pool ? 2 : 0);
+    auto kern = mode == 1 ? dwconv_mfma_k<T, K, S, NWV, 1> : (mode == 2 ? dwconv_mfma_k<T, K, S, NWV, 2> : dwconv_mfma_k<T, K, S, NWV, 0>);
+    static bool attr_done[3] = {false, false, false};
+    if (!attr_done[mode]) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_done[add ? 1 : 0] = true;
+        attr_done[mode] = true;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NWV * 64), lds, s, (const T*)x, (const T*)w, (const T*)add,
-                       (T*)y, g);
+                       (T*)pool, (T*)y, g);
     return check_launch("dwconv_mfma");
 }
 
 // -1: not covered (the caller falls back to the vector-ALU tiled kernel).
 template <typename T, int K>
-static int launch_mfma_best(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH,
-                            int PW, bool flip, hipStream_t s) {
+static int launch_mfma_best(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W,
+                            int C, int PH, int PW, bool flip, hipStream_t s) {
     const int OH = H + 2 * PH - K + 1, OW = W + 2 * PW - K + 1;
     if (OH < 1 || OW < 1 || C % 8 != 0) return -1;
     if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return -1;
     if (add && ((OH | OW) & 1 || (reinterpret_cast<uintptr_t>(add) & 15) != 0)) return -1;
+    if (pool && (add || flip || OH != H || OW != W || ((H | W | PW) & 1) || (reinterpret_cast<uintptr_t>(pool) & 15) != 0))
+        return -1;
     // strips of 14 columns (tile 56 wide) or 8 (tile 32 wide): whichever pads the output width less
     const bool s14 = (long long)cdiv(OW, 56) * 56 <= (long long)cdiv(OW, 32) * 32;
     const int tw = s14 ? 56 : 32;
@@ -360,19 +402,19 @@ static int launch_mfma_best(const void* x, const void* w, const void* add, void*
     bool w8 = t8 >= 192;
     if (getenv("PDW_MFMA_NWV")) w8 = atoi(getenv("PDW_MFMA_NWV")) == 8;
     if (s14) {
-        if (w8) return launch_mfma<T, K, 14, 8>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
-        return launch_mfma<T, K, 14, 4>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
+        if (w8) return launch_mfma<T, K, 14, 8>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+        return launch_mfma<T, K, 14, 4>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
     }
-    if (w8) return launch_mfma<T, K, 8, 8>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
-    return launch_mfma<T, K, 8, 4>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
+    if (w8) return launch_mfma<T, K, 8, 8>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+    return launch_mfma<T, K, 8, 4>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
 }
 
 template <int K>
-static int launch_mfma_dtype(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH,
-                             int PW, bool flip, int dtype, hipStream_t s) {
+static int launch_mfma_dtype(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W,
+                             int C, int PH, int PW, bool flip, int dtype, hipStream_t s) {
     switch (dtype) {
-        case kF16: return launch_mfma_best<f16_t, K>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
-        case kBF16: return launch_mfma_best<bf16_t, K>(x, w, add, y, B, H, W, C, PH, PW, flip, s);
+        case kF16: return launch_mfma_best<f16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+        case kBF16: return launch_mfma_best<bf16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
         default: return -1;
     }
 }

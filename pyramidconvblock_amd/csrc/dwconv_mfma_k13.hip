@@ -5,9 +5,9 @@
 
 namespace pdw {
 
-int dwconv_mfma_k13(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k13(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s) {
-    return launch_mfma_dtype<13>(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
+    return launch_mfma_dtype<13>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
 }
 
 }  // namespace pdw

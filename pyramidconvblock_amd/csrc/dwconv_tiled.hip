@@ -25,38 +25,38 @@ int dwconv_tiled_kw15(const void* x, const void* w, void* y, int B, int H, int W
 int dwconv_tiled_kw17(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int PH, int PW,
                       bool flip, int dtype, hipStream_t s);
 
-int dwconv_mfma_k3(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k3(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k5(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k5(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k7(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k7(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k9(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k9(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k11(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k11(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k13(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k13(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k15(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k15(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
-int dwconv_mfma_k17(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int PH, int PW,
+int dwconv_mfma_k17(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
 
 // Matrix-core kernel for square filters and 16-bit types; -1 when it does not cover the case.
-static int dwconv_mfma_launch(const void* x, const void* w, const void* add, void* y, int B, int H, int W, int C, int KH,
+static int dwconv_mfma_launch(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int KH,
                               int KW, int PH, int PW, bool flip, int dtype, hipStream_t s) {
     if (KH != KW || dtype == kF32) return -1;
     const char* e = getenv("PDW_MFMA");
     if (e && atoi(e) == 0) return -1;
     switch (KW) {
-        case 3: return dwconv_mfma_k3(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 5: return dwconv_mfma_k5(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 7: return dwconv_mfma_k7(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 9: return dwconv_mfma_k9(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 11: return dwconv_mfma_k11(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 13: return dwconv_mfma_k13(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 15: return dwconv_mfma_k15(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
-        case 17: return dwconv_mfma_k17(x, w, add, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 3: return dwconv_mfma_k3(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 5: return dwconv_mfma_k5(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 7: return dwconv_mfma_k7(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 9: return dwconv_mfma_k9(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 11: return dwconv_mfma_k11(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 13: return dwconv_mfma_k13(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 15: return dwconv_mfma_k15(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 17: return dwconv_mfma_k17(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
         default: return -1;
     }
 }
@@ -65,11 +65,11 @@ static int dwconv_mfma_launch(const void* x, const void* w, const void* add, voi
 // kernel), otherwise the launch status.  With flip the 180-degree rotated filter is used: the
 // caller passes gy as x with padding k-1-p, which yields the input gradient.
 int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
-                        int PW, bool flip, int dtype, hipStream_t s, const void* add) {
+                        int PW, bool flip, int dtype, hipStream_t s, const void* add, void* pool) {
     if (KH > 31 || H + 2 * PH - KH + 1 < 1 || W + 2 * PW - KW + 1 < 1) return -1;
     {
-        const int r = dwconv_mfma_launch(x, w, add, y, B, H, W, C, KH, KW, PH, PW, flip, dtype, s);
-        if (r != -1 || add) return r;   // only the matrix-core kernel adds the pooled gradient
+        const int r = dwconv_mfma_launch(x, w, add, pool, y, B, H, W, C, KH, KW, PH, PW, flip, dtype, s);
+        if (r != -1 || add || pool) return r;   // only the matrix-core kernel has the fused forms
     }
     switch (KW) {
         case 3: return dwconv_tiled_kw3(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);

@@ -30,9 +30,10 @@ int reduce_defer_flush(hipStream_t s);
 
 // dwconv_tiled.hip: LDS-tiled forward / input gradient for stride 1, dilation 1, odd KW <= 17.
 // Returns -1 if the case is not covered (the caller then uses the direct kernel).
-// `add` (optional, [B, OH/2, OW/2, C]): y += a quarter of add at [i/2, j/2]; -1 if the case with it is not covered.
+// `add` (optional, [B, OH/2, OW/2, C]): y += a quarter of add at [i/2, j/2].  `pool` (optional, [B, H/2, W/2, C]):
+// receives the 2x2 average pool of x.  -1 if the case with either is not covered.
 int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
-                        int PW, bool flip, int dtype, hipStream_t s, const void* add = nullptr);
+                        int PW, bool flip, int dtype, hipStream_t s, const void* add = nullptr, void* pool = nullptr);
 
 // dwconv_wgrad_tiled.hip: LDS-tiled weight gradient for stride 1, dilation 1, odd square filters <= 17.
 size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype);

@@ -25,14 +25,26 @@ def _conv_args(x_shape, w_shape, stride, padding, dilation):
     return (B, H, W, C, KH, KW, stride[0], stride[1], padding[0], padding[1], dilation[0], dilation[1])
 
 
-def dwconv_forward(x, weight, stride, padding, dilation):
-    """y[B,OH,OW,C] = depthwise cross-correlation of x[B,H,W,C] with weight[k1,k2,C]."""
+def dwconv_forward(x, weight, stride, padding, dilation, pool_to=None):
+    """y[B,OH,OW,C] = depthwise cross-correlation of x[B,H,W,C] with weight[k1,k2,C].  With pool_to = (h, w)
+    the result is (y, xp): xp[B,h,w,C] the adaptive average pool of x, from the same kernel when it can be."""
     dev = _lib.require_device(x, weight)
     L = _lib.lib()
     args = _conv_args(x.shape, weight.shape, stride, padding, dilation)
     OH = L.pdw_conv_out_size(args[1], args[4], stride[0], padding[0], dilation[0])
     OW = L.pdw_conv_out_size(args[2], args[5], stride[1], padding[1], dilation[1])
     y = torch.empty((x.shape[0], OH, OW, x.shape[3]), device=dev, dtype=x.dtype)
+    if pool_to is not None:
+        h, w = int(pool_to[0]), int(pool_to[1])
+        xp = torch.empty((x.shape[0], h, w, x.shape[3]), device=dev, dtype=x.dtype)
+        if y.numel() and xp.numel():
+            with _lib.on_device(dev):
+                _lib.check(L.pdw_dwconv_fwd_pool(x.data_ptr(), weight.data_ptr(), y.data_ptr(), xp.data_ptr(), *args,
+                                                 h, w, _lib.dtype_code(x.dtype), _lib.stream_ptr(dev)),
+                           "pdw_dwconv_fwd_pool")
+            return y, xp
+        from . import ops
+        return dwconv_forward(x, weight, stride, padding, dilation), ops.avgpool_forward(x, (h, w))
     if y.numel():
         with _lib.on_device(dev):
             _lib.check(L.pdw_dwconv_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), *args,

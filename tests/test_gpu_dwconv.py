@@ -207,3 +207,22 @@ def test_deferred_reductions_ride_on_a_dense_layer():
         assert torch.equal(d0, ref[0]) and torch.equal(d1, ref[1]) and torch.equal(y, ref[2])
     y = ops.dense_forward(a, w, flush_reductions=True)   # nothing recorded: a plain dense layer
     assert torch.equal(y, ref[2])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 16, 24, 32, 13, (8, 12)), (1, 56, 56, 24, 9, (28, 28)), (2, 12, 10, 8, 3, (6, 5)),
+                                   (2, 14, 18, 16, 5, (5, 7)), (1, 40, 36, 12, 7, (20, 18)), (2, 60, 64, 16, 13, (30, 32)),
+                                   (1, 20, 20, 16, 11, (10, 10))])
+def test_forward_with_pooled_input(oracle, dtype, shape):
+    """Conv output plus the average pool of the conv's input from one entry point: the fused kernel (exact
+    halving, even padding, 16-bit, C % 8 == 0) and the two-kernel path behind it."""
+    from pyramidconvblock_amd.dwconv import dwconv_forward
+
+    B, H, W, C, k, hw = shape
+    gen = torch.Generator().manual_seed(H + W + k)
+    x = randn(gen, B, H, W, C).to(dtype)
+    w = (randn(gen, k, k, C) / k).to(dtype)
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    y, xp = dwconv_forward(x.cuda(), w.cuda(), *geo, pool_to=hw)
+    assert_close(y, oracle.dwconv_fwd(x.double().numpy(), w.double().numpy(), 1, k // 2, 1), dtype, "y")
+    assert_close(xp, oracle.avgpool_fwd(x.double().numpy(), hw), dtype, "pooled input")
