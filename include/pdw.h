@@ -213,12 +213,14 @@ int pdw_dense_supported(int K, int NO, int dtype);
 int pdw_dense_fwd(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
                   long long N, int K, int NO, int P, int dtype, void *stream);
 
-/* pdw_dense_fwd that also writes colsum[t][k] = sum of x[n,k] over the rows n of the t-th group of 32 rows (fp32,
- * ceil(N/32) x K): with 32 | P these are per-chunk sums of each image, which pdw_pool_branch_fwd_parts /
+/* pdw_dense_fwd that also writes colsum[t][k] = sum of x[n,k] over the rows n of the t-th group of R rows (fp32,
+ * ceil(N/R) x K, R = pdw_dense_colsum_rows(), the kernel's row tile): with R | P these are per-chunk sums of each
+ * image, which pdw_pool_branch_fwd_parts /
  * _bwd_parts take in place of a second pass over x (the x.mean of conv_block.py:46 and its gradient ride on
  * conv_up, conv_block.py:37, and on the input gradient of conv_out, conv_block.py:44).  K = 64 or 128 only:
  * pdw_dense_colsum_supported. */
 int pdw_dense_colsum_supported(int K, int NO, int dtype);
+int pdw_dense_colsum_rows(void);
 int pdw_dense_fwd_colsum(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
                          float *colsum, long long N, int K, int NO, int P, int dtype, void *stream);
 

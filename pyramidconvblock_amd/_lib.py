@@ -51,6 +51,7 @@ _SIGS = {
     "pdw_pool_branch_fwd_parts": (c_int, [c_void_p, c_int] + [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
     "pdw_pool_branch_bwd_parts": (c_int, [c_void_p, c_int] + [c_void_p] * 7 + [c_size_t] + [c_int] * 4 + [c_void_p]),
     "pdw_dense_colsum_supported": (c_int, [c_int] * 3),
+    "pdw_dense_colsum_rows": (c_int, []),
     "pdw_dense_fwd_colsum": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong]
                              + [c_int] * 4 + [c_void_p]),
     "pdw_block_mid_fwd": (c_int, [c_void_p] * 3 + [c_int] * 7 + [c_void_p, c_int] + [c_void_p] * 5 + [c_int] * 3

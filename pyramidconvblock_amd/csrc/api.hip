@@ -378,6 +378,8 @@ int pdw_dense_colsum_supported(int K, int NO, int dtype) {
     return (dense_colsum_supported(K, NO, dtype) && dense_wgrad_supported(K, NO, dtype)) ? 1 : 0;
 }
 
+int pdw_dense_colsum_rows(void) { return dense_colsum_rows(); }
+
 int pdw_dense_fwd_colsum(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
                          float* colsum, long long N, int K, int NO, int P, int dtype, void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd_colsum: unknown dtype %d", dtype), 1;

@@ -39,6 +39,23 @@ __device__ __forceinline__ f32x16 mfma32(const Frag& a, const Frag& b, f32x16 c,
                                                   0);
 }
 
+// Development aid (-DPDW_STAMP=1|2|3): wall-clock stamps (10 ns units) of the phases of each wavefront's first
+// tile, for one of the instantiations, read back with pdw_debug_stamps().
+#ifdef PDW_STAMP
+__device__ unsigned long long g_stamps[8192 * 8];
+#define STAMP(i)                                                                                                  \
+    do {                                                                                                          \
+        if constexpr ((PDW_STAMP == 1 && !KMAJOR && !COLSUM) || (PDW_STAMP == 2 && !KMAJOR && COLSUM) ||          \
+                      (PDW_STAMP == 3 && KMAJOR && COLSUM)) {                                                     \
+            __builtin_amdgcn_sched_barrier(0);                                                                    \
+            if (lane == 0) g_stamps[(bid * 4 + wave) * 8 + (i)] = __builtin_amdgcn_s_memrealtime();        \
+            __builtin_amdgcn_sched_barrier(0);                                                                    \
+        }                                                                                                         \
+    } while (0)
+#else
+#define STAMP(i)
+#endif
+
 constexpr int kKT = 8;  // k tiles of 16  (inner dimension <= 128)
 constexpr int kNT = 4;  // feature tiles of 32 (<= 128 features)
 
@@ -143,19 +160,38 @@ template <typename T, bool KMAJOR, bool COLSUM>
 __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T* __restrict__ W,
                                                 const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                 T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
-                                                int NO, int P, int nkt, int nnt, int nblocks, uint32_t* dsm) {
+                                                int NO, int P, int nkt, int nnt, int bid, int nblocks, uint32_t* dsm) {
     T* wl = reinterpret_cast<T*>(dsm);
-    const int ldw = K + 8;
+    // The weights are multiplied as NOP x KP (whole feature tiles, 4 or 8 steps of the inner dimension) with zeros
+    // in the padding, so that the multiplication below is straight-line code without predicates.
+    const int KP = nkt > 4 ? 128 : 64, NOP = nnt * 32;
+    const int ldw = KP + 8;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int ldt = (K > NO ? K : NO) + 8;             // pitch of the per-wave tile buffer (elements)
-    T* tl = wl + NO * ldw + wave * 32 * ldt;
+    T* tl = wl + NOP * ldw + wave * 32 * ldt;
+    // bias[o] + rowbias[image][o] for the (at most two) images of the wavefront's current tile: [2][NOP] floats
+    float* bl = reinterpret_cast<float*>(wl + NOP * ldw + 4 * 32 * ldt) + wave * 2 * NOP;
+    const bool hasb = bias != nullptr || rowbias != nullptr;
+    const int bcol = 4 * l32;                           // this lane's 4 columns of that table (row `half`)
+    const int nimg = rowbias ? (int)((N + P - 1) / P) : 1;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias && bcol < NO) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bv[i] = to_f32(bias[bcol + i]);
+    }
+    if (K != KP || NO != NOP) {  // uniform
+        for (int i = tid; i < NOP * ldw / 8; i += 256) reinterpret_cast<uint4*>(wl)[i] = make_uint4(0u, 0u, 0u, 0u);
+        __syncthreads();
+    }
     const long long ntiles = (N + 31) / 32;
-    const long long gw = (long long)blockIdx.x * 4 + wave, nw = (long long)nblocks * 4;
+    const long long gw = (long long)bid * 4 + wave, nw = (long long)nblocks * 4;
     const int cpk = K / 8;                              // 16-byte chunks per input row
     const int nin = 32 * cpk;                           // chunks per input tile (<= 512)
     constexpr int LP = 8;                               // chunk loads per lane (K <= 128)
+    STAMP(0);
     Frag raw[LP];
+    float4 brow = make_float4(0.f, 0.f, 0.f, 0.f);
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
         const T* base = X + t * 32 * K;
         const long long rows_left = N - t * 32;         // rows of this tile that exist
@@ -164,6 +200,10 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         for (int i = 0; i < LP; ++i) {
             const int cidx = i * 64 + lane;
             raw[i] = cidx < valid ? *reinterpret_cast<const Frag*>(base + (long long)cidx * 8) : Frag{{0u, 0u, 0u, 0u}};
+        }
+        if (rowbias) {  // the tile's per-image rows ride behind its data: a tile of 32 rows meets two images at most
+            const int img = min((int)(t * 32 / P) + half, nimg - 1);
+            if (bcol < NO) brow = *reinterpret_cast<const float4*>(rowbias + (long long)img * NO + bcol);
         }
     };
     // The weights are requested first and written to LDS after the first tile's loads have been issued: loads
@@ -208,11 +248,16 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     strided_offsets<LP>(lane, 64, cpk, ldt, 8, 32, oin);
     strided_offsets<LO>(lane, 64, cpr, ldt, 8, 32, oout);
     __syncthreads();
+    STAMP(1);
     for (long long tile = gw; tile < ntiles; tile += nw) {
+        [[maybe_unused]] const bool first = tile == gw;
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
 #pragma unroll
         for (int i = 0; i < LP; ++i)
             if (oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
+        if (hasb && bcol < NOP)
+            *reinterpret_cast<float4*>(bl + half * NOP + bcol) =
+                make_float4(bv[0] + brow.x, bv[1] + brow.y, bv[2] + brow.z, bv[3] + brow.w);
         float cs[8];
         if constexpr (COLSUM) {
 #pragma unroll
@@ -235,6 +280,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 xf[kt] = Frag{{0u, 0u, 0u, 0u}};
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // fragments are in registers: the buffer may be overwritten
+        if (first) STAMP(2);
         if (tile + nw < ntiles) load_tile(tile + nw);  // next tile in flight during the MFMAs and the store
         if constexpr (COLSUM) {
             float* tf = reinterpret_cast<float*>(tl);  // [512 / K lane groups][K]
@@ -258,46 +304,53 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // read before the result tile is written to the same buffer
         }
-        const long long m = tile * 32 + l32;
-        const float* rb = rowbias ? rowbias + (long long)((int)(m < N ? m : N - 1) / P) * NO : nullptr;
+        if (first) STAMP(3);
+        // this lane's row of the bias table: the image of tile row l32 relative to the tile's first image
+        const float* blr = bl + 4 * half;
+        if (rowbias) {
+            const long long m = tile * 32 + l32;
+            const int img = min((int)((m < N ? m : N - 1) / P), nimg - 1);
+            blr += (img - (int)(tile * 32 / P)) * NOP;
+        }
         for (int nt = 0; nt < nnt; ++nt) {
+            // all LDS reads of the feature tile are issued before its first MFMA
+            const T* wr = wl + (nt * 32 + l32) * ldw + 8 * half;
+            Frag wf[kKT];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
+            if (nkt > 4) {
+#pragma unroll
+                for (int kt = 4; kt < 8; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
+            }
+            float4 r4[4];
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+                r4[g4] = hasb ? *reinterpret_cast<const float4*>(blr + nt * 32 + g4 * 8) : make_float4(0.f, 0.f, 0.f, 0.f);
             f32x16 acc;
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-            float4 r4[4];  // this lane's per-image terms, requested before the MFMA chain
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const int n0 = nt * 32 + g4 * 8 + half * 4;
-                r4[g4] = (rb && n0 < NO) ? *reinterpret_cast<const float4*>(rb + n0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int kt = 0; kt < 4; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
+            if (nkt > 4) {
+#pragma unroll
+                for (int kt = 4; kt < 8; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
             }
-            const int n = nt * 32 + l32;
-            const T* wr = wl + (n < NO ? n : 0) * ldw + 8 * half;
-#pragma unroll
-            for (int kt = 0; kt < kKT; ++kt)
-                if (kt < nkt) {
-                    Frag wf = Frag{{0u, 0u, 0u, 0u}};
-                    if (n < NO && kt * 16 + 8 * half < K) wf = *reinterpret_cast<const Frag*>(wr + kt * 16);
-                    acc = mfma32(wf, xf[kt], acc, T());
-                }
             // lane owns row l32 of the tile and features n0..n0+3 of each accumulator group
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int n0 = nt * 32 + g4 * 8 + half * 4;
                 if (n0 < NO) {
                     float o[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[i] = acc[g4 * 4 + i];
-                    if (bias) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) o[i] += to_f32(bias[n0 + i]);
-                    }
-                    o[0] += r4[g4].x, o[1] += r4[g4].y, o[2] += r4[g4].z, o[3] += r4[g4].w;
+                    o[0] = acc[g4 * 4] + r4[g4].x, o[1] = acc[g4 * 4 + 1] + r4[g4].y;
+                    o[2] = acc[g4 * 4 + 2] + r4[g4].z, o[3] = acc[g4 * 4 + 3] + r4[g4].w;
                     store_f32<T, 4>(tl + l32 * ldt + n0, o);
                 }
             }
+            if (first && nt < 2) STAMP(4 + nt);
         }
         // coalesced copy-out of the 32 x NO tile (same wavefront wrote it: no workgroup barrier needed)
         __builtin_amdgcn_s_waitcnt(0xc07f);
+        if (first) STAMP(6);
         {
             const long long rows_left = N - tile * 32;
             const int valid = (rows_left >= 32 ? 32 : (int)rows_left) * cpr;
@@ -312,33 +365,43 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // copy-out reads done before the next tile overwrites the buffer
+        if (first) STAMP(7);
     }
 }
 
 template <typename T, bool KMAJOR, bool COLSUM>
-__global__ __launch_bounds__(256, 3) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
+__global__ __launch_bounds__(256, 2) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
                                                     const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                     T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
                                                     int NO, int P, int nkt, int nnt) {
     extern __shared__ uint32_t dsm[];
-    dense_rows_body<T, KMAJOR, COLSUM>(X, W, bias, rowbias, Y, colsum, N, K, NO, P, nkt, nnt, gridDim.x, dsm);
+    dense_rows_body<T, KMAJOR, COLSUM>(X, W, bias, rowbias, Y, colsum, N, K, NO, P, nkt, nnt, blockIdx.x, gridDim.x, dsm);
 }
 
-// The same with the deferred partial-sum reductions of a backward pass in the workgroups behind the first
-// `nblocks`: they are a few microseconds of latency that need no launch of their own when a dense layer runs
+// The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
+// workgroups: they are a few microseconds of latency that need no launch of their own when a dense layer runs
 // after the last of the kernels that produce the partials.
 template <typename T, bool KMAJOR>
-__global__ __launch_bounds__(256, 3) void dense_rows_rider_k(const T* __restrict__ X, const T* __restrict__ W,
+__global__ __launch_bounds__(256, 2) void dense_rows_rider_k(const T* __restrict__ X, const T* __restrict__ W,
                                                           const T* __restrict__ bias,
                                                           const float* __restrict__ rowbias, T* __restrict__ Y,
                                                           long long N, int K, int NO, int P, int nkt, int nnt,
                                                           int nblocks, const ReduceJobs jobs) {
     extern __shared__ uint32_t dsm[];
-    if ((int)blockIdx.x >= nblocks) {
-        reduce_jobs_block(jobs, blockIdx.x - nblocks, reinterpret_cast<float(*)[32]>(dsm));
-        return;
+#if defined(PDW_STAMP) && PDW_STAMP == 4
+    if (threadIdx.x == 0) g_stamps[blockIdx.x * 8] = __builtin_amdgcn_s_memrealtime();
+#endif
+    const int nride = (int)gridDim.x - nblocks;
+    if ((int)blockIdx.x < nride) {
+        reduce_jobs_block(jobs, blockIdx.x, reinterpret_cast<float*>(dsm));
+    } else {
+        dense_rows_body<T, KMAJOR, false>(X, W, bias, rowbias, Y, nullptr, N, K, NO, P, nkt, nnt, blockIdx.x - nride,
+                                          nblocks, dsm);
     }
-    dense_rows_body<T, KMAJOR, false>(X, W, bias, rowbias, Y, nullptr, N, K, NO, P, nkt, nnt, nblocks, dsm);
+#if defined(PDW_STAMP) && PDW_STAMP == 4
+    __syncthreads();
+    if (threadIdx.x == 0) g_stamps[blockIdx.x * 8 + 1] = __builtin_amdgcn_s_memrealtime();
+#endif
 }
 
 // dW partials.  A workgroup of 4 wavefronts walks 64-row stages b, b + gridDim.x, ...: the stage's rows
@@ -348,10 +411,9 @@ __global__ __launch_bounds__(256, 3) void dense_rows_rider_k(const T* __restrict
 constexpr int kWgRows = 64;
 
 template <typename T, int MT, int NT>
-__global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A, const T* __restrict__ Bm,
-                                                        float* __restrict__ part, long long N, int M, int NO,
-                                                        int stages_per_block) {
-    extern __shared__ uint32_t dsm[];
+__device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const T* __restrict__ Bm,
+                                                 float* __restrict__ part, long long N, int M, int NO, int nblocks,
+                                                 uint32_t* dsm) {
     const int lda = M + 8, ldb = NO + 8;  // LDS row pitches (elements)
     const int buf_elems = kWgRows * (lda + ldb);
     T* lds = reinterpret_cast<T*>(dsm);
@@ -373,9 +435,8 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A,
     Frag pa[PA], pb[PB];
     const long long nstages = (N + kWgRows - 1) / kWgRows;
     // workgroup b takes stages b, b + gridDim.x, ...: at any moment the chip reads one contiguous window
-    const long long st0 = blockIdx.x, sstep = gridDim.x;
+    const long long st0 = blockIdx.x, sstep = nblocks;
     const long long st1 = nstages;
-    (void)stages_per_block;
 
     auto fetch = [&](long long st) {
         const long long r0 = st * kWgRows;
@@ -472,11 +533,34 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A,
         }
 }
 
+template <typename T, int MT, int NT>
+__global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A, const T* __restrict__ Bm,
+                                                        float* __restrict__ part, long long N, int M, int NO) {
+    extern __shared__ uint32_t dsm[];
+    dense_wgrad_body<T, MT, NT>(A, Bm, part, N, M, NO, gridDim.x, dsm);
+}
+
+// The same with earlier summations in the workgroups behind the first `nblocks` (one workgroup of the product per
+// compute unit leaves room for a second one beside it from the start).
+template <typename T, int MT, int NT>
+__global__ __launch_bounds__(256, 2) void dense_wgrad_rider_k(const T* __restrict__ A, const T* __restrict__ Bm,
+                                                              float* __restrict__ part, long long N, int M, int NO,
+                                                              int nblocks, const ReduceJobs jobs) {
+    extern __shared__ uint32_t dsm[];
+    if ((int)blockIdx.x >= nblocks) {
+        reduce_jobs_block(jobs, blockIdx.x - nblocks, reinterpret_cast<float*>(dsm));
+        return;
+    }
+    dense_wgrad_body<T, MT, NT>(A, Bm, part, N, M, NO, nblocks, dsm);
+}
+
 static bool dense_dims_ok(int K, int NO, int dtype) {
     return dtype != kF32 && K >= 8 && K <= 16 * kKT && K % 8 == 0 && NO >= 8 && NO <= 32 * kNT && NO % 8 == 0;
 }
 
 int dense_rows_supported(int K, int NO, int dtype) { return dense_dims_ok(K, NO, dtype) ? 1 : 0; }
+
+int dense_colsum_rows() { return 32; }
 
 int dense_colsum_supported(int K, int NO, int dtype) {
     return (dense_dims_ok(K, NO, dtype) && (K == 64 || K == 128)) ? 1 : 0;
@@ -493,15 +577,32 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 15) ||
         (reinterpret_cast<uintptr_t>(rowbias) & 15))
         return -1;
+    if (rowbias && P < 32) {
+        // The kernel's bias table holds two images per 32-row tile; smaller images get their rows in a second pass.
+        if (int e = dense_rows_launch(x, w, w_kmajor, bias, nullptr, y, N, K, NO, P, dtype, s, colsum, rider)) return e;
+        const long long full = N / P, rest = N - full * P;
+        if (full > 0)
+            if (int e = add_rowbias_launch(y, rowbias, (int)full, P, NO, dtype, s)) return e;
+        if (rest > 0)
+            return add_rowbias_launch(static_cast<char*>(y) + (size_t)full * P * NO * 2, rowbias + full * NO, 1, (int)rest,
+                                      NO, dtype, s);
+        return 0;
+    }
     const int nkt = cdiv(K, 16), nnt = cdiv(NO, 32);
     const long long ntiles = (N + 31) / 32;
     long long blocks = (ntiles + 3) / 4;  // one row tile per wavefront until the cap
     const int cap = getenv("PDW_DENSE_BLOCKS") ? atoi(getenv("PDW_DENSE_BLOCKS")) : 512;
     if (blocks > cap) blocks = cap;  // persistent workgroups: the weights are staged to LDS once each
     if (blocks < 1) blocks = 1;
-    const size_t lds = ((size_t)NO * (K + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2;
+    const size_t lds = ((size_t)nnt * 32 * ((nkt > 4 ? 128 : 64) + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2 +
+                       ((bias || rowbias) ? (size_t)4 * 2 * nnt * 32 * sizeof(float) : 0);
     if (rider) {
-        const unsigned total = (unsigned)blocks + (unsigned)rider->first_block[rider->njobs];
+        // The summations come first in the grid and take resident slots of their own from the start (the slots
+        // are two per compute unit; waiting for finished row workgroups would put their latency behind the
+        // product's): as long as they are few, the product gives up that many of its persistent workgroups.
+        const int nride = rider->first_block[rider->njobs];
+        if (blocks + nride > cap && nride <= cap / 4) blocks = cap - nride;
+        const unsigned total = (unsigned)blocks + (unsigned)nride;
 #define PDW_RIDE(T, KM)                                                                                           \
     hipLaunchKernelGGL((dense_rows_rider_k<T, KM>), dim3(total), dim3(256), lds, s, (const T*)x, (const T*)w,     \
                        (const T*)bias, rowbias, (T*)y, N, K, NO, P > 0 ? P : 1, nkt, nnt, (int)blocks, *rider)
@@ -560,8 +661,15 @@ static int dense_wgrad_go(const void* a, const void* b, void* dw, void* ws, long
     dense_wgrad_plan(N, &blocks, &spb);
     size_t lds = (size_t)2 * kWgRows * (M + 8 + NO + 8) * 2;
     if (lds < 4 * 16 * 64 * sizeof(float)) lds = 4 * 16 * 64 * sizeof(float);
-    hipLaunchKernelGGL((dense_wgrad_k<T, MT, NT>), dim3(blocks), dim3(256), lds, s, (const T*)a, (const T*)b,
-                       (float*)ws, N, M, NO, spb);
+    // While reductions are being deferred, the ones recorded so far run in this launch; its own joins the list.
+    ReduceJobs jobs;
+    if (reduce_defer_take(&jobs) > 0) {
+        hipLaunchKernelGGL((dense_wgrad_rider_k<T, MT, NT>), dim3(blocks + jobs.first_block[jobs.njobs]), dim3(256), lds,
+                           s, (const T*)a, (const T*)b, (float*)ws, N, M, NO, blocks, jobs);
+    } else {
+        hipLaunchKernelGGL((dense_wgrad_k<T, MT, NT>), dim3(blocks), dim3(256), lds, s, (const T*)a, (const T*)b,
+                           (float*)ws, N, M, NO);
+    }
     if (int e = check_launch("dense_wgrad")) return e;
     return wgrad_reduce_launch<T>((const float*)ws, dw, blocks, M * NO, s);
 }
@@ -586,3 +694,9 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
 }
 
 }  // namespace pdw
+
+#ifdef PDW_STAMP
+extern "C" int pdw_debug_stamps(unsigned long long* host, int n) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pdw::g_stamps), sizeof(unsigned long long) * n);
+}
+#endif

@@ -122,13 +122,13 @@ __global__ __launch_bounds__(256) void dwconv_wgrad_direct(const T* __restrict__
 
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restrict__ part, T* __restrict__ dw,
-                                                          int nparts, int n) {
-    __shared__ float red[8][32];
-    reduce_parts_block<T>(part, dw, nparts, n, blockIdx.x, red);
+                                                          int nparts, int n, int vec) {
+    __shared__ float red[kReduceLds];
+    reduce_parts_any<T>(part, dw, nparts, n, blockIdx.x, vec, red);
 }
 
 __global__ __launch_bounds__(256) void wgrad_reduce_many(const ReduceJobs jobs) {
-    __shared__ float red[8][32];
+    __shared__ float red[kReduceLds];
     reduce_jobs_block(jobs, blockIdx.x, red);
 }
 
@@ -246,14 +246,16 @@ size_t dwconv_wgrad_direct_workspace(int B, int H, int W, int C, int KH, int KW,
 
 template <typename T>
 int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStream_t s) {
+    const int vec = reduce_vec_ok(part, dw, n, (int)sizeof(T)) ? kReduceVec : 1;
     if (t_defer && t_jobs.njobs < kMaxReduceJobs) {
         const int j = t_jobs.njobs++;
         t_jobs.part[j] = part, t_jobs.out[j] = dw, t_jobs.nparts[j] = nparts, t_jobs.n[j] = n;
         t_jobs.dtype[j] = dtype_of<T>();
-        t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv(n, 32);
+        t_jobs.vec[j] = vec;
+        t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv(n, 32 * vec);
         return 0;
     }
-    hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, 32)), dim3(256), 0, s, part, (T*)dw, nparts, n);
+    hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, 32 * vec)), dim3(256), 0, s, part, (T*)dw, nparts, n, vec);
     return check_launch("wgrad_reduce_parts");
 }
 template int wgrad_reduce_launch<float>(const float*, void*, int, int, hipStream_t);

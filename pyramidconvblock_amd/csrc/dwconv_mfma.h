@@ -101,7 +101,7 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
     constexpr bool ADD = MODE == 1;
     using Sh = MfmaShape<K, S, NWV>;
     constexpr int V = 8, NT = NWV * 64, CS = Sh::CS, TH = Sh::TH, TW = Sh::TW;
-    constexpr int KP = Sh::KP, NVB = Sh::NVB, NPH = Sh::NPH, WR = Sh::WR, ROWS_IN = Sh::ROWS_IN, NCOL = Sh::NCOL;
+    constexpr int NVB = Sh::NVB, NPH = Sh::NPH, WR = Sh::WR, ROWS_IN = Sh::ROWS_IN, NCOL = Sh::NCOL;
     constexpr int NQ = (S / 2 + 2 * NVB + 1) / 2;  // 64-bit operand registers per copy of a lane's window
     constexpr int UPP = NT / (CS / V);
     constexpr int NPRE = (ROWS_IN * NCOL + UPP - 1) / UPP;  // passes: a whole window sits in registers

@@ -79,11 +79,12 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
 
 // dense.hip: thin dense layers on the matrix cores (16-bit types, inner dims <= 128); -1 = not covered
 int dense_rows_supported(int K, int NO, int dtype);
-// colsum (optional, fp32 [ceil(N/32)][K], K = 64 or 128): per-32-row sums of x, see dense_colsum_supported
+// colsum (optional, fp32 [ceil(N/R)][K], K = 64 or 128, R = dense_colsum_rows()): sums of x over groups of R rows
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
                       long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum = nullptr,
                       const struct ReduceJobs* rider = nullptr);
 int dense_colsum_supported(int K, int NO, int dtype);
+int dense_colsum_rows();
 int dense_wgrad_supported(int M, int NO, int dtype);
 size_t dense_wgrad_workspace(long long N, int M, int NO);
 int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,

@@ -6,36 +6,91 @@
 namespace pdw {
 
 // Pass 2 of wgrad (shared with the tiled kernels): dw[e] = sum over parts in a fixed order.
-// Block = 32 outputs x 8 part lanes; lane q adds parts q, q+8, ... and the 8 lanes are combined
-// through LDS, so the reads of one part are contiguous and many parts are in flight.
-template <typename T>
+// Block = 32 output lanes x 8 part lanes; an output lane owns V consecutive outputs (V = 4: 16-byte loads, a
+// quarter of the workgroups), part lane q adds parts q, q+8, ... and the 8 lanes are combined through LDS, so the
+// reads of one part are contiguous and many parts are in flight.  V = 4 needs n % 4 == 0 and 16-byte aligned
+// partials (reduce_vec_ok).
+constexpr int kReduceVec = 4;
+constexpr int kReduceLds = 8 * 32 * kReduceVec;  // floats of LDS a workgroup needs
+
+template <typename T, int V>
 __device__ __forceinline__ void reduce_parts_block(const float* __restrict__ part, T* __restrict__ dw, int nparts, int n,
-                                                   int blk, float (*red)[32]) {
+                                                   int blk, float* red) {
+    constexpr int ROW = 32 * V;  // red[8][ROW]
     const int el = threadIdx.x & 31, q = threadIdx.x >> 5;
-    const int e = blk * 32 + el;
-    float s0 = 0.f, s1 = 0.f;
+    const int e = (blk * 32 + el) * V;
+    float s0[V], s1[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) s0[i] = 0.f, s1[i] = 0.f;
+    auto ld = [&](int p, float (&v)[V]) {
+        if constexpr (V == 4) {
+            const float4 t = *reinterpret_cast<const float4*>(part + (long long)p * n + e);
+            v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+        } else {
+            v[0] = part[(long long)p * n + e];
+        }
+    };
     if (e < n) {
         int p = q;
-        for (; p + 56 < nparts; p += 64) {  // eight loads in flight per lane: the pass is pure latency
-            float v[8];
+        for (; p + 120 < nparts; p += 128) {  // sixteen loads in flight per lane: the pass is pure latency
+            float v[16][V];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part[(long long)(p + 8 * u) * n + e];
-            s0 += (v[0] + v[2]) + (v[4] + v[6]);
-            s1 += (v[1] + v[3]) + (v[5] + v[7]);
+            for (int u = 0; u < 16; ++u) ld(p + 8 * u, v[u]);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                s0[i] += ((v[0][i] + v[2][i]) + (v[4][i] + v[6][i])) + ((v[8][i] + v[10][i]) + (v[12][i] + v[14][i]));
+                s1[i] += ((v[1][i] + v[3][i]) + (v[5][i] + v[7][i])) + ((v[9][i] + v[11][i]) + (v[13][i] + v[15][i]));
+            }
+        }
+        for (; p + 56 < nparts; p += 64) {
+            float v[8][V];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ld(p + 8 * u, v[u]);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                s0[i] += (v[0][i] + v[2][i]) + (v[4][i] + v[6][i]);
+                s1[i] += (v[1][i] + v[3][i]) + (v[5][i] + v[7][i]);
+            }
         }
         for (; p + 8 < nparts; p += 16) {
-            s0 += part[(long long)p * n + e];
-            s1 += part[(long long)(p + 8) * n + e];
+            float a[V], b[V];
+            ld(p, a), ld(p + 8, b);
+#pragma unroll
+            for (int i = 0; i < V; ++i) s0[i] += a[i], s1[i] += b[i];
         }
-        if (p < nparts) s0 += part[(long long)p * n + e];
+        if (p < nparts) {
+            float a[V];
+            ld(p, a);
+#pragma unroll
+            for (int i = 0; i < V; ++i) s0[i] += a[i];
+        }
     }
-    red[q][el] = s0 + s1;
+#pragma unroll
+    for (int i = 0; i < V; ++i) red[q * ROW + el * V + i] = s0[i] + s1[i];
     __syncthreads();
     if (q == 0 && e < n) {
-        const float s = ((red[0][el] + red[1][el]) + (red[2][el] + red[3][el])) +
-                        ((red[4][el] + red[5][el]) + (red[6][el] + red[7][el]));
-        dw[e] = from_f32<T>(s);
+        float o[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const int c = el * V + i;
+            o[i] = ((red[c] + red[ROW + c]) + (red[2 * ROW + c] + red[3 * ROW + c])) +
+                   ((red[4 * ROW + c] + red[5 * ROW + c]) + (red[6 * ROW + c] + red[7 * ROW + c]));
+        }
+        store_f32<T, V>(dw + e, o);
     }
+}
+
+// Whether the 4-wide form applies to a summation.
+inline bool reduce_vec_ok(const float* part, const void* dw, int n, int esize) {
+    return n % kReduceVec == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0 &&
+           (reinterpret_cast<uintptr_t>(dw) & (size_t)(kReduceVec * esize - 1)) == 0;
+}
+
+template <typename T>
+__device__ __forceinline__ void reduce_parts_any(const float* part, T* dw, int nparts, int n, int blk, int vec,
+                                                 float* red) {
+    if (vec == kReduceVec) reduce_parts_block<T, kReduceVec>(part, dw, nparts, n, blk, red);
+    else reduce_parts_block<T, 1>(part, dw, nparts, n, blk, red);
 }
 
 // Several such reductions in one launch: the weight gradients of a backward pass are each a few microseconds of
@@ -45,19 +100,22 @@ struct ReduceJobs {
     const float* part[kMaxReduceJobs];
     void* out[kMaxReduceJobs];
     int nparts[kMaxReduceJobs], n[kMaxReduceJobs], dtype[kMaxReduceJobs];
+    int vec[kMaxReduceJobs];  // outputs per lane: kReduceVec or 1
     int first_block[kMaxReduceJobs + 1];
     int njobs;
 };
 
-// Workgroup `wg` (of 256 threads) of the table's grid; red: 8 x 32 floats of LDS.
-__device__ __forceinline__ void reduce_jobs_block(const ReduceJobs& jobs, int wg, float (*red)[32]) {
+// Workgroup `wg` (of 256 threads) of the table's grid; red: kReduceLds floats of LDS.
+__device__ __forceinline__ void reduce_jobs_block(const ReduceJobs& jobs, int wg, float* red) {
     int j = 0;
     while (j + 1 < jobs.njobs && wg >= jobs.first_block[j + 1]) ++j;  // uniform: scalar ALU
     const int blk = wg - jobs.first_block[j];
+    const float* part = jobs.part[j];
+    const int nparts = jobs.nparts[j], n = jobs.n[j], vec = jobs.vec[j];
     switch (jobs.dtype[j]) {
-        case kF32: reduce_parts_block<float>(jobs.part[j], (float*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
-        case kF16: reduce_parts_block<f16_t>(jobs.part[j], (f16_t*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
-        default: reduce_parts_block<bf16_t>(jobs.part[j], (bf16_t*)jobs.out[j], jobs.nparts[j], jobs.n[j], blk, red); break;
+        case kF32: reduce_parts_any<float>(part, (float*)jobs.out[j], nparts, n, blk, vec, red); break;
+        case kF16: reduce_parts_any<f16_t>(part, (f16_t*)jobs.out[j], nparts, n, blk, vec, red); break;
+        default: reduce_parts_any<bf16_t>(part, (bf16_t*)jobs.out[j], nparts, n, blk, vec, red); break;
     }
 }
 

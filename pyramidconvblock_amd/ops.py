@@ -232,9 +232,14 @@ def dense_supported(K, NO, dtype):
     return bool(_lib.lib().pdw_dense_supported(int(K), int(NO), _lib.dtype_code(dtype)))
 
 
+def dense_colsum_rows() -> int:
+    """Rows per chunk sum of dense_forward(..., colsum=True): the row tile of the dense kernel."""
+    return int(_lib.lib().pdw_dense_colsum_rows())
+
+
 def dense_colsum_supported(K, NO, dtype, rows_per_image) -> bool:
     """Whether dense_forward(..., colsum=True) can deliver per-image chunk sums for this shape."""
-    return (dtype in _lib._DTYPES and rows_per_image % 32 == 0
+    return (dtype in _lib._DTYPES and rows_per_image % dense_colsum_rows() == 0
             and bool(_lib.lib().pdw_dense_colsum_supported(int(K), int(NO), _lib.dtype_code(dtype))))
 
 
@@ -244,7 +249,7 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
 
     w is [NO, K] (nn.Linear layout) or, with w_kmajor, [K, NO].  rowbias is fp32 [B, NO], one row per
     `rows_per_image` consecutive rows of x.  With colsum (see dense_colsum_supported) the result is
-    (y, parts): parts fp32 [N / 32, K], the sums of x over each group of 32 consecutive rows.  With
+    (y, parts): parts fp32 [N / R, K], the sums of x over each group of R = dense_colsum_rows() consecutive rows.  With
     flush_reductions, inside _lib.deferred_reductions, the summations recorded so far run in this launch."""
     dev = _lib.require_device(x, w)
     K = x.shape[-1]
@@ -253,7 +258,8 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
     N = x.numel() // K
     y = torch.empty(x.shape[:-1] + (NO,), device=dev, dtype=x.dtype)
     if colsum:
-        parts = torch.empty(((N + 31) // 32, K), device=dev, dtype=torch.float32)
+        R = dense_colsum_rows()
+        parts = torch.empty(((N + R - 1) // R, K), device=dev, dtype=torch.float32)
         if N:
             _launch("pdw_dense_fwd_colsum", dev, x.data_ptr(), w.data_ptr(), 1 if w_kmajor else 0,
                     bias.data_ptr() if bias is not None else None, rowbias.data_ptr() if rowbias is not None else None,

@@ -184,8 +184,8 @@ def test_deferred_reductions_match_immediate_ones():
 
 
 def test_deferred_reductions_ride_on_a_dense_layer():
-    """The recorded summations executed inside a dense layer's launch give the same weight gradients, and the
-    dense result is unchanged."""
+    """The recorded summations executed inside later launches (the conv's inside the dense weight gradient's, that
+    one's inside a dense layer's) give the same weight gradients, and the dense result is unchanged."""
     from pyramidconvblock_amd import _lib, ops
     from pyramidconvblock_amd.dwconv import dwconv_wgrad
 

@@ -185,10 +185,11 @@ def test_spatial_sum_and_rowbias(dtype, shape):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("K,NO", [(128, 64), (64, 128), (96, 48), (48, 96), (64, 32), (32, 64), (8, 8), (120, 104), (16, 24)])
-@pytest.mark.parametrize("N,P", [(3 * 35, 35), (1, 1), (4 * 3136, 3136)])
+@pytest.mark.parametrize("N,P", [(3 * 35, 35), (1, 1), (4 * 3136, 3136), (100, 33), (50, 7), (96, 32)])
 def test_dense_layers(dtype, K, NO, N, P):
     """Matrix-core dense kernels against float64: forward in both weight layouts with bias and per-image
-    row bias, and the weight gradient."""
+    row bias (images that end inside a 32-row tile, images shorter than a tile, a last image cut short), and
+    the weight gradient."""
     from pyramidconvblock_amd import ops
 
     if not (ops.dense_supported(K, NO, dtype) and ops.dense_supported(NO, K, dtype)):
@@ -197,8 +198,8 @@ def test_dense_layers(dtype, K, NO, N, P):
     x = randn(gen, N, K).to(dtype)
     w = (randn(gen, NO, K) / K ** 0.5).to(dtype)
     b = randn(gen, NO).to(dtype)
-    rb = randn(gen, N // P, NO)
-    ref = x.double() @ w.double().t() + b.double() + rb.double().repeat_interleave(P, 0)
+    rb = randn(gen, (N + P - 1) // P, NO)
+    ref = x.double() @ w.double().t() + b.double() + rb.double().repeat_interleave(P, 0)[:N]
     y = ops.dense_forward(x.cuda(), w.cuda(), bias=b.cuda(), rowbias=rb.cuda(), rows_per_image=P)
     assert_close(y, ref.numpy(), dtype, "dense fwd")
     g = randn(gen, N, NO).to(dtype)
@@ -247,7 +248,8 @@ def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
     assert ops.dense_colsum_supported(K, NO, dtype, P)
     y, parts = ops.dense_forward(x, w, w_kmajor=kmajor, colsum=True)
     assert torch.equal(y, ops.dense_forward(x, w, w_kmajor=kmajor))
-    ref = x.double().view(B * P // 32, 32, K).sum(1)
+    R = ops.dense_colsum_rows()
+    ref = x.double().view(B * P // R, R, K).sum(1)
     assert (parts.double() - ref).abs().max().item() <= 1e-5 * max(1.0, ref.abs().max().item())
     wp = (randn(gen, K, K) / 11).to(dtype).cuda()
     bp = randn(gen, K).to(dtype).cuda()
