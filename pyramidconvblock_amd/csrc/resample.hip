@@ -304,24 +304,30 @@ __global__ __launch_bounds__(256) void gate_bwd_k(const T* __restrict__ x, const
 
 // U items per thread, every load of a thread requested before the first use (a streaming kernel lives on the number
 // of loads in flight); items past the end read the last item's data and store nothing.
-constexpr int kGateItems = 4;  // full-resolution items per thread of the paired kernels
+constexpr int kGateItems = 8;  // full-resolution items per thread of the paired kernels
+constexpr int kGateAhead = 2;  // items whose loads are in flight when an item is stored
 
 template <typename T, int VEC, int U>
 __device__ __forceinline__ void gate_fwd_items(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
                                                long long first, long long step, long long total) {
+    // A rolling pipeline: the loads of item u + kGateAhead are issued before item u is stored, so that a
+    // thread's reads and writes alternate.  With every thread of the grid resident at once, "load everything,
+    // then store everything" puts the whole kernel's reads before the whole kernel's writes.
     const int G = I / 2, GV = G / VEC;
     ChanVec<T, VEC> a[U], b[U];
     long long m[U];
     int c[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
+    auto load = [&](int u) {
         const long long idx = min(first + u * step, total - 1);
         c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
         a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
         b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
-    }
+    };
+#pragma unroll
+    for (int u = 0; u < kGateAhead && u < U; ++u) load(u);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+        if (u + kGateAhead < U) load(u + kGateAhead);
         float o[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) o[v] = to_f32(a[u].v[v]) * to_f32(b[u].v[v]) * s;
@@ -337,16 +343,18 @@ __device__ __forceinline__ void gate_bwd_items(const T* __restrict__ x, const T*
     ChanVec<T, VEC> a[U], b[U], g[U];
     long long m[U];
     int c[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
+    auto load = [&](int u) {
         const long long idx = min(first + u * step, total - 1);
         c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
         a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
         b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
         g[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(gy + m[u] * ldg + c[u]);
-    }
+    };
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+    for (int u = 0; u < kGateAhead && u < U; ++u) load(u);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {  // loads run kGateAhead items ahead of the stores, as in gate_fwd_items
+        if (u + kGateAhead < U) load(u + kGateAhead);
         float ga[VEC], gb[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -1035,6 +1043,9 @@ __global__ __launch_bounds__(256) void block_mid_fwd_k(const T* __restrict__ xf,
     }
 }
 
+#if defined(PDW_STAMP) && PDW_STAMP == 5
+__device__ unsigned long long g_stamps5[8192 * 2];
+#endif
 template <typename T>
 __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy, const T* __restrict__ xf,
                                                        const T* __restrict__ xh, T* __restrict__ gxf,
@@ -1044,19 +1055,27 @@ __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy,
     extern __shared__ float sm[];
     constexpr int VEC = 8;
     unsigned bid = blockIdx.x;
+#if defined(PDW_STAMP) && PDW_STAMP == 5
+    if (threadIdx.x == 0) g_stamps5[blockIdx.x * 2] = __builtin_amdgcn_s_memrealtime();
+#endif
     if (bid < (unsigned)(job.B + job.D)) {
         pool_branch_bwd_v8_block<T>(job.part, job.nchunks, job.B, job.D, job.inv_p, (const T*)job.wp, (const T*)job.m,
                                     job.gs, job.dmean, (T*)job.gbias, (T*)job.gbias2, (T*)job.gwp, (int)bid, sm);
-        return;
-    }
-    bid -= job.B + job.D;
-    if (bid < nblk_full) {
-        const long long first = (long long)bid * (kGateItems * 256) + threadIdx.x;
-        if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
     } else {
-        const long long idx = (long long)(bid - nblk_full) * blockDim.x + threadIdx.x;
-        if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
+        bid -= job.B + job.D;
+        if (bid < nblk_full) {
+            const long long first = (long long)bid * (kGateItems * 256) + threadIdx.x;
+            if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
+        } else {
+            const long long idx = (long long)(bid - nblk_full) * blockDim.x + threadIdx.x;
+            if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
+        }
     }
+#if defined(PDW_STAMP) && PDW_STAMP == 5
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) g_stamps5[blockIdx.x * 2 + 1] = __builtin_amdgcn_s_memrealtime();
+#endif
 }
 
 // y[b,p,c] += v[b,c]  (v in fp32, one rounding)
@@ -1479,3 +1498,9 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
 }
 
 }  // namespace pdw
+
+#if defined(PDW_STAMP) && PDW_STAMP == 5
+extern "C" int pdw_debug_stamps5(unsigned long long* host, int n) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pdw::g_stamps5), sizeof(unsigned long long) * n);
+}
+#endif

@@ -24,8 +24,7 @@ def _pixel_stride(t: torch.Tensor) -> int:
 
 
 def _launch(name, dev, *args):
-    with _lib.on_device(dev):
-        _lib.check(getattr(_lib.lib(), name)(*args, _lib.stream_ptr(dev)), name)
+    _lib.call(name, dev, *args)
 
 
 def avgpool_forward(x, out_hw):
