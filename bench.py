@@ -287,15 +287,12 @@ def main():
     m = make_block(D, k, dtype)
     fwd, fwd_bwd = stepper(m)
     t_eager = time_gpu(fwd_bwd, args.steps, args.warmup)
-    # The step the metric is quoted on: the same forward+backward captured once (HIP graph plus the list of
-    # C-ABI calls it was built from) and replayed: identical kernels and results, without the per-launch
-    # overhead of Python and autograd.  The step holds library kernels only, so replay() issues the recorded
-    # calls on the stream (graph_ms_per_step is the same step launched as a graph).
+    # The step the metric is quoted on: the same forward+backward captured once into a HIP graph
+    # and replayed (identical kernels and results; removes the per-launch host overhead).
     from pyramidconvblock_amd.graphs import GraphedForward, GraphedStep
 
     graphed = GraphedStep(m, x, g)
     t_step = time_gpu(graphed.replay, args.steps, args.warmup)
-    t_graph = time_gpu(graphed.graph.replay, args.steps, args.warmup)
     for p in m.parameters():
         p.grad = None
     bytes_f, bytes_fb = block_alg_bytes(B, H, W, D, k, 2)
@@ -317,9 +314,7 @@ def main():
         "config": {"workload": "ConvBlock(dim=128,kernel_size=13) fwd+bwd, bf16, x[32,56,56,128] N(0,1) seed 0, "
                                "default-init weights, grad_out N(0,1)"},
         "eager_ms_per_step": t_eager * 1e3,
-        "graph_ms_per_step": t_graph * 1e3,
-        "launch": ("recorded C-ABI calls of one captured step, issued on the stream" if graphed.replays_calls
-                   else "one HIP graph replay per step") + " (eager Python launch time in eager_ms_per_step)",
+        "launch": "one HIP graph replay per step (eager launch time in eager_ms_per_step)",
         "block_hbm_frac_fwd_bwd": bytes_fb / (t_step * HBM_PEAK),
         "block_alg_bytes_fwd_bwd": bytes_fb,
         "block_dwconv_valu_frac_fwd_bwd": flops_fb / (t_step * VALU_PEAK),

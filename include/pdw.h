@@ -32,11 +32,6 @@ enum { PDW_F32 = 0, PDW_F16 = 1, PDW_BF16 = 2 };
 
 /* ABI version of the library (bumped when a signature changes). */
 int pdw_version(void);
-
-/* Kernels launched through this library so far, by all threads of the process.  A caller that records a
- * sequence of calls (stream capture, or a list of calls to issue again) compares the difference over the sequence
- * with the number of kernels it saw, to know that the sequence holds nothing but this library's launches. */
-unsigned long long pdw_launch_count(void);
 /* Text of the last error raised on the calling thread ("" if none). */
 const char *pdw_last_error(void);
 

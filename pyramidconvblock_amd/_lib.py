@@ -23,7 +23,6 @@ _lib = None
 _CONV = [c_int] * 12  # B,H,W,C,KH,KW,SH,SW,PH,PW,DH,DW
 _SIGS = {
     "pdw_version": (c_int, []),
-    "pdw_launch_count": (ctypes.c_ulonglong, []),
     "pdw_last_error": (c_char_p, []),
     "pdw_conv_out_size": (c_int, [c_int] * 5),
     "pdw_dwconv_fwd": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
@@ -134,56 +133,6 @@ class on_device:
         return False
 
 
-class _Recorder:  # process-wide: a backward pass makes its calls on the autograd engine's thread
-    calls = None
-    lock = threading.Lock()
-
-
-_rec = _Recorder
-
-
-def call(name: str, dev: torch.device, *args) -> None:
-    """One stream-ordered entry point of the library: fn(*args, stream of `dev`), an error status raised as
-    RuntimeError.  While a `recorded_calls` block is open on this thread the call is also noted down."""
-    fn = getattr(lib(), name)
-    with on_device(dev):
-        check(fn(*args, stream_ptr(dev)), name)
-    calls = _rec.calls
-    if calls is not None:
-        with _rec.lock:
-            calls.append((fn, args, True, name))
-
-
-class recorded_calls:
-    """Collects the library calls made inside the block, by any thread, as (function, arguments, takes_stream,
-    name), in order, for `replay_calls`.  The arguments are the raw pointers and extents of the calls: they stay
-    meaningful only while the tensors behind them are alive and in place (as in a captured graph's memory pool).
-    Nothing else may use the library while the block is open."""
-
-    def __enter__(self):
-        with _rec.lock:
-            if _rec.calls is not None:
-                raise RuntimeError("recorded_calls: already recording")
-            _rec.calls = self.calls = []
-        self.first_launch = lib().pdw_launch_count()
-        return self
-
-    def __exit__(self, *exc):
-        _rec.calls = None
-        self.kernels = lib().pdw_launch_count() - self.first_launch
-        return False
-
-
-def replay_calls(calls, dev: torch.device) -> None:
-    """Issues recorded calls again, on `dev`'s current stream."""
-    with on_device(dev):
-        st = stream_ptr(dev)
-        for fn, args, takes_stream, name in calls:
-            status = fn(*args, st) if takes_stream else fn(*args)
-            if status:
-                check(status, name)
-
-
 _defer = threading.local()
 
 
@@ -196,16 +145,13 @@ class deferred_reductions:
 
     def __enter__(self):
         check(lib().pdw_reduce_defer_begin(), "pdw_reduce_defer_begin")
-        calls = _rec.calls
-        if calls is not None:
-            with _rec.lock:
-                calls.append((lib().pdw_reduce_defer_begin, (), False, "pdw_reduce_defer_begin"))
         _defer.keep = []
         return self
 
     def __exit__(self, *exc):
         try:
-            call("pdw_reduce_defer_flush", self.dev)
+            with on_device(self.dev):
+                check(lib().pdw_reduce_defer_flush(stream_ptr(self.dev)), "pdw_reduce_defer_flush")
         finally:
             _defer.keep = None
         return False

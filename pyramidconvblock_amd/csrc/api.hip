@@ -1,7 +1,6 @@
 // C ABI of libpdw.so (declared in include/pdw.h): argument validation and dispatch to
 // the kernel launchers.  No allocation, no synchronisation, no global mutable state
 // besides the per-thread error text.
-#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -21,15 +20,12 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
-static std::atomic<unsigned long long> g_launches{0};
-
 int check_launch(const char* what) {
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("%s: launch failed: %s", what, hipGetErrorString(e));
         return 2;
     }
-    g_launches.fetch_add(1, std::memory_order_relaxed);
     return 0;
 }
 
@@ -64,8 +60,6 @@ using namespace pdw;
 extern "C" {
 
 int pdw_version(void) { return 4; }
-
-unsigned long long pdw_launch_count(void) { return g_launches.load(std::memory_order_relaxed); }
 
 const char* pdw_last_error(void) { return g_err; }
 

@@ -160,6 +160,18 @@ int reduce_defer_flush(hipStream_t s) {
     return r;
 }
 
+int reduce_defer_room() { return t_defer ? kMaxReduceJobs - t_jobs.njobs : 0; }
+
+// Records out[o * D + d] = sum_b g[b * D + o] * m[b * D + d] (see outer_sum_block); only while deferring.
+int reduce_defer_outer(const float* g, const void* m, void* out, int B, int D, int dtype) {
+    if (reduce_defer_room() < 1 || dtype == kF32 || D % 4 != 0) return -1;
+    const int j = t_jobs.njobs++;
+    t_jobs.part[j] = g, t_jobs.aux[j] = m, t_jobs.out[j] = out, t_jobs.nparts[j] = B, t_jobs.n[j] = D * D;
+    t_jobs.dtype[j] = dtype, t_jobs.vec[j] = 0, t_jobs.dim[j] = D;
+    t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv((long long)D * D, kOuterBlock);
+    return 0;
+}
+
 // Hands the recorded jobs to a caller that runs them inside another kernel's grid; the later flush then finds
 // nothing left to do.  Returns the number of jobs.
 int reduce_defer_take(ReduceJobs* out) {

@@ -254,6 +254,7 @@ static WgradMfmaPlan plan_wgrad_mfma(int B, int H, int W, int C, int PH, int PW)
     long long want_h = ((long long)B * g.slices * g.tiles_w + 255) / 256;  // images*slices per CU column
     int tiles_h = (int)(256 / ((long long)B * g.slices * g.tiles_w > 0 ? (long long)B * g.slices * g.tiles_w : 1));
     (void)want_h;
+    if (getenv("PDW_WG_TILEMUL")) tiles_h *= atoi(getenv("PDW_WG_TILEMUL"));
     if (tiles_h < 1) tiles_h = 1;
     if (tiles_h > g.OH) tiles_h = g.OH;
     int th = cdiv(g.OH, tiles_h);

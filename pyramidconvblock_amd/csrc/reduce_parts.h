@@ -93,14 +93,52 @@ __device__ __forceinline__ void reduce_parts_any(const float* part, T* dw, int n
     else reduce_parts_block<T, 1>(part, dw, nparts, n, blk, red);
 }
 
+// out[o * D + d] = sum over b < B of g[b * D + o] * m[b * D + d]: the weight gradient of a small dense layer
+// applied to one row per image (g: fp32 output gradients, m: its inputs), 1024 outputs per workgroup of 256
+// threads, D % 4 == 0.  The same kind of deferred work as the sums of partials: nothing needs it before the
+// backward pass is over.
+constexpr int kOuterBlock = 1024;
+
+template <typename T>
+__device__ __forceinline__ void outer_sum_block(const float* __restrict__ g, const T* __restrict__ m,
+                                                T* __restrict__ out, int B, int D, int blk, int tid) {
+    const int e = (blk * 256 + tid) * 4;
+    if (e >= D * D) return;
+    const int o = e / D, d = e - o * D;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    int b = 0;
+    for (; b + 8 <= B; b += 8) {  // sixteen loads in flight
+        float gv[8], mv[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            gv[u] = g[(long long)(b + u) * D + o];
+            load_f32<T, 4>(m + (long long)(b + u) * D + d, mv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = fmaf(gv[u], mv[u][i], acc[i]);
+    }
+    for (; b < B; ++b) {
+        float mv[4];
+        const float gv = g[(long long)b * D + o];
+        load_f32<T, 4>(m + (long long)b * D + d, mv);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(gv, mv[i], acc[i]);
+    }
+    store_f32<T, 4>(out + e, acc);
+}
+
 // Several such reductions in one launch: the weight gradients of a backward pass are each a few microseconds of
 // latency, and nothing reads them before the pass is over.
 constexpr int kMaxReduceJobs = 8;
 struct ReduceJobs {
     const float* part[kMaxReduceJobs];
     void* out[kMaxReduceJobs];
+    const void* aux[kMaxReduceJobs];  // outer products: the second factor (element type of `out`)
     int nparts[kMaxReduceJobs], n[kMaxReduceJobs], dtype[kMaxReduceJobs];
-    int vec[kMaxReduceJobs];  // outputs per lane: kReduceVec or 1
+    int vec[kMaxReduceJobs];  // outputs per lane: kReduceVec or 1; 0 = outer product (n = D * D, nparts = B)
+    int dim[kMaxReduceJobs];  // outer products: D
     int first_block[kMaxReduceJobs + 1];
     int njobs;
 };
@@ -112,6 +150,13 @@ __device__ __forceinline__ void reduce_jobs_block(const ReduceJobs& jobs, int wg
     const int blk = wg - jobs.first_block[j];
     const float* part = jobs.part[j];
     const int nparts = jobs.nparts[j], n = jobs.n[j], vec = jobs.vec[j];
+    if (vec == 0) {  // outer product; fp32 outputs are not produced this way
+        if (jobs.dtype[j] == kF16)
+            outer_sum_block<f16_t>(part, (const f16_t*)jobs.aux[j], (f16_t*)jobs.out[j], nparts, jobs.dim[j], blk, threadIdx.x);
+        else
+            outer_sum_block<bf16_t>(part, (const bf16_t*)jobs.aux[j], (bf16_t*)jobs.out[j], nparts, jobs.dim[j], blk, threadIdx.x);
+        return;
+    }
     switch (jobs.dtype[j]) {
         case kF32: reduce_parts_any<float>(part, (float*)jobs.out[j], nparts, n, blk, vec, red); break;
         case kF16: reduce_parts_any<f16_t>(part, (f16_t*)jobs.out[j], nparts, n, blk, vec, red); break;

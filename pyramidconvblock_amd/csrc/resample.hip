@@ -1051,18 +1051,20 @@ __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy,
                                                        const T* __restrict__ xh, T* __restrict__ gxf,
                                                        T* __restrict__ gxh, int h, int w, int I, int ldg, float s,
                                                        unsigned nblk_full, long long total_full,
-                                                       long long total_half, const PoolBwdJob job) {
+                                                       long long total_half, const PoolBwdJob job, unsigned npool) {
+    // npool = B + D, or B when the per-feature part (the gradients of the pooled layer's weight and bias) is
+    // left to deferred work
     extern __shared__ float sm[];
     constexpr int VEC = 8;
     unsigned bid = blockIdx.x;
 #if defined(PDW_STAMP) && PDW_STAMP == 5
     if (threadIdx.x == 0) g_stamps5[blockIdx.x * 2] = __builtin_amdgcn_s_memrealtime();
 #endif
-    if (bid < (unsigned)(job.B + job.D)) {
+    if (bid < npool) {
         pool_branch_bwd_v8_block<T>(job.part, job.nchunks, job.B, job.D, job.inv_p, (const T*)job.wp, (const T*)job.m,
                                     job.gs, job.dmean, (T*)job.gbias, (T*)job.gbias2, (T*)job.gwp, (int)bid, sm);
     } else {
-        bid -= job.B + job.D;
+        bid -= npool;
         if (bid < nblk_full) {
             const long long first = (long long)bid * (kGateItems * 256) + threadIdx.x;
             if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
@@ -1313,15 +1315,28 @@ int block_mid_bwd_launch(const void* gy, const void* xf, const void* xh, void* g
     const PoolBwdJob job{parts, nparts, B, D, 1.f / (float)P, wp, m, gs, dmean, gbias, gbias2, gwp};
     const size_t la = (size_t)17 * D * sizeof(float), lb = (size_t)(B + 16 * D) * sizeof(float);
     const size_t lds = la > lb ? la : lb;
+    // While reductions are deferred (and the table has room) the weight and bias gradients of the pooled layer
+    // join them: they are sums over the images of what the per-image workgroups leave in `gs`, nothing reads
+    // them before the backward pass is over, and their D workgroups are the slowest of this launch.
+    const bool later = reduce_defer_room() >= (gbias2 ? 3 : 2) && D % 4 == 0;
+    const unsigned npool = later ? B : B + D;
     if (dtype == kF16)
-        hipLaunchKernelGGL((block_mid_bwd_k<f16_t>), dim3(bf + bh + B + D), dim3(256), lds, s, (const f16_t*)gy,
+        hipLaunchKernelGGL((block_mid_bwd_k<f16_t>), dim3(bf + bh + npool), dim3(256), lds, s, (const f16_t*)gy,
                            (const f16_t*)xf, (const f16_t*)xh, (f16_t*)gxf, (f16_t*)gxh, h, w, I, ldg, sc, bf, tf, th,
-                           job);
+                           job, npool);
     else
-        hipLaunchKernelGGL((block_mid_bwd_k<bf16_t>), dim3(bf + bh + B + D), dim3(256), lds, s, (const bf16_t*)gy,
+        hipLaunchKernelGGL((block_mid_bwd_k<bf16_t>), dim3(bf + bh + npool), dim3(256), lds, s, (const bf16_t*)gy,
                            (const bf16_t*)xf, (const bf16_t*)xh, (bf16_t*)gxf, (bf16_t*)gxh, h, w, I, ldg, sc, bf, tf,
-                           th, job);
-    return check_launch("block_mid_bwd");
+                           th, job, npool);
+    if (int e = check_launch("block_mid_bwd")) return e;
+    if (later) {
+        if (reduce_defer_outer(gs, m, gwp, B, D, dtype) != 0) return set_error("block_mid_bwd: deferred job refused"), 1;
+        int e = dtype == kF16 ? wgrad_reduce_launch<f16_t>(gs, gbias, B, D, s) : wgrad_reduce_launch<bf16_t>(gs, gbias, B, D, s);
+        if (!e && gbias2)
+            e = dtype == kF16 ? wgrad_reduce_launch<f16_t>(gs, gbias2, B, D, s) : wgrad_reduce_launch<bf16_t>(gs, gbias2, B, D, s);
+        return e;
+    }
+    return 0;
 }
 
 int gate_fwd_launch(const void* x, void* y, long long M, int I, int ldy, int dtype, hipStream_t s) {

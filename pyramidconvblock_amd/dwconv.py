@@ -38,14 +38,17 @@ def dwconv_forward(x, weight, stride, padding, dilation, pool_to=None):
         h, w = int(pool_to[0]), int(pool_to[1])
         xp = torch.empty((x.shape[0], h, w, x.shape[3]), device=dev, dtype=x.dtype)
         if y.numel() and xp.numel():
-            _lib.call("pdw_dwconv_fwd_pool", dev, x.data_ptr(), weight.data_ptr(), y.data_ptr(), xp.data_ptr(), *args,
-                      h, w, _lib.dtype_code(x.dtype))
+            with _lib.on_device(dev):
+                _lib.check(L.pdw_dwconv_fwd_pool(x.data_ptr(), weight.data_ptr(), y.data_ptr(), xp.data_ptr(), *args,
+                                                 h, w, _lib.dtype_code(x.dtype), _lib.stream_ptr(dev)),
+                           "pdw_dwconv_fwd_pool")
             return y, xp
         from . import ops
         return dwconv_forward(x, weight, stride, padding, dilation), ops.avgpool_forward(x, (h, w))
     if y.numel():
-        _lib.call("pdw_dwconv_fwd", dev, x.data_ptr(), weight.data_ptr(), y.data_ptr(), *args,
-                  _lib.dtype_code(x.dtype))
+        with _lib.on_device(dev):
+            _lib.check(L.pdw_dwconv_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), *args,
+                                        _lib.dtype_code(x.dtype), _lib.stream_ptr(dev)), "pdw_dwconv_fwd")
     return y
 
 
@@ -53,6 +56,7 @@ def dwconv_dgrad(gy, weight, in_shape, stride, padding, dilation, pooled_grad=No
     """dx[in_shape]; with pooled_grad [B,h,w,C] the gradient of an adaptive average pool of the same
     tensor to (h, w) is added to it."""
     dev = _lib.require_device(gy, weight)
+    L = _lib.lib()
     dx = torch.empty(in_shape, device=dev, dtype=gy.dtype)
     if dx.numel():
         if gy.numel() == 0:
@@ -62,13 +66,15 @@ def dwconv_dgrad(gy, weight, in_shape, stride, padding, dilation, pooled_grad=No
                 ops.avgpool_backward(pooled_grad, (in_shape[1], in_shape[2]), out=dx, accumulate=True)
             return dx
         args = _conv_args(in_shape, weight.shape, stride, padding, dilation)
-        if pooled_grad is None:
-            _lib.call("pdw_dwconv_dgrad", dev, gy.data_ptr(), weight.data_ptr(), dx.data_ptr(), *args,
-                      _lib.dtype_code(gy.dtype))
-        else:
-            gp = pooled_grad.contiguous()
-            _lib.call("pdw_dwconv_dgrad_addpool", dev, gy.data_ptr(), weight.data_ptr(), gp.data_ptr(), dx.data_ptr(),
-                      *args, gp.shape[1], gp.shape[2], _lib.dtype_code(gy.dtype))
+        with _lib.on_device(dev):
+            if pooled_grad is None:
+                _lib.check(L.pdw_dwconv_dgrad(gy.data_ptr(), weight.data_ptr(), dx.data_ptr(), *args,
+                                              _lib.dtype_code(gy.dtype), _lib.stream_ptr(dev)), "pdw_dwconv_dgrad")
+            else:
+                gp = pooled_grad.contiguous()
+                _lib.check(L.pdw_dwconv_dgrad_addpool(gy.data_ptr(), weight.data_ptr(), gp.data_ptr(), dx.data_ptr(),
+                                                      *args, gp.shape[1], gp.shape[2], _lib.dtype_code(gy.dtype),
+                                                      _lib.stream_ptr(dev)), "pdw_dwconv_dgrad_addpool")
     return dx
 
 
@@ -82,8 +88,9 @@ def dwconv_wgrad(x, gy, w_shape, stride, padding, dilation):
     code = _lib.dtype_code(x.dtype)
     nbytes = L.pdw_dwconv_wgrad_workspace_bytes(*args, code)
     ws = torch.empty(max(nbytes, 4) // 4 + 1, device=dev, dtype=torch.float32)
-    _lib.call("pdw_dwconv_wgrad", dev, x.data_ptr(), gy.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel() * 4,
-              *args, code)
+    with _lib.on_device(dev):
+        _lib.check(L.pdw_dwconv_wgrad(x.data_ptr(), gy.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel() * 4,
+                                      *args, code, _lib.stream_ptr(dev)), "pdw_dwconv_wgrad")
     _lib.keep_until_flush(ws)
     return dw
 

@@ -24,7 +24,8 @@ def _pixel_stride(t: torch.Tensor) -> int:
 
 
 def _launch(name, dev, *args):
-    _lib.call(name, dev, *args)
+    with _lib.on_device(dev):
+        _lib.check(getattr(_lib.lib(), name)(*args, _lib.stream_ptr(dev)), name)
 
 
 def avgpool_forward(x, out_hw):
@@ -193,6 +194,7 @@ def block_mid_backward(xf, xh, gy, parts, P, m, w_pool):
             h, w, I, _pixel_stride(gy), parts.data_ptr(), parts.shape[0] // B, m.data_ptr(), w_pool.data_ptr(),
             gbias[0].data_ptr(), gbias[1].data_ptr(), gwp.data_ptr(), dmean.data_ptr(), ws.data_ptr(), ws.numel() * 4,
             int(P), D, _lib.dtype_code(xf.dtype))
+    _lib.keep_until_flush(ws)  # inside deferred_reductions gbias and gw_pool are summed from it at the flush
     return gxf, gxh, gbias, gwp, dmean
 
 
