@@ -75,9 +75,12 @@ int pdw_dwconv_dgrad_addpool(const void *gy, const void *w, const void *gp, void
  * fp32 partial results.  Between pdw_reduce_defer_begin() and pdw_reduce_defer_flush(stream), on the calling host
  * thread, that last step is only recorded (up to 8 of them, further ones run at once as usual), and the flush
  * runs all recorded ones in a single launch on `stream`: the outputs are not valid, and the workspaces must not
- * be reused or freed, until then.  No counterpart in the reference (its backward launches every kernel
- * separately, dwconv_triton.py:358-385); the ConvBlock backward (conv_block.py:36-49 under autograd) uses it
- * for its four weight gradients. */
+ * be reused or freed, until then.  Two entry points take recorded work along in spare workgroups of their own
+ * launch, after which the list is empty again: pdw_dense_wgrad (what was recorded before it; its own summation is
+ * recorded afterwards) and pdw_dense_fwd_flush below.  pdw_block_mid_bwd records the gradients of the pooled
+ * layer's weight and bias (gw_pool, gbias, gbias2) in the same way instead of computing them in its own launch.
+ * No counterpart in the reference (its backward launches every kernel separately, dwconv_triton.py:358-385);
+ * the ConvBlock backward (conv_block.py:36-49 under autograd) uses it for its weight gradients. */
 int pdw_reduce_defer_begin(void);
 int pdw_reduce_defer_flush(void *stream);
 /* pdw_dense_fwd that also runs the reductions recorded so far (see above) in spare workgroups of its own launch;
@@ -193,7 +196,9 @@ int pdw_pool_branch_bwd_parts(const float *parts, int nparts, const void *m, con
  * pdw_pool_branch_fwd_parts, and pdw_gate_pair_bwd together with pdw_pool_branch_bwd_parts (same arguments, same
  * results; the mean branch is a handful of latency-bound workgroups that ride in the gate kernel's grid).  When
  * the combination is not covered (fp32, D > 128, unaligned slices) the two kernels are launched one after the
- * other.  P = positions per image of the tensor whose chunk sums `parts` holds (conv_block.py:40-49). */
+ * other.  P = positions per image of the tensor whose chunk sums `parts` holds (conv_block.py:40-49).  Between
+ * pdw_reduce_defer_begin and the flush, pdw_block_mid_bwd leaves gw_pool, gbias and gbias2 to the deferred work
+ * (they are sums over the images of values it writes into `workspace`, which must stay in place until then). */
 int pdw_block_mid_fwd(const void *xf, const void *xh, void *y, int B, int H, int W, int h, int w, int I, int ldy,
                       const float *parts, int nparts, const void *w_pool, const void *b_pool, const void *b_out,
                       void *m, float *rowbias, int P, int D, int dtype, void *stream);

@@ -175,11 +175,9 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     const bool hasb = bias != nullptr || rowbias != nullptr;
     const int bcol = 4 * l32;                           // this lane's 4 columns of that table (row `half`)
     const int nimg = rowbias ? (int)((N + P - 1) / P) : 1;
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias && bcol < NO) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) bv[i] = to_f32(bias[bcol + i]);
-    }
+    // this lane's four bias values: an unconditional 8-byte load (of the weights when there is no bias), converted
+    // where the table is written, so that nothing waits for it before the weights and the first tile are requested
+    const ChanVec<T, 4> braw = *reinterpret_cast<const ChanVec<T, 4>*>(bias && bcol < NO ? bias + bcol : W);
     if (K != KP || NO != NOP) {  // uniform
         for (int i = tid; i < NOP * ldw / 8; i += 256) reinterpret_cast<uint4*>(wl)[i] = make_uint4(0u, 0u, 0u, 0u);
         __syncthreads();
@@ -255,9 +253,12 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
 #pragma unroll
         for (int i = 0; i < LP; ++i)
             if (oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
-        if (hasb && bcol < NOP)
+        if (hasb && bcol < NOP) {
+            const bool hb = bias != nullptr && bcol < NO;
             *reinterpret_cast<float4*>(bl + half * NOP + bcol) =
-                make_float4(bv[0] + brow.x, bv[1] + brow.y, bv[2] + brow.z, bv[3] + brow.w);
+                make_float4((hb ? to_f32(braw.v[0]) : 0.f) + brow.x, (hb ? to_f32(braw.v[1]) : 0.f) + brow.y,
+                            (hb ? to_f32(braw.v[2]) : 0.f) + brow.z, (hb ? to_f32(braw.v[3]) : 0.f) + brow.w);
+        }
         float cs[8];
         if constexpr (COLSUM) {
 #pragma unroll
@@ -575,7 +576,8 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     if (N == 0) return 0;
     if (N > 0x7fffffffLL) return -1;
     if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 15) ||
-        (reinterpret_cast<uintptr_t>(rowbias) & 15))
+        (reinterpret_cast<uintptr_t>(rowbias) & 15) || (reinterpret_cast<uintptr_t>(bias) & 7) ||
+        (reinterpret_cast<uintptr_t>(w) & 15))
         return -1;
     if (rowbias && P < 32) {
         // The kernel's bias table holds two images per 32-row tile; smaller images get their rows in a second pass.

@@ -831,6 +831,17 @@ __device__ __forceinline__ void pool_branch_fwd_v8_body(const float* __restrict_
             const bool ok = o < D && v * 8 < D;
             wv[pass][i] = *reinterpret_cast<const ChanVec<T, 8>*>(wp + (ok ? (long long)o * D + v * 8 : 0));
         }
+    // the biases of this thread's outputs, requested here as well: read where they are added, after the last
+    // barrier, they would be eight dependent trips to memory at the end of the workgroup
+    // (unconditional loads from a readable address, converted where they are used: no branch, no early wait)
+    const T* bpp = bp ? bp : wp;
+    const T* bop = bo ? bo : wp;
+    T braw[4][2];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int oc = min(ol + 32 * pass, D - 1);
+        braw[pass][0] = bpp[oc], braw[pass][1] = bop[oc];
+    }
     colsum_coop(part + (long long)b * nchunks * D, nchunks, D, sm, sm + D);
     if (tid < D) {
         const T mv = from_f32<T>(sm[tid] * inv_p);
@@ -853,11 +864,8 @@ __device__ __forceinline__ void pool_branch_fwd_v8_body(const float* __restrict_
         acc += __shfl_xor(acc, 1);
         acc += __shfl_xor(acc, 2);
         acc += __shfl_xor(acc, 4);
-        if (sub == 0 && o < D) {
-            if (bp) acc += to_f32(bp[o]);
-            if (bo) acc += to_f32(bo[o]);
-            rowbias[(long long)b * D + o] = acc;
-        }
+        acc += (bp ? to_f32(braw[pass][0]) : 0.f) + (bo ? to_f32(braw[pass][1]) : 0.f);
+        if (sub == 0 && o < D) rowbias[(long long)b * D + o] = acc;
     }
 }
 
