@@ -214,25 +214,44 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
     const T* gb = gy + b * H * W * ldg + c;
-    constexpr int NC = 10;  // candidate destinations per axis kept in registers (enough for scale >= 1/3)
+    // The candidate ranges are generous (up to 10 wide when the output is twice the input); the destinations
+    // that really weigh in are a contiguous run of about 2 * out/in.  Up to NS of them per axis are handled
+    // without branches: weights beyond the run are zero and addresses clamped, so the NS loads of a row are issued
+    // together (a load behind a per-lane `continue` is a trip to memory of its own).
+    constexpr int NC = 10, NS = 5;
+    int i0 = ihi + 1, i1 = ilo - 1, j0 = jhi + 1, j1 = jlo - 1;
     if (ihi - ilo < NC && jhi - jlo < NC) {
-        float wy[NC], wx[NC];
 #pragma unroll
-        for (int q = 0; q < NC; ++q) {
-            wy[q] = ilo + q <= ihi ? bl_weight(ilo + q, sy, h, m) : 0.f;
-            wx[q] = jlo + q <= jhi ? bl_weight(jlo + q, sx, w, n) : 0.f;
+        for (int q = NC - 1; q >= 0; --q) {
+            if (ilo + q <= ihi && bl_weight(ilo + q, sy, h, m) != 0.f) i0 = ilo + q;
+            if (jlo + q <= jhi && bl_weight(jlo + q, sx, w, n) != 0.f) j0 = jlo + q;
         }
 #pragma unroll
-        for (int p = 0; p < NC; ++p) {
-            if (wy[p] == 0.f) continue;
+        for (int q = 0; q < NC; ++q) {
+            if (ilo + q <= ihi && bl_weight(ilo + q, sy, h, m) != 0.f) i1 = ilo + q;
+            if (jlo + q <= jhi && bl_weight(jlo + q, sx, w, n) != 0.f) j1 = jlo + q;
+        }
+    }
+    if (i1 - i0 < NS && j1 - j0 < NS && i1 >= i0 && j1 >= j0) {
+        float wy[NS], wx[NS];
+        int jo[NS];
 #pragma unroll
-            for (int q = 0; q < NC; ++q) {
-                if (wx[q] == 0.f) continue;
-                float gv[VEC];
-                load_f32<T, VEC>(gb + ((long long)(ilo + p) * W + (jlo + q)) * ldg, gv);
+        for (int q = 0; q < NS; ++q) {
+            wy[q] = i0 + q <= i1 ? bl_weight(i0 + q, sy, h, m) : 0.f;
+            wx[q] = j0 + q <= j1 ? bl_weight(j0 + q, sx, w, n) : 0.f;
+            jo[q] = min(j0 + q, j1) * ldg;
+        }
+#pragma unroll
+        for (int p = 0; p < NS; ++p) {
+            const T* gr = gb + (long long)min(i0 + p, i1) * W * ldg;
+            ChanVec<T, VEC> gv[NS];
+#pragma unroll
+            for (int q = 0; q < NS; ++q) gv[q] = *reinterpret_cast<const ChanVec<T, VEC>*>(gr + jo[q]);
+#pragma unroll
+            for (int q = 0; q < NS; ++q) {
                 const float ww = wy[p] * wx[q];
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, gv[v], acc[v]);
+                for (int v = 0; v < VEC; ++v) acc[v] = fmaf(ww, to_f32(gv[q].v[v]), acc[v]);
             }
         }
     } else {
