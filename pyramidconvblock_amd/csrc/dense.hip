@@ -156,11 +156,21 @@ struct WTransposer {
 // need per-image sums of X over the positions and would otherwise read X a second time.  Chunk i*64+lane of a tile
 // is 8 columns of one row, and with 64 % (K/8) == 0 a lane keeps the same 8 columns for every chunk: 8 running
 // sums per lane, combined over the 512/K lanes that share them through the tile buffer once the fragments are out.
-template <typename T, bool KMAJOR, bool COLSUM>
+//
+// SK, SNO: the inner dimension and the feature count as compile-time constants (0: taken from the arguments).
+// With both fixed (and then K % 16 == 0, NO % 32 == 0) a full tile is whole passes of 64 chunks in and out and
+// whole MFMA steps, and its code has no per-lane predicates and no loop bounds to test: those were a third of the
+// generic kernel's vector-ALU work.
+template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0>
 __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T* __restrict__ W,
                                                 const T* __restrict__ bias, const float* __restrict__ rowbias,
-                                                T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
-                                                int NO, int P, int nkt, int nnt, int bid, int nblocks, uint32_t* dsm) {
+                                                T* __restrict__ Y, float* __restrict__ colsum, long long N, int Kd,
+                                                int NOd, int P, int nktd, int nntd, int bid, int nblocks,
+                                                uint32_t* dsm) {
+    constexpr bool STATIC = SK > 0 && SNO > 0;
+    static_assert(!STATIC || (SK % 16 == 0 && SNO % 32 == 0 && SK <= 128 && SNO <= 128), "static dense shape");
+    const int K = STATIC ? SK : Kd, NO = STATIC ? SNO : NOd;
+    const int nkt = STATIC ? SK / 16 : nktd, nnt = STATIC ? SNO / 32 : nntd;
     T* wl = reinterpret_cast<T*>(dsm);
     // The weights are multiplied as NOP x KP (whole feature tiles, 4 or 8 steps of the inner dimension) with zeros
     // in the padding, so that the multiplication below is straight-line code without predicates.
@@ -193,11 +203,22 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
         const T* base = X + t * 32 * K;
         const long long rows_left = N - t * 32;         // rows of this tile that exist
-        const int valid = rows_left >= 32 ? nin : (int)rows_left * cpk;
+        if (STATIC && rows_left >= 32) {
 #pragma unroll
-        for (int i = 0; i < LP; ++i) {
-            const int cidx = i * 64 + lane;
-            raw[i] = cidx < valid ? *reinterpret_cast<const Frag*>(base + (long long)cidx * 8) : Frag{{0u, 0u, 0u, 0u}};
+            for (int i = 0; i < LP; ++i) {
+                if (i * 64 < nin)
+                    raw[i] = *reinterpret_cast<const Frag*>(base + (long long)(i * 64 + lane) * 8);
+                else
+                    raw[i] = Frag{{0u, 0u, 0u, 0u}};
+            }
+        } else {
+            const int valid = rows_left >= 32 ? nin : (int)rows_left * cpk;
+#pragma unroll
+            for (int i = 0; i < LP; ++i) {
+                const int cidx = i * 64 + lane;
+                raw[i] = cidx < valid ? *reinterpret_cast<const Frag*>(base + (long long)cidx * 8)
+                                      : Frag{{0u, 0u, 0u, 0u}};
+            }
         }
         if (rowbias) {  // the tile's per-image rows ride behind its data: a tile of 32 rows meets two images at most
             const int img = min((int)(t * 32 / P) + half, nimg - 1);
@@ -252,7 +273,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
 #pragma unroll
         for (int i = 0; i < LP; ++i)
-            if (oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
+            if (STATIC ? i * 64 < nin : oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
         if (hasb && bcol < NOP) {
             const bool hb = bias != nullptr && bcol < NO;
             *reinterpret_cast<float4*>(bl + half * NOP + bcol) =
@@ -275,7 +296,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         Frag xf[kKT];
 #pragma unroll
         for (int kt = 0; kt < kKT; ++kt) {
-            if (kt < nkt && kt * 16 + 8 * half < K)
+            if (kt < nkt && (STATIC || kt * 16 + 8 * half < K))
                 xf[kt] = *reinterpret_cast<const Frag*>(tl + l32 * ldt + kt * 16 + 8 * half);
             else
                 xf[kt] = Frag{{0u, 0u, 0u, 0u}};
@@ -340,7 +361,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int n0 = nt * 32 + g4 * 8 + half * 4;
-                if (n0 < NO) {
+                if (STATIC || n0 < NO) {
                     float o[4];
                     o[0] = acc[g4 * 4] + r4[g4].x, o[1] = acc[g4 * 4 + 1] + r4[g4].y;
                     o[2] = acc[g4 * 4 + 2] + r4[g4].z, o[3] = acc[g4 * 4 + 3] + r4[g4].w;
@@ -354,15 +375,30 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         if (first) STAMP(6);
         {
             const long long rows_left = N - tile * 32;
-            const int valid = (rows_left >= 32 ? 32 : (int)rows_left) * cpr;
             T* yb = Y + tile * 32 * NO;
-            Frag ov[LO];
+            if (STATIC && rows_left >= 32) {  // (an array of its own: one array written on both paths ends up in scratch)
+                Frag of[LO];
 #pragma unroll
-            for (int i = 0; i < LO; ++i) ov[i] = *reinterpret_cast<const Frag*>(tl + (oout[i] >= 0 ? oout[i] : 0));
+                for (int i = 0; i < LO; ++i)
+                    if (i * 64 < 32 * cpr) of[i] = *reinterpret_cast<const Frag*>(tl + oout[i]);
 #pragma unroll
-            for (int i = 0; i < LO; ++i) {
-                const int cidx = i * 64 + lane;
-                if (cidx < valid) *reinterpret_cast<Frag*>(yb + (long long)cidx * 8) = ov[i];
+                for (int i = 0; i < LO; ++i)
+                    if (i * 64 < 32 * cpr) *reinterpret_cast<Frag*>(yb + (long long)(i * 64 + lane) * 8) = of[i];
+            } else {
+                const int valid = (rows_left >= 32 ? 32 : (int)rows_left) * cpr;
+                Frag ov[LO];
+#pragma unroll
+                for (int i = 0; i < LO; ++i) ov[i] = *reinterpret_cast<const Frag*>(tl + (oout[i] >= 0 ? oout[i] : 0));
+                // (naming the registers keeps the reads together: a read whose only use is a conditional store is
+                // otherwise moved to that store, one LDS latency per chunk)
+#pragma unroll
+                for (int i = 0; i < LO; ++i)
+                    asm volatile("" : "+v"(ov[i].v[0]), "+v"(ov[i].v[1]), "+v"(ov[i].v[2]), "+v"(ov[i].v[3]));
+#pragma unroll
+                for (int i = 0; i < LO; ++i) {
+                    const int cidx = i * 64 + lane;
+                    if (cidx < valid) *reinterpret_cast<Frag*>(yb + (long long)cidx * 8) = ov[i];
+                }
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // copy-out reads done before the next tile overwrites the buffer
@@ -370,19 +406,20 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     }
 }
 
-template <typename T, bool KMAJOR, bool COLSUM>
+template <typename T, bool KMAJOR, bool COLSUM, int SK, int SNO>
 __global__ __launch_bounds__(256, 2) void dense_rows_k(const T* __restrict__ X, const T* __restrict__ W,
                                                     const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                     T* __restrict__ Y, float* __restrict__ colsum, long long N, int K,
                                                     int NO, int P, int nkt, int nnt) {
     extern __shared__ uint32_t dsm[];
-    dense_rows_body<T, KMAJOR, COLSUM>(X, W, bias, rowbias, Y, colsum, N, K, NO, P, nkt, nnt, blockIdx.x, gridDim.x, dsm);
+    dense_rows_body<T, KMAJOR, COLSUM, SK, SNO>(X, W, bias, rowbias, Y, colsum, N, K, NO, P, nkt, nnt, blockIdx.x,
+                                                gridDim.x, dsm);
 }
 
 // The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
 // workgroups: they are a few microseconds of latency that need no launch of their own when a dense layer runs
 // after the last of the kernels that produce the partials.
-template <typename T, bool KMAJOR>
+template <typename T, bool KMAJOR, int SK, int SNO>
 __global__ __launch_bounds__(256, 2) void dense_rows_rider_k(const T* __restrict__ X, const T* __restrict__ W,
                                                           const T* __restrict__ bias,
                                                           const float* __restrict__ rowbias, T* __restrict__ Y,
@@ -396,8 +433,8 @@ __global__ __launch_bounds__(256, 2) void dense_rows_rider_k(const T* __restrict
     if ((int)blockIdx.x < nride) {
         reduce_jobs_block(jobs, blockIdx.x, reinterpret_cast<float*>(dsm));
     } else {
-        dense_rows_body<T, KMAJOR, false>(X, W, bias, rowbias, Y, nullptr, N, K, NO, P, nkt, nnt, blockIdx.x - nride,
-                                          nblocks, dsm);
+        dense_rows_body<T, KMAJOR, false, SK, SNO>(X, W, bias, rowbias, Y, nullptr, N, K, NO, P, nkt, nnt,
+                                                   blockIdx.x - nride, nblocks, dsm);
     }
 #if defined(PDW_STAMP) && PDW_STAMP == 4
     __syncthreads();
@@ -598,6 +635,7 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     if (blocks < 1) blocks = 1;
     const size_t lds = ((size_t)nnt * 32 * ((nkt > 4 ? 128 : 64) + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2 +
                        ((bias || rowbias) ? (size_t)4 * 2 * nnt * 32 * sizeof(float) : 0);
+    const int shape = getenv("PDW_DENSE_GENERIC") ? 0 : (K == 128 && NO == 64) ? 1 : (K == 64 && NO == 128) ? 2 : 0;
     if (rider) {
         // The summations come first in the grid and take resident slots of their own from the start (the slots
         // are two per compute unit; waiting for finished row workgroups would put their latency behind the
@@ -605,31 +643,50 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
         const int nride = rider->first_block[rider->njobs];
         if (blocks + nride > cap && nride <= cap / 4) blocks = cap - nride;
         const unsigned total = (unsigned)blocks + (unsigned)nride;
-#define PDW_RIDE(T, KM)                                                                                           \
-    hipLaunchKernelGGL((dense_rows_rider_k<T, KM>), dim3(total), dim3(256), lds, s, (const T*)x, (const T*)w,     \
-                       (const T*)bias, rowbias, (T*)y, N, K, NO, P > 0 ? P : 1, nkt, nnt, (int)blocks, *rider)
+        // shapes of the block's layers as compile-time constants (shape = 0: from the arguments)
+#define PDW_RIDE(T, KM, SK, SNO)                                                                                    \
+    hipLaunchKernelGGL((dense_rows_rider_k<T, KM, SK, SNO>), dim3(total), dim3(256), lds, s, (const T*)x,            \
+                       (const T*)w, (const T*)bias, rowbias, (T*)y, N, K, NO, P > 0 ? P : 1, nkt, nnt, (int)blocks,   \
+                       *rider)
+#define PDW_RIDE_S(T, KM)                 \
+    if (shape == 1)                       \
+        PDW_RIDE(T, KM, 128, 64);         \
+    else if (shape == 2)                  \
+        PDW_RIDE(T, KM, 64, 128);         \
+    else                                  \
+        PDW_RIDE(T, KM, 0, 0)
         if (dtype == kF16) {
-            if (w_kmajor) PDW_RIDE(f16_t, true); else PDW_RIDE(f16_t, false);
+            if (w_kmajor) { PDW_RIDE_S(f16_t, true); } else { PDW_RIDE_S(f16_t, false); }
         } else {
-            if (w_kmajor) PDW_RIDE(bf16_t, true); else PDW_RIDE(bf16_t, false);
+            if (w_kmajor) { PDW_RIDE_S(bf16_t, true); } else { PDW_RIDE_S(bf16_t, false); }
         }
+#undef PDW_RIDE_S
 #undef PDW_RIDE
         return check_launch("dense_rows_rider");
     }
-#define PDW_GO(T, KM, CSUM)                                                                                    \
-    hipLaunchKernelGGL((dense_rows_k<T, KM, CSUM>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x,        \
+#define PDW_GO(T, KM, CSUM, SK, SNO)                                                                             \
+    hipLaunchKernelGGL((dense_rows_k<T, KM, CSUM, SK, SNO>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x, \
                        (const T*)w, (const T*)bias, rowbias, (T*)y, colsum, N, K, NO, P > 0 ? P : 1, nkt, nnt)
-#define PDW_GO2(T, KM)            \
-    if (colsum)                   \
-        PDW_GO(T, KM, true);      \
-    else                          \
-        PDW_GO(T, KM, false)
+#define PDW_GO_S(T, KM, CSUM)             \
+    if (shape == 1)                       \
+        PDW_GO(T, KM, CSUM, 128, 64);     \
+    else if (shape == 2)                  \
+        PDW_GO(T, KM, CSUM, 64, 128);     \
+    else                                  \
+        PDW_GO(T, KM, CSUM, 0, 0)
+#define PDW_GO2(T, KM)                    \
+    if (colsum) {                         \
+        PDW_GO_S(T, KM, true);            \
+    } else {                              \
+        PDW_GO_S(T, KM, false);           \
+    }
     if (dtype == kF16) {
-        if (w_kmajor) { PDW_GO2(f16_t, true); } else { PDW_GO2(f16_t, false); }
+        if (w_kmajor) { PDW_GO2(f16_t, true) } else { PDW_GO2(f16_t, false) }
     } else {
-        if (w_kmajor) { PDW_GO2(bf16_t, true); } else { PDW_GO2(bf16_t, false); }
+        if (w_kmajor) { PDW_GO2(bf16_t, true) } else { PDW_GO2(bf16_t, false) }
     }
 #undef PDW_GO2
+#undef PDW_GO_S
 #undef PDW_GO
     return check_launch("dense_rows");
 }
