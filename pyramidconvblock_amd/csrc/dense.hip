@@ -448,10 +448,13 @@ __global__ __launch_bounds__(256, 2) void dense_rows_rider_k(const T* __restrict
 // the k-major MFMA fragments (8 consecutive rows of one feature) from LDS with 16-bit reads.
 constexpr int kWgRows = 64;
 
-template <typename T, int MT, int NT>
+// EXACT: M = 32 MT and NO = 32 NT, as compile-time facts: the staging map is shifts and masks, every pass is a
+// whole one and no fragment needs a clamp or a zero (the generic form spends a quarter of its time on those).
+template <typename T, int MT, int NT, bool EXACT>
 __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const T* __restrict__ Bm,
-                                                 float* __restrict__ part, long long N, int M, int NO, int nblocks,
+                                                 float* __restrict__ part, long long N, int Md, int NOd, int nblocks,
                                                  uint32_t* dsm) {
+    const int M = EXACT ? 32 * MT : Md, NO = EXACT ? 32 * NT : NOd;
     const int lda = M + 8, ldb = NO + 8;  // LDS row pitches (elements)
     const int buf_elems = kWgRows * (lda + ldb);
     T* lds = reinterpret_cast<T*>(dsm);
@@ -478,6 +481,15 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
 
     auto fetch = [&](long long st) {
         const long long r0 = st * kWgRows;
+        if (EXACT && r0 + kWgRows <= N) {  // a whole stage of an exact shape: contiguous, nothing to test
+            const T* ab = A + r0 * M + tid * 8;
+            const T* bb = Bm + r0 * NO + tid * 8;
+#pragma unroll
+            for (int p = 0; p < PA; ++p) pa[p] = *reinterpret_cast<const Frag*>(ab + p * 2048);
+#pragma unroll
+            for (int p = 0; p < PB; ++p) pb[p] = *reinterpret_cast<const Frag*>(bb + p * 2048);
+            return;
+        }
 #pragma unroll
         for (int p = 0; p < PA; ++p) {
             const int idx = tid + p * 256;
@@ -499,12 +511,12 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
 #pragma unroll
         for (int p = 0; p < PA; ++p) {
             const int idx = tid + p * 256;
-            if (idx < nva) *reinterpret_cast<Frag*>(la + (idx / va) * lda + (idx % va) * 8) = pa[p];
+            if (EXACT || idx < nva) *reinterpret_cast<Frag*>(la + (idx / va) * lda + (idx % va) * 8) = pa[p];
         }
 #pragma unroll
         for (int p = 0; p < PB; ++p) {
             const int idx = tid + p * 256;
-            if (idx < nvb) *reinterpret_cast<Frag*>(lb + (idx / vb) * ldb + (idx % vb) * 8) = pb[p];
+            if (EXACT || idx < nvb) *reinterpret_cast<Frag*>(lb + (idx / vb) * ldb + (idx % vb) * 8) = pb[p];
         }
     };
 
@@ -521,8 +533,8 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
         Frag af[MT], bf[NT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-            const int m = min(t * 32 + l32, M - 1);
-            const bool ok = t * 32 + l32 < M;
+            const int m = EXACT ? t * 32 + l32 : min(t * 32 + l32, M - 1);
+            const bool ok = EXACT || t * 32 + l32 < M;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t lo = ld16(la + (2 * j) * lda + m), hi = ld16(la + (2 * j + 1) * lda + m);
@@ -531,8 +543,8 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const int n = min(t * 32 + l32, NO - 1);
-            const bool ok = t * 32 + l32 < NO;
+            const int n = EXACT ? t * 32 + l32 : min(t * 32 + l32, NO - 1);
+            const bool ok = EXACT || t * 32 + l32 < NO;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t lo = ld16(lb + (2 * j) * ldb + n), hi = ld16(lb + (2 * j + 1) * ldb + n);
@@ -563,7 +575,7 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
                 const float4 a = *reinterpret_cast<const float4*>(red + idx), b = *reinterpret_cast<const float4*>(red + 1024 + idx);
                 const float4 c = *reinterpret_cast<const float4*>(red + 2048 + idx), d = *reinterpret_cast<const float4*>(red + 3072 + idx);
                 const int m = mt * 32 + 8 * (i / 4) + 4 * (l >> 5) + (i % 4), n = nt * 32 + (l & 31);
-                if (m < M && n < NO)  // NO % 8 == 0: the four values are in range together
+                if (EXACT || (m < M && n < NO))  // NO % 8 == 0: the four values are in range together
                     *reinterpret_cast<float4*>(pout + (long long)m * NO + n) =
                         make_float4((a.x + b.x) + (c.x + d.x), (a.y + b.y) + (c.y + d.y), (a.z + b.z) + (c.z + d.z),
                                     (a.w + b.w) + (c.w + d.w));
@@ -571,16 +583,16 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
         }
 }
 
-template <typename T, int MT, int NT>
+template <typename T, int MT, int NT, bool EXACT>
 __global__ __launch_bounds__(256, 2) void dense_wgrad_k(const T* __restrict__ A, const T* __restrict__ Bm,
                                                         float* __restrict__ part, long long N, int M, int NO) {
     extern __shared__ uint32_t dsm[];
-    dense_wgrad_body<T, MT, NT>(A, Bm, part, N, M, NO, gridDim.x, dsm);
+    dense_wgrad_body<T, MT, NT, EXACT>(A, Bm, part, N, M, NO, gridDim.x, dsm);
 }
 
 // The same with earlier summations in the workgroups behind the first `nblocks` (one workgroup of the product per
 // compute unit leaves room for a second one beside it from the start).
-template <typename T, int MT, int NT>
+template <typename T, int MT, int NT, bool EXACT>
 __global__ __launch_bounds__(256, 2) void dense_wgrad_rider_k(const T* __restrict__ A, const T* __restrict__ Bm,
                                                               float* __restrict__ part, long long N, int M, int NO,
                                                               int nblocks, const ReduceJobs jobs) {
@@ -589,7 +601,7 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_rider_k(const T* __restric
         reduce_jobs_block(jobs, blockIdx.x - nblocks, reinterpret_cast<float*>(dsm));
         return;
     }
-    dense_wgrad_body<T, MT, NT>(A, Bm, part, N, M, NO, nblocks, dsm);
+    dense_wgrad_body<T, MT, NT, EXACT>(A, Bm, part, N, M, NO, nblocks, dsm);
 }
 
 static bool dense_dims_ok(int K, int NO, int dtype) {
@@ -714,7 +726,7 @@ size_t dense_wgrad_workspace(long long N, int M, int NO) {
     return (size_t)blocks * M * NO * sizeof(float);
 }
 
-template <typename T, int MT, int NT>
+template <typename T, int MT, int NT, bool EXACT>
 static int dense_wgrad_go(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, hipStream_t s) {
     int blocks, spb;
     dense_wgrad_plan(N, &blocks, &spb);
@@ -723,11 +735,11 @@ static int dense_wgrad_go(const void* a, const void* b, void* dw, void* ws, long
     // While reductions are being deferred, the ones recorded so far run in this launch; its own joins the list.
     ReduceJobs jobs;
     if (reduce_defer_take(&jobs) > 0) {
-        hipLaunchKernelGGL((dense_wgrad_rider_k<T, MT, NT>), dim3(blocks + jobs.first_block[jobs.njobs]), dim3(256), lds,
-                           s, (const T*)a, (const T*)b, (float*)ws, N, M, NO, blocks, jobs);
+        hipLaunchKernelGGL((dense_wgrad_rider_k<T, MT, NT, EXACT>), dim3(blocks + jobs.first_block[jobs.njobs]),
+                           dim3(256), lds, s, (const T*)a, (const T*)b, (float*)ws, N, M, NO, blocks, jobs);
     } else {
-        hipLaunchKernelGGL((dense_wgrad_k<T, MT, NT>), dim3(blocks), dim3(256), lds, s, (const T*)a, (const T*)b,
-                           (float*)ws, N, M, NO);
+        hipLaunchKernelGGL((dense_wgrad_k<T, MT, NT, EXACT>), dim3(blocks), dim3(256), lds, s, (const T*)a,
+                           (const T*)b, (float*)ws, N, M, NO);
     }
     if (int e = check_launch("dense_wgrad")) return e;
     return wgrad_reduce_launch<T>((const float*)ws, dw, blocks, M * NO, s);
@@ -736,8 +748,11 @@ static int dense_wgrad_go(const void* a, const void* b, void* dw, void* ws, long
 template <typename T>
 static int dense_wgrad_t(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, hipStream_t s) {
     const int mt = cdiv(M, 32), nt = cdiv(NO, 32);
+    // the block's two layer shapes (64 x 128 and 128 x 64) have variants with the extents as constants
+    if (M == 64 && NO == 128 && !getenv("PDW_DENSE_GENERIC")) return dense_wgrad_go<T, 2, 4, true>(a, b, dw, ws, N, M, NO, s);
+    if (M == 128 && NO == 64 && !getenv("PDW_DENSE_GENERIC")) return dense_wgrad_go<T, 4, 2, true>(a, b, dw, ws, N, M, NO, s);
 #define PDW_CASE(MT, NT) \
-    if (mt == MT && nt == NT) return dense_wgrad_go<T, MT, NT>(a, b, dw, ws, N, M, NO, s);
+    if (mt == MT && nt == NT) return dense_wgrad_go<T, MT, NT, false>(a, b, dw, ws, N, M, NO, s);
     PDW_CASE(1, 1) PDW_CASE(1, 2) PDW_CASE(2, 1) PDW_CASE(2, 2) PDW_CASE(1, 3) PDW_CASE(3, 1) PDW_CASE(2, 3)
     PDW_CASE(3, 2) PDW_CASE(1, 4) PDW_CASE(4, 1) PDW_CASE(2, 4) PDW_CASE(4, 2)
 #undef PDW_CASE
