@@ -333,12 +333,18 @@ __device__ __forceinline__ void gate_fwd_items(const T* __restrict__ x, T* __res
     // thread's reads and writes alternate.  With every thread of the grid resident at once, "load everything,
     // then store everything" puts the whole kernel's reads before the whole kernel's writes.
     const int G = I / 2, GV = G / VEC;
+    // item -> (pixel, channel vector): a shift and a mask for the usual power-of-two channel counts; the general
+    // 64-bit division costs more vector-ALU time per item than the gate itself
+    const int sh = (GV & (GV - 1)) == 0 ? 31 - __builtin_clz(GV) : -1;
     ChanVec<T, VEC> a[U], b[U];
     long long m[U];
     int c[U];
     auto load = [&](int u) {
         const long long idx = min(first + u * step, total - 1);
-        c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
+        if (sh >= 0)
+            c[u] = ((int)idx & (GV - 1)) * VEC, m[u] = idx >> sh;
+        else
+            c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
         a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
         b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
     };
@@ -359,12 +365,16 @@ __device__ __forceinline__ void gate_bwd_items(const T* __restrict__ x, const T*
                                                int I, int ldg, float s, long long first, long long step,
                                                long long total) {
     const int G = I / 2, GV = G / VEC;
+    const int sh = (GV & (GV - 1)) == 0 ? 31 - __builtin_clz(GV) : -1;  // as in gate_fwd_items
     ChanVec<T, VEC> a[U], b[U], g[U];
     long long m[U];
     int c[U];
     auto load = [&](int u) {
         const long long idx = min(first + u * step, total - 1);
-        c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
+        if (sh >= 0)
+            c[u] = ((int)idx & (GV - 1)) * VEC, m[u] = idx >> sh;
+        else
+            c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
         a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
         b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
         g[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(gy + m[u] * ldg + c[u]);
