@@ -604,6 +604,24 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_rider_k(const T* __restric
     dense_wgrad_body<T, MT, NT, EXACT>(A, Bm, part, N, M, NO, nblocks, dsm);
 }
 
+// Input gradient and weight gradient of one dense layer (y = x W^T, W[O][I]) in one launch, for the block's
+// conv_out shape O = 128, I = 64: dx[N][I] = gy W (dense_rows_body, W as W[k][o]) and the partials of
+// dW[O][I] = gy^T x (dense_wgrad_body).  Both read gy and neither fills the chip alone (the weight gradient is one
+// workgroup per compute unit, the row product waits on memory in lockstep): the weight gradient's workgroups come
+// first in the grid, one per compute unit, and the row product's persistent workgroups take the second slot.
+template <typename T, bool COLSUM>
+__global__ __launch_bounds__(256, 2) void dense_bwd_pair_k(const T* __restrict__ gy, const T* __restrict__ W,
+                                                           const T* __restrict__ xin, T* __restrict__ dx,
+                                                           float* __restrict__ colsum, float* __restrict__ part,
+                                                           long long N, int nwg, int nrows) {
+    extern __shared__ uint32_t dsm[];
+    if ((int)blockIdx.x < nwg)
+        dense_wgrad_body<T, 4, 2, true>(gy, xin, part, N, 128, 64, nwg, dsm);
+    else
+        dense_rows_body<T, true, COLSUM, 128, 64>(gy, W, nullptr, nullptr, dx, colsum, N, 128, 64, 1, 8, 2,
+                                                  blockIdx.x - nwg, nrows, dsm);
+}
+
 static bool dense_dims_ok(int K, int NO, int dtype) {
     return dtype != kF32 && K >= 8 && K <= 16 * kKT && K % 8 == 0 && NO >= 8 && NO <= 32 * kNT && NO % 8 == 0;
 }
@@ -765,6 +783,40 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
     if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15)) return -1;
     if (dtype == kF16) return dense_wgrad_t<f16_t>(a, b, dw, ws, N, M, NO, s);
     return dense_wgrad_t<bf16_t>(a, b, dw, ws, N, M, NO, s);
+}
+
+int dense_bwd_pair_supported(int O, int I, int dtype) { return (dtype != kF32 && O == 128 && I == 64) ? 1 : 0; }
+
+// -1: shape not covered.  ws: dense_wgrad_workspace(N, O, I) bytes.
+int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* dx, float* colsum, void* dw, void* ws,
+                          long long N, int O, int I, int dtype, hipStream_t s) {
+    if (!dense_bwd_pair_supported(O, I, dtype)) return -1;
+    if (N <= 0 || N > 0x7fffffffLL) return -1;
+    const void* ptrs[5] = {gy, w, xin, dx, colsum};
+    for (const void* p : ptrs)
+        if (reinterpret_cast<uintptr_t>(p) & 15) return -1;
+    int nwg, spb;
+    dense_wgrad_plan(N, &nwg, &spb);
+    const long long ntiles = (N + 31) / 32;
+    long long nrows = (ntiles + 3) / 4;
+    const int cap = getenv("PDW_PAIR_ROWS") ? atoi(getenv("PDW_PAIR_ROWS")) : 256;  // the second slot of every CU
+    if (nrows > cap) nrows = cap;
+    const size_t lds_rows = ((size_t)64 * (128 + 8) + 4 * 32 * (128 + 8)) * 2;
+    const size_t lds_wg = (size_t)2 * kWgRows * (128 + 8 + 64 + 8) * 2;
+    const size_t lds = lds_rows > lds_wg ? lds_rows : lds_wg;
+    const dim3 grid((unsigned)(nwg + nrows));
+#define PDW_PAIR(T, CS)                                                                                              \
+    hipLaunchKernelGGL((dense_bwd_pair_k<T, CS>), grid, dim3(256), lds, s, (const T*)gy, (const T*)w, (const T*)xin, \
+                       (T*)dx, colsum, (float*)ws, N, nwg, (int)nrows)
+    if (dtype == kF16) {
+        if (colsum) PDW_PAIR(f16_t, true); else PDW_PAIR(f16_t, false);
+    } else {
+        if (colsum) PDW_PAIR(bf16_t, true); else PDW_PAIR(bf16_t, false);
+    }
+#undef PDW_PAIR
+    if (int e = check_launch("dense_bwd_pair")) return e;
+    if (dtype == kF16) return wgrad_reduce_launch<f16_t>((const float*)ws, dw, nwg, O * I, s);
+    return wgrad_reduce_launch<bf16_t>((const float*)ws, dw, nwg, O * I, s);
 }
 
 }  // namespace pdw

@@ -289,6 +289,34 @@ def dense_wgrad(a, b):
     return dw
 
 
+def dense_backward_pair_supported(O, I, dtype) -> bool:
+    """Whether dense_backward_pair covers a layer with weight [O, I]."""
+    return dtype in _lib._DTYPES and bool(_lib.lib().pdw_dense_bwd_pair_supported(int(O), int(I), _lib.dtype_code(dtype)))
+
+
+def dense_backward_pair(gy, w, x, colsum=False):
+    """Both gradients of y = x W^T that need gy, one launch: (dx [..., I], parts or None, dw [O, I]) with
+    dx = gy W, dw = gy^T x and, with colsum, parts as in dense_forward(gy, ..., colsum=True)."""
+    dev = _lib.require_device(gy, w, x)
+    O, I = w.shape
+    N = gy.numel() // O
+    assert gy.shape[-1] == O and x.shape[-1] == I and x.numel() // I == N
+    assert gy.is_contiguous() and w.is_contiguous() and x.is_contiguous()
+    dx = torch.empty(gy.shape[:-1] + (I,), device=dev, dtype=gy.dtype)
+    dw = torch.empty((O, I), device=dev, dtype=gy.dtype)
+    parts = None
+    if colsum:
+        R = dense_colsum_rows()
+        parts = torch.empty(((N + R - 1) // R, O), device=dev, dtype=torch.float32)
+    nbytes = _lib.lib().pdw_dense_wgrad_workspace_bytes(N, O, I)
+    ws = torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
+    _launch("pdw_dense_bwd_pair", dev, gy.data_ptr(), w.data_ptr(), x.data_ptr(), dx.data_ptr(),
+            parts.data_ptr() if parts is not None else None, dw.data_ptr(), ws.data_ptr(), ws.numel() * 4, N, O, I,
+            _lib.dtype_code(gy.dtype))
+    _lib.keep_until_flush(ws)
+    return dx, parts, dw
+
+
 def _pool_ws(B, P, D, dev):
     nbytes = _lib.lib().pdw_pool_branch_workspace_bytes(B, P, D)
     return torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)

@@ -297,3 +297,32 @@ def test_block_mid_matches_separate_launches(dtype, B, hw, I, D):
     r1 = ops.block_mid_backward(xf, xh, g, parts, P, m0, wp)
     for t0, t1 in zip(tuple(a0) + tuple(b0), r1):
         assert same(t0, t1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N", [1, 70, 96 * 7, 32 * 56 * 56])
+def test_dense_backward_pair_matches_separate_launches(dtype, N):
+    """Input gradient (with column sums) and weight gradient of a 64 -> 128 layer from one launch: the same bits
+    as the two launches it replaces, and the same with the summation deferred."""
+    from pyramidconvblock_amd import _lib, ops
+
+    O, I = 128, 64
+    assert ops.dense_backward_pair_supported(O, I, dtype) and not ops.dense_backward_pair_supported(64, 128, dtype)
+    gen = torch.Generator().manual_seed(N)
+    gy = randn(gen, N, O).to(dtype).cuda()
+    x = randn(gen, N, I).to(dtype).cuda()
+    w = (randn(gen, O, I) / 8).to(dtype).cuda()
+    colsum = N % ops.dense_colsum_rows() == 0
+    if colsum:
+        dx0, parts0 = ops.dense_forward(gy, w, w_kmajor=True, colsum=True)
+    else:
+        dx0, parts0 = ops.dense_forward(gy, w, w_kmajor=True), None
+    dw0 = ops.dense_wgrad(gy, x)
+    dx1, parts1, dw1 = ops.dense_backward_pair(gy, w, x, colsum=colsum)
+    assert torch.equal(dx1, dx0) and torch.equal(dw1, dw0)
+    assert (parts1 is None) == (parts0 is None) and (parts0 is None or torch.equal(parts1, parts0))
+    assert_close(dw1, (gy.double().t() @ x.double()).cpu().numpy(), dtype, "pair wgrad")
+    with _lib.deferred_reductions(gy.device):
+        dx2, _, dw2 = ops.dense_backward_pair(gy, w, x, colsum=colsum)
+    torch.cuda.synchronize()
+    assert torch.equal(dx2, dx0) and torch.equal(dw2, dw0)
