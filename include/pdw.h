@@ -235,15 +235,17 @@ size_t pdw_dense_wgrad_workspace_bytes(long long N, int M, int NO);
 int pdw_dense_wgrad(const void *a, const void *b, void *dw, void *workspace, size_t workspace_bytes, long long N,
                     int M, int NO, int dtype, void *stream);
 
-/* Both gradients of a dense layer y = x W^T (W[O][I]) that need gy, in one launch: dx[N,I] = gy W and
- * dw[O,I] = gy^T x (workspace and summation as pdw_dense_wgrad, size pdw_dense_wgrad_workspace_bytes(N, O, I)); with
+/* Both gradients of a dense layer y = x W^T (W[O][I]) that need gy, in one launch: dx[N,I] = gy W
+ * (+ rowbias[n / P], fp32 [ceil(N/P), I], may be NULL; P >= 32) and dw[O,I] = gy^T x (workspace and summation as pdw_dense_wgrad, size pdw_dense_wgrad_workspace_bytes(N, O, I)); with
  * colsum != NULL also the sums of gy over groups of pdw_dense_colsum_rows() rows, as pdw_dense_fwd_colsum.  The two
  * products share the chip instead of following each other (each alone leaves half of it waiting on memory).
- * Covered: 16-bit, O = 128, I = 64 (pdw_dense_bwd_pair_supported): the backward of conv_out, conv_block.py:44, in
- * ConvBlock(128); other shapes take pdw_dense_fwd(w_kmajor) and pdw_dense_wgrad. */
+ * Covered: 16-bit, (O, I) = (128, 64) or (64, 128) (pdw_dense_bwd_pair_supported): the backward of conv_out and
+ * conv_up, conv_block.py:44 and :37, in ConvBlock(128); other shapes take pdw_dense_fwd(w_kmajor) and
+ * pdw_dense_wgrad.  Unlike pdw_dense_wgrad it carries no recorded summations along. */
 int pdw_dense_bwd_pair_supported(int O, int I, int dtype);
 int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, float *colsum, void *dw, void *workspace,
-                       size_t workspace_bytes, long long N, int O, int I, int dtype, void *stream);
+                       size_t workspace_bytes, const float *rowbias, int P, long long N, int O, int I, int dtype,
+                       void *stream);
 
 #ifdef __cplusplus
 }

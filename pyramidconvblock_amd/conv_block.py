@@ -16,6 +16,8 @@ gradients as a batched split-K product.
 """
 from __future__ import annotations
 
+import os as _os
+
 import torch
 from torch import nn
 from torch.nn import functional as F
@@ -257,7 +259,13 @@ class ConvBlockFunction(torch.autograd.Function):
             a2d = da.view(N, I)
             grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
             dx = None
-            if fast_up:
+            if (fast_up and ctx.needs_input_grad[0] and N > 0 and x.dtype == dt and dmean is not None
+                    and ops.dense_backward_pair_supported(I, D, dt, H * W) and not _os.environ.get("PDW_NO_UP_PAIR")):
+                # both products that read da share the pass's last large launch; the summations recorded on the
+                # way run as one small launch when the block of deferred work closes
+                dx, _, grad_w_up = ops.dense_backward_pair(da, w_up.detach().contiguous(), x.contiguous(),
+                                                           rowbias=dmean, rows_per_image=H * W)
+            elif fast_up:
                 grad_w_up = ops.dense_wgrad(da, x)
                 if ctx.needs_input_grad[0]:
                     # the last kernel of the pass: the recorded summations ride in its grid

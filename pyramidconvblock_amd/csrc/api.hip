@@ -449,17 +449,20 @@ int pdw_dense_bwd_pair_supported(int O, int I, int dtype) {
 }
 
 int pdw_dense_bwd_pair(const void* gy, const void* w, const void* x, void* dx, float* colsum, void* dw, void* workspace,
-                       size_t workspace_bytes, long long N, int O, int I, int dtype, void* stream) {
+                       size_t workspace_bytes, const float* rowbias, int P, long long N, int O, int I, int dtype,
+                       void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_dense_bwd_pair: unknown dtype %d", dtype), 1;
     if (N < 1 || O < 1 || I < 1) return set_error("pdw_dense_bwd_pair: bad extents N=%lld O=%d I=%d", N, O, I), 1;
     if (!gy || !w || !x || !dx || !dw) return set_error("pdw_dense_bwd_pair: null pointer"), 1;
     const size_t need = dense_wgrad_workspace(N, O, I);
     if (!workspace || workspace_bytes < need)
         return set_error("pdw_dense_bwd_pair: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
-    const int r = dense_bwd_pair_launch(gy, w, x, dx, colsum, dw, workspace, N, O, I, dtype, (hipStream_t)stream);
+    if (rowbias && P < 1) return set_error("pdw_dense_bwd_pair: rowbias needs P >= 1"), 1;
+    const int r = dense_bwd_pair_launch(gy, w, x, dx, colsum, dw, workspace, rowbias, P, N, O, I, dtype,
+                                        (hipStream_t)stream);
     if (r == -1)
-        return set_error("pdw_dense_bwd_pair: O=%d I=%d dtype=%d not covered (see pdw_dense_bwd_pair_supported)", O, I,
-                         dtype), 3;
+        return set_error("pdw_dense_bwd_pair: O=%d I=%d dtype=%d (P=%d) not covered (see pdw_dense_bwd_pair_supported)",
+                         O, I, dtype, P), 3;
     return r;
 }
 

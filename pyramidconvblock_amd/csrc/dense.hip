@@ -605,21 +605,22 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_rider_k(const T* __restric
 }
 
 // Input gradient and weight gradient of one dense layer (y = x W^T, W[O][I]) in one launch, for the block's
-// conv_out shape O = 128, I = 64: dx[N][I] = gy W (dense_rows_body, W as W[k][o]) and the partials of
-// dW[O][I] = gy^T x (dense_wgrad_body).  Both read gy and neither fills the chip alone (the weight gradient is one
+// two layer shapes (O, I) = (128, 64) and (64, 128): dx[N][I] = gy W (dense_rows_body, W as W[k][o]) and the
+// partials of dW[O][I] = gy^T x (dense_wgrad_body).  Both read gy and neither fills the chip alone (the weight gradient is one
 // workgroup per compute unit, the row product waits on memory in lockstep): the weight gradient's workgroups come
 // first in the grid, one per compute unit, and the row product's persistent workgroups take the second slot.
-template <typename T, bool COLSUM>
+template <typename T, bool COLSUM, int O, int I>
 __global__ __launch_bounds__(256, 2) void dense_bwd_pair_k(const T* __restrict__ gy, const T* __restrict__ W,
                                                            const T* __restrict__ xin, T* __restrict__ dx,
                                                            float* __restrict__ colsum, float* __restrict__ part,
-                                                           long long N, int nwg, int nrows) {
+                                                           const float* __restrict__ rowbias, int P, long long N,
+                                                           int nwg, int nrows) {
     extern __shared__ uint32_t dsm[];
     if ((int)blockIdx.x < nwg)
-        dense_wgrad_body<T, 4, 2, true>(gy, xin, part, N, 128, 64, nwg, dsm);
+        dense_wgrad_body<T, O / 32, I / 32, true>(gy, xin, part, N, O, I, nwg, dsm);
     else
-        dense_rows_body<T, true, COLSUM, 128, 64>(gy, W, nullptr, nullptr, dx, colsum, N, 128, 64, 1, 8, 2,
-                                                  blockIdx.x - nwg, nrows, dsm);
+        dense_rows_body<T, true, COLSUM, O, I>(gy, W, nullptr, rowbias, dx, colsum, N, O, I, P, O / 16, I / 32,
+                                               blockIdx.x - nwg, nrows, dsm);
 }
 
 static bool dense_dims_ok(int K, int NO, int dtype) {
@@ -785,12 +786,15 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
     return dense_wgrad_t<bf16_t>(a, b, dw, ws, N, M, NO, s);
 }
 
-int dense_bwd_pair_supported(int O, int I, int dtype) { return (dtype != kF32 && O == 128 && I == 64) ? 1 : 0; }
+int dense_bwd_pair_supported(int O, int I, int dtype) {
+    return (dtype != kF32 && ((O == 128 && I == 64) || (O == 64 && I == 128))) ? 1 : 0;
+}
 
 // -1: shape not covered.  ws: dense_wgrad_workspace(N, O, I) bytes.
 int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* dx, float* colsum, void* dw, void* ws,
-                          long long N, int O, int I, int dtype, hipStream_t s) {
+                          const float* rowbias, int P, long long N, int O, int I, int dtype, hipStream_t s) {
     if (!dense_bwd_pair_supported(O, I, dtype)) return -1;
+    if (rowbias && (P < 32 || (reinterpret_cast<uintptr_t>(rowbias) & 15))) return -1;  // two images per tile at most
     if (N <= 0 || N > 0x7fffffffLL) return -1;
     const void* ptrs[5] = {gy, w, xin, dx, colsum};
     for (const void* p : ptrs)
@@ -801,18 +805,24 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
     long long nrows = (ntiles + 3) / 4;
     const int cap = getenv("PDW_PAIR_ROWS") ? atoi(getenv("PDW_PAIR_ROWS")) : 256;  // the second slot of every CU
     if (nrows > cap) nrows = cap;
-    const size_t lds_rows = ((size_t)64 * (128 + 8) + 4 * 32 * (128 + 8)) * 2;
-    const size_t lds_wg = (size_t)2 * kWgRows * (128 + 8 + 64 + 8) * 2;
+    if (colsum && !dense_colsum_supported(O, I, dtype)) return -1;
+    // rows product: K = O, NO = I (inner dimension padded to 64 or 128 in LDS); weight gradient: M = O, NO = I
+    const size_t lds_rows = ((size_t)I * ((O > 64 ? 128 : 64) + 8) + 4 * 32 * ((O > I ? O : I) + 8)) * 2 +
+                            (rowbias ? (size_t)4 * 2 * I * sizeof(float) : 0);
+    const size_t lds_wg = (size_t)2 * kWgRows * (O + 8 + I + 8) * 2;
     const size_t lds = lds_rows > lds_wg ? lds_rows : lds_wg;
     const dim3 grid((unsigned)(nwg + nrows));
-#define PDW_PAIR(T, CS)                                                                                              \
-    hipLaunchKernelGGL((dense_bwd_pair_k<T, CS>), grid, dim3(256), lds, s, (const T*)gy, (const T*)w, (const T*)xin, \
-                       (T*)dx, colsum, (float*)ws, N, nwg, (int)nrows)
-    if (dtype == kF16) {
-        if (colsum) PDW_PAIR(f16_t, true); else PDW_PAIR(f16_t, false);
-    } else {
-        if (colsum) PDW_PAIR(bf16_t, true); else PDW_PAIR(bf16_t, false);
+#define PDW_PAIR(T, CS, OO, II)                                                                                      \
+    hipLaunchKernelGGL((dense_bwd_pair_k<T, CS, OO, II>), grid, dim3(256), lds, s, (const T*)gy, (const T*)w,        \
+                       (const T*)xin, (T*)dx, colsum, (float*)ws, rowbias, P > 0 ? P : 1, N, nwg, (int)nrows)
+#define PDW_PAIR_T(T)                                           \
+    if (O == 128) {                                             \
+        if (colsum) PDW_PAIR(T, true, 128, 64); else PDW_PAIR(T, false, 128, 64); \
+    } else {                                                    \
+        if (colsum) PDW_PAIR(T, true, 64, 128); else PDW_PAIR(T, false, 64, 128); \
     }
+    if (dtype == kF16) { PDW_PAIR_T(f16_t) } else { PDW_PAIR_T(bf16_t) }
+#undef PDW_PAIR_T
 #undef PDW_PAIR
     if (int e = check_launch("dense_bwd_pair")) return e;
     if (dtype == kF16) return wgrad_reduce_launch<f16_t>((const float*)ws, dw, nwg, O * I, s);

@@ -122,9 +122,9 @@ __global__ __launch_bounds__(256) void dwconv_wgrad_direct(const T* __restrict__
 
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_parts(const float* __restrict__ part, T* __restrict__ dw,
-                                                          int nparts, int n, int vec) {
+                                                          int nparts, int n, int vec, int ql) {
     __shared__ float red[kReduceLds];
-    reduce_parts_any<T>(part, dw, nparts, n, blockIdx.x, vec, red);
+    reduce_parts_any<T>(part, dw, nparts, n, blockIdx.x, vec, ql, red);
 }
 
 __global__ __launch_bounds__(256) void wgrad_reduce_many(const ReduceJobs jobs) {
@@ -137,8 +137,22 @@ __global__ __launch_bounds__(256) void wgrad_reduce_many(const ReduceJobs jobs) 
 static thread_local bool t_defer = false;
 static thread_local ReduceJobs t_jobs;
 
-int reduce_jobs_launch(const ReduceJobs& jobs, hipStream_t s) {
-    if (jobs.njobs == 0) return 0;
+// Part lanes of a stand-alone summation: 32 when 8 would need more than one round of loads.
+static int standalone_part_lanes(int nparts) { return nparts > 128 ? 32 : 8; }
+
+// A launch of its own has the whole chip's slots: the jobs that were laid out for riding (few workgroups, 8 part
+// lanes) are laid out again with as many part lanes as make their loads a single round.
+int reduce_jobs_launch(const ReduceJobs& recorded, hipStream_t s) {
+    if (recorded.njobs == 0) return 0;
+    ReduceJobs jobs = recorded;
+    for (int j = 0; j < jobs.njobs; ++j) {
+        int nb = recorded.first_block[j + 1] - recorded.first_block[j];
+        if (recorded.vec[j] != 0) {
+            jobs.ql[j] = standalone_part_lanes(jobs.nparts[j]);
+            nb = cdiv(jobs.n[j], reduce_block_outputs(jobs.vec[j], jobs.ql[j]));
+        }
+        jobs.first_block[j + 1] = jobs.first_block[j] + nb;
+    }
     hipLaunchKernelGGL(wgrad_reduce_many, dim3(jobs.first_block[jobs.njobs]), dim3(256), 0, s, jobs);
     return check_launch("wgrad_reduce_many");
 }
@@ -167,7 +181,7 @@ int reduce_defer_outer(const float* g, const void* m, void* out, int B, int D, i
     if (reduce_defer_room() < 1 || dtype == kF32 || D % 4 != 0) return -1;
     const int j = t_jobs.njobs++;
     t_jobs.part[j] = g, t_jobs.aux[j] = m, t_jobs.out[j] = out, t_jobs.nparts[j] = B, t_jobs.n[j] = D * D;
-    t_jobs.dtype[j] = dtype, t_jobs.vec[j] = 0, t_jobs.dim[j] = D;
+    t_jobs.dtype[j] = dtype, t_jobs.vec[j] = 0, t_jobs.ql[j] = 8, t_jobs.dim[j] = D;
     t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv((long long)D * D, kOuterBlock);
     return 0;
 }
@@ -263,11 +277,13 @@ int wgrad_reduce_launch(const float* part, void* dw, int nparts, int n, hipStrea
         const int j = t_jobs.njobs++;
         t_jobs.part[j] = part, t_jobs.out[j] = dw, t_jobs.nparts[j] = nparts, t_jobs.n[j] = n;
         t_jobs.dtype[j] = dtype_of<T>();
-        t_jobs.vec[j] = vec;
-        t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv(n, 32 * vec);
+        t_jobs.vec[j] = vec, t_jobs.ql[j] = 8;
+        t_jobs.first_block[j + 1] = t_jobs.first_block[j] + cdiv(n, reduce_block_outputs(vec, 8));
         return 0;
     }
-    hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, 32 * vec)), dim3(256), 0, s, part, (T*)dw, nparts, n, vec);
+    const int ql = standalone_part_lanes(nparts);
+    hipLaunchKernelGGL((wgrad_reduce_parts<T>), dim3(cdiv(n, reduce_block_outputs(vec, ql))), dim3(256), 0, s, part,
+                       (T*)dw, nparts, n, vec, ql);
     return check_launch("wgrad_reduce_parts");
 }
 template int wgrad_reduce_launch<float>(const float*, void*, int, int, hipStream_t);

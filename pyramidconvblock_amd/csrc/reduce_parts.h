@@ -6,19 +6,21 @@
 namespace pdw {
 
 // Pass 2 of wgrad (shared with the tiled kernels): dw[e] = sum over parts in a fixed order.
-// Block = 32 output lanes x 8 part lanes; an output lane owns V consecutive outputs (V = 4: 16-byte loads, a
-// quarter of the workgroups), part lane q adds parts q, q+8, ... and the 8 lanes are combined through LDS, so the
-// reads of one part are contiguous and many parts are in flight.  V = 4 needs n % 4 == 0 and 16-byte aligned
-// partials (reduce_vec_ok).
+// Block = EL output lanes x QL part lanes (EL * QL = 256); an output lane owns V consecutive outputs (V = 4:
+// 16-byte loads), part lane q adds parts q, q + QL, ... with up to sixteen loads in flight, and the QL lanes are
+// combined through LDS, so the reads of one part are contiguous and many parts are in flight.  The pass is pure
+// latency.  QL = 8 keeps the workgroups few (they ride in other kernels' grids, where resident slots are scarce);
+// QL = 32 takes 256 parts in one round of loads, for the stand-alone launch.  V = 4 needs n % 4 == 0 and 16-byte
+// aligned partials (reduce_vec_ok).  The order of the additions, and so the result, depends on QL.
 constexpr int kReduceVec = 4;
 constexpr int kReduceLds = 8 * 32 * kReduceVec;  // floats of LDS a workgroup needs
 
-template <typename T, int V>
+template <typename T, int V, int QL>
 __device__ __forceinline__ void reduce_parts_block(const float* __restrict__ part, T* __restrict__ dw, int nparts, int n,
                                                    int blk, float* red) {
-    constexpr int ROW = 32 * V;  // red[8][ROW]
-    const int el = threadIdx.x & 31, q = threadIdx.x >> 5;
-    const int e = (blk * 32 + el) * V;
+    constexpr int EL = 256 / QL, ROW = EL * V;  // red[QL][ROW]
+    const int el = threadIdx.x % EL, q = threadIdx.x / EL;
+    const int e = (blk * EL + el) * V;
     float s0[V], s1[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) s0[i] = 0.f, s1[i] = 0.f;
@@ -32,29 +34,29 @@ __device__ __forceinline__ void reduce_parts_block(const float* __restrict__ par
     };
     if (e < n) {
         int p = q;
-        for (; p + 120 < nparts; p += 128) {  // sixteen loads in flight per lane: the pass is pure latency
+        for (; p + 15 * QL < nparts; p += 16 * QL) {  // sixteen loads in flight per lane
             float v[16][V];
 #pragma unroll
-            for (int u = 0; u < 16; ++u) ld(p + 8 * u, v[u]);
+            for (int u = 0; u < 16; ++u) ld(p + QL * u, v[u]);
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 s0[i] += ((v[0][i] + v[2][i]) + (v[4][i] + v[6][i])) + ((v[8][i] + v[10][i]) + (v[12][i] + v[14][i]));
                 s1[i] += ((v[1][i] + v[3][i]) + (v[5][i] + v[7][i])) + ((v[9][i] + v[11][i]) + (v[13][i] + v[15][i]));
             }
         }
-        for (; p + 56 < nparts; p += 64) {
+        for (; p + 7 * QL < nparts; p += 8 * QL) {
             float v[8][V];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) ld(p + 8 * u, v[u]);
+            for (int u = 0; u < 8; ++u) ld(p + QL * u, v[u]);
 #pragma unroll
             for (int i = 0; i < V; ++i) {
                 s0[i] += (v[0][i] + v[2][i]) + (v[4][i] + v[6][i]);
                 s1[i] += (v[1][i] + v[3][i]) + (v[5][i] + v[7][i]);
             }
         }
-        for (; p + 8 < nparts; p += 16) {
+        for (; p + QL < nparts; p += 2 * QL) {
             float a[V], b[V];
-            ld(p, a), ld(p + 8, b);
+            ld(p, a), ld(p + QL, b);
 #pragma unroll
             for (int i = 0; i < V; ++i) s0[i] += a[i], s1[i] += b[i];
         }
@@ -68,6 +70,17 @@ __device__ __forceinline__ void reduce_parts_block(const float* __restrict__ par
 #pragma unroll
     for (int i = 0; i < V; ++i) red[q * ROW + el * V + i] = s0[i] + s1[i];
     __syncthreads();
+    if constexpr (QL == 32) {  // 32 rows -> 8, by the threads of the first 8 part lanes
+        if (q < 8) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const int c = el * V + i;
+                red[q * ROW + c] = (red[q * ROW + c] + red[(q + 8) * ROW + c]) +
+                                   (red[(q + 16) * ROW + c] + red[(q + 24) * ROW + c]);
+            }
+        }
+        __syncthreads();
+    }
     if (q == 0 && e < n) {
         float o[V];
 #pragma unroll
@@ -86,11 +99,19 @@ inline bool reduce_vec_ok(const float* part, const void* dw, int n, int esize) {
            (reinterpret_cast<uintptr_t>(dw) & (size_t)(kReduceVec * esize - 1)) == 0;
 }
 
+// Outputs one workgroup covers, for `vec` outputs per lane and `ql` part lanes.
+inline int reduce_block_outputs(int vec, int ql) { return 256 / ql * vec; }
+
 template <typename T>
-__device__ __forceinline__ void reduce_parts_any(const float* part, T* dw, int nparts, int n, int blk, int vec,
+__device__ __forceinline__ void reduce_parts_any(const float* part, T* dw, int nparts, int n, int blk, int vec, int ql,
                                                  float* red) {
-    if (vec == kReduceVec) reduce_parts_block<T, kReduceVec>(part, dw, nparts, n, blk, red);
-    else reduce_parts_block<T, 1>(part, dw, nparts, n, blk, red);
+    if (vec == kReduceVec) {
+        if (ql == 32) reduce_parts_block<T, kReduceVec, 32>(part, dw, nparts, n, blk, red);
+        else reduce_parts_block<T, kReduceVec, 8>(part, dw, nparts, n, blk, red);
+    } else {
+        if (ql == 32) reduce_parts_block<T, 1, 32>(part, dw, nparts, n, blk, red);
+        else reduce_parts_block<T, 1, 8>(part, dw, nparts, n, blk, red);
+    }
 }
 
 // out[o * D + d] = sum over b < B of g[b * D + o] * m[b * D + d]: the weight gradient of a small dense layer
@@ -138,6 +159,7 @@ struct ReduceJobs {
     const void* aux[kMaxReduceJobs];  // outer products: the second factor (element type of `out`)
     int nparts[kMaxReduceJobs], n[kMaxReduceJobs], dtype[kMaxReduceJobs];
     int vec[kMaxReduceJobs];  // outputs per lane: kReduceVec or 1; 0 = outer product (n = D * D, nparts = B)
+    int ql[kMaxReduceJobs];   // part lanes: 8 or 32
     int dim[kMaxReduceJobs];  // outer products: D
     int first_block[kMaxReduceJobs + 1];
     int njobs;
@@ -149,7 +171,7 @@ __device__ __forceinline__ void reduce_jobs_block(const ReduceJobs& jobs, int wg
     while (j + 1 < jobs.njobs && wg >= jobs.first_block[j + 1]) ++j;  // uniform: scalar ALU
     const int blk = wg - jobs.first_block[j];
     const float* part = jobs.part[j];
-    const int nparts = jobs.nparts[j], n = jobs.n[j], vec = jobs.vec[j];
+    const int nparts = jobs.nparts[j], n = jobs.n[j], vec = jobs.vec[j], ql = jobs.ql[j];
     if (vec == 0) {  // outer product; fp32 outputs are not produced this way
         if (jobs.dtype[j] == kF16)
             outer_sum_block<f16_t>(part, (const f16_t*)jobs.aux[j], (f16_t*)jobs.out[j], nparts, jobs.dim[j], blk, threadIdx.x);
@@ -158,9 +180,9 @@ __device__ __forceinline__ void reduce_jobs_block(const ReduceJobs& jobs, int wg
         return;
     }
     switch (jobs.dtype[j]) {
-        case kF32: reduce_parts_any<float>(part, (float*)jobs.out[j], nparts, n, blk, vec, red); break;
-        case kF16: reduce_parts_any<f16_t>(part, (f16_t*)jobs.out[j], nparts, n, blk, vec, red); break;
-        default: reduce_parts_any<bf16_t>(part, (bf16_t*)jobs.out[j], nparts, n, blk, vec, red); break;
+        case kF32: reduce_parts_any<float>(part, (float*)jobs.out[j], nparts, n, blk, vec, ql, red); break;
+        case kF16: reduce_parts_any<f16_t>(part, (f16_t*)jobs.out[j], nparts, n, blk, vec, ql, red); break;
+        default: reduce_parts_any<bf16_t>(part, (bf16_t*)jobs.out[j], nparts, n, blk, vec, ql, red); break;
     }
 }
 

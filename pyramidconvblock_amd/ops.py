@@ -289,14 +289,17 @@ def dense_wgrad(a, b):
     return dw
 
 
-def dense_backward_pair_supported(O, I, dtype) -> bool:
-    """Whether dense_backward_pair covers a layer with weight [O, I]."""
-    return dtype in _lib._DTYPES and bool(_lib.lib().pdw_dense_bwd_pair_supported(int(O), int(I), _lib.dtype_code(dtype)))
+def dense_backward_pair_supported(O, I, dtype, rows_per_image=None) -> bool:
+    """Whether dense_backward_pair covers a layer with weight [O, I] (and a per-image term over images of
+    rows_per_image rows)."""
+    return (dtype in _lib._DTYPES and (rows_per_image is None or rows_per_image >= 32)
+            and bool(_lib.lib().pdw_dense_bwd_pair_supported(int(O), int(I), _lib.dtype_code(dtype))))
 
 
-def dense_backward_pair(gy, w, x, colsum=False):
+def dense_backward_pair(gy, w, x, colsum=False, rowbias=None, rows_per_image=1):
     """Both gradients of y = x W^T that need gy, one launch: (dx [..., I], parts or None, dw [O, I]) with
-    dx = gy W, dw = gy^T x and, with colsum, parts as in dense_forward(gy, ..., colsum=True)."""
+    dx = gy W + rowbias[image] (rowbias fp32 [B, I] or None), dw = gy^T x and, with colsum, parts as in
+    dense_forward(gy, ..., colsum=True)."""
     dev = _lib.require_device(gy, w, x)
     O, I = w.shape
     N = gy.numel() // O
@@ -311,7 +314,8 @@ def dense_backward_pair(gy, w, x, colsum=False):
     nbytes = _lib.lib().pdw_dense_wgrad_workspace_bytes(N, O, I)
     ws = torch.empty(nbytes // 4 + 1, device=dev, dtype=torch.float32)
     _launch("pdw_dense_bwd_pair", dev, gy.data_ptr(), w.data_ptr(), x.data_ptr(), dx.data_ptr(),
-            parts.data_ptr() if parts is not None else None, dw.data_ptr(), ws.data_ptr(), ws.numel() * 4, N, O, I,
+            parts.data_ptr() if parts is not None else None, dw.data_ptr(), ws.data_ptr(), ws.numel() * 4,
+            rowbias.data_ptr() if rowbias is not None else None, int(rows_per_image), N, O, I,
             _lib.dtype_code(gy.dtype))
     _lib.keep_until_flush(ws)
     return dx, parts, dw

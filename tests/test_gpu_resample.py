@@ -307,7 +307,7 @@ def test_dense_backward_pair_matches_separate_launches(dtype, N):
     from pyramidconvblock_amd import _lib, ops
 
     O, I = 128, 64
-    assert ops.dense_backward_pair_supported(O, I, dtype) and not ops.dense_backward_pair_supported(64, 128, dtype)
+    assert ops.dense_backward_pair_supported(O, I, dtype) and not ops.dense_backward_pair_supported(96, 64, dtype)
     gen = torch.Generator().manual_seed(N)
     gy = randn(gen, N, O).to(dtype).cuda()
     x = randn(gen, N, I).to(dtype).cuda()
@@ -326,3 +326,13 @@ def test_dense_backward_pair_matches_separate_launches(dtype, N):
         dx2, _, dw2 = ops.dense_backward_pair(gy, w, x, colsum=colsum)
     torch.cuda.synchronize()
     assert torch.equal(dx2, dx0) and torch.equal(dw2, dw0)
+    # the other covered shape (128 -> 64 layer), with a per-image term on the input gradient
+    if N >= 64:
+        P = 32 if N % 32 == 0 else N
+        rb = randn(gen, (N + P - 1) // P, O).cuda()
+        w2 = (randn(gen, I, O) / 8).to(dtype).cuda()
+        assert ops.dense_backward_pair_supported(I, O, dtype, P)
+        dxa = ops.dense_forward(x, w2, w_kmajor=True, rowbias=rb, rows_per_image=P)
+        dwa = ops.dense_wgrad(x, gy)
+        dxb, _, dwb = ops.dense_backward_pair(x, w2, gy, rowbias=rb, rows_per_image=P)
+        assert torch.equal(dxb, dxa) and torch.equal(dwb, dwa)
