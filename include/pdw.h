@@ -102,6 +102,17 @@ int pdw_dwconv_wgrad(const void *x, const void *gy, void *dw, void *workspace, s
                      int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW, int DH,
                      int DW, int dtype, void *stream);
 
+/* Two pdw_dwconv_wgrad calls of one pyramid block as one call: the same batch, channel count and odd square
+ * filter (stride 1, padding K/2, dilation 1) on two tensors of different extents, each with its own workspace
+ * (sized by pdw_dwconv_wgrad_workspace_bytes).  For 16-bit types the two problems share one launch, the second
+ * one's workgroups starting as compute units finish with the first; otherwise this is the two calls in turn.
+ * Results are bitwise those of the separate calls.  Replaces the two launches of
+ * _depthwise_conv_weight_grad_kernel (dwconv_triton.py:377-385) that the backward of conv_block.py:41 makes
+ * for the block's two scales. */
+int pdw_dwconv_wgrad_pair(const void *x0, const void *gy0, void *dw0, void *workspace0, size_t workspace0_bytes,
+                          int H0, int W0, const void *x1, const void *gy1, void *dw1, void *workspace1,
+                          size_t workspace1_bytes, int H1, int W1, int B, int C, int K, int dtype, void *stream);
+
 /* Adaptive average pooling x[B,H,W,C] -> y[B,h,w,C]; bin i covers [floor(i*H/h), ceil((i+1)*H/h)).
  * Replaces F.adaptive_avg_pool2d at conv_block.py:16 and the launch at avgpool_triton.py:225-229
  * (kernel :14-107; integer bin arithmetic here instead of the fp16 one at :42-47). */

@@ -33,6 +33,7 @@ _SIGS = {
     "pdw_dwconv_dgrad_addpool": (c_int, [c_void_p] * 4 + _CONV + [c_int, c_int, c_int, c_void_p]),
     "pdw_dwconv_wgrad_workspace_bytes": (c_size_t, _CONV + [c_int]),
     "pdw_dwconv_wgrad": (c_int, [c_void_p] * 4 + [c_size_t] + _CONV + [c_int, c_void_p]),
+    "pdw_dwconv_wgrad_pair": (c_int, ([c_void_p] * 4 + [c_size_t] + [c_int] * 2) * 2 + [c_int] * 4 + [c_void_p]),
     "pdw_avgpool_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
     "pdw_avgpool_bwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
     "pdw_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),

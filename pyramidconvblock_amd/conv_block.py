@@ -23,7 +23,7 @@ from torch import nn
 from torch.nn import functional as F
 
 from . import _lib, ops
-from .dwconv import OptimizedDepthwiseConv2d, dwconv_dgrad, dwconv_forward, dwconv_wgrad
+from .dwconv import OptimizedDepthwiseConv2d, dwconv_dgrad, dwconv_forward, dwconv_wgrad, dwconv_wgrad_pair
 
 
 class GateFunction(torch.autograd.Function):
@@ -230,6 +230,11 @@ class ConvBlockFunction(torch.autograd.Function):
             waiting = []                                               # pooled gradients not yet added to da
             if gcs is None and _is_pair(scales):
                 gcs = ops.gate_pair_backward(convs[0], convs[1], dcat)
+            srcs = [pooled[i] if scales[i] != 1. else a for i in range(ns)]
+            if (gcs is not None and ns == 2 and w_dw[0].shape == w_dw[1].shape and w_dw[0].shape[0] == w_dw[0].shape[1]
+                    and w_dw[0].shape[0] % 2 == 1 and all(t.is_contiguous() and t.dtype == dt for t in (*srcs, *gcs))):
+                # the weight gradients of both scales in one launch (the smaller problem fills the larger one's tail)
+                grad_w_dw[0], grad_w_dw[1] = dwconv_wgrad_pair(srcs[0], gcs[0], srcs[1], gcs[1], w_dw[0].shape)
             for i in order:
                 s = scales[i]
                 w = w_dw[i].detach().to(dt).contiguous()
@@ -244,7 +249,8 @@ class ConvBlockFunction(torch.autograd.Function):
                     gc = ops.bilinear_gate_backward(c, dslice)
                 else:
                     gc = ops.gate_backward(c, dslice)
-                grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo)
+                if grad_w_dw[i] is None:
+                    grad_w_dw[i] = dwconv_wgrad(src, gc, w.shape, *geo)
                 if s != 1.:
                     waiting.append(dwconv_dgrad(gc, w, src.shape, *geo))
                 elif da is None:

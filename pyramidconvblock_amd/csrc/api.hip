@@ -163,6 +163,31 @@ int pdw_dwconv_wgrad(const void* x, const void* gy, void* dw, void* workspace, s
                                       (hipStream_t)stream);
 }
 
+int pdw_dwconv_wgrad_pair(const void* x0, const void* gy0, void* dw0, void* workspace0, size_t workspace0_bytes, int H0,
+                          int W0, const void* x1, const void* gy1, void* dw1, void* workspace1, size_t workspace1_bytes,
+                          int H1, int W1, int B, int C, int K, int dtype, void* stream) {
+    const int P = K / 2;
+    if (int e = check_conv("pdw_dwconv_wgrad_pair", x0, gy0, dw0, B, H0, W0, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (int e = check_conv("pdw_dwconv_wgrad_pair", x1, gy1, dw1, B, H1, W1, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (!(K & 1)) return set_error("pdw_dwconv_wgrad_pair: odd filter size needed (K=%d)", K), 1;
+    if (!dw0 || !dw1) return set_error("pdw_dwconv_wgrad_pair: null dw"), 1;
+    const size_t need0 = pdw_dwconv_wgrad_workspace_bytes(B, H0, W0, C, K, K, 1, 1, P, P, 1, 1, dtype);
+    const size_t need1 = pdw_dwconv_wgrad_workspace_bytes(B, H1, W1, C, K, K, 1, 1, P, P, 1, 1, dtype);
+    if (!workspace0 || workspace0_bytes < need0 || !workspace1 || workspace1_bytes < need1)
+        return set_error("pdw_dwconv_wgrad_pair: workspaces of %zu and %zu bytes given, %zu and %zu needed",
+                         workspace0_bytes, workspace1_bytes, need0, need1), 1;
+    if (B > 0) {
+        const int r = dwconv_wgrad_pair_launch(x0, gy0, dw0, workspace0, H0, W0, x1, gy1, dw1, workspace1, H1, W1, B, C,
+                                               K, P, P, dtype, (hipStream_t)stream);
+        if (r != -1) return r;
+    }
+    if (int e = pdw_dwconv_wgrad(x0, gy0, dw0, workspace0, workspace0_bytes, B, H0, W0, C, K, K, 1, 1, P, P, 1, 1, dtype,
+                                 stream))
+        return e;
+    return pdw_dwconv_wgrad(x1, gy1, dw1, workspace1, workspace1_bytes, B, H1, W1, C, K, K, 1, 1, P, P, 1, 1, dtype,
+                            stream);
+}
+
 int pdw_avgpool_fwd(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
     if (int e = check_resample("pdw_avgpool_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
     return avgpool_fwd_launch(x, y, B, H, W, C, h, w, dtype, (hipStream_t)stream);

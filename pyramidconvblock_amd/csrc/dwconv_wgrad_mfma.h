@@ -48,9 +48,23 @@ struct WgradMfmaShape {
     static constexpr int NTILE = NUB * NVG * 2;    // accumulator tiles (4 registers each) per lane
 };
 
+// One launch can hold two independent problems of the same filter size (the two resolutions of a pyramid block):
+// workgroups from `first1` on work on problem 1.  Its workgroups start as compute units finish their workgroup of
+// problem 0, so the second problem fills the first one's tail instead of paying a launch, a ramp and a tail of its
+// own.  A single problem is first1 = gridDim.x.
 template <typename T, int K, int NWV>
-__global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __restrict__ x, const T* __restrict__ gy,
-                                                                   float* __restrict__ part, const WgradMfmaGeom g) {
+__global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __restrict__ x0, const T* __restrict__ gy0,
+                                                                   float* __restrict__ part0, const WgradMfmaGeom g0,
+                                                                   const T* __restrict__ x1, const T* __restrict__ gy1,
+                                                                   float* __restrict__ part1, const WgradMfmaGeom g1,
+                                                                   const unsigned first1) {
+    const bool second = blockIdx.x >= first1;  // uniform
+    const T* __restrict__ x = second ? x1 : x0;
+    const T* __restrict__ gy = second ? gy1 : gy0;
+    float* __restrict__ part = second ? part1 : part0;
+    const WgradMfmaGeom g = second ? g1 : g0;
+    const unsigned my_block = second ? blockIdx.x - first1 : blockIdx.x;
+    const unsigned my_blocks = second ? gridDim.x - first1 : first1;
     using Sh = WgradMfmaShape<K>;
     constexpr int V = 8, NT = NWV * 64, CS = Sh::CS, NUB = Sh::NUB, NVG = Sh::NVG, NTILE = Sh::NTILE;
     constexpr int NPX = 6, NPG = 4;  // staging passes of the x / gy windows requested at once (more: staged directly)
@@ -63,7 +77,7 @@ __global__ __launch_bounds__(NWV * 64, 1) void dwconv_wgrad_mfma_k(const T* __re
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it branches uniformly
-    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int bid = xcd_remap(my_block, my_blocks);
     const int sl = bid % g.slices, chunk = bid / g.slices;
     const int c0 = sl * CS;
     const int tiles_per_img = g.tiles_h * g.tiles_w;
@@ -302,9 +316,34 @@ static int wgrad_mfma_launch_t(const void* x, const void* gy, void* dw, void* ws
         attr_done = true;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)p.nblocks), dim3(NWV * 64), p.lds, s, (const T*)x, (const T*)gy, (float*)ws,
-                       p.g);
+                       p.g, (const T*)x, (const T*)gy, (float*)ws, p.g, (unsigned)p.nblocks);
     if (int e = check_launch("dwconv_wgrad_mfma")) return e;
     return wgrad_reduce_launch<T>((const float*)ws, dw, p.g.nchunks, K * K * C, s);
+}
+
+// Two problems (same batch, channels and filter size, different extents) in one launch; -1: not covered.
+template <typename T, int K>
+static int wgrad_mfma_pair_launch_t(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                                    const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                                    hipStream_t s) {
+    constexpr int NWV = 8;
+    for (const void* ptr : {xa, gya, xb, gyb})
+        if (reinterpret_cast<uintptr_t>(ptr) & 15) return -1;
+    const WgradMfmaPlan pa = plan_wgrad_mfma<T, K, NWV>(B, Ha, Wa, C, PH, PW);
+    const WgradMfmaPlan pb = plan_wgrad_mfma<T, K, NWV>(B, Hb, Wb, C, PH, PW);
+    if (!pa.ok || !pb.ok || pa.nblocks % 8 != 0) return -1;  // a multiple of 8: problem 1 keeps its XCD mapping
+    auto kern = dwconv_wgrad_mfma_k<T, K, NWV>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(pa.nblocks + pb.nblocks)), dim3(NWV * 64), pa.lds > pb.lds ? pa.lds : pb.lds,
+                       s, (const T*)xa, (const T*)gya, (float*)wsa, pa.g, (const T*)xb, (const T*)gyb, (float*)wsb, pb.g,
+                       (unsigned)pa.nblocks);
+    if (int e = check_launch("dwconv_wgrad_mfma pair")) return e;
+    if (int e = wgrad_reduce_launch<T>((const float*)wsa, dwa, pa.g.nchunks, K * K * C, s)) return e;
+    return wgrad_reduce_launch<T>((const float*)wsb, dwb, pb.g.nchunks, K * K * C, s);
 }
 
 }  // namespace pdw

@@ -18,4 +18,14 @@ int dwconv_wgrad_mfma_k3(const void* x, const void* gy, void* dw, void* ws, int 
     return -1;
 }
 
+int dwconv_wgrad_mfma_pair_k3(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s) {
+    if (dtype == kF16)
+        return wgrad_mfma_pair_launch_t<f16_t, 3>(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, s);
+    if (dtype == kBF16)
+        return wgrad_mfma_pair_launch_t<bf16_t, 3>(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, s);
+    return -1;
+}
+
 }  // namespace pdw

@@ -58,6 +58,31 @@ size_t dwconv_wgrad_mfma_ws_k17(int B, int H, int W, int C, int PH, int PW, int 
 int dwconv_wgrad_mfma_k17(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int PH,
                             int PW, int dtype, hipStream_t s);
 
+int dwconv_wgrad_mfma_pair_k3(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k5(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k7(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k9(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k11(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k13(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k15(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+int dwconv_wgrad_mfma_pair_k17(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                               const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
+                               int dtype, hipStream_t s);
+
 // Matrix-core variant (16-bit types): workspace bytes (0 = not covered) and launch (-1 = not covered).
 static bool wgrad_mfma_enabled(int dtype) {
     if (dtype == kF32) return false;
@@ -90,6 +115,25 @@ static int wgrad_mfma_launch(const void* x, const void* gy, void* dw, void* ws, 
         case 13: return dwconv_wgrad_mfma_k13(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
         case 15: return dwconv_wgrad_mfma_k15(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
         case 17: return dwconv_wgrad_mfma_k17(x, gy, dw, ws, B, H, W, C, PH, PW, dtype, s);
+        default: return -1;
+    }
+}
+
+// Two weight gradients of the same filter size, batch and channel count in one matrix-core launch (stride 1,
+// dilation 1, square filter); -1 when that kernel does not cover both, and the caller runs them one by one.
+int dwconv_wgrad_pair_launch(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                             const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int K, int PH, int PW,
+                             int dtype, hipStream_t s) {
+    if (!wgrad_mfma_enabled(dtype) || getenv("PDW_NO_WGRAD_PAIR")) return -1;
+    switch (K) {
+        case 3: return dwconv_wgrad_mfma_pair_k3(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 5: return dwconv_wgrad_mfma_pair_k5(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 7: return dwconv_wgrad_mfma_pair_k7(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 9: return dwconv_wgrad_mfma_pair_k9(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 11: return dwconv_wgrad_mfma_pair_k11(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 13: return dwconv_wgrad_mfma_pair_k13(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 15: return dwconv_wgrad_mfma_pair_k15(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
+        case 17: return dwconv_wgrad_mfma_pair_k17(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
         default: return -1;
     }
 }

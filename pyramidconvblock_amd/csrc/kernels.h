@@ -41,6 +41,9 @@ int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int
 size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype);
 int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int KH,
                               int KW, int PH, int PW, int dtype, hipStream_t s);
+int dwconv_wgrad_pair_launch(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
+                             const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int K, int PH, int PW,
+                             int dtype, hipStream_t s);
 
 // resample.hip: adaptive average pool, bilinear resize, gate
 int avgpool_fwd_launch(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, hipStream_t s);

@@ -95,6 +95,35 @@ def dwconv_wgrad(x, gy, w_shape, stride, padding, dilation):
     return dw
 
 
+def dwconv_wgrad_pair(x0, gy0, x1, gy1, w_shape):
+    """The weight gradients of two 'same' convolutions (stride 1, padding k // 2) with filters of one odd square
+    shape `w_shape` on tensors of different extents, as one call of the library: (dw0, dw1)."""
+    dev = _lib.require_device(x0, gy0, x1, gy1)
+    L = _lib.lib()
+    K, C = int(w_shape[0]), int(w_shape[2])
+    B = x0.shape[0]
+    if (w_shape[0] != w_shape[1] or K % 2 == 0 or x0.shape != gy0.shape or x1.shape != gy1.shape or x1.shape[0] != B
+            or x0.shape[3] != C or x1.shape[3] != C or x1.dtype != x0.dtype):
+        raise ValueError("dwconv_wgrad_pair: two same-padded convolutions with one odd square filter shape needed")
+    dws = [torch.empty(tuple(w_shape), device=dev, dtype=x0.dtype) for _ in range(2)]
+    if x0.numel() == 0 or x1.numel() == 0:
+        geo = ((1, 1), (K // 2, K // 2), (1, 1))
+        return dwconv_wgrad(x0, gy0, w_shape, *geo), dwconv_wgrad(x1, gy1, w_shape, *geo)
+    code = _lib.dtype_code(x0.dtype)
+    wss = []
+    for x in (x0, x1):
+        nbytes = L.pdw_dwconv_wgrad_workspace_bytes(B, x.shape[1], x.shape[2], C, K, K, 1, 1, K // 2, K // 2, 1, 1, code)
+        wss.append(torch.empty(max(nbytes, 4) // 4 + 1, device=dev, dtype=torch.float32))
+    with _lib.on_device(dev):
+        _lib.check(L.pdw_dwconv_wgrad_pair(x0.data_ptr(), gy0.data_ptr(), dws[0].data_ptr(), wss[0].data_ptr(),
+                                           wss[0].numel() * 4, x0.shape[1], x0.shape[2], x1.data_ptr(), gy1.data_ptr(),
+                                           dws[1].data_ptr(), wss[1].data_ptr(), wss[1].numel() * 4, x1.shape[1],
+                                           x1.shape[2], B, C, K, code, _lib.stream_ptr(dev)), "pdw_dwconv_wgrad_pair")
+    for ws in wss:
+        _lib.keep_until_flush(ws)
+    return dws[0], dws[1]
+
+
 class DepthwiseConv2DFunction(torch.autograd.Function):
     """apply(input[B,H,W,C], weight[k1,k2,C], stride, padding, dilation, dtype) -> output[B,OH,OW,C] of `dtype`.
 

@@ -109,6 +109,28 @@ def test_wgrad_is_deterministic():
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("case", [(32, 56, 56, 28, 28, 64, 13), (2, 20, 24, 10, 12, 40, 9), (3, 9, 11, 17, 5, 8, 3),
+                                  (1, 30, 30, 15, 15, 16, 17)])
+def test_wgrad_pair_is_the_two_separate_calls(dtype, case):
+    """pdw_dwconv_wgrad_pair (two problems in one launch for 16-bit types, two launches otherwise) gives bitwise
+    the results of two pdw_dwconv_wgrad calls, immediately and with the summations deferred."""
+    from pyramidconvblock_amd import _lib
+    from pyramidconvblock_amd.dwconv import dwconv_wgrad, dwconv_wgrad_pair
+
+    B, H0, W0, H1, W1, C, k = case
+    gen = torch.Generator().manual_seed(7)
+    t = [randn(gen, B, H, W, C).to(dtype).cuda() for H, W in ((H0, W0), (H0, W0), (H1, W1), (H1, W1))]
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    want = [dwconv_wgrad(t[0], t[1], (k, k, C), *geo), dwconv_wgrad(t[2], t[3], (k, k, C), *geo)]
+    got = dwconv_wgrad_pair(t[0], t[1], t[2], t[3], (k, k, C))
+    with _lib.deferred_reductions(t[0].device):
+        later = dwconv_wgrad_pair(t[0], t[1], t[2], t[3], (k, k, C))
+    torch.cuda.synchronize()
+    for w, g, l in zip(want, got, later):
+        assert torch.equal(w, g) and torch.equal(w, l)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_full_size_properties(dtype):
     """Size-independent checks at the benchmark shape: delta kernel = identity, linearity in w,
