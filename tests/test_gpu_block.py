@@ -54,3 +54,48 @@ def test_config4_fp16(oracle):
 @pytest.mark.parametrize("k", [9, 15])
 def test_config5_ragged(oracle, dtype, k):
     _block_case(oracle, 200, k, (3, 57, 61, 200), dtype, dist="uniform")
+
+
+@pytest.mark.parametrize("case", [
+    (128, 13, (1, 8, 8, 128), torch.bfloat16),     # one image, a few rows per dense launch
+    (128, 9, (3, 10, 14, 128), torch.float16),     # extents not multiples of 4
+    (128, 3, (2, 4, 6, 128), torch.bfloat16),      # pooled map of 2 x 3
+    (128, 13, (2, 58, 62, 128), torch.bfloat16),   # wider than a conv tile
+    (64, 7, (5, 12, 12, 64), torch.bfloat16),      # layer widths without the paired dense launch
+    (256, 5, (2, 8, 8, 256), torch.bfloat16),      # layer widths the dense kernels leave to the BLAS library
+    (128, 11, (2, 16, 16, 128), torch.float32),
+])
+def test_small_and_odd_even_extents(oracle, case):
+    """Even extents take the fused two-scale path (paired launches, deferred summations); small and unusual
+    sizes exercise its tails, partial tiles and fallbacks."""
+    dim, k, shape, dtype = case
+    _block_case(oracle, dim, k, shape, dtype)
+
+
+@pytest.mark.parametrize("bias", [(True, True), (True, False), (False, False)])
+def test_bias_combinations(oracle, bias):
+    import pyramid_dwconv
+
+    torch.manual_seed(3)
+    dtype = torch.bfloat16
+    m = pyramid_dwconv.ConvBlock(dim=128, bias=bias[0], out_bias=bias[1], kernel_size=9)
+    with torch.no_grad():
+        for n, p in m.named_parameters():
+            if n.endswith("bias"):
+                p.normal_(0, 0.5)   # the default initialisation leaves some of them at zero
+    gen = torch.Generator().manual_seed(3)
+    shape = (3, 12, 16, 128)
+    x, g = randn(gen, *shape).to(dtype), randn(gen, *shape).to(dtype)
+    m = m.to(dtype)
+    params = {n: p.detach().double().numpy() for n, p in m.state_dict().items()}
+    yo, cache = oracle.convblock_fwd(x.double().numpy(), params)
+    dxo, go = oracle.convblock_bwd(cache, g.double().numpy())
+    m = m.cuda()
+    xd = x.cuda().requires_grad_()
+    y = m(xd)
+    assert_close(y, yo, dtype, "y")
+    torch.autograd.backward(y, g.cuda())
+    assert_close(xd.grad, dxo, dtype, "dx")
+    for n, p in m.named_parameters():
+        assert p.grad is not None, n
+        assert_close(p.grad, go[n], dtype, "grad " + n)
