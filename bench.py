@@ -159,6 +159,9 @@ def kernel_rooflines(B, H, W, D, k, dtype):
          2.0 * N * D * I),
         ("dense_wgrad", lambda i: ops.dense_wgrad(a[i % 4], xin[i % 4]), 4, es * (N * D + N * I + D * I),
          2.0 * N * D * I),
+        # both gradients of conv_up as the block's backward runs them: one launch, gy read once
+        ("dense_bwd_pair", lambda i: ops.dense_backward_pair(a[i % 4], wup, xin[i % 4]), 4,
+         es * (2 * N * D + N * I + 2 * D * I), 4.0 * N * D * I),
     ):
         t = time_kernel_events(fn, nb_)
         out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=fl))
@@ -168,7 +171,7 @@ def kernel_rooflines(B, H, W, D, k, dtype):
 def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     """Launches one hot kernel `iters` times at its shape inside the headline block (for rocprofv3 runs).
     name: {fwd,dgrad,wgrad}_{full,half} | avgpool_fwd | avgpool_bwd | bilinear_fwd | bilinear_bwd |
-    dense_{fwd,dgrad,wgrad} (the conv_up layer: [N,D] <-> [N,D/2])"""
+    dense_{fwd,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pair = both gradients in one launch)"""
     from pyramidconvblock_amd import avgpool, dwconv, up
 
     I, G = D // 2, D // 4
@@ -196,7 +199,8 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         rb = torch.randn(B, D, device="cuda")
         fn = {"fwd": lambda: ops.dense_forward(xin, wup),
               "dgrad": lambda: ops.dense_forward(ain, wup, w_kmajor=True, rowbias=rb, rows_per_image=H * W),
-              "wgrad": lambda: ops.dense_wgrad(ain, xin)}[res]
+              "wgrad": lambda: ops.dense_wgrad(ain, xin),
+              "pair": lambda: ops.dense_backward_pair(ain, wup, xin, rowbias=rb, rows_per_image=H * W)}[res]
     else:
         a = torch.randn(B, H, W, I, device="cuda").to(dtype)
         p = torch.randn(B, h, w, I, device="cuda").to(dtype)
