@@ -264,17 +264,30 @@ static WgradMfmaPlan plan_wgrad_mfma(int B, int H, int W, int C, int PH, int PW)
     if (getenv("PDW_WG_XP") && atoi(getenv("PDW_WG_XP")) >= g.TW / 2 + 4 * Sh::NVG) g.XP = atoi(getenv("PDW_WG_XP"));
     if (getenv("PDW_WG_GP") && atoi(getenv("PDW_WG_GP")) >= g.TW / 2) g.GP = atoi(getenv("PDW_WG_GP"));
     auto lds_of = [&](int th) { return ((size_t)(th + K - 1) * Sh::CS * g.XP + (size_t)th * (Sh::CS * g.GP + 1)) * 4; };
-    // tile height: about one tile per CU, within LDS and the staging registers
-    long long want_h = ((long long)B * g.slices * g.tiles_w + 255) / 256;  // images*slices per CU column
-    int tiles_h = (int)(256 / ((long long)B * g.slices * g.tiles_w > 0 ? (long long)B * g.slices * g.tiles_w : 1));
-    (void)want_h;
+    // tile height: about one tile per CU, within LDS.  Where LDS forces lower tiles than that, the count of tile
+    // rows is chosen for the shortest run: rounds of tiles per workgroup times (tile rows + 66), the 66 being what a
+    // tile costs beside its rows (halo, staging latency, the final sum), fitted to measurements at K = 13 and 17.
+    const long long per_row = (long long)B * g.slices * g.tiles_w;  // tiles per row of tiles, all slices
+    int tiles_h = (int)(256 / (per_row > 0 ? per_row : 1));
     if (getenv("PDW_WG_TILEMUL")) tiles_h *= atoi(getenv("PDW_WG_TILEMUL"));
     if (tiles_h < 1) tiles_h = 1;
     if (tiles_h > g.OH) tiles_h = g.OH;
     int th = cdiv(g.OH, tiles_h);
     if (th < 4) th = g.OH < 4 ? g.OH : 4;
-    while (th > 1 && lds_of(th) > 150 * 1024) --th;
-    if (lds_of(th) > 150 * 1024) return p;
+    if (lds_of(th) > 150 * 1024) {
+        while (th > 1 && lds_of(th) > 150 * 1024) --th;
+        if (lds_of(th) > 150 * 1024) return p;
+        const int first = cdiv(g.OH, th);
+        const int cap_s = 256 / g.slices > 1 ? 256 / g.slices : 1;
+        long long best = -1;
+        for (int cand = first; cand <= 2 * first + 2 && cand <= g.OH; ++cand) {
+            const int thc = cdiv(g.OH, cand);
+            if (thc < 4 || lds_of(thc) > 150 * 1024) continue;
+            const long long rounds = cdiv((long long)B * cdiv(g.OH, thc) * g.tiles_w, (long long)cap_s);
+            const long long cost = rounds * (thc + 66);
+            if (best < 0 || cost < best) best = cost, th = thc;
+        }
+    }
     g.TH = th;
     g.tiles_h = cdiv(g.OH, th);
     const long long ntiles = (long long)B * g.tiles_h * g.tiles_w;
