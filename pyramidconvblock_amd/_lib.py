@@ -113,7 +113,13 @@ def require_device(*tensors: torch.Tensor) -> torch.device:
     return dev
 
 
+_scope = threading.local()
+
+
 def stream_ptr(dev: torch.device) -> int:
+    held = getattr(_scope, "held", None)
+    if held is not None and held[0] == dev:
+        return held[1]
     return torch.cuda.current_stream(dev).cuda_stream
 
 
@@ -124,6 +130,9 @@ class on_device:
         self.dev, self.prev = dev, None
 
     def __enter__(self):
+        held = getattr(_scope, "held", None)
+        if held is not None and held[0] == self.dev:
+            return self  # launch_scope made it current
         idx = self.dev.index if self.dev.index is not None else torch.cuda.current_device()
         cur = torch.cuda.current_device()
         if idx != cur:
@@ -134,6 +143,29 @@ class on_device:
     def __exit__(self, *exc):
         if self.prev is not None:
             torch.cuda.set_device(self.prev)
+        return False
+
+
+class launch_scope:
+    """A run of launches on one device from one host thread (an autograd node's forward or backward): `dev` is made
+    current and its current stream looked up once instead of per launch.  The stream must not be switched inside."""
+
+    def __init__(self, dev: torch.device):
+        self.dev = dev
+        self.guard = on_device(dev)
+        self.outer = None
+
+    def __enter__(self):
+        self.outer = getattr(_scope, "held", None)
+        _scope.held = None
+        self.guard.__enter__()
+        _scope.held = (self.dev, torch.cuda.current_stream(self.dev).cuda_stream)
+        return self
+
+    def __exit__(self, *exc):
+        _scope.held = None
+        self.guard.__exit__(*exc)
+        _scope.held = self.outer
         return False
 
 

@@ -96,6 +96,16 @@ class ConvBlockFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, *w_dw):
+        with _lib.launch_scope(_lib.require_device(x)):  # one device and stream look-up for all launches
+            return ConvBlockFunction._forward(ctx, x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, *w_dw)
+
+    @staticmethod
+    def backward(ctx, gy):
+        with _lib.launch_scope(_lib.require_device(gy)):
+            return ConvBlockFunction._backward(ctx, gy)
+
+    @staticmethod
+    def _forward(ctx, x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, *w_dw):
         dev = _lib.require_device(x)
         x = x.detach().contiguous()
         B, H, W, D = x.shape
@@ -167,7 +177,7 @@ class ConvBlockFunction(torch.autograd.Function):
         return y
 
     @staticmethod
-    def backward(ctx, gy):
+    def _backward(ctx, gy):
         scales = ctx.scales
         ns = len(scales)
         saved = ctx.saved_tensors
