@@ -258,6 +258,30 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
                        size_t workspace_bytes, const float *rowbias, int P, long long N, int O, int I, int dtype,
                        void *stream);
 
+/* The whole block of conv_block.py:25-49 (scales (1, 1/2), conv_up without bias) as one host call each way: the
+ * launch sequence of the entry points above (5 launches forward; 6 launches and one summation launch backward)
+ * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
+ * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense
+ * kernels and pdw_dense_bwd_pair cover (D = 128, I = 64), odd K.  All tensors channels-last and contiguous, all
+ * parameters in `dtype`: x, y[B,H,W,D]; w_up[I,D]; w_dw0, w_dw1[K,K,I]; w_pool[D,D]; w_out[D,I]; b_pool, b_out[D] or
+ * NULL.  The forward writes what the backward reads again: a = conv_up(x), c0 = conv(a), xp = pool(a)[B,H/2,W/2,I],
+ * c1 = conv(xp), cat[B,H,W,I] (the gated scales), m[B,D] (per-image mean of x).  The backward overwrites dx and the
+ * parameter gradients (gb_pool, gb_out may be NULL).  Workspaces: device scratch of the stated size, free for reuse
+ * when the call's work on `stream` is done.  Results are bitwise those of the separate calls.
+ * Replaces the Python-level sequence of ConvBlock.forward, conv_block.py:36-49, and its autograd backward. */
+int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype);
+size_t pdw_convblock_fwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype);
+int pdw_convblock_fwd(const void *x, const void *w_up, const void *w_dw0, const void *w_dw1, const void *w_pool,
+                      const void *b_pool, const void *w_out, const void *b_out, void *a, void *c0, void *xp, void *c1,
+                      void *cat, void *m, void *y, void *workspace, size_t workspace_bytes, int B, int H, int W,
+                      int D, int I, int K, int dtype, void *stream);
+size_t pdw_convblock_bwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype);
+int pdw_convblock_bwd(const void *gy, const void *x, const void *a, const void *c0, const void *xp, const void *c1,
+                      const void *cat, const void *m, const void *w_up, const void *w_dw0, const void *w_dw1,
+                      const void *w_pool, const void *w_out, void *dx, void *gw_up, void *gw_dw0, void *gw_dw1,
+                      void *gw_pool, void *gb_pool, void *gw_out, void *gb_out, void *workspace,
+                      size_t workspace_bytes, int B, int H, int W, int D, int I, int K, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

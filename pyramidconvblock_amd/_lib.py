@@ -34,6 +34,11 @@ _SIGS = {
     "pdw_dwconv_wgrad_workspace_bytes": (c_size_t, _CONV + [c_int]),
     "pdw_dwconv_wgrad": (c_int, [c_void_p] * 4 + [c_size_t] + _CONV + [c_int, c_void_p]),
     "pdw_dwconv_wgrad_pair": (c_int, ([c_void_p] * 4 + [c_size_t] + [c_int] * 2) * 2 + [c_int] * 4 + [c_void_p]),
+    "pdw_convblock_supported": (c_int, [c_int] * 7),
+    "pdw_convblock_fwd_workspace_bytes": (c_size_t, [c_int] * 7),
+    "pdw_convblock_fwd": (c_int, [c_void_p] * 16 + [c_size_t] + [c_int] * 7 + [c_void_p]),
+    "pdw_convblock_bwd_workspace_bytes": (c_size_t, [c_int] * 7),
+    "pdw_convblock_bwd": (c_int, [c_void_p] * 22 + [c_size_t] + [c_int] * 7 + [c_void_p]),
     "pdw_avgpool_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
     "pdw_avgpool_bwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),
     "pdw_bilinear_fwd": (c_int, [c_void_p] * 2 + [c_int] * 8 + [c_void_p]),

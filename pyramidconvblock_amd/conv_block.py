@@ -85,6 +85,23 @@ def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
     return torch.bmm(a, b).float().sum(0)
 
 
+def _block_call_ok(x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, w_dw) -> bool:
+    """Whether pdw_convblock_fwd / _bwd cover this call: scales (1, 1/2), no conv_up bias, everything contiguous and
+    of x's 16-bit dtype, one odd square depthwise filter shape, and shapes the library accepts."""
+    if _os.environ.get("PDW_BLOCK_STEPWISE") or b_up is not None or tuple(scales) != (1., 0.5) or x.dim() != 4:
+        return False
+    dt = x.dtype
+    tensors = [w_up, w_out, w_pool, *w_dw] + [b for b in (b_out, b_pool) if b is not None]
+    if len(w_dw) != 2 or any(t.dtype != dt or not t.is_contiguous() or t.device != x.device for t in tensors):
+        return False
+    B, H, W, D = x.shape
+    I, K = w_up.shape[0], w_dw[0].shape[0]
+    if (dt not in (torch.float16, torch.bfloat16) or tuple(w_up.shape) != (I, D) or tuple(w_out.shape) != (D, I)
+            or tuple(w_pool.shape) != (D, D) or any(tuple(w.shape) != (K, K, I) for w in w_dw)):
+        return False
+    return bool(_lib.lib().pdw_convblock_supported(B, H, W, D, I, K, _lib.dtype_code(dt)))
+
+
 def _is_pair(scales) -> bool:
     return len(scales) == 2 and scales[0] == 1. and scales[1] != 1.
 
@@ -111,6 +128,29 @@ class ConvBlockFunction(torch.autograd.Function):
         B, H, W, D = x.shape
         dt = x.dtype
         I = w_up.shape[0]
+        ctx.block_call = None
+        if _block_call_ok(x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, w_dw):
+            # the whole launch sequence below as one call of the library (same kernels, same order, same results)
+            K = w_dw[0].shape[0]
+            L, code = _lib.lib(), _lib.dtype_code(dt)
+            new = lambda *shape: torch.empty(shape, device=dev, dtype=dt)
+            a, c0, cat = new(B, H, W, I), new(B, H, W, I), new(B, H, W, I)
+            xp, c1 = new(B, H // 2, W // 2, I), new(B, H // 2, W // 2, I)
+            m, y = new(B, D), new(B, H, W, D)
+            ws = torch.empty(L.pdw_convblock_fwd_workspace_bytes(B, H, W, D, I, K, code) // 4 + 1, device=dev,
+                             dtype=torch.float32)
+            _lib.check(L.pdw_convblock_fwd(x.data_ptr(), w_up.data_ptr(), w_dw[0].data_ptr(), w_dw[1].data_ptr(),
+                                           w_pool.data_ptr(), b_pool.data_ptr() if b_pool is not None else None,
+                                           w_out.data_ptr(), b_out.data_ptr() if b_out is not None else None,
+                                           a.data_ptr(), c0.data_ptr(), xp.data_ptr(), c1.data_ptr(), cat.data_ptr(),
+                                           m.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel() * 4, B, H, W, D, I, K,
+                                           code, _lib.stream_ptr(dev)), "pdw_convblock_fwd")
+            ctx.block_call = (B, H, W, D, I, K, code)
+            ctx.fast = (True, True)
+            ctx.scales = tuple(scales)
+            ctx.has_bias = (False, b_out is not None, b_pool is not None)
+            ctx.save_for_backward(x, a, cat, m, w_up, w_out, w_pool, *w_dw, c0, c1, xp)
+            return y
         fast_up = (ops.dense_supported(D, I, dt) and ops.dense_supported(I, D, dt) and w_up.dtype == dt
                    and (b_up is None or b_up.dtype == dt))
         same_dt = w_pool.dtype == dt and all(b is None or b.dtype == dt for b in (b_pool, b_out))
@@ -193,6 +233,25 @@ class ConvBlockFunction(torch.autograd.Function):
         N = B * H * W
         gy = gy.to(dt).contiguous()
         g2d = gy.view(N, D)
+        if ctx.block_call is not None:
+            dev = gy.device
+            L = _lib.lib()
+            shape = ctx.block_call
+            like = lambda t: torch.empty_like(t, memory_format=torch.contiguous_format)
+            dx, gw_up, gw_out, gw_pool = like(x), like(w_up), like(w_out), like(w_pool)
+            gw_dw = [like(w_dw[0]), like(w_dw[1])]
+            gb_out = torch.empty(D, device=dev, dtype=dt) if ctx.has_bias[1] else None
+            gb_pool = torch.empty(D, device=dev, dtype=dt) if ctx.has_bias[2] else None
+            ws = torch.empty(L.pdw_convblock_bwd_workspace_bytes(*shape) // 4 + 1, device=dev, dtype=torch.float32)
+            _lib.check(L.pdw_convblock_bwd(gy.data_ptr(), x.data_ptr(), a.data_ptr(), convs[0].data_ptr(),
+                                           pooled[1].data_ptr(), convs[1].data_ptr(), cat.data_ptr(), m.data_ptr(),
+                                           w_up.data_ptr(), w_dw[0].data_ptr(), w_dw[1].data_ptr(), w_pool.data_ptr(),
+                                           w_out.data_ptr(), dx.data_ptr(), gw_up.data_ptr(), gw_dw[0].data_ptr(),
+                                           gw_dw[1].data_ptr(), gw_pool.data_ptr(),
+                                           gb_pool.data_ptr() if gb_pool is not None else None, gw_out.data_ptr(),
+                                           gb_out.data_ptr() if gb_out is not None else None, ws.data_ptr(),
+                                           ws.numel() * 4, *shape, _lib.stream_ptr(dev)), "pdw_convblock_bwd")
+            return (dx, None, gw_up, None, gw_out, gb_out, gw_pool, gb_pool, *gw_dw)
 
         fast_up, fast_out = ctx.fast
         pool_fast = w_pool.dtype == dt and B > 0

@@ -1,0 +1,179 @@
+// The pyramid block of conv_block.py:25-49 as one host call each way: the launch sequence that the Python operator
+// makes through the single entry points (5 launches forward, 7 backward), for callers that cannot afford an
+// interpreter between launches.  Host code only: every step is one of the library's own entry points, in the order
+// and with the arguments of pyramidconvblock_amd/conv_block.py, so the results are bitwise the same.
+#include <stdint.h>
+
+#include "../../include/pdw.h"
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+using namespace pdw;
+
+size_t up256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// Hands out 256-byte aligned pieces of the caller's workspace.
+struct Carver {
+    char* p;
+    size_t left;
+    bool ok = true;
+    void* take(size_t bytes) {
+        bytes = up256(bytes);
+        if (bytes > left) {
+            ok = false;
+            return nullptr;
+        }
+        void* r = p;
+        p += bytes, left -= bytes;
+        return r;
+    }
+};
+
+struct Shape {
+    int B, H, W, D, I, K, dtype;
+    int h, w, P, R, es;
+    long long N, nt;  // rows of the dense layers, row tiles (chunk sums)
+};
+
+Shape shape_of(int B, int H, int W, int D, int I, int K, int dtype) {
+    Shape s{B, H, W, D, I, K, dtype, H / 2, W / 2, H * W, pdw_dense_colsum_rows(), 2, 0, 0};
+    s.N = (long long)B * H * W;
+    s.nt = (s.N + s.R - 1) / s.R;
+    return s;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype) {
+    if (dtype != kF16 && dtype != kBF16) return 0;
+    if (B < 1 || H < 4 || W < 4 || (H & 1) || (W & 1) || K < 1 || !(K & 1) || D < 8 || I < 16 || (I & 15)) return 0;
+    if ((long long)B * H * W * (D > I ? D : I) > 0x7fffffffLL) return 0;
+    if ((H * W) % pdw_dense_colsum_rows()) return 0;
+    return pdw_dense_supported(D, I, dtype) && pdw_dense_supported(I, D, dtype) && pdw_dense_colsum_supported(D, I, dtype) &&
+           pdw_dense_bwd_pair_supported(D, I, dtype) && pdw_dense_bwd_pair_supported(I, D, dtype);
+}
+
+size_t pdw_convblock_fwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
+    if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
+    const Shape s = shape_of(B, H, W, D, I, K, dtype);
+    return up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4);
+}
+
+int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const void* w_dw1, const void* w_pool,
+                      const void* b_pool, const void* w_out, const void* b_out, void* a, void* c0, void* xp, void* c1,
+                      void* cat, void* m, void* y, void* workspace, size_t workspace_bytes, int B, int H, int W, int D,
+                      int I, int K, int dtype, void* stream) {
+    if (!pdw_convblock_supported(B, H, W, D, I, K, dtype))
+        return set_error("pdw_convblock_fwd: shape not covered (B=%d H=%d W=%d D=%d I=%d K=%d dtype=%d)", B, H, W, D, I, K,
+                         dtype), 1;
+    for (const void* ptr : {x, w_up, w_dw0, w_dw1, w_pool, w_out, (const void*)a, (const void*)c0, (const void*)xp,
+                            (const void*)c1, (const void*)cat, (const void*)m, (const void*)y, (const void*)workspace})
+        if (!ptr) return set_error("pdw_convblock_fwd: null pointer"), 1;
+    const Shape s = shape_of(B, H, W, D, I, K, dtype);
+    if (workspace_bytes < pdw_convblock_fwd_workspace_bytes(B, H, W, D, I, K, dtype))
+        return set_error("pdw_convblock_fwd: workspace of %zu bytes given, %zu needed", workspace_bytes,
+                         pdw_convblock_fwd_workspace_bytes(B, H, W, D, I, K, dtype)), 1;
+    Carver ws{(char*)workspace, workspace_bytes};
+    float* xparts = (float*)ws.take((size_t)s.nt * D * 4);  // sums of x over each row tile
+    float* yp = (float*)ws.take((size_t)B * D * 4);         // mean branch: one row per image
+    const int pad = K / 2;
+    // conv_up, with the tile sums of x for the mean branch                                   (conv_block.py:37, 46)
+    if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) return e;
+    // full-resolution conv, which also pools its input for the second scale                  (conv_block.py:14-16)
+    if (int e = pdw_dwconv_fwd_pool(a, w_dw0, c0, xp, B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, s.h, s.w, dtype, stream))
+        return e;
+    if (int e = pdw_dwconv_fwd(xp, w_dw1, c1, B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream)) return e;
+    // both gates into cat, mean -> conv_pool (+ both biases) into yp                          (conv_block.py:40-49)
+    if (int e = pdw_block_mid_fwd(c0, c1, cat, B, H, W, s.h, s.w, I, I, xparts, (int)(s.nt / B), w_pool, b_pool, b_out, m,
+                                  yp, s.P, D, dtype, stream))
+        return e;
+    // conv_out plus the per-image row                                                        (conv_block.py:44, 49)
+    return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
+}
+
+size_t pdw_convblock_bwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
+    if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
+    const Shape s = shape_of(B, H, W, D, I, K, dtype);
+    const int pad = K / 2;
+    const size_t full = (size_t)s.N * I * s.es, half = (size_t)B * s.h * s.w * I * s.es;
+    return up256(full) /* dcat */ + up256((size_t)s.nt * D * 4) /* gparts */ +
+           up256(pdw_dense_wgrad_workspace_bytes(s.N, D, I)) + up256(full) /* gcf */ + up256(half) /* gch */ +
+           up256((size_t)2 * D * s.es) /* gbias */ + up256((size_t)B * D * 4) /* dmean */ +
+           up256(pdw_pool_branch_workspace_bytes(B, s.P, D)) +
+           up256(pdw_dwconv_wgrad_workspace_bytes(B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, dtype)) +
+           up256(pdw_dwconv_wgrad_workspace_bytes(B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype)) +
+           up256(half) /* dxp */ + up256(full) /* da */ + up256(pdw_dense_wgrad_workspace_bytes(s.N, I, D));
+}
+
+int pdw_convblock_bwd(const void* gy, const void* x, const void* a, const void* c0, const void* xp, const void* c1,
+                      const void* cat, const void* m, const void* w_up, const void* w_dw0, const void* w_dw1,
+                      const void* w_pool, const void* w_out, void* dx, void* gw_up, void* gw_dw0, void* gw_dw1,
+                      void* gw_pool, void* gb_pool, void* gw_out, void* gb_out, void* workspace, size_t workspace_bytes,
+                      int B, int H, int W, int D, int I, int K, int dtype, void* stream) {
+    if (!pdw_convblock_supported(B, H, W, D, I, K, dtype))
+        return set_error("pdw_convblock_bwd: shape not covered (B=%d H=%d W=%d D=%d I=%d K=%d dtype=%d)", B, H, W, D, I, K,
+                         dtype), 1;
+    for (const void* ptr : {gy, x, a, c0, xp, c1, cat, m, w_up, w_dw0, w_dw1, w_pool, w_out, (const void*)dx,
+                            (const void*)gw_up, (const void*)gw_dw0, (const void*)gw_dw1, (const void*)gw_pool,
+                            (const void*)gw_out, (const void*)workspace})
+        if (!ptr) return set_error("pdw_convblock_bwd: null pointer"), 1;
+    const size_t need = pdw_convblock_bwd_workspace_bytes(B, H, W, D, I, K, dtype);
+    if (workspace_bytes < need)
+        return set_error("pdw_convblock_bwd: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
+    const Shape s = shape_of(B, H, W, D, I, K, dtype);
+    const int pad = K / 2;
+    const size_t full = (size_t)s.N * I * s.es, half = (size_t)B * s.h * s.w * I * s.es;
+    Carver ws{(char*)workspace, workspace_bytes};
+    void* dcat = ws.take(full);
+    float* gparts = (float*)ws.take((size_t)s.nt * D * 4);
+    const size_t b_po = pdw_dense_wgrad_workspace_bytes(s.N, D, I);
+    void* ws_po = ws.take(b_po);
+    void* gcf = ws.take(full);
+    void* gch = ws.take(half);
+    char* gbias = (char*)ws.take((size_t)2 * D * s.es);
+    float* dmean = (float*)ws.take((size_t)B * D * 4);
+    const size_t b_pool_ws = pdw_pool_branch_workspace_bytes(B, s.P, D);
+    void* ws_pool = ws.take(b_pool_ws);
+    const size_t b_w0 = pdw_dwconv_wgrad_workspace_bytes(B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, dtype);
+    const size_t b_w1 = pdw_dwconv_wgrad_workspace_bytes(B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype);
+    void* ws_w0 = ws.take(b_w0);
+    void* ws_w1 = ws.take(b_w1);
+    void* dxp = ws.take(half);
+    void* da = ws.take(full);
+    const size_t b_pu = pdw_dense_wgrad_workspace_bytes(s.N, I, D);
+    void* ws_pu = ws.take(b_pu);
+    if (!ws.ok) return set_error("pdw_convblock_bwd: workspace layout exceeds %zu bytes", workspace_bytes), 1;
+
+    // the final summations of all weight gradients run as one launch at the end
+    if (int e = pdw_reduce_defer_begin()) return e;
+    int e = 0;
+    do {
+        // conv_out: gradient of cat, weight gradient, and the tile sums of gy for the mean branch   (conv_block.py:44)
+        if ((e = pdw_dense_bwd_pair(gy, w_out, cat, dcat, gparts, gw_out, ws_po, up256(b_po), nullptr, 1, s.N, D, I,
+                                    dtype, stream)))
+            break;
+        // both gates and the mean branch                                                            (conv_block.py:40-49)
+        if ((e = pdw_block_mid_bwd(dcat, c0, c1, gcf, gch, B, H, W, s.h, s.w, I, I, gparts, (int)(s.nt / B), m, w_pool,
+                                   gb_out ? gb_out : (void*)gbias, gb_pool ? gb_pool : (void*)(gbias + (size_t)D * s.es),
+                                   gw_pool, dmean, ws_pool, up256(b_pool_ws), s.P, D, dtype, stream)))
+            break;
+        // depthwise convs: weight gradients of both scales, then the input gradients, pooled scale first
+        if ((e = pdw_dwconv_wgrad_pair(a, gcf, gw_dw0, ws_w0, up256(b_w0), H, W, xp, gch, gw_dw1, ws_w1, up256(b_w1), s.h,
+                                       s.w, B, I, K, dtype, stream)))
+            break;
+        if ((e = pdw_dwconv_dgrad(gch, w_dw1, dxp, B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream))) break;
+        if ((e = pdw_dwconv_dgrad_addpool(gcf, w_dw0, dxp, da, B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, s.h, s.w, dtype,
+                                          stream)))
+            break;
+        // conv_up: input gradient (plus the mean branch's per-image term) and weight gradient        (conv_block.py:37)
+        e = pdw_dense_bwd_pair(da, w_up, x, dx, nullptr, gw_up, ws_pu, up256(b_pu), dmean, s.P, s.N, I, D, dtype, stream);
+    } while (false);
+    const int f = pdw_reduce_defer_flush(stream);  // also ends the deferral after an error
+    return e ? e : f;
+}
+
+}  // extern "C"

@@ -99,3 +99,38 @@ def test_bias_combinations(oracle, bias):
     for n, p in m.named_parameters():
         assert p.grad is not None, n
         assert_close(p.grad, go[n], dtype, "grad " + n)
+
+
+@pytest.mark.parametrize("case", [(128, 13, (4, 56, 56, 128), torch.bfloat16), (128, 9, (3, 8, 16, 128), torch.float16),
+                                  (128, 3, (1, 4, 8, 128), torch.bfloat16)])
+@pytest.mark.parametrize("out_bias", [True, False])
+def test_single_call_block_is_the_stepwise_block(case, out_bias, monkeypatch):
+    """pdw_convblock_fwd / _bwd (the block's launch sequence as one library call each way) give bitwise the results
+    of the operator making the same launches one by one."""
+    import pyramid_dwconv
+    from pyramidconvblock_amd import _lib
+
+    dim, k, shape, dtype = case
+    B, H, W, D = shape
+    assert _lib.lib().pdw_convblock_supported(B, H, W, D, D // 2, k, _lib.dtype_code(dtype)) == 1
+    torch.manual_seed(5)
+    m = pyramid_dwconv.ConvBlock(dim=dim, kernel_size=k, out_bias=out_bias).to(dtype).cuda()
+    gen = torch.Generator().manual_seed(5)
+    x = randn(gen, *shape).to(dtype).cuda()
+    g = randn(gen, *shape).to(dtype).cuda()
+
+    def run():
+        for p in m.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_()
+        y = m(xi)
+        torch.autograd.backward(y, g)
+        torch.cuda.synchronize()
+        return [y.detach(), xi.grad] + [p.grad for p in m.parameters()]
+
+    single = run()
+    monkeypatch.setenv("PDW_BLOCK_STEPWISE", "1")
+    stepwise = run()
+    assert len(single) == len(stepwise)
+    for i, (s, t) in enumerate(zip(single, stepwise)):
+        assert s is not None and torch.equal(s, t), f"result {i} differs"
