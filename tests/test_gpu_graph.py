@@ -6,15 +6,16 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def test_graph_replays_match_eager():
+@pytest.mark.parametrize("dim", [64, 128])  # 128: the block runs as one library call per direction
+def test_graph_replays_match_eager(dim):
     import pyramid_dwconv
     from pyramidconvblock_amd.graphs import GraphedStep
 
     torch.manual_seed(0)
-    m = pyramid_dwconv.ConvBlock(64, kernel_size=9).to(torch.bfloat16).cuda()
+    m = pyramid_dwconv.ConvBlock(dim, kernel_size=9).to(torch.bfloat16).cuda()
     gen = torch.Generator().manual_seed(1)
-    x = torch.randn(4, 28, 30, 64, generator=gen).to(torch.bfloat16).cuda()
-    g = torch.randn(4, 28, 30, 64, generator=gen).to(torch.bfloat16).cuda()
+    x = torch.randn(4, 28, 32, dim, generator=gen).to(torch.bfloat16).cuda()
+    g = torch.randn(4, 28, 32, dim, generator=gen).to(torch.bfloat16).cuda()
     step = GraphedStep(m, x, g)
     graph_grads = [step.x.grad] + step.param_grads
 
@@ -31,7 +32,7 @@ def test_graph_replays_match_eager():
 
     for rep in range(4):
         if rep == 2:  # new input data through the static buffers
-            step.x.data.copy_(torch.randn(4, 28, 30, 64, generator=gen).to(torch.bfloat16))
+            step.x.data.copy_(torch.randn(4, 28, 32, dim, generator=gen).to(torch.bfloat16))
         ref = eager(step.x)
         step.y.zero_()
         for t in graph_grads:
