@@ -43,6 +43,34 @@ def test_argument_validation_without_gpu():
     assert b"workspace" in L.pdw_last_error()
 
 
+def test_single_call_block_host_logic_without_gpu():
+    """pdw_convblock_*: which shapes are covered, workspace sizes, and rejection before any HIP call."""
+    from pyramidconvblock_amd import _lib
+
+    L = _lib.lib()
+    BF16, F16, F32 = 2, 1, 0
+    assert L.pdw_convblock_supported(32, 56, 56, 128, 64, 13, BF16) == 1
+    assert L.pdw_convblock_supported(1, 4, 8, 128, 64, 3, F16) == 1
+    for bad in ((32, 56, 56, 128, 64, 13, F32),    # 16-bit types only
+                (32, 57, 56, 128, 64, 13, BF16),   # odd extent: the pooled scale is not an exact half
+                (32, 56, 56, 128, 64, 12, BF16),   # even filter
+                (32, 56, 56, 64, 32, 13, BF16),    # widths without the paired dense backward
+                (0, 56, 56, 128, 64, 13, BF16),
+                (2, 6, 6, 128, 64, 3, BF16)):      # 36 rows per image: not whole row tiles
+        assert L.pdw_convblock_supported(*bad) == 0, bad
+        assert L.pdw_convblock_fwd_workspace_bytes(*bad) == 0 and L.pdw_convblock_bwd_workspace_bytes(*bad) == 0
+    shape = (32, 56, 56, 128, 64, 13, BF16)
+    fwd, bwd = L.pdw_convblock_fwd_workspace_bytes(*shape), L.pdw_convblock_bwd_workspace_bytes(*shape)
+    n = 32 * 56 * 56
+    assert fwd >= n // L.pdw_dense_colsum_rows() * 128 * 4 + 32 * 128 * 4
+    assert bwd >= 3 * n * 64 * 2 + L.pdw_dense_wgrad_workspace_bytes(n, 128, 64) * 2
+    assert L.pdw_convblock_fwd(*([None] * 16), 0, *shape, None) != 0 and b"null" in L.pdw_last_error()
+    assert L.pdw_convblock_fwd(*([1] * 16), 16, *shape, None) != 0 and b"workspace" in L.pdw_last_error()
+    assert L.pdw_convblock_bwd(*([1] * 22), 16, *shape, None) != 0 and b"workspace" in L.pdw_last_error()
+    assert L.pdw_convblock_bwd(*([1] * 22), 1 << 40, 32, 57, 56, 128, 64, 13, BF16, None) != 0
+    assert b"not covered" in L.pdw_last_error()
+
+
 def test_module_structure_and_seeded_init_match_reference_recipe():
     import pyramid_dwconv
     from oracle import torch_path
