@@ -250,7 +250,7 @@ int pdw_dense_wgrad(const void *a, const void *b, void *dw, void *workspace, siz
  * (+ rowbias[n / P], fp32 [ceil(N/P), I], may be NULL; P >= 32) and dw[O,I] = gy^T x (workspace and summation as pdw_dense_wgrad, size pdw_dense_wgrad_workspace_bytes(N, O, I)); with
  * colsum != NULL also the sums of gy over groups of pdw_dense_colsum_rows() rows, as pdw_dense_fwd_colsum.  The two
  * products share the chip instead of following each other (each alone leaves half of it waiting on memory).
- * Covered: 16-bit, (O, I) = (128, 64) or (64, 128) (pdw_dense_bwd_pair_supported): the backward of conv_out and
+ * Covered: 16-bit, (O, I) = (128, 64), (64, 128), (64, 32) or (32, 64) (pdw_dense_bwd_pair_supported): the backward of conv_out and
  * conv_up, conv_block.py:44 and :37, in ConvBlock(128); other shapes take pdw_dense_fwd(w_kmajor) and
  * pdw_dense_wgrad.  Unlike pdw_dense_wgrad it carries no recorded summations along. */
 int pdw_dense_bwd_pair_supported(int O, int I, int dtype);
@@ -262,7 +262,7 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
  * launch sequence of the entry points above (5 launches forward; 6 launches and one summation launch backward)
  * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
  * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense
- * kernels and pdw_dense_bwd_pair cover (D = 128, I = 64), odd K.  All tensors channels-last and contiguous, all
+ * kernels and pdw_dense_bwd_pair cover (D = 128, I = 64 or D = 64, I = 32), odd K.  All tensors channels-last and contiguous, all
  * parameters in `dtype`: x, y[B,H,W,D]; w_up[I,D]; w_dw0, w_dw1[K,K,I]; w_pool[D,D]; w_out[D,I]; b_pool, b_out[D] or
  * NULL.  The forward writes what the backward reads again: a = conv_up(x), c0 = conv(a), xp = pool(a)[B,H/2,W/2,I],
  * c1 = conv(xp), cat[B,H,W,I] (the gated scales), m[B,D] (per-image mean of x).  The backward overwrites dx and the

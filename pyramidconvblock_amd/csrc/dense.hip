@@ -787,7 +787,9 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
 }
 
 int dense_bwd_pair_supported(int O, int I, int dtype) {
-    return (dtype != kF32 && ((O == 128 && I == 64) || (O == 64 && I == 128))) ? 1 : 0;
+    return (dtype != kF32 && ((O == 128 && I == 64) || (O == 64 && I == 128) || (O == 64 && I == 32) || (O == 32 && I == 64)))
+               ? 1
+               : 0;
 }
 
 // -1: shape not covered.  ws: dense_wgrad_workspace(N, O, I) bytes.
@@ -805,7 +807,7 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
     long long nrows = (ntiles + 3) / 4;
     const int cap = getenv("PDW_PAIR_ROWS") ? atoi(getenv("PDW_PAIR_ROWS")) : 256;  // the second slot of every CU
     if (nrows > cap) nrows = cap;
-    if (colsum && !dense_colsum_supported(O, I, dtype)) return -1;
+    if (colsum && (O < 64 || !dense_colsum_supported(O, I, dtype))) return -1;
     // rows product: K = O, NO = I (inner dimension padded to 64 or 128 in LDS); weight gradient: M = O, NO = I
     const size_t lds_rows = ((size_t)I * ((O > 64 ? 128 : 64) + 8) + 4 * 32 * ((O > I ? O : I) + 8)) * 2 +
                             (rowbias ? (size_t)4 * 2 * I * sizeof(float) : 0);
@@ -818,8 +820,12 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
 #define PDW_PAIR_T(T)                                           \
     if (O == 128) {                                             \
         if (colsum) PDW_PAIR(T, true, 128, 64); else PDW_PAIR(T, false, 128, 64); \
-    } else {                                                    \
+    } else if (O == 64 && I == 128) {                           \
         if (colsum) PDW_PAIR(T, true, 64, 128); else PDW_PAIR(T, false, 64, 128); \
+    } else if (O == 64) {                                       \
+        if (colsum) PDW_PAIR(T, true, 64, 32); else PDW_PAIR(T, false, 64, 32); \
+    } else {                                                    \
+        PDW_PAIR(T, false, 32, 64);                             \
     }
     if (dtype == kF16) { PDW_PAIR_T(f16_t) } else { PDW_PAIR_T(bf16_t) }
 #undef PDW_PAIR_T

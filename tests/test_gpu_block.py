@@ -102,7 +102,7 @@ def test_bias_combinations(oracle, bias):
 
 
 @pytest.mark.parametrize("case", [(128, 13, (4, 56, 56, 128), torch.bfloat16), (128, 9, (3, 8, 16, 128), torch.float16),
-                                  (128, 3, (1, 4, 8, 128), torch.bfloat16)])
+                                  (128, 3, (1, 4, 8, 128), torch.bfloat16), (64, 7, (5, 12, 16, 64), torch.bfloat16)])
 @pytest.mark.parametrize("out_bias", [True, False])
 def test_single_call_block_is_the_stepwise_block(case, out_bias, monkeypatch):
     """pdw_convblock_fwd / _bwd (the block's launch sequence as one library call each way) give bitwise the results

@@ -301,12 +301,13 @@ def test_block_mid_matches_separate_launches(dtype, B, hw, I, D):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N", [1, 70, 96 * 7, 32 * 56 * 56])
-def test_dense_backward_pair_matches_separate_launches(dtype, N):
-    """Input gradient (with column sums) and weight gradient of a 64 -> 128 layer from one launch: the same bits
+@pytest.mark.parametrize("widths", [(128, 64), (64, 32)])
+def test_dense_backward_pair_matches_separate_launches(dtype, N, widths):
+    """Input gradient (with column sums) and weight gradient of an I -> O layer from one launch: the same bits
     as the two launches it replaces, and the same with the summation deferred."""
     from pyramidconvblock_amd import _lib, ops
 
-    O, I = 128, 64
+    O, I = widths
     assert ops.dense_backward_pair_supported(O, I, dtype) and not ops.dense_backward_pair_supported(96, 64, dtype)
     gen = torch.Generator().manual_seed(N)
     gy = randn(gen, N, O).to(dtype).cuda()
