@@ -250,7 +250,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep and forward-only timings")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep, the forward-only timings and the batch-size sweep")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel event timings")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
                     "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, dense_{fwd,dgrad,wgrad}, copy")
@@ -337,6 +337,18 @@ def main():
             sweep[f"k{kk}"] = {"fwd_ms": tf * 1e3, "fwd_bwd_ms": tfb * 1e3, "hbm_frac_fwd": bf / (tf * HBM_PEAK),
                                "hbm_frac_fwd_bwd": bfb / (tfb * HBM_PEAK)}
         result["sweep"] = sweep
+        # The same block at other batch sizes (not the metric: how the fixed cost per launch amortises)
+        batches = {}
+        for bb in (8, 64, 128):
+            xb = torch.randn(bb, H, W, D, generator=gen).to(dtype).cuda().requires_grad_()
+            gb = torch.randn(bb, H, W, D, generator=gen).to(dtype).cuda()
+            tb = time_gpu(GraphedStep(m, xb, gb).replay, args.steps, args.warmup)
+            for p in m.parameters():
+                p.grad = None
+            batches[f"B{bb}"] = {"fwd_bwd_ms": tb * 1e3,
+                                 "hbm_frac_fwd_bwd": block_alg_bytes(bb, H, W, D, k, 2)[1] / (tb * HBM_PEAK)}
+            del xb, gb
+        result["batch_sweep"] = batches
 
     if not args.no_kernels:
         ks = kernel_rooflines(B, H, W, D, k, dtype)
