@@ -128,14 +128,14 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         const int th_i = rem / g.tiles_w;
         row0 = th_i * TH, col0 = (rem - th_i * g.tiles_w) * TW;
     };
-    // ---- filter slice (requested first: it is in LDS by the time the window arrives)
-    constexpr int NW = K * K * CS, IT = (NW + NT - 1) / NT;
-    uint32_t val[IT];
+    // ---- filter slice, 8 channels of a tap per load (requested first: it is in LDS by the time the window arrives)
+    constexpr int NW = K * K * (CS / 8), IT = (NW + NT - 1) / NT;
+    uint4 val[IT];
 #pragma unroll
     for (int s = 0; s < IT; ++s) {  // all loads of a thread in flight together
         const int idx = min(tid + s * NT, NW - 1);
-        const int ch = idx % CS, uv = idx / CS;
-        val[s] = bits16(w[(long long)uv * g.C + min(c0 + ch, g.C - 1)]);
+        const int oct = idx & 1, uv = idx >> 1;
+        val[s] = *reinterpret_cast<const uint4*>(w + uv * g.C + min(c0 + 8 * oct, g.C - 8));  // C % 8 == 0
     }
     int nb = 0, nrow0 = 0, ncol0 = 0;  // tile whose window is in flight
     if (chunk < g.ntiles) {
@@ -143,8 +143,8 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         st.issue(x + (long long)nb * g.H * g.W * g.C, g.H, g.W, g.C, nrow0 - g.PH, ncol0 - g.PW);
     }
 
-    // ---- filter operands in LDS (rotated for the input gradient), zero elsewhere: cleared here, filled after the
-    // first window has been written (the window is what the workgroup waits for; the filter arrived long before)
+    // ---- filter operands in LDS (rotated for the input gradient), zero elsewhere: cleared here, filled behind a
+    // barrier that does not wait for the loads in flight, while the window is still on its way
     {
         uint4* wz = reinterpret_cast<uint4*>(wl);  // both copies: 2 * WR * WPITCH elements, a multiple of 8
         for (int i = tid; i < WR * WPITCH / 4; i += NT) wz[i] = make_uint4(0u, 0u, 0u, 0u);
@@ -155,15 +155,25 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
         for (int s = 0; s < IT; ++s) {
             const int idx = tid + s * NT;
             if (idx < NW) {
-                const int ch = idx % CS, uv = idx / CS;
+                const int oct = idx & 1, uv = idx >> 1;
                 const int u = uv / K, v = uv - u * K;
                 const int uu = g.flip ? K - 1 - u : u, vv = g.flip ? K - 1 - v : v;
-                const unsigned short val16 = (unsigned short)(c0 + ch < g.C ? val[s] : 0u);
-                wls[(3 + uu) * WPITCH + ((vv >> 2) * 16 + ch) * 4 + (vv & 3)] = val16;
-                wls[(WR + 3 + uu) * WPITCH + (((vv + 1) >> 2) * 16 + ch) * 4 + ((vv + 1) & 3)] = val16;
+                const bool chok = c0 + 8 * oct < g.C;
+                const uint32_t d[4] = {val[s].x, val[s].y, val[s].z, val[s].w};
+                unsigned short* w0 = wls + (3 + uu) * WPITCH + ((vv >> 2) * 16 + 8 * oct) * 4 + (vv & 3);
+                unsigned short* w1 = wls + (WR + 3 + uu) * WPITCH + (((vv + 1) >> 2) * 16 + 8 * oct) * 4 + ((vv + 1) & 3);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const unsigned short val16 = (unsigned short)(chok ? (d[e >> 1] >> (16 * (e & 1))) & 0xffffu : 0u);
+                    w0[4 * e] = val16;
+                    w1[4 * e] = val16;
+                }
             }
         }
     };
+    // LDS accesses of this wavefront are complete, then the workgroup barrier: unlike __syncthreads this leaves
+    // global loads in flight
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
     // ---- this lane's operand addresses: wavefront = unit row, lane = (channel bq, q)
     const int bq = lane >> 2, q = lane & 3;
@@ -175,11 +185,11 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
     for (int tile = chunk; tile < g.ntiles; tile += g.nchunks) {
         int b, orow0, ocol0;
         origin(tile, b, orow0, ocol0);
-        __syncthreads();  // the previous window is fully consumed
+        lds_barrier();  // the previous window is fully consumed; first tile: the filter area is cleared
+        if (tile == chunk) fill_filter();  // waits for the filter's loads only
         st.commit_begin();
 #pragma unroll
         for (int it = 0; it < NPRE; ++it) st.commit_next(xl, it, g.H, g.W, orow0 - g.PH, ocol0 - g.PW);
-        if (tile == chunk) fill_filter();  // the barrier above lies between the clearing and these writes
         __syncthreads();
         if constexpr (MODE == 2) {
             // 2x2 means of the tile's own input pixels (H = OH, W = OW, both even, PW even: a window dword is one of
@@ -390,7 +400,9 @@ static int launch_mfma_best(const void* x, const void* w, const void* add, void*
                             int C, int PH, int PW, bool flip, hipStream_t s) {
     const int OH = H + 2 * PH - K + 1, OW = W + 2 * PW - K + 1;
     if (OH < 1 || OW < 1 || C % 8 != 0) return -1;
-    if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return -1;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(w) & 15) != 0)
+        return -1;
     if (add && ((OH | OW) & 1 || (reinterpret_cast<uintptr_t>(add) & 15) != 0)) return -1;
     if (pool && (add || flip || OH != H || OW != W || ((H | W | PW) & 1) || (reinterpret_cast<uintptr_t>(pool) & 15) != 0))
         return -1;
