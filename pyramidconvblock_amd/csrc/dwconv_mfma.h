@@ -106,12 +106,13 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
     constexpr int UPP = NT / (CS / V);
     constexpr int NPRE = (ROWS_IN * NCOL + UPP - 1) / UPP;  // passes: a whole window sits in registers
     constexpr int NE = S / 2;                               // column pairs per strip
-    constexpr int WPITCH = (16 * NVB + 8) * 4;              // elements per filter row in LDS
+    constexpr int WPITCH = (16 * NVB + 4) * 4;              // elements per filter row in LDS
     static_assert(S % 2 == 0 && K % 2 == 1 && (NWV == 4 || NWV == 8), "bad shape");
     extern __shared__ uint32_t smem[];
     uint32_t* xl = smem;                                                  // [ROWS_IN][CS][CPn]
-    // filter operands: wl[copy][3 + u][vb][channel] as 4 columns (8 bytes) each, copy 1 shifted by one column; the
-    // row pitch of 16 NVB + 8 operands puts the 4 filter rows an MFMA reads 64 bytes apart modulo 128: no bank conflicts
+    // filter operands: wl[copy][3 + u][vb][channel] as 4 columns (8 bytes) each, copy 1 shifted by one column; a
+    // row pitch of 16 NVB + 4 operands puts consecutive filter rows an odd multiple of 32 bytes apart modulo 256,
+    // measured the best of the paddings 0..24 (the 4 rows an MFMA's lanes read then fall on different banks)
     T* wl = reinterpret_cast<T*>(smem + ROWS_IN * CS * g.CPn);
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -364,7 +365,7 @@ static int launch_mfma(const void* x, const void* w, const void* add, void* pool
     g.ntiles = (int)ntiles;
     // LDS: pitch = pairs per channel row.  A lane's operand reads start at pitch * channel + S/2 * strip: measured
     // on the part, a pitch of 4 mod 8 is free of bank conflicts for strips of 14 columns, an odd one for strips of 8.
-    const size_t wbytes = (size_t)(2 * Sh::WR + 1) * (16 * Sh::NVB + 8) * 8;  // + the row the last prefetch reads
+    const size_t wbytes = (size_t)(2 * Sh::WR + 1) * (16 * Sh::NVB + 4) * 8;  // + the row the last prefetch reads
     auto lds_of = [&](int p) { return (size_t)Sh::ROWS_IN * Sh::CS * p * 4 + wbytes; };
     int pitch = Sh::NCOL;
     while (S == 14 ? pitch % 8 != 4 : pitch % 2 != 1) ++pitch;
