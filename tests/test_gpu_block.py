@@ -64,6 +64,8 @@ def test_config5_ragged(oracle, dtype, k):
     (64, 7, (5, 12, 12, 64), torch.bfloat16),      # layer widths without the paired dense launch
     (256, 5, (2, 8, 8, 256), torch.bfloat16),      # layer widths the dense kernels leave to the BLAS library
     (128, 11, (2, 16, 16, 128), torch.float32),
+    (64, 7, (3, 8, 16, 64), torch.float16),        # narrow block through the single library call per direction
+    (128, 17, (2, 24, 32, 128), torch.float16),
 ])
 def test_small_and_odd_even_extents(oracle, case):
     """Even extents take the fused two-scale path (paired launches, deferred summations); small and unusual
