@@ -228,6 +228,7 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
             // Operands of a phase: the lane's window at pair offsets 0 and 1 (operand pairs must start at an even
             // register) and the 2 NVB filter operands.  They are requested one phase ahead, all at the top of the
             // phase, so the LDS latency lies under the 4 S NVB MFMAs of the current phase.
+            constexpr bool REUSE = NWV == 4;
             struct Ops {
                 uint2 P0[NQ], P1[NQ], ae[NVB], ao[NVB];
             };
@@ -236,7 +237,15 @@ __global__ __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) void dwconv_mfma_k(cons
 #pragma unroll
                 for (int i = 0; i < NQ; ++i) {
                     if (2 * i < NE + 2 * NVB - 1) o.P0[i] = make_uint2(xr[2 * i], xr[2 * i + 1]);
-                    if (2 * i + 1 < NE + 2 * NVB - 1) o.P1[i] = make_uint2(xr1[2 * i], xr1[2 * i + 1]);
+                    if constexpr (!REUSE)
+                        if (2 * i + 1 < NE + 2 * NVB - 1) o.P1[i] = make_uint2(xr1[2 * i], xr1[2 * i + 1]);
+                }
+                if constexpr (REUSE) {
+                    // one wavefront per SIMD: the loop is bound by LDS traffic and the vector ALU is idle, so the
+                    // copy at pair offset 1 is put together from the registers of the first (2 moves per operand)
+#pragma unroll
+                    for (int i = 0; i < NQ; ++i)
+                        if (2 * i + 1 < NE + 2 * NVB - 1) o.P1[i] = make_uint2(o.P0[i].y, o.P0[i + 1 < NQ ? i + 1 : i].x);
                 }
 #pragma unroll
                 for (int vb = 0; vb < NVB; ++vb) {
