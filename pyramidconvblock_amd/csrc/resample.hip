@@ -1102,11 +1102,14 @@ __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy,
                                     job.gs, job.dmean, (T*)job.gbias, (T*)job.gbias2, (T*)job.gwp, (int)bid, sm);
     } else {
         bid -= npool;
-        if (bid < nblk_full) {
-            const long long first = (long long)bid * (kGateItems * 256) + threadIdx.x;
+        // the half-resolution workgroups (16 gathered taps per item, the slowest to finish) come first in the grid
+        const unsigned nblk_half = gridDim.x - npool - nblk_full;
+        if (bid >= nblk_half) {
+            const long long first = (long long)(bid - nblk_half) * (kGateItems * 256) + threadIdx.x;
             if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
         } else {
-            const long long idx = (long long)(bid - nblk_full) * blockDim.x + threadIdx.x;
+            __builtin_amdgcn_s_setprio(2);
+            const long long idx = (long long)bid * blockDim.x + threadIdx.x;
             if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
         }
     }
