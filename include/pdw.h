@@ -17,7 +17,15 @@
  *     call.  Arithmetic is fp32 (bf16/fp16 products are exact in fp32), one rounding on store.
  *   - Return value: 0 on success; non-zero on invalid arguments or a failed launch, with a
  *     message available from pdw_last_error() (thread-local).
- *   - Re-entrant; no global mutable state except the per-thread error text.
+ *   - Callable from several host threads at once.  The library keeps three pieces of state: the per-thread
+ *     error text, the per-thread list of summations recorded between pdw_reduce_defer_begin() and
+ *     pdw_reduce_defer_flush(), and a once-per-process set-up of each large kernel's LDS limit (guarded by
+ *     std::call_once).  It reads no environment variables: every launch plan is a function of the arguments.
+ *   - Non-finite inputs: the matrix-core convolution kernels multiply a window of input pixels somewhat larger
+ *     than the filter by zero-padded filter operands, so an Inf or NaN input pixel can turn outputs up to
+ *     PDW_NONFINITE_REACH pixels beyond the filter's own footprint into NaN (0 * Inf).  Outputs further away, and
+ *     all outputs for finite inputs, are unaffected.  The reference masks its loads (dwconv_triton.py:55-86), so
+ *     there the value reaches the footprint only.
  */
 #ifndef PDW_H_
 #define PDW_H_
@@ -29,6 +37,10 @@ extern "C" {
 #endif
 
 enum { PDW_F32 = 0, PDW_F16 = 1, PDW_BF16 = 2 };
+
+/* See "Non-finite inputs" above: extra pixels, in every direction, by which a non-finite input value can reach
+ * beyond the K x K footprint of the filter. */
+#define PDW_NONFINITE_REACH 16
 
 /* ABI version of the library (bumped when a signature changes). */
 int pdw_version(void);
@@ -218,7 +230,7 @@ int pdw_block_mid_bwd(const void *gy, const void *xf, const void *xh, void *gxf,
                       const void *w_pool, void *gbias, void *gbias2, void *gw_pool, float *dmean, void *workspace,
                       size_t workspace_bytes, int P, int D, int dtype, void *stream);
 
-/* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 4 == 0;
+/* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 8 == 0;
  * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).
  *   y[n,o] = sum_k x[n,k] * W(o,k) + bias[o] + rowbias[n / P][o]        x[N,K] -> y[N,NO]
  * W(o,k) = w[o*K + k] (w_kmajor == 0, the nn.Linear layout) or w[k*NO + o] (w_kmajor != 0, which gives the

@@ -16,8 +16,6 @@ gradients as a batched split-K product.
 """
 from __future__ import annotations
 
-import os as _os
-
 import torch
 from torch import nn
 from torch.nn import functional as F
@@ -66,6 +64,11 @@ class SimpleGate(nn.Module):
 
 _BMM_FP32_OUT = [True]
 
+# Test hooks (module attributes, never read from the environment): run the block as one Python-level call per
+# launch instead of the library's single call per direction / run conv_up's two gradients as separate launches.
+FORCE_STEPWISE = False
+NO_UP_PAIR = False
+
 
 def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
     """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I], as a batched product over S slabs of N summed in fp32."""
@@ -88,7 +91,7 @@ def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
 def _block_call_ok(x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, w_dw) -> bool:
     """Whether pdw_convblock_fwd / _bwd cover this call: scales (1, 1/2), no conv_up bias, everything contiguous and
     of x's 16-bit dtype, one odd square depthwise filter shape, and shapes the library accepts."""
-    if _os.environ.get("PDW_BLOCK_STEPWISE") or b_up is not None or tuple(scales) != (1., 0.5) or x.dim() != 4:
+    if FORCE_STEPWISE or b_up is not None or tuple(scales) != (1., 0.5) or x.dim() != 4:
         return False
     dt = x.dtype
     tensors = [w_up, w_out, w_pool, *w_dw] + [b for b in (b_out, b_pool) if b is not None]
@@ -335,7 +338,7 @@ class ConvBlockFunction(torch.autograd.Function):
             grad_b_up = a2d.float().sum(0).to(w_up.dtype) if ctx.has_bias[0] else None
             dx = None
             if (fast_up and ctx.needs_input_grad[0] and N > 0 and x.dtype == dt and dmean is not None
-                    and ops.dense_backward_pair_supported(I, D, dt, H * W) and not _os.environ.get("PDW_NO_UP_PAIR")):
+                    and ops.dense_backward_pair_supported(I, D, dt, H * W) and not NO_UP_PAIR):
                 # both products that read da share the pass's last large launch; the summations recorded on the
                 # way run as one small launch when the block of deferred work closes
                 dx, _, grad_w_up = ops.dense_backward_pair(da, w_up.detach().contiguous(), x.contiguous(),

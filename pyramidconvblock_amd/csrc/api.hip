@@ -1,6 +1,7 @@
 // C ABI of libpdw.so (declared in include/pdw.h): argument validation and dispatch to
-// the kernel launchers.  No allocation, no synchronisation, no global mutable state
-// besides the per-thread error text.
+// the kernel launchers.  No allocation, no synchronisation; the only state is the per-thread
+// error text here, the per-thread list of deferred summations (dwconv_direct.hip) and the
+// once-per-process LDS-limit set-up next to each large kernel's launcher.
 #include <stdarg.h>
 #include <stdio.h>
 

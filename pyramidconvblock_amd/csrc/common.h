@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace pdw {
 
@@ -56,6 +57,14 @@ inline int pick_vec(int C, size_t elem, const void* const* ptrs, int nptrs) {
 }
 
 inline int cdiv(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+// Planner overrides for experiments (PDW_* environment variables): read only in a build with -DPDW_TUNE.
+// The shipped library never looks at the environment; every planner then takes its own choice.
+#ifdef PDW_TUNE
+inline const char* tune_env(const char* name) { return getenv(name); }
+#else
+inline const char* tune_env(const char*) { return nullptr; }
+#endif
 
 // Thread-local last-error text returned through the C ABI.
 void set_error(const char* fmt, ...);

@@ -39,22 +39,6 @@ __device__ __forceinline__ f32x16 mfma32(const Frag& a, const Frag& b, f32x16 c,
                                                   0);
 }
 
-// Development aid (-DPDW_STAMP=1|2|3): wall-clock stamps (10 ns units) of the phases of each wavefront's first
-// tile, for one of the instantiations, read back with pdw_debug_stamps().
-#ifdef PDW_STAMP
-__device__ unsigned long long g_stamps[8192 * 8];
-#define STAMP(i)                                                                                                  \
-    do {                                                                                                          \
-        if constexpr ((PDW_STAMP == 1 && !KMAJOR && !COLSUM) || (PDW_STAMP == 2 && !KMAJOR && COLSUM) ||          \
-                      (PDW_STAMP == 3 && KMAJOR && COLSUM)) {                                                     \
-            __builtin_amdgcn_sched_barrier(0);                                                                    \
-            if (lane == 0) g_stamps[(bid * 4 + wave) * 8 + (i)] = __builtin_amdgcn_s_memrealtime();        \
-            __builtin_amdgcn_sched_barrier(0);                                                                    \
-        }                                                                                                         \
-    } while (0)
-#else
-#define STAMP(i)
-#endif
 
 constexpr int kKT = 8;  // k tiles of 16  (inner dimension <= 128)
 constexpr int kNT = 4;  // feature tiles of 32 (<= 128 features)
@@ -197,7 +181,6 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     const int cpk = K / 8;                              // 16-byte chunks per input row
     const int nin = 32 * cpk;                           // chunks per input tile (<= 512)
     constexpr int LP = 8;                               // chunk loads per lane (K <= 128)
-    STAMP(0);
     Frag raw[LP];
     float4 brow = make_float4(0.f, 0.f, 0.f, 0.f);
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
@@ -267,7 +250,6 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     strided_offsets<LP>(lane, 64, cpk, ldt, 8, 32, oin);
     strided_offsets<LO>(lane, 64, cpr, ldt, 8, 32, oout);
     __syncthreads();
-    STAMP(1);
     for (long long tile = gw; tile < ntiles; tile += nw) {
         [[maybe_unused]] const bool first = tile == gw;
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
@@ -302,7 +284,6 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 xf[kt] = Frag{{0u, 0u, 0u, 0u}};
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // fragments are in registers: the buffer may be overwritten
-        if (first) STAMP(2);
         if (tile + nw < ntiles) load_tile(tile + nw);  // next tile in flight during the MFMAs and the store
         if constexpr (COLSUM) {
             float* tf = reinterpret_cast<float*>(tl);  // [512 / K lane groups][K]
@@ -326,7 +307,6 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // read before the result tile is written to the same buffer
         }
-        if (first) STAMP(3);
         // this lane's row of the bias table: the image of tile row l32 relative to the tile's first image
         const float* blr = bl + 4 * half;
         if (rowbias) {
@@ -368,11 +348,9 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                     store_f32<T, 4>(tl + l32 * ldt + n0, o);
                 }
             }
-            if (first && nt < 2) STAMP(4 + nt);
         }
         // coalesced copy-out of the 32 x NO tile (same wavefront wrote it: no workgroup barrier needed)
         __builtin_amdgcn_s_waitcnt(0xc07f);
-        if (first) STAMP(6);
         {
             const long long rows_left = N - tile * 32;
             T* yb = Y + tile * 32 * NO;
@@ -402,7 +380,6 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // copy-out reads done before the next tile overwrites the buffer
-        if (first) STAMP(7);
     }
 }
 
@@ -426,9 +403,6 @@ __global__ __launch_bounds__(256, 2) void dense_rows_rider_k(const T* __restrict
                                                           long long N, int K, int NO, int P, int nkt, int nnt,
                                                           int nblocks, const ReduceJobs jobs) {
     extern __shared__ uint32_t dsm[];
-#if defined(PDW_STAMP) && PDW_STAMP == 4
-    if (threadIdx.x == 0) g_stamps[blockIdx.x * 8] = __builtin_amdgcn_s_memrealtime();
-#endif
     const int nride = (int)gridDim.x - nblocks;
     if ((int)blockIdx.x < nride) {
         reduce_jobs_block(jobs, blockIdx.x, reinterpret_cast<float*>(dsm));
@@ -436,10 +410,6 @@ __global__ __launch_bounds__(256, 2) void dense_rows_rider_k(const T* __restrict
         dense_rows_body<T, KMAJOR, false, SK, SNO>(X, W, bias, rowbias, Y, nullptr, N, K, NO, P, nkt, nnt,
                                                    blockIdx.x - nride, nblocks, dsm);
     }
-#if defined(PDW_STAMP) && PDW_STAMP == 4
-    __syncthreads();
-    if (threadIdx.x == 0) g_stamps[blockIdx.x * 8 + 1] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 // dW partials.  A workgroup of 4 wavefronts walks 64-row stages b, b + gridDim.x, ...: the stage's rows
@@ -661,12 +631,12 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     const int nkt = cdiv(K, 16), nnt = cdiv(NO, 32);
     const long long ntiles = (N + 31) / 32;
     long long blocks = (ntiles + 3) / 4;  // one row tile per wavefront until the cap
-    const int cap = getenv("PDW_DENSE_BLOCKS") ? atoi(getenv("PDW_DENSE_BLOCKS")) : 512;
+    const int cap = tune_env("PDW_DENSE_BLOCKS") ? atoi(tune_env("PDW_DENSE_BLOCKS")) : 512;
     if (blocks > cap) blocks = cap;  // persistent workgroups: the weights are staged to LDS once each
     if (blocks < 1) blocks = 1;
     const size_t lds = ((size_t)nnt * 32 * ((nkt > 4 ? 128 : 64) + 8) + 4 * 32 * ((K > NO ? K : NO) + 8)) * 2 +
                        ((bias || rowbias) ? (size_t)4 * 2 * nnt * 32 * sizeof(float) : 0);
-    const int shape = getenv("PDW_DENSE_GENERIC") ? 0 : (K == 128 && NO == 64) ? 1 : (K == 64 && NO == 128) ? 2 : 0;
+    const int shape = tune_env("PDW_DENSE_GENERIC") ? 0 : (K == 128 && NO == 64) ? 1 : (K == 64 && NO == 128) ? 2 : 0;
     if (rider) {
         // The summations come first in the grid and take resident slots of their own from the start (the slots
         // are two per compute unit; waiting for finished row workgroups would put their latency behind the
@@ -724,7 +694,7 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
 
 static void dense_wgrad_plan(long long N, int* blocks, int* stages_per_block) {
     const long long nstages = (N + kWgRows - 1) / kWgRows;
-    long long nb = getenv("PDW_DWG_BLOCKS") ? atoi(getenv("PDW_DWG_BLOCKS")) : 256;
+    long long nb = tune_env("PDW_DWG_BLOCKS") ? atoi(tune_env("PDW_DWG_BLOCKS")) : 256;
     if (nb > nstages) nb = nstages;
     if (nb < 1) nb = 1;
     const long long spb = (nstages + nb - 1) / nb;
@@ -768,8 +738,8 @@ template <typename T>
 static int dense_wgrad_t(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, hipStream_t s) {
     const int mt = cdiv(M, 32), nt = cdiv(NO, 32);
     // the block's two layer shapes (64 x 128 and 128 x 64) have variants with the extents as constants
-    if (M == 64 && NO == 128 && !getenv("PDW_DENSE_GENERIC")) return dense_wgrad_go<T, 2, 4, true>(a, b, dw, ws, N, M, NO, s);
-    if (M == 128 && NO == 64 && !getenv("PDW_DENSE_GENERIC")) return dense_wgrad_go<T, 4, 2, true>(a, b, dw, ws, N, M, NO, s);
+    if (M == 64 && NO == 128 && !tune_env("PDW_DENSE_GENERIC")) return dense_wgrad_go<T, 2, 4, true>(a, b, dw, ws, N, M, NO, s);
+    if (M == 128 && NO == 64 && !tune_env("PDW_DENSE_GENERIC")) return dense_wgrad_go<T, 4, 2, true>(a, b, dw, ws, N, M, NO, s);
 #define PDW_CASE(MT, NT) \
     if (mt == MT && nt == NT) return dense_wgrad_go<T, MT, NT, false>(a, b, dw, ws, N, M, NO, s);
     PDW_CASE(1, 1) PDW_CASE(1, 2) PDW_CASE(2, 1) PDW_CASE(2, 2) PDW_CASE(1, 3) PDW_CASE(3, 1) PDW_CASE(2, 3)
@@ -805,7 +775,7 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
     dense_wgrad_plan(N, &nwg, &spb);
     const long long ntiles = (N + 31) / 32;
     long long nrows = (ntiles + 3) / 4;
-    const int cap = getenv("PDW_PAIR_ROWS") ? atoi(getenv("PDW_PAIR_ROWS")) : 256;  // the second slot of every CU
+    const int cap = tune_env("PDW_PAIR_ROWS") ? atoi(tune_env("PDW_PAIR_ROWS")) : 256;  // the second slot of every CU
     if (nrows > cap) nrows = cap;
     if (colsum && (O < 64 || !dense_colsum_supported(O, I, dtype))) return -1;
     // rows product: K = O, NO = I (inner dimension padded to 64 or 128 in LDS); weight gradient: M = O, NO = I
@@ -837,8 +807,3 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
 
 }  // namespace pdw
 
-#ifdef PDW_STAMP
-extern "C" int pdw_debug_stamps(unsigned long long* host, int n) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pdw::g_stamps), sizeof(unsigned long long) * n);
-}
-#endif

@@ -26,6 +26,7 @@
 // filter is staged, the next ones as soon as the operand registers are free) and written to LDS in passes,
 // and the results leave through LDS as 16-byte stores.
 #pragma once
+#include <mutex>
 #include <stdlib.h>
 
 #include "common.h"
@@ -379,26 +380,23 @@ static int launch_mfma(const void* x, const void* w, const void* add, void* pool
     int pitch = Sh::NCOL;
     while (S == 14 ? pitch % 8 != 4 : pitch % 2 != 1) ++pitch;
     if (lds_of(pitch) > 160 * 1024) pitch = Sh::NCOL;
-    if (getenv("PDW_MFMA_PITCH") && atoi(getenv("PDW_MFMA_PITCH")) >= Sh::NCOL) pitch = atoi(getenv("PDW_MFMA_PITCH"));
+    if (tune_env("PDW_MFMA_PITCH") && atoi(tune_env("PDW_MFMA_PITCH")) >= Sh::NCOL) pitch = atoi(tune_env("PDW_MFMA_PITCH"));
     if (lds_of(pitch) > 160 * 1024) return -1;
     g.CPn = pitch;
     size_t lds = lds_of(pitch);
-    if (getenv("PDW_MFMA_LDSMIN") && lds < (size_t)atoi(getenv("PDW_MFMA_LDSMIN"))) lds = atoi(getenv("PDW_MFMA_LDSMIN"));
+    if (tune_env("PDW_MFMA_LDSMIN") && lds < (size_t)atoi(tune_env("PDW_MFMA_LDSMIN"))) lds = atoi(tune_env("PDW_MFMA_LDSMIN"));
     // persistent workgroups: as many as are resident at once, tiles dealt out as evenly as they divide
     const int resident = (int)((160 * 1024) / (lds + 1024)) >= 2 && NWV == 4 ? 2 : 1;
     const int cap = (256 * resident) / g.slices > 1 ? (256 * resident) / g.slices : 1;
     const long long rounds = cdiv(ntiles, (long long)cap);
     long long nch = cdiv(ntiles, rounds);
-    if (getenv("PDW_MFMA_NCH")) nch = atoi(getenv("PDW_MFMA_NCH"));
+    if (tune_env("PDW_MFMA_NCH")) nch = atoi(tune_env("PDW_MFMA_NCH"));
     g.nchunks = (int)(nch < 1 ? 1 : nch);
     const long long nblocks = (long long)g.nchunks * g.slices;
     const int mode = add ? 1 : (pool ? 2 : 0);
     auto kern = mode == 1 ? dwconv_mfma_k<T, K, S, NWV, 1> : (mode == 2 ? dwconv_mfma_k<T, K, S, NWV, 2> : dwconv_mfma_k<T, K, S, NWV, 0>);
-    static bool attr_done[3] = {false, false, false};
-    if (!attr_done[mode]) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_done[mode] = true;
-    }
+    static std::once_flag attr_once[3];
+    std::call_once(attr_once[mode], [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(NWV * 64), lds, s, (const T*)x, (const T*)w, (const T*)add,
                        (T*)pool, (T*)y, g);
     return check_launch("dwconv_mfma");
@@ -422,7 +420,7 @@ static int launch_mfma_best(const void* x, const void* w, const void* add, void*
     // 8 wavefronts per workgroup (tile 32 rows) when that still yields a workgroup for most CUs
     const long long t8 = (long long)B * cdiv(OH, 32) * cdiv(OW, tw) * cdiv(C, 16);
     bool w8 = t8 >= 192;
-    if (getenv("PDW_MFMA_NWV")) w8 = atoi(getenv("PDW_MFMA_NWV")) == 8;
+    if (tune_env("PDW_MFMA_NWV")) w8 = atoi(tune_env("PDW_MFMA_NWV")) == 8;
     if (s14) {
         if (w8) return launch_mfma<T, K, 14, 8>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
         return launch_mfma<T, K, 14, 4>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);

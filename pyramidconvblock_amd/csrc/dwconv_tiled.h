@@ -19,6 +19,7 @@
 // A zero tap multiplies the pixel one column outside the window, so a non-finite value there
 // would leak into the output (0 * inf); finite inputs are unaffected.
 #pragma once
+#include <mutex>
 #include <stdlib.h>
 
 #include "common.h"
@@ -394,7 +395,7 @@ static int launch_tiled(const TiledPlan& plan, const void* x, const void* w, voi
     // Persistent workgroups: as many as fit on the chip at once (LDS allows `occ` per CU, at most 3), then
     // trimmed so the tiles divide as evenly as possible among them.
     int occ = (int)((160 * 1024) / (lds + 512));
-    const int occ_max = getenv("PDW_OCC") ? atoi(getenv("PDW_OCC")) : 3;
+    const int occ_max = tune_env("PDW_OCC") ? atoi(tune_env("PDW_OCC")) : 3;
     occ = occ < 1 ? 1 : (occ > occ_max ? occ_max : occ);
     const int target = (256 * occ) / g.slices > 1 ? (256 * occ) / g.slices : 1;
     int nch = (int)(ntiles < target ? ntiles : target);
@@ -407,21 +408,18 @@ static int launch_tiled(const TiledPlan& plan, const void* x, const void* w, voi
             if (eff >= beste) beste = eff, nch = cand;
         }
     }
-    if (getenv("PDW_NCH")) nch = atoi(getenv("PDW_NCH"));
+    if (tune_env("PDW_NCH")) nch = atoi(tune_env("PDW_NCH"));
     g.nchunks = nch < 1 ? 1 : nch;
     const long long nblocks = (long long)g.nchunks * g.slices;
-    const void* ptrs[1] = {x};
-    const int vec = pick_vec(C, sizeof(T), ptrs, 1);
+    const void* ptrs[3] = {x, w, y};  // all three are moved with the same channel vectors
+    const int vec = pick_vec(C, sizeof(T), ptrs, 3);
 #define PDW_GO(V)                                                                                            \
     {                                                                                                        \
         auto kern = dwconv_tiled_k<T, KW, R, Q, CS, V>;                                                      \
         const int upp = 256 / (CS / V);                                                                      \
         g.step_r = upp / g.CPn, g.step_u = upp % g.CPn;                                                      \
-        static bool attr_done = false;                                                                       \
-        if (!attr_done) {                                                                                    \
-            (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
-            attr_done = true;                                                                                \
-        }                                                                                                    \
+        static std::once_flag attr_once;                                                                       \
+        std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });                                                                                                    \
         hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), lds, s, (const T*)x, (const T*)w, (T*)y, g); \
     }
     if constexpr (sizeof(T) == 2) {
@@ -446,11 +444,11 @@ static int launch_best(const void* x, const void* w, void* y, int B, int H, int 
     const TiledPlan* ps[3] = {&p0, &p1, &p2};
     for (int i = 0; i < 3; ++i)
         if (ps[i]->cost >= 0 && (best < 0 || ps[i]->cost < best)) best = ps[i]->cost, pick = i;
-    const char* force = getenv("PDW_PATCH");
+    const char* force = tune_env("PDW_PATCH");
     if (force && atoi(force) >= 0 && atoi(force) < 3) pick = atoi(force);
     TiledPlan p = pick >= 0 ? *ps[pick] : p0;
     if (pick < 0 || p.cost < 0) return -1;
-    if (getenv("PDW_NRG") && getenv("PDW_NST")) p.nrg = atoi(getenv("PDW_NRG")), p.nst = atoi(getenv("PDW_NST"));
+    if (tune_env("PDW_NRG") && tune_env("PDW_NST")) p.nrg = atoi(tune_env("PDW_NRG")), p.nst = atoi(tune_env("PDW_NST"));
     switch (pick) {
         case 0: return launch_tiled<T, KW, 8, 2, 32>(p, x, w, y, B, H, W, C, KH, PH, PW, flip, s);
         case 1: return launch_tiled<T, KW, 14, 1, 32>(p, x, w, y, B, H, W, C, KH, PH, PW, flip, s);

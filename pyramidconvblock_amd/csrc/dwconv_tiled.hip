@@ -46,7 +46,7 @@ int dwconv_mfma_k17(const void* x, const void* w, const void* add, void* pool, v
 static int dwconv_mfma_launch(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int KH,
                               int KW, int PH, int PW, bool flip, int dtype, hipStream_t s) {
     if (KH != KW || dtype == kF32) return -1;
-    const char* e = getenv("PDW_MFMA");
+    const char* e = tune_env("PDW_MFMA");
     if (e && atoi(e) == 0) return -1;
     switch (KW) {
         case 3: return dwconv_mfma_k3(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);

@@ -21,6 +21,7 @@
 //
 // Both windows are staged in LDS channel-major, [row][channel][column pair], as in dwconv_mfma.h.
 #pragma once
+#include <mutex>
 #include <stdlib.h>
 
 #include "common.h"
@@ -261,15 +262,15 @@ static WgradMfmaPlan plan_wgrad_mfma(int B, int H, int W, int C, int PH, int PW)
         return n;
     };
     g.XP = pad(g.TW / 2 + 4 * Sh::NVG), g.GP = pad(g.TW / 2);
-    if (getenv("PDW_WG_XP") && atoi(getenv("PDW_WG_XP")) >= g.TW / 2 + 4 * Sh::NVG) g.XP = atoi(getenv("PDW_WG_XP"));
-    if (getenv("PDW_WG_GP") && atoi(getenv("PDW_WG_GP")) >= g.TW / 2) g.GP = atoi(getenv("PDW_WG_GP"));
+    if (tune_env("PDW_WG_XP") && atoi(tune_env("PDW_WG_XP")) >= g.TW / 2 + 4 * Sh::NVG) g.XP = atoi(tune_env("PDW_WG_XP"));
+    if (tune_env("PDW_WG_GP") && atoi(tune_env("PDW_WG_GP")) >= g.TW / 2) g.GP = atoi(tune_env("PDW_WG_GP"));
     auto lds_of = [&](int th) { return ((size_t)(th + K - 1) * Sh::CS * g.XP + (size_t)th * (Sh::CS * g.GP + 1)) * 4; };
     // tile height: about one tile per CU, within LDS.  Where LDS forces lower tiles than that, the count of tile
     // rows is chosen for the shortest run: rounds of tiles per workgroup times (tile rows + 66), the 66 being what a
     // tile costs beside its rows (halo, staging latency, the final sum), fitted to measurements at K = 13 and 17.
     const long long per_row = (long long)B * g.slices * g.tiles_w;  // tiles per row of tiles, all slices
     int tiles_h = (int)(256 / (per_row > 0 ? per_row : 1));
-    if (getenv("PDW_WG_TILEMUL")) tiles_h *= atoi(getenv("PDW_WG_TILEMUL"));
+    if (tune_env("PDW_WG_TILEMUL")) tiles_h *= atoi(tune_env("PDW_WG_TILEMUL"));
     if (tiles_h < 1) tiles_h = 1;
     if (tiles_h > g.OH) tiles_h = g.OH;
     int th = cdiv(g.OH, tiles_h);
@@ -323,11 +324,8 @@ static int wgrad_mfma_launch_t(const void* x, const void* gy, void* dw, void* ws
     const WgradMfmaPlan p = plan_wgrad_mfma<T, K, NWV>(B, H, W, C, PH, PW);
     if (!p.ok) return -1;
     auto kern = dwconv_wgrad_mfma_k<T, K, NWV>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_done = true;
-    }
+    static std::once_flag attr_once;
+    std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)p.nblocks), dim3(NWV * 64), p.lds, s, (const T*)x, (const T*)gy, (float*)ws,
                        p.g, (const T*)x, (const T*)gy, (float*)ws, p.g, (unsigned)p.nblocks);
     if (int e = check_launch("dwconv_wgrad_mfma")) return e;
@@ -346,11 +344,8 @@ static int wgrad_mfma_pair_launch_t(const void* xa, const void* gya, void* dwa, 
     const WgradMfmaPlan pb = plan_wgrad_mfma<T, K, NWV>(B, Hb, Wb, C, PH, PW);
     if (!pa.ok || !pb.ok || pa.nblocks % 8 != 0) return -1;  // a multiple of 8: problem 1 keeps its XCD mapping
     auto kern = dwconv_wgrad_mfma_k<T, K, NWV>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_done = true;
-    }
+    static std::once_flag attr_once;
+    std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)(pa.nblocks + pb.nblocks)), dim3(NWV * 64), pa.lds > pb.lds ? pa.lds : pb.lds,
                        s, (const T*)xa, (const T*)gya, (float*)wsa, pa.g, (const T*)xb, (const T*)gyb, (float*)wsb, pb.g,
                        (unsigned)pa.nblocks);

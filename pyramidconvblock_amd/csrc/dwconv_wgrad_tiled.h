@@ -17,6 +17,7 @@
 // Pass 2 sums the partials in a fixed order (wgrad_reduce_parts).  No atomics anywhere, so the
 // result is bit-reproducible.
 #pragma once
+#include <mutex>
 #include <stdlib.h>
 
 #include "common.h"
@@ -234,8 +235,8 @@ static WgradPlan plan_wgrad(int B, int H, int W, int C, int PH, int PW) {
             }
         }
     if (best < 0) return p;
-    if (getenv("PDW_WG_TH") && getenv("PDW_WG_NSP")) {
-        g.TH = atoi(getenv("PDW_WG_TH")), g.NSP = atoi(getenv("PDW_WG_NSP"));
+    if (tune_env("PDW_WG_TH") && tune_env("PDW_WG_NSP")) {
+        g.TH = atoi(tune_env("PDW_WG_TH")), g.NSP = atoi(tune_env("PDW_WG_NSP"));
         const int tw = 2 * g.NSP * R;
         g.tiles_h = cdiv(g.OH, g.TH), g.tiles_w = cdiv(g.OW, tw);
         g.CPX = (tw + K - 1 + PK - 1) / PK, g.CPG = tw / PK;
@@ -247,7 +248,7 @@ static WgradPlan plan_wgrad(int B, int H, int W, int C, int PH, int PW) {
     if (ntiles > 0x7fffffffLL) return p;
     g.ntiles = (int)ntiles;
     int nch = best_nch;
-    if (getenv("PDW_WG_NCH")) nch = atoi(getenv("PDW_WG_NCH"));
+    if (tune_env("PDW_WG_NCH")) nch = atoi(tune_env("PDW_WG_NCH"));
     g.nchunks = nch < 1 ? 1 : nch;
     p.nblocks = g.nchunks * g.slices;
     p.ok = true;
@@ -273,11 +274,8 @@ static int wgrad_tiled_launch_t(const void* x, const void* gy, void* dw, void* w
 #define PDW_GO(V)                                                                                                 \
     {                                                                                                             \
         auto kern = dwconv_wgrad_tiled_k<T, K, R, USPLIT, V>;                                                     \
-        static bool attr_done = false;                                                                            \
-        if (!attr_done) {                                                                                         \
-            (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
-            attr_done = true;                                                                                     \
-        }                                                                                                         \
+        static std::once_flag attr_once;                                                                            \
+        std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });                                                                                                         \
         hipLaunchKernelGGL(kern, dim3((unsigned)p.nblocks), dim3(256), p.lds, s, (const T*)x, (const T*)gy,       \
                            (float*)ws, g);                                                                        \
     }

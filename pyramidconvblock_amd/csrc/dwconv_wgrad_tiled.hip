@@ -86,7 +86,7 @@ int dwconv_wgrad_mfma_pair_k17(const void* xa, const void* gya, void* dwa, void*
 // Matrix-core variant (16-bit types): workspace bytes (0 = not covered) and launch (-1 = not covered).
 static bool wgrad_mfma_enabled(int dtype) {
     if (dtype == kF32) return false;
-    const char* e = getenv("PDW_MFMA");
+    const char* e = tune_env("PDW_MFMA");
     return !(e && atoi(e) == 0);
 }
 static size_t wgrad_mfma_workspace(int B, int H, int W, int C, int K, int PH, int PW, int dtype) {
@@ -124,7 +124,7 @@ static int wgrad_mfma_launch(const void* x, const void* gy, void* dw, void* ws, 
 int dwconv_wgrad_pair_launch(const void* xa, const void* gya, void* dwa, void* wsa, int Ha, int Wa, const void* xb,
                              const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int K, int PH, int PW,
                              int dtype, hipStream_t s) {
-    if (!wgrad_mfma_enabled(dtype) || getenv("PDW_NO_WGRAD_PAIR")) return -1;
+    if (!wgrad_mfma_enabled(dtype) || tune_env("PDW_NO_WGRAD_PAIR")) return -1;
     switch (K) {
         case 3: return dwconv_wgrad_mfma_pair_k3(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
         case 5: return dwconv_wgrad_mfma_pair_k5(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);

@@ -1080,9 +1080,6 @@ __global__ __launch_bounds__(256) void block_mid_fwd_k(const T* __restrict__ xf,
     }
 }
 
-#if defined(PDW_STAMP) && PDW_STAMP == 5
-__device__ unsigned long long g_stamps5[8192 * 2];
-#endif
 template <typename T>
 __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy, const T* __restrict__ xf,
                                                        const T* __restrict__ xh, T* __restrict__ gxf,
@@ -1094,9 +1091,6 @@ __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy,
     extern __shared__ float sm[];
     constexpr int VEC = 8;
     unsigned bid = blockIdx.x;
-#if defined(PDW_STAMP) && PDW_STAMP == 5
-    if (threadIdx.x == 0) g_stamps5[blockIdx.x * 2] = __builtin_amdgcn_s_memrealtime();
-#endif
     if (bid < npool) {
         pool_branch_bwd_v8_block<T>(job.part, job.nchunks, job.B, job.D, job.inv_p, (const T*)job.wp, (const T*)job.m,
                                     job.gs, job.dmean, (T*)job.gbias, (T*)job.gbias2, (T*)job.gwp, (int)bid, sm);
@@ -1113,11 +1107,6 @@ __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy,
             if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
         }
     }
-#if defined(PDW_STAMP) && PDW_STAMP == 5
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (threadIdx.x == 0) g_stamps5[blockIdx.x * 2 + 1] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 // y[b,p,c] += v[b,c]  (v in fp32, one rounding)
@@ -1554,8 +1543,3 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
 
 }  // namespace pdw
 
-#if defined(PDW_STAMP) && PDW_STAMP == 5
-extern "C" int pdw_debug_stamps5(unsigned long long* host, int n) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pdw::g_stamps5), sizeof(unsigned long long) * n);
-}
-#endif

@@ -23,6 +23,12 @@ def _pixel_stride(t: torch.Tensor) -> int:
     return ld
 
 
+def _aligned(t):
+    """The dense matrix-core kernels move 16-byte pieces: a view whose storage offset is not a multiple of 16
+    bytes (a slice of a larger parameter buffer, say) is copied to a fresh, aligned allocation."""
+    return t if t is None or t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+
+
 def _launch(name, dev, *args):
     with _lib.on_device(dev):
         _lib.check(getattr(_lib.lib(), name)(*args, _lib.stream_ptr(dev)), name)
@@ -253,6 +259,7 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
     (y, parts): parts fp32 [N / R, K], the sums of x over each group of R = dense_colsum_rows() consecutive rows.  With
     flush_reductions, inside _lib.deferred_reductions, the summations recorded so far run in this launch."""
     dev = _lib.require_device(x, w)
+    x, w, bias, rowbias = _aligned(x), _aligned(w), _aligned(bias), _aligned(rowbias)
     K = x.shape[-1]
     NO = w.shape[1] if w_kmajor else w.shape[0]
     assert (w.shape[0] if w_kmajor else w.shape[1]) == K and x.is_contiguous() and w.is_contiguous()
@@ -277,6 +284,7 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
 def dense_wgrad(a, b):
     """dw[m, o] = sum_n a[n, m] * b[n, o] over all leading dimensions; returns [M, NO] in a's dtype."""
     dev = _lib.require_device(a, b)
+    a, b = _aligned(a), _aligned(b)
     M, NO = a.shape[-1], b.shape[-1]
     N = a.numel() // M
     assert b.numel() // NO == N and a.is_contiguous() and b.is_contiguous()
@@ -301,6 +309,7 @@ def dense_backward_pair(gy, w, x, colsum=False, rowbias=None, rows_per_image=1):
     dx = gy W + rowbias[image] (rowbias fp32 [B, I] or None), dw = gy^T x and, with colsum, parts as in
     dense_forward(gy, ..., colsum=True)."""
     dev = _lib.require_device(gy, w, x)
+    gy, w, x, rowbias = _aligned(gy), _aligned(w), _aligned(x), _aligned(rowbias)
     O, I = w.shape
     N = gy.numel() // O
     assert gy.shape[-1] == O and x.shape[-1] == I and x.numel() // I == N

@@ -131,7 +131,8 @@ def test_single_call_block_is_the_stepwise_block(case, out_bias, monkeypatch):
         return [y.detach(), xi.grad] + [p.grad for p in m.parameters()]
 
     single = run()
-    monkeypatch.setenv("PDW_BLOCK_STEPWISE", "1")
+    from pyramidconvblock_amd import conv_block
+    monkeypatch.setattr(conv_block, "FORCE_STEPWISE", True)
     stepwise = run()
     assert len(single) == len(stepwise)
     for i, (s, t) in enumerate(zip(single, stepwise)):
