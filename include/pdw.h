@@ -114,6 +114,21 @@ int pdw_dwconv_wgrad(const void *x, const void *gy, void *dw, void *workspace, s
                      int B, int H, int W, int C, int KH, int KW, int SH, int SW, int PH, int PW, int DH,
                      int DW, int dtype, void *stream);
 
+/* pdw_dwconv_wgrad for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments and bitwise the same result, but the fp32 partial sums
+ * go to a buffer of pdw_static_scratch_bytes() (32 MiB) that is part of the library's device image instead of a
+ * caller-supplied workspace.  The call allocates and frees nothing.  Extents whose
+ * pdw_dwconv_wgrad_workspace_bytes exceeds that size are rejected with an error (use pdw_dwconv_wgrad).  Every
+ * call on a device shares that device's one buffer, so calls that overlap on one device (two streams, two host
+ * threads) race; the kernels overwrite what they read of it, nothing has to be cleared between calls.  Not
+ * available between pdw_reduce_defer_begin and the flush.  The buffer's address on the current device is looked
+ * up on the first call there (hipGetSymbolAddress); pdw_static_scratch_init() does that ahead of time, e.g.
+ * before a graph capture begins.  No counterpart in the reference. */
+size_t pdw_static_scratch_bytes(void);
+int pdw_static_scratch_init(void);
+int pdw_dwconv_wgrad_static(const void *x, const void *gy, void *dw, int B, int H, int W, int C, int KH, int KW,
+                            int SH, int SW, int PH, int PW, int DH, int DW, int dtype, void *stream);
+
 /* Two pdw_dwconv_wgrad calls of one pyramid block as one call: the same batch, channel count and odd square
  * filter (stride 1, padding K/2, dilation 1) on two tensors of different extents, each with its own workspace
  * (sized by pdw_dwconv_wgrad_workspace_bytes).  For 16-bit types the two problems share one launch, the second

@@ -33,6 +33,9 @@ _SIGS = {
     "pdw_dwconv_dgrad_addpool": (c_int, [c_void_p] * 4 + _CONV + [c_int, c_int, c_int, c_void_p]),
     "pdw_dwconv_wgrad_workspace_bytes": (c_size_t, _CONV + [c_int]),
     "pdw_dwconv_wgrad": (c_int, [c_void_p] * 4 + [c_size_t] + _CONV + [c_int, c_void_p]),
+    "pdw_static_scratch_bytes": (c_size_t, []),
+    "pdw_static_scratch_init": (c_int, []),
+    "pdw_dwconv_wgrad_static": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
     "pdw_dwconv_wgrad_pair": (c_int, ([c_void_p] * 4 + [c_size_t] + [c_int] * 2) * 2 + [c_int] * 4 + [c_void_p]),
     "pdw_convblock_supported": (c_int, [c_int] * 7),
     "pdw_convblock_fwd_workspace_bytes": (c_size_t, [c_int] * 7),

@@ -5,6 +5,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "../../include/pdw.h"
 #include "common.h"
 #include "kernels.h"
@@ -51,6 +53,34 @@ static int check_resample(const char* fn, const void* a, const void* b, int B, i
     if (B > 0 && (!a || !b)) return set_error("%s: null pointer", fn), 1;
     if ((long long)H * h >= 0x7fffffffLL || (long long)W * w >= 0x7fffffffLL)
         return set_error("%s: extents too large", fn), 1;
+    return 0;
+}
+
+// Scratch of the entry point that allocates nothing (pdw_dwconv_wgrad_static): one copy of this array lives on every
+// device the library is loaded on, at that device's own address.  The name is a host-side stand-in; device
+// code and HIP calls get the address hipGetSymbolAddress returns for the current device.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device, looked up once per device (with that device current).
+static int static_scratch(const char* fn, void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error("%s: hipGetDevice: %s", fn, hipGetErrorString(e)), 2;
+    if (dev < 0 || dev >= kMaxDevices) return set_error("%s: device index %d not supported", fn, dev), 2;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return set_error("%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e)), 2;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
     return 0;
 }
 
@@ -162,6 +192,29 @@ int pdw_dwconv_wgrad(const void* x, const void* gy, void* dw, void* workspace, s
     }
     return dwconv_wgrad_direct_launch(x, gy, dw, workspace, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype,
                                       (hipStream_t)stream);
+}
+
+size_t pdw_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int pdw_static_scratch_init(void) {
+    void* p = nullptr;
+    return static_scratch("pdw_static_scratch_init", &p);
+}
+
+int pdw_dwconv_wgrad_static(const void* x, const void* gy, void* dw, int B, int H, int W, int C, int KH, int KW, int SH,
+                            int SW, int PH, int PW, int DH, int DW, int dtype, void* stream) {
+    if (int e = check_conv("pdw_dwconv_wgrad_static", x, gy, dw, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype))
+        return e;
+    if (reduce_deferring())
+        return set_error("pdw_dwconv_wgrad_static: not available between pdw_reduce_defer_begin and the flush (the "
+                         "shared scratch would have to stay untouched until then)"), 1;
+    const size_t need = pdw_dwconv_wgrad_workspace_bytes(B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype);
+    if (need > kStaticScratchBytes)
+        return set_error("pdw_dwconv_wgrad_static: these extents need %zu bytes of scratch, the static buffer holds "
+                         "%zu; use pdw_dwconv_wgrad with a workspace", need, kStaticScratchBytes), 1;
+    void* ws = nullptr;
+    if (int e = static_scratch("pdw_dwconv_wgrad_static", &ws)) return e;
+    return pdw_dwconv_wgrad(x, gy, dw, ws, kStaticScratchBytes, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype, stream);
 }
 
 int pdw_dwconv_wgrad_pair(const void* x0, const void* gy0, void* dw0, void* workspace0, size_t workspace0_bytes, int H0,

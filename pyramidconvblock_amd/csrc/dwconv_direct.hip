@@ -174,6 +174,8 @@ int reduce_defer_flush(hipStream_t s) {
     return r;
 }
 
+bool reduce_deferring() { return t_defer; }
+
 int reduce_defer_room() { return t_defer ? kMaxReduceJobs - t_jobs.njobs : 0; }
 
 // Records out[o * D + d] = sum_b g[b * D + o] * m[b * D + d] (see outer_sum_block); only while deferring.

@@ -26,6 +26,7 @@ struct ReduceJobs;
 int reduce_defer_take(ReduceJobs* out);  // moves the recorded jobs out (0 = none); the flush then has nothing to do
 int reduce_jobs_launch(const ReduceJobs& jobs, hipStream_t s);
 int reduce_defer_begin();
+bool reduce_deferring();  // between reduce_defer_begin and the flush on this thread
 int reduce_defer_room();  // jobs that can still be recorded (0 when not deferring)
 int reduce_defer_outer(const float* g, const void* m, void* out, int B, int D, int dtype);  // -1: not recorded
 int reduce_defer_flush(hipStream_t s);
