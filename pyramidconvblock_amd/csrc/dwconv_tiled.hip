@@ -42,6 +42,42 @@ int dwconv_mfma_k15(const void* x, const void* w, const void* add, void* pool, v
 int dwconv_mfma_k17(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
                     bool flip, int dtype, hipStream_t s);
 
+int dwconv_tz_k3(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k5(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k7(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k9(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k11(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k13(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k15(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+int dwconv_tz_k17(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
+                   bool flip, int dtype, hipStream_t s);
+
+// Block-Toeplitz kernel on the dense matrix cores (dwconv_tz.h): square odd filters, 16-bit types, C % 8 == 0.
+static int dwconv_tz_launch(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int KH,
+                            int KW, int PH, int PW, bool flip, int dtype, hipStream_t s) {
+    if (KH != KW || dtype == kF32) return -1;
+    const char* e = tune_env("PDW_TZ");
+    if (e && atoi(e) == 0) return -1;
+    switch (KW) {
+        case 3: return dwconv_tz_k3(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 5: return dwconv_tz_k5(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 7: return dwconv_tz_k7(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 9: return dwconv_tz_k9(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 11: return dwconv_tz_k11(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 13: return dwconv_tz_k13(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 15: return dwconv_tz_k15(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        case 17: return dwconv_tz_k17(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+        default: return -1;
+    }
+}
+
 // Matrix-core kernel for square filters and 16-bit types; -1 when it does not cover the case.
 static int dwconv_mfma_launch(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int KH,
                               int KW, int PH, int PW, bool flip, int dtype, hipStream_t s) {
@@ -67,6 +103,10 @@ static int dwconv_mfma_launch(const void* x, const void* w, const void* add, voi
 int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
                         int PW, bool flip, int dtype, hipStream_t s, const void* add, void* pool) {
     if (KH > 31 || H + 2 * PH - KH + 1 < 1 || W + 2 * PW - KW + 1 < 1) return -1;
+    {
+        const int r = dwconv_tz_launch(x, w, add, pool, y, B, H, W, C, KH, KW, PH, PW, flip, dtype, s);
+        if (r != -1) return r;
+    }
     {
         const int r = dwconv_mfma_launch(x, w, add, pool, y, B, H, W, C, KH, KW, PH, PW, flip, dtype, s);
         if (r != -1 || add || pool) return r;   // only the matrix-core kernel has the fused forms

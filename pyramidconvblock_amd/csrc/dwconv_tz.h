@@ -1,0 +1,473 @@
+// Depthwise convolution as a block-Toeplitz product on the dense matrix cores: forward and input gradient for
+// 16-bit types, stride 1, dilation 1, odd square filters up to 17 (the input gradient is the same kernel run on gy
+// with the 180-degree rotated filter and padding k-1-p).
+//
+// For one channel, a patch of 4 x 4 outputs is a product of the filter, spread out as a 16 x (K+3)(K+3) matrix
+//     A[(di,dj)][(r,s)] = w[r - di][s - dj]          (zero where the tap falls outside the filter)
+// with the patch's (K+3) x (K+3) input window as a vector.  v_mfma_f32_16x16x32_{bf16,f16} computes
+// D[m][n] += sum_k A[m][k] B[k][n] with m = one of the patch's 16 outputs, n = one of 16 patches and k running over
+// 32 window positions per instruction: 4 "k groups" of 8 consecutive columns of one window row, which is what one
+// lane holds (lane = n + 16 * group for B, m + 16 * group for A).  A window row is ICB = ceil((K+3)/8) groups wide,
+// so a patch takes NM = ceil((K+3) * ICB / 4) instructions (8 at K = 13: 169 of every 256 multiply-adds fall on a
+// real tap, on the pipe that runs at four times the rate of the 4x4x4 block form).  A depends on the channel only:
+// each wavefront owns CPW channels and keeps their A operands in registers for the whole kernel.
+//
+// The 16 patches of an instruction lie side by side (4 columns apart) in NI = 16 / NPC images, and a wavefront
+// walks down the rows four at a time.  Moving down by 4 rows shifts every B operand by ICB instructions, so the
+// operands live in a register ring: a step reads only the 4 new window rows from LDS (ICB operands of 16 bytes per
+// lane) for NM instructions.  That is what makes the kernel a stream: per step and channel 2 LDS reads, 8 MFMAs.
+//
+// A workgroup (8 wavefronts, CS = 8 CPW channels) owns a band of BR output rows x 4 NPC columns of NI images.  Its
+// input window is staged once in LDS, channel-major: xl[image][channel][row][column] as 16-bit values, so that 8
+// consecutive columns of a channel are 16 contiguous bytes.  Threads load 2 x 2 pixels x 8 channels (four 16-byte
+// loads), interleave column pairs with byte permutes and write dwords; the passes of this copy are requested two
+// ahead and committed only as far as the next step needs, so steps start while the lower rows are still on their
+// way and the loads, the MFMAs and the stores of a band overlap.  Results are rounded once, transposed through a
+// small double-buffered LDS tile (pixel-major, one dword of padding per 4 pixels keeps the 4-byte scatter free of
+// bank conflicts) and leave as 16-byte stores, one step behind the MFMAs.
+//
+// MODE 1 (input gradient of a tensor that was also average-pooled 2x2): y += add[i/2, j/2] / 4 in the store.
+// MODE 2 (forward): the 2x2 average pool of x is written to `pool` by the staging threads, which hold exactly the
+// four pixels of a pool window in registers (needs even padding, so that windows do not straddle threads).
+//
+// Zero entries of A multiply real pixels of the window (and the window is wider than K+3 where (K+3) % 8 != 0), so a
+// non-finite input value reaches outputs up to 3 + 8 ICB - (K+3) pixels beyond its K x K footprint as NaN.
+#pragma once
+#include <mutex>
+
+#include "common.h"
+#include "kernels.h"
+#include "tile_common.h"
+
+namespace pdw {
+
+typedef float tz_f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ tz_f32x4 mfma16(uint4 a, uint4 b, tz_f32x4 c, bf16_t) {
+    typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ tz_f32x4 mfma16(uint4 a, uint4 b, tz_f32x4 c, f16_t) {
+    typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), c, 0, 0, 0);
+}
+
+template <int K, int NPC, int CS>
+struct TzShape {
+    static constexpr int NT = 512, NWV = 8;
+    static constexpr int IC = K + 3;                  // window columns (and rows) of a 4 x 4 patch
+    static constexpr int ICB = (IC + 7) / 8;          // k groups per window row
+    static constexpr int NKG = IC * ICB;              // k groups of a patch
+    static constexpr int NM = (NKG + 3) / 4;          // MFMAs per patch (group of 16) and channel
+    static constexpr int PER = (NM + ICB - 1) / ICB;  // row groups (of 4 rows) an operand ring spans
+    static constexpr int RING = PER * ICB;            // operands in the ring
+    static constexpr int NI = 16 / NPC;               // images side by side in one instruction
+    static constexpr int TW = 4 * NPC;                // output columns of a workgroup
+    static constexpr int NH = CS / 8;                 // 8-channel pieces per pixel
+    static constexpr int CPW = CS / 8;                // channels per wavefront
+    static constexpr int WCOLS = 4 * (NPC - 1) + 8 * ICB;  // window columns the operands touch
+    static constexpr int RP = (2 * WCOLS + 7) / 8 * 8;     // bytes per window row of a channel
+    static constexpr int OPX = 2 * CS;                     // bytes per pixel of the result tile
+    static constexpr int OROWP = TW * OPX + NPC * 4;       // bytes per row of the result tile (4 per 4 pixels padding)
+    static constexpr int OLB = NI * 4 * OROWP;             // one result tile: 4 rows of every image
+    static constexpr int WTH = 4 * PER + 3, WTW = 8 * ICB + 4;  // zero-bordered filter table [channel][WTH][WTW]
+    static constexpr int WTB = CS * WTH * WTW * 2;
+    static constexpr int R2B = (2 * OLB > 2 * WTB ? 2 * OLB : 2 * WTB + 15) / 16 * 16;  // result tiles / two filter tables (shared)
+    static_assert(K % 2 == 1 && K >= 3 && K <= 17, "odd filters up to 17");
+    static_assert(NPC == 16 || NPC == 8, "patches per image row");
+    static_assert(CS == 8 || CS == 16, "channels per workgroup");
+    static constexpr int win_rows(int BR) { return BR + 4 * (PER - 1); }  // BR % 4 == 0
+    static constexpr int chp(int BR) {                                   // bytes per channel plane, = 8 mod 16
+        const int b = win_rows(BR) * RP;
+        return b % 16 == 8 ? b : b + 8;
+    }
+    static constexpr size_t lds_bytes(int BR) { return (size_t)NI * CS * chp(BR) + R2B; }
+};
+
+struct TzGeom {
+    int B, H, W, C;    // input extents
+    int OH, OW;        // output extents
+    int PH, PW;        // padding
+    int BR;            // output rows of a band (multiple of 4)
+    int nbands, ncolt, nslices;
+    int CHP;           // LDS bytes per channel plane
+    int flip;          // 1: 180-degree rotated filter (input gradient)
+    int AH, AW;        // extents of the half-resolution addend / pooled output
+};
+
+// 8 values of T: a + b / 4, rounded once more (what an accumulating pool gradient does to a stored tensor).
+template <typename T>
+__device__ __forceinline__ uint4 tz_add_quarter(uint4 a, uint4 b) {
+    union U {
+        uint4 u;
+        T t[8];
+    } ua, ub, uo;
+    ua.u = a, ub.u = b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) uo.t[i] = from_f32<T>(to_f32(ua.t[i]) + 0.25f * to_f32(ub.t[i]));
+    return uo.u;
+}
+
+template <typename T, int K, int NPC, int CS, int MODE>
+__global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, const T* __restrict__ w,
+                                                      const T* __restrict__ add, T* __restrict__ pool,
+                                                      T* __restrict__ y, const TzGeom g) {
+    using Sh = TzShape<K, NPC, CS>;
+    constexpr int NT = Sh::NT, ICB = Sh::ICB, NKG = Sh::NKG, NM = Sh::NM, PER = Sh::PER, RING = Sh::RING;
+    constexpr int NI = Sh::NI, TW = Sh::TW, NH = Sh::NH, CPW = Sh::CPW, RP = Sh::RP, OPX = Sh::OPX, OROWP = Sh::OROWP;
+    constexpr int OLB = Sh::OLB, WTH = Sh::WTH, WTW = Sh::WTW;
+    extern __shared__ uint32_t smem[];
+    char* const xl = reinterpret_cast<char*>(smem);        // [NI][CS] planes of CHP bytes: [row][column] of T
+    char* const r2 = xl + NI * CS * g.CHP;                 // filter table, then the two result tiles
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int sl = bid % g.nslices;
+    bid /= g.nslices;
+    const int ct = bid % g.ncolt;
+    bid /= g.ncolt;
+    const int band = bid % g.nbands, ig = bid / g.nbands;
+    const int c0 = sl * CS, ocol0 = ct * TW, orow0 = band * g.BR, b0 = ig * NI;
+    const int rows_valid = min(g.BR, g.OH - orow0), cols_valid = min(TW, g.OW - ocol0);
+    const int nsteps = (rows_valid + 3) >> 2;
+    const int NROWS = 4 * (nsteps + PER - 1);              // window rows the steps read
+    const int WCP = (4 * ((cols_valid + 3) / 4 - 1) + 8 * ICB) / 2;  // column pairs the used patches read
+    const long long img_in = (long long)g.H * g.W * g.C, img_out = (long long)g.OH * g.OW * g.C;
+
+    // ---- filter slice, 8 channels of a tap per load: requested before the window, so that waiting for it leaves
+    // the window's loads in flight
+    constexpr int NWL = (K * K * NH + NT - 1) / NT;
+    uint4 wval[NWL];
+#pragma unroll
+    for (int i = 0; i < NWL; ++i) {
+        const int idx = min(tid + i * NT, K * K * NH - 1);
+        wval[i] = *reinterpret_cast<const uint4*>(w + (idx / NH) * g.C + min(c0 + 8 * (idx % NH), g.C - 8));
+    }
+
+    // ---- staging.  The window arrives in passes of GP row groups (of 4 rows), requested two ahead into two
+    // register buffers; pass p is committed to LDS right before the first step that reads one of its rows.  A
+    // thread's item is (row pair of the pass, image, column pair cp, 8-channel piece h), h fastest, the same in
+    // every pass.
+    constexpr int GP = PER % 2 == 0 ? 2 : PER;                   // row groups per pass
+    constexpr int NLD = (2 * GP * NI * (Sh::WCOLS / 2) * NH + NT - 1) / NT;  // items per thread and pass
+    constexpr int P0 = (PER + GP - 1) / GP;                      // passes the first step needs
+    constexpr int UNR = PER % 2 == 0 ? (PER % 4 == 0 ? PER : 2 * PER) : 2 * PER;  // steps per trip: PER | UNR, 2 GP | UNR
+    static_assert(UNR % PER == 0 && UNR % (2 * GP) == 0 && P0 <= 2, "staging schedule");
+    // Loads go through a buffer descriptor over the workgroup's images: an offset past its end (an image beyond the
+    // batch, or one of the markers for a row / column / channel outside the tensor) reads as zero and moves no
+    // data, which is the zero padding.  NI * H * W * C < 2^29 elements (guarded on the host), so valid byte
+    // offsets stay below 2^30 and any sum with a marker stays past the end.
+    constexpr uint32_t kNoCol = 0x40000000u, kNoRow = 0x80000000u;
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(x + (long long)b0 * img_in), (short)0, (int)(min(NI, g.B - b0) * img_in * 2), 0x00020000);
+    auto xload = [&](uint32_t off) {
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (int)off, 0, 0);
+        return make_uint4(v.x, v.y, v.z, v.w);
+    };
+    uint32_t icol[NLD][2];  // byte offsets of the item's two columns (image and channel piece included), or kNoCol
+    int irpw[NLD];          // row pair within a pass, -1: no item
+    int idst[NLD];          // LDS byte offset of the item in pass 0
+#pragma unroll
+    for (int l = 0; l < NLD; ++l) {
+        const int idx = tid + l * NT;
+        const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI, rpw = idx / NH / WCP / NI;
+        irpw[l] = rpw < 2 * GP ? rpw : -1;
+        const int ic = ocol0 - g.PW + 2 * cp;
+        const bool any = c0 + 8 * h < g.C && rpw < 2 * GP;
+        const uint32_t ioff = (uint32_t)img * (uint32_t)img_in + (uint32_t)(c0 + 8 * h);
+        icol[l][0] = any && ic >= 0 && ic < g.W ? (ioff + (uint32_t)(ic * g.C)) * 2u : kNoCol;
+        icol[l][1] = any && ic + 1 >= 0 && ic + 1 < g.W ? (ioff + (uint32_t)((ic + 1) * g.C)) * 2u : kNoCol;
+        idst[l] = (img * CS + 8 * h) * g.CHP + (2 * min(rpw, 2 * GP - 1)) * RP + 4 * cp;
+    }
+    uint4 buf[2][NLD][4];
+    auto issue = [&](uint4 (&bf)[NLD][4], int pass) {  // rows beyond the window read nothing
+#pragma unroll
+        for (int l = 0; l < NLD; ++l) {
+            const int wr = 4 * GP * pass + 2 * max(irpw[l], 0);  // window row
+            const int ir = orow0 - g.PH + wr;
+            const uint32_t r0 = wr < NROWS && ir >= 0 && ir < g.H ? (uint32_t)(ir * g.W * g.C) * 2u : kNoRow;
+            const uint32_t r1 = wr < NROWS && ir + 1 >= 0 && ir + 1 < g.H ? (uint32_t)((ir + 1) * g.W * g.C) * 2u : kNoRow;
+            bf[l][0] = xload(r0 + icol[l][0]);
+            bf[l][1] = xload(r0 + icol[l][1]);
+            bf[l][2] = xload(r1 + icol[l][0]);
+            bf[l][3] = xload(r1 + icol[l][1]);
+        }
+    };
+    auto commit = [&](const uint4 (&bf)[NLD][4], int pass) {
+#pragma unroll
+        for (int l = 0; l < NLD; ++l) {
+            const int wr = 4 * GP * pass + 2 * irpw[l];
+            if (irpw[l] >= 0 && wr < NROWS) {
+                const uint32_t a0[4] = {bf[l][0].x, bf[l][0].y, bf[l][0].z, bf[l][0].w};
+                const uint32_t a1[4] = {bf[l][1].x, bf[l][1].y, bf[l][1].z, bf[l][1].w};
+                const uint32_t a2[4] = {bf[l][2].x, bf[l][2].y, bf[l][2].z, bf[l][2].w};
+                const uint32_t a3[4] = {bf[l][3].x, bf[l][3].y, bf[l][3].z, bf[l][3].w};
+                char* dst = xl + idst[l] + pass * (4 * GP * RP);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    // column pair of channels 2j and 2j+1, the item's two rows
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j) * g.CHP) = __builtin_amdgcn_perm(a1[j], a0[j], 0x05040100u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * g.CHP) = __builtin_amdgcn_perm(a1[j], a0[j], 0x07060302u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x05040100u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
+                }
+                if constexpr (MODE == 2) {
+                    // the thread holds one window of the 2x2 pool (H, W, PH, PW even): the band that owns these rows
+                    // writes it
+                    const int idx = tid + l * NT;
+                    const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI;
+                    const int ir = orow0 - g.PH + wr, ic = ocol0 - g.PW + 2 * cp;
+                    if (b0 + img < g.B && c0 + 8 * h < g.C && ir >= orow0 && ir < orow0 + rows_valid && ic >= ocol0 &&
+                        ic < ocol0 + cols_valid) {
+                        union U {
+                            uint4 u;
+                            T t[8];
+                        } p0, p1, p2, p3, o;
+                        p0.u = bf[l][0], p1.u = bf[l][1], p2.u = bf[l][2], p3.u = bf[l][3];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            o.t[e] = from_f32<T>((((to_f32(p0.t[e]) + to_f32(p1.t[e])) + to_f32(p2.t[e])) + to_f32(p3.t[e])) * 0.25f);
+                        *reinterpret_cast<uint4*>(pool + (((long long)(b0 + img) * g.AH + (ir >> 1)) * g.AW + (ic >> 1)) * g.C + c0 + 8 * h) = o.u;
+                    }
+                }
+            }
+        }
+    };
+    issue(buf[0], 0);
+    issue(buf[1], 1);
+
+    // LDS accesses of this wavefront complete, then the workgroup barrier; global loads and stores stay in flight
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // ---- filter table wt[copy][channel][3 + u][3 + v] (rotated for the input gradient), zero elsewhere; copy 1 is
+    // the same table one element to the left, so that a run of 8 values that starts at an odd index is dword
+    // aligned in it
+    constexpr int WTC = CS * WTH * WTW;  // elements per copy
+    unsigned short* const wt = reinterpret_cast<unsigned short*>(r2);
+    {
+        uint4* wz = reinterpret_cast<uint4*>(r2);
+        for (int i = tid; i < (2 * Sh::WTB + 15) / 16; i += NT) wz[i] = make_uint4(0u, 0u, 0u, 0u);
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < NWL; ++i) {
+            const int idx = tid + i * NT;
+            const int h = idx % NH, uv = idx / NH;
+            const int u = uv / K, v = uv - u * K;
+            if (idx < K * K * NH && c0 + 8 * h < g.C) {
+                const uint32_t d[4] = {wval[i].x, wval[i].y, wval[i].z, wval[i].w};
+                const int uu = g.flip ? K - 1 - u : u, vv = g.flip ? K - 1 - v : v;
+                unsigned short* wp = wt + ((8 * h) * WTH + 3 + uu) * WTW + 3 + vv;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const unsigned short val = (unsigned short)((d[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+                    wp[e * WTH * WTW] = val;
+                    wp[WTC + e * WTH * WTW - 1] = val;
+                }
+            }
+        }
+        lds_barrier();
+    }
+    // ---- this wavefront's A operands: lane = (m = 4 di + dj, k group kg); operand t covers k groups 4t .. 4t+3
+    const int ln = lane & 15, kg = lane >> 4;
+    uint4 A[CPW][NM];
+    {
+        const int di = ln >> 2, dj = ln & 3;
+#pragma unroll
+        for (int q = 0; q < CPW; ++q) {
+#pragma unroll
+            for (int t = 0; t < NM; ++t) {
+                const int kap = 4 * t + kg;
+                const int r = kap / ICB, cb = kap - r * ICB;
+                const int v0 = 8 * cb - dj + 3;  // first of the lane's 8 table columns
+                const uint32_t* wp = reinterpret_cast<const uint32_t*>(
+                    wt + (v0 & 1) * WTC + ((wv * CPW + q) * WTH + r - di + 3) * WTW + (v0 & ~1));
+                const bool real = kap < NKG;
+                A[q][t] = make_uint4(real ? wp[0] : 0u, real ? wp[1] : 0u, real ? wp[2] : 0u, real ? wp[3] : 0u);
+            }
+        }
+    }
+
+    // ---- per-lane addresses
+    // B operands: lane = (patch n = image * NPC + pc, k group kg); operand a = ICB * rowgroup + i covers window rows
+    // 4 rowgroup + (4i + kg) / ICB, column block (4i + kg) % ICB
+    const int pimg = ln / NPC, pc = ln % NPC;
+    const char* xb[CPW][ICB];
+#pragma unroll
+    for (int q = 0; q < CPW; ++q)
+#pragma unroll
+        for (int i = 0; i < ICB; ++i)
+            xb[q][i] = xl + (pimg * CS + wv * CPW + q) * g.CHP + ((4 * i + kg) / ICB) * RP + ((4 * i + kg) % ICB) * 16 + pc * 8;
+    // results: register r of a lane is output (row kg, column 4 pc + r) of patch n
+    char* const olw = r2 + (pimg * 4 + kg) * OROWP + (4 * pc) * OPX + pc * 4 + 2 * (wv * CPW);
+    // store phase: one 16-byte piece (image, row, column, h) of a result tile per thread
+    const int sh = tid % NH, scol = (tid / NH) % TW, srow = (tid / NH / TW) % 4, simg = tid / NH / TW / 4;
+    const bool s_ok = simg < NI && b0 + simg < g.B && scol < cols_valid && c0 + 8 * sh < g.C;
+    const char* const olr = r2 + (min(simg, NI - 1) * 4 + srow) * OROWP + scol * OPX + (scol >> 2) * 4 + 16 * sh;
+    T* const ybase = y + (b0 + min(simg, NI - 1)) * img_out + ((long long)(orow0 + srow) * g.OW + ocol0 + scol) * g.C + c0 + 8 * sh;
+    uint4 addv = make_uint4(0u, 0u, 0u, 0u);
+    auto add_fetch = [&](int s) {
+        if constexpr (MODE == 1) {
+            const int b = min(b0 + min(simg, NI - 1), g.B - 1);
+            const int ar = min((orow0 + 4 * s + srow) >> 1, g.AH - 1), ac = min((ocol0 + scol) >> 1, g.AW - 1);
+            addv = *reinterpret_cast<const uint4*>(add + (((long long)b * g.AH + ar) * g.AW + ac) * g.C + min(c0 + 8 * sh, g.C - 8));
+        }
+    };
+    auto store = [&](int s) {
+        const char* src = olr + (s & 1) * OLB;
+        uint4 v;
+        v.x = *reinterpret_cast<const uint32_t*>(src), v.y = *reinterpret_cast<const uint32_t*>(src + 4);
+        v.z = *reinterpret_cast<const uint32_t*>(src + 8), v.w = *reinterpret_cast<const uint32_t*>(src + 12);
+        if (s_ok && 4 * s + srow < rows_valid) {
+            if constexpr (MODE == 1) v = tz_add_quarter<T>(v, addv);
+            *reinterpret_cast<uint4*>(ybase + (long long)(4 * s) * g.OW * g.C) = v;
+        }
+    };
+
+    uint4 ring[CPW][RING];
+    auto load_group = [&](int slotgroup, int byteoff) {  // window rows byteoff / RP .. + 3 -> ICB operands per channel
+#pragma unroll
+        for (int q = 0; q < CPW; ++q)
+#pragma unroll
+            for (int i = 0; i < ICB; ++i) {
+                const uint2 lo = *reinterpret_cast<const uint2*>(xb[q][i] + byteoff);
+                const uint2 hi = *reinterpret_cast<const uint2*>(xb[q][i] + byteoff + 8);
+                ring[q][slotgroup * ICB + i] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            }
+    };
+    // the passes the first step reads, then the ring's first PER - 1 row groups
+    commit(buf[0], 0);
+    issue(buf[0], 2);
+    if constexpr (P0 == 2) {
+        commit(buf[1], 1);
+        issue(buf[1], 3);
+    }
+    lds_barrier();
+#pragma unroll
+    for (int j = 0; j < PER - 1; ++j) load_group(j, 4 * j * RP);
+    for (int s0 = 0; s0 < nsteps; s0 += UNR) {
+#pragma unroll
+        for (int j = 0; j < UNR; ++j) {
+            const int s = s0 + j;
+            if (s < nsteps) {
+                if ((j + PER - 1) % GP == 0) {  // the step's last row group opens a new pass (j is unrolled)
+                    const int bi = ((j + PER - 1) / GP) % 2;
+                    const int pass = (s + PER - 1) / GP;
+                    if (pass >= P0) {
+                        commit(buf[bi], pass);
+                        issue(buf[bi], pass + 2);
+                    }
+                }
+                lds_barrier();  // the step's window rows are in LDS; the previous result tile is complete
+                if (s > 0) store(s - 1);
+                add_fetch(s);
+                load_group((j + PER - 1) % PER, 4 * (j + PER - 1) * RP);
+                tz_f32x4 acc[CPW];
+#pragma unroll
+                for (int q = 0; q < CPW; ++q) acc[q] = tz_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < NM; ++t)
+#pragma unroll
+                    for (int q = 0; q < CPW; ++q) acc[q] = mfma16(A[q][t], ring[q][(ICB * j + t) % RING], acc[q], T());
+                char* dst = olw + (s & 1) * OLB;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if constexpr (CPW == 2) {
+                        union {
+                            T t[2];
+                            uint32_t u;
+                        } o;
+                        o.t[0] = from_f32<T>(acc[0][r]), o.t[1] = from_f32<T>(acc[1][r]);
+                        *reinterpret_cast<uint32_t*>(dst + r * OPX) = o.u;
+                    } else {
+                        *reinterpret_cast<T*>(dst + r * OPX) = from_f32<T>(acc[0][r]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < CPW; ++q)
+#pragma unroll
+            for (int i = 0; i < ICB; ++i) xb[q][i] += 4 * UNR * RP;
+    }
+    lds_barrier();
+    store(nsteps - 1);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Host side
+
+// Band height: the choice with the shortest estimated run, rounds of workgroups over 256 compute units times the
+// rows a workgroup moves (window rows plus a fixed cost of about 8 rows' worth).
+template <int K, int NPC, int CS>
+static int tz_pick_band(int B, int OH, int OW, int C) {
+    using Sh = TzShape<K, NPC, CS>;
+    const long long per_band = (long long)cdiv(B, Sh::NI) * cdiv(C, CS) * cdiv(OW, Sh::TW);
+    int best = 0;
+    double best_cost = 0;
+    for (int br = 4; br <= ((OH + 3) / 4) * 4; br += 4) {
+        if (Sh::lds_bytes(br) > 160 * 1024) break;
+        const long long wgs = per_band * cdiv(OH, br);
+        const double cost = (double)cdiv(wgs, 256) * (Sh::win_rows(br) + 8);
+        if (best == 0 || cost <= best_cost) best = br, best_cost = cost;
+    }
+    return best;
+}
+
+template <typename T, int K, int NPC, int CS>
+static int launch_tz(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
+                     int PH, int PW, bool flip, hipStream_t s) {
+    using Sh = TzShape<K, NPC, CS>;
+    TzGeom g;
+    g.B = B, g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0;
+    g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
+    g.AH = add ? g.OH / 2 : H / 2, g.AW = add ? g.OW / 2 : W / 2;
+    if ((long long)H * W * C * Sh::NI > 0x1fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL) return -1;
+    g.BR = tz_pick_band<K, NPC, CS>(B, g.OH, g.OW, C);
+    if (g.BR < 4) return -1;
+    g.nbands = cdiv(g.OH, g.BR), g.ncolt = cdiv(g.OW, Sh::TW), g.nslices = cdiv(C, CS);
+    g.CHP = Sh::chp(g.BR);
+    const long long nblocks = (long long)cdiv(B, Sh::NI) * g.nbands * g.ncolt * g.nslices;
+    if (nblocks > 0x7fffffffLL) return -1;
+    const size_t lds = Sh::lds_bytes(g.BR);
+    const int mode = add ? 1 : (pool ? 2 : 0);
+    auto kern = mode == 1 ? dwconv_tz_k<T, K, NPC, CS, 1> : (mode == 2 ? dwconv_tz_k<T, K, NPC, CS, 2> : dwconv_tz_k<T, K, NPC, CS, 0>);
+    static std::once_flag attr_once[3];
+    std::call_once(attr_once[mode], [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(Sh::NT), lds, s, (const T*)x, (const T*)w, (const T*)add,
+                       (T*)pool, (T*)y, g);
+    return check_launch("dwconv_tz");
+}
+
+// -1: not covered (the caller falls back to the other kernels).
+template <typename T, int K>
+static int launch_tz_best(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
+                          int PH, int PW, bool flip, hipStream_t s) {
+    const int OH = H + 2 * PH - K + 1, OW = W + 2 * PW - K + 1;
+    if (OH < 1 || OW < 1 || C % 8 != 0 || B < 1) return -1;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(w) & 15) != 0)
+        return -1;
+    if (add && ((OH | OW) & 1 || (reinterpret_cast<uintptr_t>(add) & 15) != 0)) return -1;
+    if (pool && (add || flip || OH != H || OW != W || ((H | W | PH | PW) & 1) || (reinterpret_cast<uintptr_t>(pool) & 15) != 0))
+        return -1;
+    // patches per image row: the width whose padding of (columns x images) is smaller, wider on ties
+    const long long pad16 = (long long)cdiv(OW, 64) * 64 * B, pad8 = (long long)cdiv(OW, 32) * 32 * cdiv(B, 2) * 2;
+    const bool wide_tile = pad16 <= pad8;
+    // 16 channels per workgroup (two per wavefront) while the operand registers allow it, else 8
+    constexpr int CS = (2 * 4 * TzShape<K, 16, 16>::NM + 2 * 4 * TzShape<K, 16, 16>::RING) <= 160 ? 16 : 8;
+    if (wide_tile) return launch_tz<T, K, 16, CS>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+    return launch_tz<T, K, 8, CS>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+}
+
+template <int K>
+static int launch_tz_dtype(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
+                           int PH, int PW, bool flip, int dtype, hipStream_t s) {
+    switch (dtype) {
+        case kF16: return launch_tz_best<f16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+        case kBF16: return launch_tz_best<bf16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+        default: return -1;
+    }
+}
+
+}  // namespace pdw
