@@ -72,7 +72,7 @@ struct TzShape {
     static constexpr int OLB = NI * 4 * OROWP;             // one result tile: 4 rows of every image
     static constexpr int WTH = 4 * PER + 3, WTW = 8 * ICB + 4;  // zero-bordered filter table [channel][WTH][WTW]
     static constexpr int WTB = CS * WTH * WTW * 2;
-    static constexpr int R2B = (2 * OLB > 2 * WTB ? 2 * OLB : 2 * WTB + 15) / 16 * 16;  // result tiles / two filter tables (shared)
+    static constexpr int R2B = (4 * OLB > 2 * WTB ? 4 * OLB : 2 * WTB + 15) / 16 * 16;  // 4 result tiles / two filter tables (shared)
     static_assert(K % 2 == 1 && K >= 3 && K <= 17, "odd filters up to 17");
     static_assert(NPC == 16 || NPC == 8, "patches per image row");
     static_assert(CS == 8 || CS == 16, "channels per workgroup");
@@ -144,15 +144,16 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
         wval[i] = *reinterpret_cast<const uint4*>(w + (idx / NH) * g.C + min(c0 + 8 * (idx % NH), g.C - 8));
     }
 
-    // ---- staging.  The window arrives in passes of GP row groups (of 4 rows), requested two ahead into two
-    // register buffers; pass p is committed to LDS right before the first step that reads one of its rows.  A
-    // thread's item is (row pair of the pass, image, column pair cp, 8-channel piece h), h fastest, the same in
-    // every pass.
-    constexpr int GP = PER % 2 == 0 ? 2 : PER;                   // row groups per pass
-    constexpr int NLD = (2 * GP * NI * (Sh::WCOLS / 2) * NH + NT - 1) / NT;  // items per thread and pass
-    constexpr int P0 = (PER + GP - 1) / GP;                      // passes the first step needs
-    constexpr int UNR = PER % 2 == 0 ? (PER % 4 == 0 ? PER : 2 * PER) : 2 * PER;  // steps per trip: PER | UNR, 2 GP | UNR
-    static_assert(UNR % PER == 0 && UNR % (2 * GP) == 0 && P0 <= 2, "staging schedule");
+    // ---- staging.  The window arrives in passes, requested two ahead into two register buffers.  Passes 0 and 1
+    // are halves of the PER + 1 row groups (of 4 rows) the first step reads, every later pass the two row groups the
+    // next step adds, so step f is preceded by the commit of pass f + 1.  A thread's item is (row pair of the pass,
+    // image, column pair cp, 8-channel piece h), h fastest, the same in every pass.
+    constexpr int RP01 = PER + 1;                                // row pairs of pass 0 and of pass 1
+    constexpr int RPMAX = RP01 > 4 ? RP01 : 4;
+    constexpr int NLD = (RPMAX * NI * (Sh::WCOLS / 2) * NH + NT - 1) / NT;  // items per thread and pass
+    constexpr int UNRF = PER % 4 == 0 ? PER / 2 : (PER % 2 == 0 ? PER : 2 * PER);  // steps per trip: even, PER | 2 UNRF
+    auto first_rowpair = [&](int pass) { return pass < 2 ? pass * RP01 : 2 * RP01 + 4 * (pass - 2); };
+    auto rowpair_count = [&](int pass) { return pass < 2 ? RP01 : 4; };
     // Loads go through a buffer descriptor over the workgroup's images: an offset past its end (an image beyond the
     // batch, or one of the markers for a row / column / channel outside the tensor) reads as zero and moves no
     // data, which is the zero padding.  NI * H * W * C < 2^29 elements (guarded on the host), so valid byte
@@ -160,34 +161,42 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     constexpr uint32_t kNoCol = 0x40000000u, kNoRow = 0x80000000u;
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<T*>(x + (long long)b0 * img_in), (short)0, (int)(min(NI, g.B - b0) * img_in * 2), 0x00020000);
-    auto xload = [&](uint32_t off) {
+    auto xload_from = [&](const __amdgpu_buffer_rsrc_t& r, uint32_t off) {
         typedef unsigned v4u __attribute__((ext_vector_type(4)));
-        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, (int)off, 0, 0);
+        const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
         return make_uint4(v.x, v.y, v.z, v.w);
     };
+    auto xload = [&](uint32_t off) { return xload_from(xrsrc, off); };
     uint32_t icol[NLD][2];  // byte offsets of the item's two columns (image and channel piece included), or kNoCol
-    int irpw[NLD];          // row pair within a pass, -1: no item
-    int idst[NLD];          // LDS byte offset of the item in pass 0
+    int irpw[NLD];          // row pair within a pass
+    int idst[NLD];          // LDS byte offset of the item in a pass that starts at window row 0
 #pragma unroll
     for (int l = 0; l < NLD; ++l) {
         const int idx = tid + l * NT;
         const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI, rpw = idx / NH / WCP / NI;
-        irpw[l] = rpw < 2 * GP ? rpw : -1;
+        irpw[l] = rpw;
         const int ic = ocol0 - g.PW + 2 * cp;
-        const bool any = c0 + 8 * h < g.C && rpw < 2 * GP;
+        const bool any = c0 + 8 * h < g.C && rpw < RPMAX;
         const uint32_t ioff = (uint32_t)img * (uint32_t)img_in + (uint32_t)(c0 + 8 * h);
         icol[l][0] = any && ic >= 0 && ic < g.W ? (ioff + (uint32_t)(ic * g.C)) * 2u : kNoCol;
         icol[l][1] = any && ic + 1 >= 0 && ic + 1 < g.W ? (ioff + (uint32_t)((ic + 1) * g.C)) * 2u : kNoCol;
-        idst[l] = (img * CS + 8 * h) * g.CHP + (2 * min(rpw, 2 * GP - 1)) * RP + 4 * cp;
+        idst[l] = (img * CS + 8 * h) * g.CHP + (2 * min(rpw, RPMAX - 1)) * RP + 4 * cp;
     }
+    // the 2x2 average pool of x (MODE 2) leaves through a buffer descriptor as well: a store past its end is dropped
+    __amdgpu_buffer_rsrc_t prsrc = xrsrc;
+    if constexpr (MODE == 2)
+        prsrc = __builtin_amdgcn_make_buffer_rsrc(pool + (long long)b0 * g.AH * g.AW * g.C, (short)0,
+                                                  (int)((long long)min(NI, g.B - b0) * g.AH * g.AW * g.C * 2), 0x00020000);
     uint4 buf[2][NLD][4];
-    auto issue = [&](uint4 (&bf)[NLD][4], int pass) {  // rows beyond the window read nothing
+    auto issue = [&](uint4 (&bf)[NLD][4], int pass) {  // rows beyond the pass or the window read nothing
+        const int wr0 = 2 * first_rowpair(pass), nrp = rowpair_count(pass);
 #pragma unroll
         for (int l = 0; l < NLD; ++l) {
-            const int wr = 4 * GP * pass + 2 * max(irpw[l], 0);  // window row
+            const int wr = wr0 + 2 * irpw[l];  // window row
             const int ir = orow0 - g.PH + wr;
-            const uint32_t r0 = wr < NROWS && ir >= 0 && ir < g.H ? (uint32_t)(ir * g.W * g.C) * 2u : kNoRow;
-            const uint32_t r1 = wr < NROWS && ir + 1 >= 0 && ir + 1 < g.H ? (uint32_t)((ir + 1) * g.W * g.C) * 2u : kNoRow;
+            const bool ok = irpw[l] < nrp && wr < NROWS;
+            const uint32_t r0 = ok && ir >= 0 && ir < g.H ? (uint32_t)(ir * g.W * g.C) * 2u : kNoRow;
+            const uint32_t r1 = ok && ir + 1 >= 0 && ir + 1 < g.H ? (uint32_t)((ir + 1) * g.W * g.C) * 2u : kNoRow;
             bf[l][0] = xload(r0 + icol[l][0]);
             bf[l][1] = xload(r0 + icol[l][1]);
             bf[l][2] = xload(r1 + icol[l][0]);
@@ -195,15 +204,16 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
         }
     };
     auto commit = [&](const uint4 (&bf)[NLD][4], int pass) {
+        const int wr0 = 2 * first_rowpair(pass), nrp = rowpair_count(pass);
 #pragma unroll
         for (int l = 0; l < NLD; ++l) {
-            const int wr = 4 * GP * pass + 2 * irpw[l];
-            if (irpw[l] >= 0 && wr < NROWS) {
+            const int wr = wr0 + 2 * irpw[l];
+            if (irpw[l] < nrp && wr < NROWS) {
                 const uint32_t a0[4] = {bf[l][0].x, bf[l][0].y, bf[l][0].z, bf[l][0].w};
                 const uint32_t a1[4] = {bf[l][1].x, bf[l][1].y, bf[l][1].z, bf[l][1].w};
                 const uint32_t a2[4] = {bf[l][2].x, bf[l][2].y, bf[l][2].z, bf[l][2].w};
                 const uint32_t a3[4] = {bf[l][3].x, bf[l][3].y, bf[l][3].z, bf[l][3].w};
-                char* dst = xl + idst[l] + pass * (4 * GP * RP);
+                char* dst = xl + idst[l] + wr0 * RP;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     // column pair of channels 2j and 2j+1, the item's two rows
@@ -212,25 +222,25 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
                     *reinterpret_cast<uint32_t*>(dst + (2 * j) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x05040100u);
                     *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
                 }
-                if constexpr (MODE == 2) {
-                    // the thread holds one window of the 2x2 pool (H, W, PH, PW even): the band that owns these rows
-                    // writes it
-                    const int idx = tid + l * NT;
-                    const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI;
-                    const int ir = orow0 - g.PH + wr, ic = ocol0 - g.PW + 2 * cp;
-                    if (b0 + img < g.B && c0 + 8 * h < g.C && ir >= orow0 && ir < orow0 + rows_valid && ic >= ocol0 &&
-                        ic < ocol0 + cols_valid) {
-                        union U {
-                            uint4 u;
-                            T t[8];
-                        } p0, p1, p2, p3, o;
-                        p0.u = bf[l][0], p1.u = bf[l][1], p2.u = bf[l][2], p3.u = bf[l][3];
+            }
+            if constexpr (MODE == 2) {
+                // the thread holds one window of the 2x2 pool (H, W, PH, PW even): the band that owns these rows writes it
+                const int idx = tid + l * NT;
+                const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI;
+                const int ir = orow0 - g.PH + wr, ic = ocol0 - g.PW + 2 * cp;
+                const bool mine = irpw[l] < nrp && c0 + 8 * h < g.C && ir >= orow0 && ir < orow0 + rows_valid && ic >= ocol0 &&
+                                  ic < ocol0 + cols_valid;
+                union U {
+                    uint4 u;
+                    T t[8];
+                } p0, p1, p2, p3, o;
+                p0.u = bf[l][0], p1.u = bf[l][1], p2.u = bf[l][2], p3.u = bf[l][3];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            o.t[e] = from_f32<T>((((to_f32(p0.t[e]) + to_f32(p1.t[e])) + to_f32(p2.t[e])) + to_f32(p3.t[e])) * 0.25f);
-                        *reinterpret_cast<uint4*>(pool + (((long long)(b0 + img) * g.AH + (ir >> 1)) * g.AW + (ic >> 1)) * g.C + c0 + 8 * h) = o.u;
-                    }
-                }
+                for (int e = 0; e < 8; ++e)
+                    o.t[e] = from_f32<T>((((to_f32(p0.t[e]) + to_f32(p1.t[e])) + to_f32(p2.t[e])) + to_f32(p3.t[e])) * 0.25f);
+                const uint32_t off = mine ? (uint32_t)(((img * g.AH + (ir >> 1)) * g.AW + (ic >> 1)) * g.C + c0 + 8 * h) * 2u : kNoRow;
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                __builtin_amdgcn_raw_buffer_store_b128(v4u{o.u.x, o.u.y, o.u.z, o.u.w}, prsrc, (int)off, 0, 0);
             }
         }
     };
@@ -300,98 +310,145 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
             xb[q][i] = xl + (pimg * CS + wv * CPW + q) * g.CHP + ((4 * i + kg) / ICB) * RP + ((4 * i + kg) % ICB) * 16 + pc * 8;
     // results: register r of a lane is output (row kg, column 4 pc + r) of patch n
     char* const olw = r2 + (pimg * 4 + kg) * OROWP + (4 * pc) * OPX + pc * 4 + 2 * (wv * CPW);
-    // store phase: one 16-byte piece (image, row, column, h) of a result tile per thread
+    // store phase: one 16-byte piece (image, row, column, h) of each 4-row result tile per thread, through buffer
+    // descriptors (an offset past the end: nothing stored / zero loaded), so that no vector memory instruction of the
+    // kernel sits behind a branch and the in-flight counts the staging waits rely on stay exact
     const int sh = tid % NH, scol = (tid / NH) % TW, srow = (tid / NH / TW) % 4, simg = tid / NH / TW / 4;
-    const bool s_ok = simg < NI && b0 + simg < g.B && scol < cols_valid && c0 + 8 * sh < g.C;
+    const bool s_ok = simg < NI && scol < cols_valid && c0 + 8 * sh < g.C;
     const char* const olr = r2 + (min(simg, NI - 1) * 4 + srow) * OROWP + scol * OPX + (scol >> 2) * 4 + 16 * sh;
-    T* const ybase = y + (b0 + min(simg, NI - 1)) * img_out + ((long long)(orow0 + srow) * g.OW + ocol0 + scol) * g.C + c0 + 8 * sh;
-    uint4 addv = make_uint4(0u, 0u, 0u, 0u);
-    auto add_fetch = [&](int s) {
+    const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        y + (long long)b0 * img_out, (short)0, (int)(min(NI, g.B - b0) * img_out * 2), 0x00020000);
+    const uint32_t ycol = (uint32_t)simg * (uint32_t)img_out + (uint32_t)((ocol0 + scol) * g.C + c0 + 8 * sh);
+    __amdgpu_buffer_rsrc_t arsrc = xrsrc;
+    if constexpr (MODE == 1)
+        arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(add + (long long)b0 * g.AH * g.AW * g.C), (short)0,
+                                                  (int)((long long)min(NI, g.B - b0) * g.AH * g.AW * g.C * 2), 0x00020000);
+    uint4 addv[2] = {make_uint4(0u, 0u, 0u, 0u), make_uint4(0u, 0u, 0u, 0u)};
+    auto add_fetch = [&](int f) {   // the addends of step f's two tiles
         if constexpr (MODE == 1) {
-            const int b = min(b0 + min(simg, NI - 1), g.B - 1);
-            const int ar = min((orow0 + 4 * s + srow) >> 1, g.AH - 1), ac = min((ocol0 + scol) >> 1, g.AW - 1);
-            addv = *reinterpret_cast<const uint4*>(add + (((long long)b * g.AH + ar) * g.AW + ac) * g.C + min(c0 + 8 * sh, g.C - 8));
+#pragma unroll
+            for (int gi = 0; gi < 2; ++gi) {
+                const int row = 4 * (2 * f + gi) + srow;
+                const bool ok = s_ok && row < rows_valid;
+                const uint32_t off = ok ? (uint32_t)(((simg * g.AH + ((orow0 + row) >> 1)) * g.AW + ((ocol0 + scol) >> 1)) * g.C + c0 + 8 * sh) * 2u : kNoRow;
+                addv[gi] = xload_from(arsrc, off);
+            }
         }
     };
-    auto store = [&](int s) {
-        const char* src = olr + (s & 1) * OLB;
-        uint4 v;
-        v.x = *reinterpret_cast<const uint32_t*>(src), v.y = *reinterpret_cast<const uint32_t*>(src + 4);
-        v.z = *reinterpret_cast<const uint32_t*>(src + 8), v.w = *reinterpret_cast<const uint32_t*>(src + 12);
-        if (s_ok && 4 * s + srow < rows_valid) {
-            if constexpr (MODE == 1) v = tz_add_quarter<T>(v, addv);
-            *reinterpret_cast<uint4*>(ybase + (long long)(4 * s) * g.OW * g.C) = v;
+    auto store = [&](int f) {   // f = -1: nothing
+#pragma unroll
+        for (int gi = 0; gi < 2; ++gi) {
+            const char* src = olr + (2 * (f & 1) + gi) * OLB;
+            uint4 v;
+            v.x = *reinterpret_cast<const uint32_t*>(src), v.y = *reinterpret_cast<const uint32_t*>(src + 4);
+            v.z = *reinterpret_cast<const uint32_t*>(src + 8), v.w = *reinterpret_cast<const uint32_t*>(src + 12);
+            if constexpr (MODE == 1) v = tz_add_quarter<T>(v, addv[gi]);
+            const int row = 4 * (2 * f + gi) + srow;
+            const bool ok = s_ok && f >= 0 && row < rows_valid;
+            const uint32_t off = ok ? (ycol + (uint32_t)((orow0 + row) * g.OW * g.C)) * 2u : kNoRow;
+            typedef unsigned v4u __attribute__((ext_vector_type(4)));
+            __builtin_amdgcn_raw_buffer_store_b128(v4u{v.x, v.y, v.z, v.w}, yrsrc, (int)off, 0, 0);
         }
     };
 
     uint4 ring[CPW][RING];
+    auto read16 = [&](const char* p) {
+        const uint2 lo = *reinterpret_cast<const uint2*>(p), hi = *reinterpret_cast<const uint2*>(p + 8);
+        return make_uint4(lo.x, lo.y, hi.x, hi.y);
+    };
     auto load_group = [&](int slotgroup, int byteoff) {  // window rows byteoff / RP .. + 3 -> ICB operands per channel
 #pragma unroll
         for (int q = 0; q < CPW; ++q)
 #pragma unroll
-            for (int i = 0; i < ICB; ++i) {
-                const uint2 lo = *reinterpret_cast<const uint2*>(xb[q][i] + byteoff);
-                const uint2 hi = *reinterpret_cast<const uint2*>(xb[q][i] + byteoff + 8);
-                ring[q][slotgroup * ICB + i] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-            }
+            for (int i = 0; i < ICB; ++i) ring[q][slotgroup * ICB + i] = read16(xb[q][i] + byteoff);
     };
     // the passes the first step reads, then the ring's first PER - 1 row groups
     commit(buf[0], 0);
     issue(buf[0], 2);
-    if constexpr (P0 == 2) {
-        commit(buf[1], 1);
-        issue(buf[1], 3);
-    }
+    commit(buf[1], 1);
+    issue(buf[1], 3);
     lds_barrier();
 #pragma unroll
     for (int j = 0; j < PER - 1; ++j) load_group(j, 4 * j * RP);
-    for (int s0 = 0; s0 < nsteps; s0 += UNR) {
-#pragma unroll
-        for (int j = 0; j < UNR; ++j) {
-            const int s = s0 + j;
-            if (s < nsteps) {
-                if ((j + PER - 1) % GP == 0) {  // the step's last row group opens a new pass (j is unrolled)
-                    const int bi = ((j + PER - 1) / GP) % 2;
-                    const int pass = (s + PER - 1) / GP;
-                    if (pass >= P0) {
-                        commit(buf[bi], pass);
-                        issue(buf[bi], pass + 2);
-                    }
-                }
-                lds_barrier();  // the step's window rows are in LDS; the previous result tile is complete
-                if (s > 0) store(s - 1);
-                add_fetch(s);
-                load_group((j + PER - 1) % PER, 4 * (j + PER - 1) * RP);
-                tz_f32x4 acc[CPW];
-#pragma unroll
-                for (int q = 0; q < CPW; ++q) acc[q] = tz_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int t = 0; t < NM; ++t)
-#pragma unroll
-                    for (int q = 0; q < CPW; ++q) acc[q] = mfma16(A[q][t], ring[q][(ICB * j + t) % RING], acc[q], T());
-                char* dst = olw + (s & 1) * OLB;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if constexpr (CPW == 2) {
-                        union {
-                            T t[2];
-                            uint32_t u;
-                        } o;
-                        o.t[0] = from_f32<T>(acc[0][r]), o.t[1] = from_f32<T>(acc[1][r]);
-                        *reinterpret_cast<uint32_t*>(dst + r * OPX) = o.u;
-                    } else {
-                        *reinterpret_cast<T*>(dst + r * OPX) = from_f32<T>(acc[0][r]);
-                    }
-                }
-            }
-        }
+    // A step is two row groups (8 output rows).  Trips of UNRF steps run without a test between the staging calls: a
+    // trip may run past the band's end, where loads read nothing, stores are dropped and only the products (no memory
+    // request among them) are skipped.  Besides its products a step
+    // stores the previous step's tiles and commits the pass the NEXT step needs; the wavefronts 0-3 do the products
+    // first and the others last, so that of the two wavefronts a SIMD holds one feeds the matrix pipe while the
+    // other moves data (both make the same memory requests in the same order: the in-flight counts stay exact).
+    const int nfat = (nsteps + 1) >> 1;
+    int fdone = 0;
+    auto stage_step = [&](int jf, int f) {
+        store(f - 1);
+        add_fetch(f);
+        commit(buf[jf % 2], f + 2);   // pass f + 2 sits in buffer f % 2 = jf % 2 (UNRF is even)
+        issue(buf[jf % 2], f + 4);
+    };
+    auto compute_step = [&](int jf, int f) {
+        // the two row groups this step adds to the ring; the second goes to the slot of the step's own first
+        // group, which the first tile still reads, so it waits in registers until the products are issued
+        load_group((2 * jf + PER - 1) % PER, 4 * (2 * jf + PER - 1) * RP);
+        uint4 late[CPW][ICB];
 #pragma unroll
         for (int q = 0; q < CPW; ++q)
 #pragma unroll
-            for (int i = 0; i < ICB; ++i) xb[q][i] += 4 * UNR * RP;
+            for (int i = 0; i < ICB; ++i) late[q][i] = read16(xb[q][i] + 4 * (2 * jf + PER) * RP);
+        tz_f32x4 acc[2][CPW];
+#pragma unroll
+        for (int gi = 0; gi < 2; ++gi)
+#pragma unroll
+            for (int q = 0; q < CPW; ++q) acc[gi][q] = tz_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < NM; ++t)
+#pragma unroll
+            for (int q = 0; q < CPW; ++q) {
+                acc[0][q] = mfma16(A[q][t], ring[q][(ICB * 2 * jf + t) % RING], acc[0][q], T());
+                const uint4 b1 = t < ICB * (PER - 1) ? ring[q][(ICB * (2 * jf + 1) + t) % RING] : late[q][t - ICB * (PER - 1) < ICB ? t - ICB * (PER - 1) : 0];
+                acc[1][q] = mfma16(A[q][t], b1, acc[1][q], T());
+            }
+#pragma unroll
+        for (int q = 0; q < CPW; ++q)
+#pragma unroll
+            for (int i = 0; i < ICB; ++i) ring[q][((2 * jf) % PER) * ICB + i] = late[q][i];
+#pragma unroll
+        for (int gi = 0; gi < 2; ++gi) {
+            char* dst = olw + (2 * (f & 1) + gi) * OLB;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if constexpr (CPW == 2) {
+                    union {
+                        T t[2];
+                        uint32_t u;
+                    } o;
+                    o.t[0] = from_f32<T>(acc[gi][0][r]), o.t[1] = from_f32<T>(acc[gi][1][r]);
+                    *reinterpret_cast<uint32_t*>(dst + r * OPX) = o.u;
+                } else {
+                    *reinterpret_cast<T*>(dst + r * OPX) = from_f32<T>(acc[gi][0][r]);
+                }
+            }
+        }
+    };
+    for (int f0 = 0; f0 < nfat; f0 += UNRF) {
+#pragma unroll
+        for (int jf = 0; jf < UNRF; ++jf) {
+            const int f = f0 + jf;
+            lds_barrier();  // the previous step's tiles are complete, its window reads done
+            if (wv < 4) {
+                if (f < nfat) compute_step(jf, f);
+                stage_step(jf, f);
+            } else {
+                stage_step(jf, f);
+                if (f < nfat) compute_step(jf, f);
+            }
+        }
+        fdone = f0 + UNRF;
+#pragma unroll
+        for (int q = 0; q < CPW; ++q)
+#pragma unroll
+            for (int i = 0; i < ICB; ++i) xb[q][i] += 4 * (2 * UNRF) * RP;
     }
     lds_barrier();
-    store(nsteps - 1);
+    store(fdone - 1);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -83,6 +83,15 @@ int dwconv_wgrad_mfma_pair_k17(const void* xa, const void* gya, void* dwa, void*
                                const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
                                int dtype, hipStream_t s);
 
+// dwconv_wgrad_tz.hip: dense matrix-core kernel (16-bit types, C % 8 == 0, K <= 14)
+size_t dwconv_wgrad_tz_workspace(int B, int H, int W, int C, int K, int PH, int PW, int dtype);
+int dwconv_wgrad_tz_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int K, int PH,
+                           int PW, int dtype, hipStream_t s);
+static bool wgrad_tz_enabled() {
+    const char* e = tune_env("PDW_WGRAD_TZ");
+    return !(e && atoi(e) == 0);
+}
+
 // Matrix-core variant (16-bit types): workspace bytes (0 = not covered) and launch (-1 = not covered).
 static bool wgrad_mfma_enabled(int dtype) {
     if (dtype == kF32) return false;
@@ -125,6 +134,9 @@ int dwconv_wgrad_pair_launch(const void* xa, const void* gya, void* dwa, void* w
                              const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int K, int PH, int PW,
                              int dtype, hipStream_t s) {
     if (!wgrad_mfma_enabled(dtype) || tune_env("PDW_NO_WGRAD_PAIR")) return -1;
+    if (wgrad_tz_enabled() && dwconv_wgrad_tz_workspace(B, Ha, Wa, C, K, PH, PW, dtype) &&
+        dwconv_wgrad_tz_workspace(B, Hb, Wb, C, K, PH, PW, dtype))
+        return -1;  // the dense matrix-core kernel covers both: two launches of it beat the shared launch of this one
     switch (K) {
         case 3: return dwconv_wgrad_mfma_pair_k3(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
         case 5: return dwconv_wgrad_mfma_pair_k5(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
@@ -142,7 +154,9 @@ int dwconv_wgrad_pair_launch(const void* xa, const void* gya, void* dwa, void* w
 // cover the case.
 size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype) {
     if (KH != KW) return 0;
-    const size_t wm = wgrad_mfma_workspace(B, H, W, C, KH, PH, PW, dtype);
+    size_t wm = wgrad_mfma_workspace(B, H, W, C, KH, PH, PW, dtype);
+    const size_t wz = wgrad_tz_enabled() ? dwconv_wgrad_tz_workspace(B, H, W, C, KH, PH, PW, dtype) : 0;
+    if (wz > wm) wm = wz;
     size_t wt = 0;
     switch (KH) {
         case 3: wt = dwconv_wgrad_tiled_ws_k3(B, H, W, C, PH, PW, dtype); break;
@@ -162,6 +176,10 @@ size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, 
 int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int KH,
                               int KW, int PH, int PW, int dtype, hipStream_t s) {
     if (KH != KW) return -1;
+    if (wgrad_tz_enabled()) {
+        const int r = dwconv_wgrad_tz_launch(x, gy, dw, ws, B, H, W, C, KH, PH, PW, dtype, s);
+        if (r != -1) return r;
+    }
     {
         const int r = wgrad_mfma_launch(x, gy, dw, ws, B, H, W, C, KH, PH, PW, dtype, s);
         if (r != -1) return r;
