@@ -1,18 +1,26 @@
 #!/usr/bin/env python3
 """Benchmark of the ConvBlock hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-sweep] [--no-kernels] [--no-configs]
+                    [--no-torch-gpu]
 
 A step is one ConvBlock forward + backward on the headline workload
-(ConvBlock(128, kernel_size=13), bf16, x [32,56,56,128], seeded synthetic data, inputs
-resident in HBM).  Prints ONE JSON line: ms per step, the forward-only time, the k = 9/13/17
-sweep, the HBM-roofline fraction of the whole block and of the dominant kernel (timed live
-with HIP events on the launch stream), and the PyTorch-CPU baseline of the same workload.
+(ConvBlock(128, kernel_size=13), bf16, x [32,56,56,128], seeded synthetic data, inputs resident in HBM),
+replayed as one HIP graph.  Consecutive steps run on different sets of buffers (inputs, saved activations,
+gradients) that together exceed the 256 MB Infinity Cache, so that a step finds its inputs in HBM and not in
+the cache: that is the headline `value` ("rotated").  The same step replayed on one set of buffers (inputs
+cache-warm) is reported beside it as `warm_ms_per_step`.
+
+Prints ONE JSON line: ms per step, the forward-only times, the k = 9/13/17 sweep, rows for the other
+workloads (stand-alone depthwise conv at C = 128; the fp16 high-resolution block; the ragged block in fp32 and
+bf16), the per-kernel timings (HIP events on the launch stream) with the roofline record of the longest launch
+of the step, the same op set through torch's own GPU operators, and the PyTorch-CPU baseline.
 """
 from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -23,21 +31,17 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-HBM_PEAK = 8.0e12  # B/s, MI355X published
-VALU_PEAK = 157.3e12  # fp32 vector FLOP/s, MI355X published
+HBM_PEAK = 8.0e12     # B/s, MI355X published
 MFMA_PEAK = 2.5e15    # dense bf16/fp16 matrix FLOP/s, MI355X published
+FP32_PEAK = 157.3e12  # fp32 vector FLOP/s, MI355X published
+MALL_BYTES = 256e6    # Infinity Cache
 
 WORKLOAD = dict(B=32, H=56, W=56, D=128, k=13, dtype="bf16")
+DTYPES = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --kernel ...`, each
-# scaled by what the same counter reads for a plain copy of known size (`bench.py --kernel copy`); the
-# runs and the scale factors are recorded under profiles/.  None = not measured.
-MEASURED_TRAFFIC = {
-    "dwconv_fwd[32x56x56x64,k=13]": (12872 + 12544) * 1024,   # fetch 13.18 MB + write 12.85 MB
-    "dwconv_dgrad[32x56x56x64,k=13]": (12872 + 12544) * 1024,  # same kernel, same shape
-    "dwconv_wgrad[32x56x56x64,k=13]": (25392 + 2704 + 2721 + 21) * 1024,  # main kernel + partial reduction
-}
 
+# ------------------------------------------------------------------------------------------------
+# Algorithmic bytes and flops
 
 def block_alg_bytes(B, H, W, D, k, esize, scales=(1.0, 0.5)):
     """Compulsory HBM traffic of the unfused op graph (each op reads each input once and writes
@@ -53,20 +57,18 @@ def block_alg_bytes(B, H, W, D, k, esize, scales=(1.0, 0.5)):
     return esize * (fwd + params), esize * (fwd + bwd + 3 * params)
 
 
-def dwconv_flops_block(B, H, W, D, k, scales=(1.0, 0.5)):
-    I = D // 2
-    N = B * H * W
-    n = B * int(H * scales[1]) * int(W * scales[1])
-    f = 2 * k * k * I * (N + n)
-    return f, 3 * f
+def conv_issue(k):
+    """Multiply-adds the matrix-core depthwise kernels issue per output (forward / input gradient: a 4 x 4 patch
+    against its (k+3)^2 window, 32 window positions per instruction) and per position (weight gradient: 16 x 16
+    taps per instruction), against the k*k that fall on a real tap."""
+    ic = k + 3
+    icb = (ic + 7) // 8
+    nm = (ic * icb + 3) // 4
+    return dict(fwd=nm * 32, wgrad=256 if k <= 14 else None, useful=k * k)
 
 
-def make_block(D, k, dtype, seed=0):
-    import pyramid_dwconv
-
-    torch.manual_seed(seed)
-    return pyramid_dwconv.ConvBlock(dim=D, kernel_size=k).to(dtype).cuda()
-
+# ------------------------------------------------------------------------------------------------
+# Timing
 
 def time_gpu(fn, steps, warmup):
     """Wall time per call of fn over `steps` calls, bracketed by device synchronisation."""
@@ -80,9 +82,20 @@ def time_gpu(fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def rotate(replayers):
+    """One callable that replays the next of `replayers` on every call."""
+    state = {"i": 0}
+
+    def fn():
+        replayers[state["i"] % len(replayers)]()
+        state["i"] += 1
+
+    return fn
+
+
 def time_kernel_events(launch, nbuf, iters=24, reps=4):
     """Average duration of one launch.  `iters` launches (launch(i) uses buffer set i % nbuf, so that
-    consecutive launches do not hit in the 256 MB Infinity Cache) are captured into a HIP graph, and the
+    consecutive launches do not hit in the Infinity Cache) are captured into a HIP graph, and the
     replays are bracketed by HIP events recorded on the stream the graph runs on, so the figure is GPU
     time per launch, free of the host's per-call overhead."""
     side = torch.cuda.Stream()
@@ -107,6 +120,121 @@ def time_kernel_events(launch, nbuf, iters=24, reps=4):
     return start.elapsed_time(stop) * 1e-3 / (iters * reps)
 
 
+# ------------------------------------------------------------------------------------------------
+# Block workloads
+
+def make_block(D, k, dtype, seed=0):
+    import pyramid_dwconv
+
+    torch.manual_seed(seed)
+    return pyramid_dwconv.ConvBlock(dim=D, kernel_size=k).to(dtype).cuda()
+
+
+def make_inputs(shape, dtype, dist, seed):
+    gen = torch.Generator().manual_seed(seed)
+    if dist == "uniform":   # U(-2, 2)
+        x = (torch.rand(*shape, generator=gen) * 4 - 2)
+    else:
+        x = torch.randn(*shape, generator=gen)
+    g = torch.randn(*shape, generator=gen)
+    return x.to(dtype).cuda(), g.to(dtype).cuda()
+
+
+def n_sets(B, H, W, D, k, esize):
+    """Buffer sets to rotate over: their inputs and saved activations (about half of the forward+backward
+    algorithmic bytes each) together exceed twice the Infinity Cache; between 3 and 24."""
+    per_set = 0.5 * block_alg_bytes(B, H, W, D, k, esize)[1]
+    return int(min(24, max(3, math.ceil(2 * MALL_BYTES / per_set))))
+
+
+def measure_block(m, shape, dtype, dist, steps, warmup, with_forward=True):
+    """ms per forward+backward step (rotated over buffer sets / one warm set) and per inference forward."""
+    from pyramidconvblock_amd.graphs import GraphedForward, GraphedStep
+
+    B, H, W, D = shape
+    k = m.gates[0].conv_spatial.weight.shape[0]
+    es = torch.empty((), dtype=dtype).element_size()
+    ns = n_sets(B, H, W, D, k, es)
+    steps_g, fwds_g = [], []
+    for i in range(ns):
+        x, g = make_inputs(shape, dtype, dist, seed=i)
+        steps_g.append(GraphedStep(m, x, g))
+        if with_forward:
+            fwds_g.append(GraphedForward(m, x))
+        for p in m.parameters():
+            p.grad = None
+    out = {"buffer_sets": ns}
+    out["fwd_bwd_ms"] = time_gpu(rotate([s.replay for s in steps_g]), steps, warmup) * 1e3
+    out["fwd_bwd_ms_warm"] = time_gpu(steps_g[0].replay, steps, warmup) * 1e3
+    if with_forward:
+        out["fwd_ms"] = time_gpu(rotate([f.replay for f in fwds_g]), steps, warmup) * 1e3
+        out["fwd_ms_warm"] = time_gpu(fwds_g[0].replay, steps, warmup) * 1e3
+    bf, bfb = block_alg_bytes(B, H, W, D, k, es)
+    out["hbm_frac_fwd_bwd"] = bfb / (out["fwd_bwd_ms"] * 1e-3 * HBM_PEAK)
+    if with_forward:
+        out["hbm_frac_fwd"] = bf / (out["fwd_ms"] * 1e-3 * HBM_PEAK)
+    return out
+
+
+def torch_gpu_block(shape, D, k, dtype, steps, warmup):
+    """The same block through torch's own GPU operators, as the reference's benchmark times its all-torch twin on
+    the same device (pyramid_dwconv/conv_block.py:52-97, :99-158): NCHW, 1x1 and grouped F.conv2d,
+    adaptive_avg_pool2d, interpolate; forward + backward, eager launches, cache-warm."""
+    import torch.nn.functional as F
+
+    B, H, W, _ = shape
+    I, G = D // 2, D // 4
+    torch.manual_seed(0)
+    P = {
+        "up": torch.randn(I, D, 1, 1) / D ** 0.5, "w0": torch.randn(I, 1, k, k) / k, "w1": torch.randn(I, 1, k, k) / k,
+        "out": torch.randn(D, 2 * G, 1, 1) / (2 * G) ** 0.5, "out_b": torch.zeros(D),
+        "pool": torch.randn(D, D, 1, 1) / D ** 0.5, "pool_b": torch.zeros(D),
+    }
+    P = {n: v.to(dtype).cuda().requires_grad_() for n, v in P.items()}
+    x = torch.randn(B, D, H, W).to(dtype).cuda().requires_grad_()
+    g = torch.randn(B, D, H, W).to(dtype).cuda()
+    scale = (I / 2) ** -0.5
+
+    def gate(a, w, s):
+        if s != 1.0:
+            a = F.adaptive_avg_pool2d(a, (int(H * s), int(W * s)))
+        c = F.conv2d(a, w, None, 1, k // 2, 1, I)
+        c1, c2 = c.chunk(2, dim=1)
+        y = c1 * (c2 / scale)
+        if s != 1.0:
+            y = F.interpolate(y, size=(H, W), mode="bilinear", align_corners=False)
+        return y
+
+    def step():
+        a = F.conv2d(x, P["up"])
+        cat = torch.cat([gate(a, P["w0"], 1.0), gate(a, P["w1"], 0.5)], dim=1)
+        y = F.conv2d(cat, P["out"], P["out_b"]) + F.conv2d(F.adaptive_avg_pool2d(x, 1), P["pool"], P["pool_b"])
+        torch.autograd.backward(y, g)
+        x.grad = None
+        for v in P.values():
+            v.grad = None
+
+    return time_gpu(step, steps, warmup) * 1e3
+
+
+# ------------------------------------------------------------------------------------------------
+# Per-kernel timings
+
+def load_traffic():
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known
+    size), as recorded in profiles/hbm_traffic_by_kernel.txt: lines `key = bytes`."""
+    out = {}
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic_by_kernel.txt")) as f:
+            for line in f:
+                if "=" in line and not line.lstrip().startswith("#"):
+                    key, _, val = line.partition("=")
+                    out[key.strip()] = float(val.split()[0])
+    except OSError:
+        pass
+    return out
+
+
 def kernel_rooflines(B, H, W, D, k, dtype):
     """Times each hot kernel of the block alone at its real shapes; returns a list of dicts."""
     from pyramidconvblock_amd import avgpool, dwconv, ops, up
@@ -115,6 +243,7 @@ def kernel_rooflines(B, H, W, D, k, dtype):
     es = torch.empty((), dtype=dtype).element_size()
     out = []
     geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    iss = conv_issue(k)
     for tag, (h, w) in (("full", (H, W)), ("half", (H // 2, W // 2))):
         n_el = B * h * w * I
         nbuf = max(2, int(600e6 // (2 * n_el * es)) + 1)
@@ -123,13 +252,14 @@ def kernel_rooflines(B, H, W, D, k, dtype):
         wt = (torch.randn(k, k, I, device="cuda") / k).to(dtype)
         conv_bytes = es * (2 * n_el + k * k * I)
         flops = 2.0 * k * k * n_el
-        for name, fn in (
-            ("dwconv_fwd", lambda i: dwconv.dwconv_forward(xs[i], wt, *geo)),
-            ("dwconv_dgrad", lambda i: dwconv.dwconv_dgrad(gs[i], wt, xs[i].shape, *geo)),
-            ("dwconv_wgrad", lambda i: dwconv.dwconv_wgrad(xs[i], gs[i], wt.shape, *geo)),
+        for name, fn, issued in (
+            ("dwconv_fwd", lambda i: dwconv.dwconv_forward(xs[i], wt, *geo), iss["fwd"]),
+            ("dwconv_dgrad", lambda i: dwconv.dwconv_dgrad(gs[i], wt, xs[i].shape, *geo), iss["fwd"]),
+            ("dwconv_wgrad", lambda i: dwconv.dwconv_wgrad(xs[i], gs[i], wt.shape, *geo), iss["wgrad"]),
         ):
             t = time_kernel_events(fn, nbuf)
-            out.append(dict(kernel=f"{name}[{B}x{h}x{w}x{I},k={k}]", seconds=t, alg_bytes=conv_bytes, flops=flops))
+            out.append(dict(kernel=f"{name}[{B}x{h}x{w}x{I},k={k}]", seconds=t, alg_bytes=conv_bytes, flops=flops,
+                            issued_flops=2.0 * issued * n_el if issued else None, pipe="mfma"))
         del xs, gs
     # resampling kernels of the half-resolution gate
     h, w = H // 2, W // 2
@@ -145,33 +275,56 @@ def kernel_rooflines(B, H, W, D, k, dtype):
         ("bilinear_bwd", lambda i: up.bilinear_backward(gbig[i], (h, w)), es * (B * H * W * G + B * h * w * G)),
     ):
         t = time_kernel_events(fn, nbuf)
-        out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=0.0))
+        out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=0.0, issued_flops=None, pipe="valu"))
     # gate and the dense conv_up layer ([N,D] <-> [N,I])
     c = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
     xin = [torch.randn(B, H, W, D, device="cuda").to(dtype) for _ in range(4)]
     wup = (torch.randn(I, D, device="cuda") / D ** 0.5).to(dtype)
     N = B * H * W
-    for name, fn, nb_, nbytes, fl in (
-        ("gate_fwd", lambda i: ops.gate_forward(c[i]), nbuf, es * 1.5 * N * I, 0.0),
-        ("gate_bwd", lambda i: ops.gate_backward(c[i], gbig[i]), nbuf, es * 2.5 * N * I, 0.0),
-        ("dense_fwd", lambda i: ops.dense_forward(xin[i], wup), 4, es * (N * D + N * I + D * I), 2.0 * N * D * I),
+    for name, fn, nb_, nbytes, fl, pipe in (
+        ("gate_fwd", lambda i: ops.gate_forward(c[i]), nbuf, es * 1.5 * N * I, 0.0, "valu"),
+        ("gate_bwd", lambda i: ops.gate_backward(c[i], gbig[i]), nbuf, es * 2.5 * N * I, 0.0, "valu"),
+        ("dense_fwd", lambda i: ops.dense_forward(xin[i], wup), 4, es * (N * D + N * I + D * I), 2.0 * N * D * I, "mfma"),
         ("dense_dgrad", lambda i: ops.dense_forward(a[i], wup, w_kmajor=True), 4, es * (N * D + N * I + D * I),
-         2.0 * N * D * I),
+         2.0 * N * D * I, "mfma"),
         ("dense_wgrad", lambda i: ops.dense_wgrad(a[i % 4], xin[i % 4]), 4, es * (N * D + N * I + D * I),
-         2.0 * N * D * I),
+         2.0 * N * D * I, "mfma"),
         # both gradients of conv_up as the block's backward runs them: one launch, gy read once
         ("dense_bwd_pair", lambda i: ops.dense_backward_pair(a[i % 4], wup, xin[i % 4]), 4,
-         es * (2 * N * D + N * I + 2 * D * I), 4.0 * N * D * I),
+         es * (2 * N * D + N * I + 2 * D * I), 4.0 * N * D * I, "mfma"),
     ):
         t = time_kernel_events(fn, nb_)
-        out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=fl))
+        out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=fl, issued_flops=fl if pipe == "mfma" else None,
+                        pipe=pipe))
     return out
+
+
+def conv_rows(B, H, W, C, dtype, ks=(9, 13, 17)):
+    """Stand-alone depthwise-conv forward, x [B,H,W,C], weight ~ N(0, 1/k^2), 'same' padding, stride 1."""
+    from pyramidconvblock_amd import dwconv
+
+    es = torch.empty((), dtype=dtype).element_size()
+    n_el = B * H * W * C
+    nbuf = max(2, int(600e6 // (2 * n_el * es)) + 1)
+    xs = [torch.randn(B, H, W, C, device="cuda").to(dtype) for _ in range(nbuf)]
+    rows = {}
+    for k in ks:
+        wt = (torch.randn(k, k, C, device="cuda") / k).to(dtype)
+        geo = ((1, 1), (k // 2, k // 2), (1, 1))
+        t = time_kernel_events(lambda i: dwconv.dwconv_forward(xs[i], wt, *geo), nbuf)
+        nbytes = es * (2 * n_el + k * k * C)
+        iss = conv_issue(k)
+        rows[f"k{k}"] = {"us": round(t * 1e6, 2), "hbm_frac": round(nbytes / t / HBM_PEAK, 4),
+                         "mfma_issue_frac": round(2.0 * iss["fwd"] * n_el / t / MFMA_PEAK, 4),
+                         "useful_tap_frac": round(iss["useful"] / iss["fwd"], 3)}
+    return rows
 
 
 def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     """Launches one hot kernel `iters` times at its shape inside the headline block (for rocprofv3 runs).
-    name: {fwd,dgrad,wgrad}_{full,half} | avgpool_fwd | avgpool_bwd | bilinear_fwd | bilinear_bwd |
-    dense_{fwd,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pair = both gradients in one launch)"""
+    name: {fwd,dgrad,wgrad}_{full,half} | conv128 (stand-alone forward at C = D) | avgpool_fwd | avgpool_bwd |
+    bilinear_fwd | bilinear_bwd | dense_{fwd,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pair = both
+    gradients in one launch) | step (whole forward+backward steps, eager) | copy"""
     from pyramidconvblock_amd import avgpool, dwconv, up
 
     I, G = D // 2, D // 4
@@ -182,6 +335,20 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         src = torch.randn(B, H, W, I, device="cuda").to(dtype)
         dst = torch.empty_like(src)
         fn = lambda: dst.copy_(src)
+    elif name == "step":
+        m = make_block(D, k, dtype)
+        x, g = make_inputs((B, H, W, D), dtype, "normal", 0)
+        x.requires_grad_()
+
+        def fn():
+            torch.autograd.backward(m(x), g)
+            x.grad = None
+            for p in m.parameters():
+                p.grad = None
+    elif name == "conv128":
+        x = torch.randn(B, H, W, D, device="cuda").to(dtype)
+        wt = (torch.randn(k, k, D, device="cuda") / k).to(dtype)
+        fn = lambda: dwconv.dwconv_forward(x, wt, *geo)
     elif op in ("fwd", "dgrad", "wgrad"):
         hh, ww = (H, W) if res == "full" else (h, w)
         x = torch.randn(B, hh, ww, I, device="cuda").to(dtype)
@@ -215,6 +382,31 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     torch.cuda.synchronize()
 
 
+# ------------------------------------------------------------------------------------------------
+# CPU baseline
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_threads():
+    """Threads for the CPU baseline: the host's processors, capped by the share the job was given
+    (OMP_NUM_THREADS where the environment sets one)."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, int(os.environ["OMP_NUM_THREADS"]))
+    except (KeyError, ValueError):
+        pass
+    return max(1, n)
+
+
 def cpu_baseline(B, H, W, D, k, dtype, threads, iters=3):
     """The reference's PyTorch path (F.conv2d groups=C, adaptive_avg_pool2d, interpolate, linear) on
     the host cores: forward+backward of the same block on the same seeded inputs."""
@@ -244,16 +436,22 @@ def cpu_baseline(B, H, W, D, k, dtype, threads, iters=3):
     return ts[len(ts) // 2]
 
 
+# ------------------------------------------------------------------------------------------------
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=60)
+    ap.add_argument("--warmup", type=int, default=12)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep, the forward-only timings and the batch-size sweep")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the k=9/17 sweep and the batch-size sweep")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel event timings")
+    ap.add_argument("--no-configs", action="store_true", help="skip the rows of the other workloads")
+    ap.add_argument("--no-torch-gpu", action="store_true", help="skip the torch-operator comparator on the GPU")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
-                    "{fwd,dgrad,wgrad}_{full,half}, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, dense_{fwd,dgrad,wgrad}, copy")
+                    "{fwd,dgrad,wgrad}_{full,half}, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
+                    "dense_{fwd,dgrad,wgrad,pair}, step, copy")
+    ap.add_argument("--torch-gpu-only", action="store_true", help="(internal) time the torch-operator comparator and exit")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -270,113 +468,154 @@ def main():
     if args.kernel:
         run_single_kernel(args.kernel, args.steps, B, H, W, D, args.k, dtype)
         return
-    gen = torch.Generator().manual_seed(0)
-    x = torch.randn(B, H, W, D, generator=gen).to(dtype).cuda().requires_grad_()
-    g = torch.randn(B, H, W, D, generator=gen).to(dtype).cuda()
-
-    def stepper(m):
-        def fwd():
-            with torch.no_grad():
-                return m(x)
-
-        def fwd_bwd():
-            y = m(x)
-            torch.autograd.backward(y, g)
-            x.grad = None
-            for p in m.parameters():
-                p.grad = None
-
-        return fwd, fwd_bwd
+    if args.torch_gpu_only:
+        print(json.dumps({"fwd_bwd_ms": torch_gpu_block((B, H, W, D), D, k, dtype, steps=10, warmup=3)}))
+        return
 
     m = make_block(D, k, dtype)
-    fwd, fwd_bwd = stepper(m)
-    t_eager = time_gpu(fwd_bwd, args.steps, args.warmup)
-    # The step the metric is quoted on: the same forward+backward captured once into a HIP graph
-    # and replayed (identical kernels and results; removes the per-launch host overhead).
-    from pyramidconvblock_amd.graphs import GraphedForward, GraphedStep
+    head = measure_block(m, (B, H, W, D), dtype, "normal", args.steps, args.warmup)
+    # eager launches of the same step (host-bound), for reference
+    x0, g0 = make_inputs((B, H, W, D), dtype, "normal", 0)
+    x0.requires_grad_()
 
-    graphed = GraphedStep(m, x, g)
-    t_step = time_gpu(graphed.replay, args.steps, args.warmup)
+    def eager():
+        torch.autograd.backward(m(x0), g0)
+        x0.grad = None
+        for p in m.parameters():
+            p.grad = None
+
+    t_eager = time_gpu(eager, args.steps, args.warmup)
     for p in m.parameters():
         p.grad = None
+    del x0, g0
     bytes_f, bytes_fb = block_alg_bytes(B, H, W, D, k, 2)
-    flops_f, flops_fb = dwconv_flops_block(B, H, W, D, k)
+    t_step = head["fwd_bwd_ms"] * 1e-3
 
     result = {
         "metric": "convblock_fwd_bwd_ms",
-        "value": t_step * 1e3,
+        "value": head["fwd_bwd_ms"],
         "unit": "ms",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": t_step * 1e3,
+        "ms_per_step": head["fwd_bwd_ms"],
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "ConvBlock(dim=128,kernel_size=13) fwd+bwd, bf16, x[32,56,56,128] N(0,1) seed 0, "
+        "config": {"workload": "ConvBlock(dim=128,kernel_size=13) fwd+bwd, bf16, x[32,56,56,128] N(0,1), "
                                "default-init weights, grad_out N(0,1)"},
+        "cache_state": f"rotated: consecutive steps use {head['buffer_sets']} different sets of inputs, activations and "
+                       "gradients (more than twice the 256 MB Infinity Cache in total), so a step's inputs come from HBM",
+        "warm_ms_per_step": head["fwd_bwd_ms_warm"],
+        "warm_note": "the same step replayed on one buffer set: inputs and weights hit in the Infinity Cache",
+        "fwd_ms": head["fwd_ms"],
+        "warm_fwd_ms": head["fwd_ms_warm"],
         "eager_ms_per_step": t_eager * 1e3,
         "launch": "one HIP graph replay per step (eager launch time in eager_ms_per_step)",
         "block_hbm_frac_fwd_bwd": bytes_fb / (t_step * HBM_PEAK),
+        "block_hbm_frac_fwd_bwd_warm": bytes_fb / (head["fwd_bwd_ms_warm"] * 1e-3 * HBM_PEAK),
+        "block_hbm_frac_fwd": bytes_f / (head["fwd_ms"] * 1e-3 * HBM_PEAK),
         "block_alg_bytes_fwd_bwd": bytes_fb,
-        "block_dwconv_valu_frac_fwd_bwd": flops_fb / (t_step * VALU_PEAK),
+        "block_alg_bytes_fwd": bytes_f,
     }
 
     if not args.no_sweep:
         sweep = {}
         for kk in (9, 13, 17):
-            mk = m if kk == k else make_block(D, kk, dtype)
-            f, fb = stepper(mk)
-            tf = time_gpu(GraphedForward(mk, x).replay, args.steps, args.warmup)
-            tfb = t_step if kk == k else time_gpu(GraphedStep(mk, x, g).replay, args.steps, args.warmup)
-            for p in mk.parameters():
-                p.grad = None
-            bf, bfb = block_alg_bytes(B, H, W, D, kk, 2)
-            sweep[f"k{kk}"] = {"fwd_ms": tf * 1e3, "fwd_bwd_ms": tfb * 1e3, "hbm_frac_fwd": bf / (tf * HBM_PEAK),
-                               "hbm_frac_fwd_bwd": bfb / (tfb * HBM_PEAK)}
+            if kk == k:
+                r = head
+            else:
+                mk = make_block(D, kk, dtype)
+                r = measure_block(mk, (B, H, W, D), dtype, "normal", args.steps, args.warmup)
+                del mk
+            sweep[f"k{kk}"] = {n: round(r[n], 5) for n in ("fwd_ms", "fwd_bwd_ms", "fwd_bwd_ms_warm", "hbm_frac_fwd",
+                                                            "hbm_frac_fwd_bwd")}
         result["sweep"] = sweep
         # The same block at other batch sizes (not the metric: how the fixed cost per launch amortises)
         batches = {}
         for bb in (8, 64, 128):
-            xb = torch.randn(bb, H, W, D, generator=gen).to(dtype).cuda().requires_grad_()
-            gb = torch.randn(bb, H, W, D, generator=gen).to(dtype).cuda()
-            tb = time_gpu(GraphedStep(m, xb, gb).replay, args.steps, args.warmup)
-            for p in m.parameters():
-                p.grad = None
-            batches[f"B{bb}"] = {"fwd_bwd_ms": tb * 1e3,
-                                 "hbm_frac_fwd_bwd": block_alg_bytes(bb, H, W, D, k, 2)[1] / (tb * HBM_PEAK)}
-            del xb, gb
+            r = measure_block(m, (bb, H, W, D), dtype, "normal", args.steps, args.warmup, with_forward=False)
+            batches[f"B{bb}"] = {"fwd_bwd_ms": round(r["fwd_bwd_ms"], 5), "hbm_frac_fwd_bwd": round(r["hbm_frac_fwd_bwd"], 4)}
         result["batch_sweep"] = batches
+
+    if not args.no_configs:
+        cfg = {}
+        # stand-alone depthwise conv forward, bf16, x [32,56,56,128], k = 9/13/17
+        cfg["dwconv_fwd_bf16_32x56x56x128"] = conv_rows(B, H, W, D, dtype)
+        # the same in fp32 (vector kernel)
+        cfg["dwconv_fwd_fp32_32x56x56x128"] = {
+            kk: {n: v for n, v in row.items() if n in ("us", "hbm_frac")}
+            for kk, row in conv_rows(B, H, W, D, torch.float32).items()}
+        # high-resolution stage: fp16, x [8,112,112,96], k = 17
+        mk = make_block(96, 17, torch.float16)
+        cfg["convblock_fp16_8x112x112x96_k17"] = {n: round(v, 5) for n, v in measure_block(
+            mk, (8, 112, 112, 96), torch.float16, "normal", args.steps, args.warmup).items()}
+        # ragged shapes: x [3,57,61,200] ~ U(-2,2), k = 9 and 15, fp32 and bf16
+        for dn in ("fp32", "bf16"):
+            for kk in (9, 15):
+                mk = make_block(200, kk, DTYPES[dn])
+                cfg[f"convblock_{dn}_3x57x61x200_k{kk}"] = {n: round(v, 5) for n, v in measure_block(
+                    mk, (3, 57, 61, 200), DTYPES[dn], "uniform", args.steps, args.warmup).items()}
+        # the headline block in fp32
+        mk = make_block(D, k, torch.float32)
+        cfg["convblock_fp32_32x56x56x128_k13"] = {n: round(v, 5) for n, v in measure_block(
+            mk, (B, H, W, D), torch.float32, "normal", args.steps, args.warmup).items()}
+        del mk
+        result["configs"] = cfg
 
     if not args.no_kernels:
         ks = kernel_rooflines(B, H, W, D, k, dtype)
-        # Dominant kernel = largest share of the step.  Forward and input gradient are the same kernel
-        # function (dwconv_mfma_k) at the same shape, so their launches count together.
-        def share(r):
-            return r["seconds"] * (2 if r["kernel"].startswith(("dwconv_fwd", "dwconv_dgrad")) else 1)
-
-        dom = max(ks, key=share)
+        traffic = load_traffic()
+        dom = max(ks, key=lambda r: r["seconds"])   # the longest launch of the step
+        ai = dom["flops"] / dom["alg_bytes"]
         result["roofline"] = {
-            "kernel": dom["kernel"], "bound": "hbm", "achieved": dom["alg_bytes"] / dom["seconds"] / 1e9,
-            "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": dom["alg_bytes"] / dom["seconds"] / HBM_PEAK,
-            "traffic": MEASURED_TRAFFIC.get(dom["kernel"]), "avg_us": dom["seconds"] * 1e6,
-            "valu_frac": dom["flops"] / dom["seconds"] / VALU_PEAK,
-            "mfma_frac": dom["flops"] / dom["seconds"] / MFMA_PEAK,
+            "kernel": dom["kernel"],
+            # the roofline that bounds it: its useful flops per algorithmic byte against the machine balance
+            "bound": "hbm" if ai < MFMA_PEAK / HBM_PEAK else "mfma",
+            "achieved": dom["alg_bytes"] / dom["seconds"] / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": dom["alg_bytes"] / dom["seconds"] / HBM_PEAK,
+            "traffic": traffic.get(dom["kernel"]), "avg_us": dom["seconds"] * 1e6,
+            "flops_per_byte": ai, "machine_flops_per_byte": MFMA_PEAK / HBM_PEAK,
+            "mfma_issue_frac": (dom["issued_flops"] / dom["seconds"] / MFMA_PEAK) if dom["issued_flops"] else None,
+            "limiter": "not the roofline: LDS operand reads and exposed load latency (profiles/)",
         }
-        result["kernels"] = [{"kernel": r["kernel"], "us": round(r["seconds"] * 1e6, 2),
-                              "hbm_frac": round(r["alg_bytes"] / r["seconds"] / HBM_PEAK, 4),
-                              "valu_frac": round(r["flops"] / r["seconds"] / VALU_PEAK, 4),
-                              "mfma_frac": round(r["flops"] / r["seconds"] / MFMA_PEAK, 4)} for r in ks]
+        result["kernels"] = []
+        for r in ks:
+            row = {"kernel": r["kernel"], "us": round(r["seconds"] * 1e6, 2),
+                   "hbm_frac": round(r["alg_bytes"] / r["seconds"] / HBM_PEAK, 4), "pipe": r["pipe"]}
+            if r["issued_flops"]:
+                row["mfma_issue_frac"] = round(r["issued_flops"] / r["seconds"] / MFMA_PEAK, 4)
+            if r["kernel"] in traffic:
+                row["traffic"] = traffic[r["kernel"]]
+            result["kernels"].append(row)
+
+    if not args.no_torch_gpu:
+        # in a child process with a time limit: the library may build its kernels on first use
+        import subprocess
+
+        try:
+            cp = subprocess.run([sys.executable, os.path.abspath(__file__), "--torch-gpu-only"], capture_output=True,
+                                text=True, timeout=240)
+            t_torch = json.loads(cp.stdout.strip().splitlines()[-1])["fwd_bwd_ms"]
+            result["torch_gpu"] = {"fwd_bwd_ms": t_torch, "speedup": t_torch / head["fwd_bwd_ms_warm"],
+                                   "what": "same block through torch-ROCm operators (NCHW conv2d 1x1 / groups=C, "
+                                           "adaptive_avg_pool2d, interpolate), eager, cache-warm; speedup against "
+                                           "warm_ms_per_step"}
+        except Exception as e:  # noqa: BLE001 - the comparator must not take the bench line down
+            result["torch_gpu"] = {"error": f"{type(e).__name__}: {e}"[:300]}
 
     if not args.no_cpu:
-        threads = min(os.cpu_count() or 1, 16)
-        t_cpu = cpu_baseline(B, H, W, D, k, dtype, threads)
-        result["cpu_baseline"] = {"value": t_cpu * 1e3, "unit": "ms", "cores": threads, "kind": "port",
-                                  "sample": "full workload: same ConvBlock fwd+bwd in bf16 through torch CPU ops "
+        threads = cpu_threads()
+        t_bf16 = cpu_baseline(B, H, W, D, k, torch.bfloat16, threads)
+        t_fp32 = cpu_baseline(B, H, W, D, k, torch.float32, threads)
+        result["cpu_baseline"] = {"value": t_bf16 * 1e3, "unit": "ms", "cores": threads, "kind": "port",
+                                  "fp32_value": t_fp32 * 1e3, "cpu_model": cpu_model(), "host_cpus": os.cpu_count(),
+                                  "sample": "full workload: same ConvBlock fwd+bwd through torch CPU ops "
                                             "(F.conv2d groups=C, adaptive_avg_pool2d, interpolate, linear), "
-                                            "median of 3 after 1 warm-up"}
+                                            "median of 3 after 1 warm-up; value in bf16, fp32_value in fp32; threads = "
+                                            "host processors capped by the job's OMP_NUM_THREADS share"}
     print(json.dumps(result))
 
 
