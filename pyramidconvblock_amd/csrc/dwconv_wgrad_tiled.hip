@@ -83,7 +83,7 @@ int dwconv_wgrad_mfma_pair_k17(const void* xa, const void* gya, void* dwa, void*
                                const void* gyb, void* dwb, void* wsb, int Hb, int Wb, int B, int C, int PH, int PW,
                                int dtype, hipStream_t s);
 
-// dwconv_wgrad_tz.hip: dense matrix-core kernel (16-bit types, C % 8 == 0, K <= 14)
+// dwconv_wgrad_tz.hip: dense matrix-core kernel (16-bit types, C % 8 == 0, K <= 17)
 size_t dwconv_wgrad_tz_workspace(int B, int H, int W, int C, int K, int PH, int PW, int dtype);
 int dwconv_wgrad_tz_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int K, int PH,
                            int PW, int dtype, hipStream_t s);

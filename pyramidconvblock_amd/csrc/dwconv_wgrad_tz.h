@@ -1,5 +1,5 @@
 // Depthwise-convolution weight gradient on the dense matrix cores (16-bit types, stride 1, dilation 1, square
-// filters up to 14):     dw[u,v,c] = sum_{b,i,j} gy[b,i,j,c] * xw[b, i+u, j+v, c],   xw[r][s] = x[r-PH][s-PW].
+// filters up to 17):     dw[u,v,c] = sum_{b,i,j} gy[b,i,j,c] * xw[b, i+u, j+v, c],   xw[r][s] = x[r-PH][s-PW].
 //
 // With u = 2a + du, v = 8b + dv and the position p = (i + du, j + dv) the sum for one channel is
 //     dw[2a+du][8b+dv] = sum_p  xw[p + (2a, 8b)] * gy[p - (du, dv)],
@@ -9,7 +9,8 @@
 //     A[(a,b)][(kr,e)]   = xw[R + kr + 2a][Cc + e + 8b]
 //     B[(kr,e)][(du,dv)] = gy[R + kr - du][Cc + e - dv]        (zero outside the band's own rows and columns)
 // One accumulator of 4 registers holds all 16 x 16 taps of a channel (169 of 256 used at K = 13), and a band of
-// BR x 56 positions takes ceil((BR+1)/4) x 8 instructions per channel.  Both operands are data, so nothing is kept
+// BR x 56 positions takes ceil((BR+1)/4) x 8 instructions per channel.  K = 17 has 9 x 3 tap blocks (a, b): they are
+// numbered a * NB + b over two instructions that share the gy operand.  Both operands are data, so nothing is kept
 // per channel but the accumulator: a wavefront owns 2 of the workgroup's 16 channels for the whole band and
 // writes their taps to the fp32 partial of the band at the end; the partials are summed in a fixed order by
 // wgrad_reduce_parts (no atomics: bit-reproducible).
@@ -35,12 +36,13 @@
 namespace pdw {
 
 // NGA: row groups (of 4 rows) the xw operand of a step spans (rows kr + 2a, a <= (K-1)/2); NCB: column blocks of 8
-// positions per band row (8: bands of 56 columns, 5: of 32).
-template <int NGA, int NCB>
+// positions per band row (8: bands of 56 columns, 5: of 32); NB: tap column blocks (2: K <= 16, 3: K = 17).
+template <int NGA, int NCB, int NB>
 struct WgTzShape {
     static constexpr int NT = 512, CS = 16, CPW = 2, NH = 2;
     static constexpr int TWG = 8 * NCB - 8;                 // gy columns of a workgroup: TWG + 7 <= 8 NCB positions
-    static constexpr int WCX = 8 * NCB + 8;                 // xw window columns the operands touch
+    static constexpr int NMF = NB == 3 ? 2 : 1;             // instructions per position block and channel
+    static constexpr int WCX = 8 * NCB + 8 * (NB - 1);      // xw window columns the operands touch
     static constexpr int WCG = 8 * NCB + 8;                 // gy window columns: 8 of padding on the left
     // LDS pitches, chosen by measurement of the operands' access patterns on this part.  xw (ds_read_b128, lane (a, b, kr)
     // at row kr + 2a, byte 16 b): rows 32 bytes (mod 128) apart run at the full rate (3.9 cycles per instruction against
@@ -49,14 +51,17 @@ struct WgTzShape {
     // further the six runs start at banks 1, 6, 11, 16, 23, 28: no two share a bank.
     static constexpr int RPX = (2 * WCX - 32 + 127) / 128 * 128 + 32;
     static constexpr int RPG = (2 * WCG - 40 + 127) / 128 * 128 + 40;
-    static constexpr int NSX = NGA + 2 + (NGA % 2), NSG = 4;    // ring slots (row groups); NSX even, >= NGA + 2
+    // ring slots (row groups).  xw: the NGA groups a step reads and the two the pass committed meanwhile covers; even,
+    // so that a pass never wraps.  gy: a step reads groups t-1 and t while a whole pass (groups t+1, t+2) is committed;
+    // where LDS is short (NGA = 5) a step commits only group t+1, one half of a pass, and 3 slots do.
+    static constexpr int NSX = NGA + 2 + (NGA % 2), NSG = NGA == 5 ? 3 : 4;
     static constexpr int GBX = 4 * RPX, GBG = 4 * RPG;      // bytes per row group of a channel
     static constexpr int CHPX = NSX * GBX + 16, CHPG = NSG * GBG + 8;   // channel planes
     static constexpr int XHALF = 64;                        // channels 8..15 sit 16 banks further: the two 8-channel
                                                             // pieces of a staging pass write different banks
     static constexpr int XB = CS * CHPX + XHALF, GCB = (CS * CHPG + 127) / 128 * 128 + 24;  // xw window; one gy copy
     static constexpr size_t lds_bytes = (size_t)XB + 2 * GCB;
-    static_assert(NGA >= 2 && NGA <= 4 && (NCB == 8 || NCB == 5), "row groups spanned, column blocks");
+    static_assert(NGA >= 2 && NGA <= 5 && (NCB == 8 || NCB == 5) && (NB == 2 || NB == 3), "row groups spanned, column blocks");
     static_assert(RPX % 128 == 32 && RPX >= 2 * WCX && RPG % 128 == 40 && RPG >= 2 * WCG && CHPX % 16 == 0 && GCB % 128 == 24,
                   "operand alignment / bank spread");
     static_assert(4 * (WCX / 2) * NH <= NT && 4 * (WCG / 2) * NH <= NT, "a pass is at most one item per thread");
@@ -71,11 +76,11 @@ struct WgTzGeom {
     int nbands, ncolt, nslices;
 };
 
-template <typename T, int NGA, int NCB>
+template <typename T, int NGA, int NCB, int NB>
 __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict__ x, const T* __restrict__ gy,
                                                             float* __restrict__ part, const WgTzGeom g) {
-    using Sh = WgTzShape<NGA, NCB>;
-    constexpr int NT = Sh::NT, CS = Sh::CS, CPW = Sh::CPW, NH = Sh::NH, TWG = Sh::TWG, RPX = Sh::RPX, RPG = Sh::RPG;
+    using Sh = WgTzShape<NGA, NCB, NB>;
+    constexpr int NT = Sh::NT, CS = Sh::CS, CPW = Sh::CPW, NH = Sh::NH, TWG = Sh::TWG, RPX = Sh::RPX, RPG = Sh::RPG, NMF = Sh::NMF;
     constexpr int NSX = Sh::NSX, NSG = Sh::NSG, GBX = Sh::GBX, GBG = Sh::GBG, CHPX = Sh::CHPX, CHPG = Sh::CHPG;
     constexpr int WCPX = Sh::WCX / 2, WCPG = Sh::WCG / 2;
     extern __shared__ uint32_t smem[];
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
         const bool any = chok && rp < 4;
         gcol[0] = any && jc >= 0 && jc < cols_valid ? (uint32_t)((j0 + jc) * g.C + c0 + 8 * ih) * 2u : kNoCol;
         gcol[1] = any && jc + 1 >= 0 && jc + 1 < cols_valid ? (uint32_t)((j0 + jc + 1) * g.C + c0 + 8 * ih) * 2u : kNoCol;
-        gdst = (8 * ih) * CHPG + (2 * min(rp, 3)) * RPG + 4 * cp;
+        gdst = (8 * ih) * CHPG + (2 * (min(rp, 3) & 1)) * RPG + 4 * cp;   // within the row group (rp >> 1) of the pass
     }
     uint4 bx[2][4], bg[2][4];
     auto issue_x = [&](uint4 (&bf)[4], int pass) {   // xw rows 8 pass .. 8 pass + 7 (window row 0 = x row i0 - PH)
@@ -166,11 +171,11 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
         }
     };
     const bool gfirst = (tid / NH) % WCPG == 0;  // the item's first column is the window's first: nothing to its left
-    auto commit_g = [&](const uint4 (&bf)[4], int pass) {
-        if (grp < 0) return;
+    auto commit_g = [&](const uint4 (&bf)[4], int pass, int half) {   // half 0 / 1: one row group of the pass; -1: both
+        if (grp < 0 || (half >= 0 && (grp >> 1) != half)) return;
         const uint32_t a0[4] = {bf[0].x, bf[0].y, bf[0].z, bf[0].w}, a1[4] = {bf[1].x, bf[1].y, bf[1].z, bf[1].w};
         const uint32_t a2[4] = {bf[2].x, bf[2].y, bf[2].z, bf[2].w}, a3[4] = {bf[3].x, bf[3].y, bf[3].z, bf[3].w};
-        char* dst = gl + gdst + ((2 * pass) & (NSG - 1)) * GBG;
+        char* dst = gl + gdst + ((2 * pass + (grp >> 1)) % NSG) * GBG;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t p00 = __builtin_amdgcn_perm(a1[j], a0[j], 0x05040100u), p01 = __builtin_amdgcn_perm(a1[j], a0[j], 0x07060302u);
@@ -212,14 +217,22 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
 
     // ---- per-lane operand addresses
     const int ln = lane & 15, kr = lane >> 4;
-    const int la = min(ln >> 1, amax), lb = ln & 1;   // A: tap block (a, b); blocks beyond the filter read valid data
+    // A: tap block (a, b) = (i / NB, i % NB) of instruction f, i = ln + 16 f; blocks beyond the filter read valid data
+    int la[NMF];
+    const char* xlane[NMF];
+#pragma unroll
+    for (int f = 0; f < NMF; ++f) {
+        la[f] = min((ln + 16 * f) / NB, amax);
+        xlane[f] = xl + (wv * CPW) * CHPX + ((wv * CPW) >> 3) * Sh::XHALF + (8 * ((ln + 16 * f) % NB)) * 2;
+    }
     const int ldu = ln >> 3, ldv = ln & 7;            // B: fine offset (du, dv)
-    const char* const xlane = xl + (wv * CPW) * CHPX + ((wv * CPW) >> 3) * Sh::XHALF + (8 * lb) * 2;
     const char* const glane = gl + (ldv & 1) * Sh::GCB + (wv * CPW) * CHPG + ((8 - ldv) & ~1) * 2;
 
-    tz_f32x4 acc[CPW];
+    tz_f32x4 acc[CPW][NMF];
 #pragma unroll
-    for (int q = 0; q < CPW; ++q) acc[q] = tz_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int q = 0; q < CPW; ++q)
+#pragma unroll
+        for (int f = 0; f < NMF; ++f) acc[q][f] = tz_f32x4{0.f, 0.f, 0.f, 0.f};
 
     // the passes the first step reads: xw groups 0 .. NGA-1, gy group 0
     constexpr int P0X = (NGA + 1) / 2;
@@ -228,15 +241,20 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
         commit_x(bx[p % 2], p);
         issue_x(bx[p % 2], p + 2);
         if (p == 0) {
-            commit_g(bg[0], 0);
-            issue_g(bg[0], 2);
+            if constexpr (NSG == 4) {
+                commit_g(bg[0], 0, -1);
+                issue_g(bg[0], 2);
+            } else {
+                commit_g(bg[0], 0, 0);
+            }
         }
     }
     auto read_a = [&](const char* p) { return *reinterpret_cast<const uint4*>(p); };   // 16-byte aligned
     // Steps in trips of 4 without a test in between (the band's last trip may run up to 3 steps past its end: their gy
-    // rows read as zero, their loads move nothing).  A step first commits what the NEXT step adds to the windows, behind
-    // the barrier that ends the previous step's reads of the ring slots it overwrites; no condition depends on data,
-    // so the loads keep their exact in-flight counts.
+    // rows read as zero, their loads move nothing).  A step first commits what the NEXT step adds to the windows (an
+    // 8-row pass of xw or of gy on alternating steps; with 3 gy slots one row group of gy every step, the pass's
+    // registers being requested again once both of its groups are in LDS), behind the barrier that ends the previous step's reads of the ring slots it
+    // overwrites; no condition depends on data, so the loads keep their exact in-flight counts.
     constexpr int UNR = 4;
     for (int s0 = 0; s0 < nsteps; s0 += UNR) {
 #pragma unroll
@@ -248,27 +266,39 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
                 commit_x(bx[bi], pass);
                 issue_x(bx[bi], pass + 2);
             }
-            if (j % 2 == 1) {          // gy row group t + 1 opens a pass
+            if constexpr (NSG == 4) {
+                if (j % 2 == 1) {       // gy row group t + 1 opens a pass
+                    const int bi = ((j + 1) / 2) % 2, pass = (t + 1) / 2;
+                    commit_g(bg[bi], pass, -1);
+                    issue_g(bg[bi], pass + 2);
+                }
+            } else {                    // gy row group t + 1: half (t + 1) % 2 of pass (t + 1) / 2
                 const int bi = ((j + 1) / 2) % 2, pass = (t + 1) / 2;
-                commit_g(bg[bi], pass);
-                issue_g(bg[bi], pass + 2);
+                commit_g(bg[bi], pass, (j + 1) % 2);
+                if ((j + 1) % 2 == 1) issue_g(bg[bi], pass + 2);
             }
-            // A: xw rows 4 t + kr + 2 a;  B: gy rows 4 t + kr - du (relative to the band)
-            const int ra = 4 * (t % NSX) + kr + 2 * la;          // row within the ring, before wrapping
-            const char* xa = xlane + (ra >= 4 * NSX ? ra - 4 * NSX : ra) * RPX;
-            const int rr = 4 * t + kr - ldu;
-            const char* gb = glane + ((rr >> 2) & (NSG - 1)) * GBG + (rr & 3) * RPG;
+            // A: xw rows 4 t + kr + 2 a;  B: gy rows 4 t + kr - du (relative to the band): group t, or t - 1 for row -1
+            const char* xa[NMF];
+#pragma unroll
+            for (int f = 0; f < NMF; ++f) {
+                const int ra = 4 * (t % NSX) + kr + 2 * la[f];      // row within the ring, before wrapping
+                xa[f] = xlane[f] + (ra >= 4 * NSX ? ra - 4 * NSX : ra) * RPX;
+            }
+            const int st = t % NSG, sp = (t + NSG - 1) % NSG;
+            const char* gb = glane + (kr < ldu ? sp * GBG + 3 * RPG : st * GBG + (kr - ldu) * RPG);
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
                 for (int q = 0; q < CPW; ++q) {
                     const uint32_t* gp = reinterpret_cast<const uint32_t*>(gb + q * CHPG + 16 * cb);
-                    acc[q] = mfma16(read_a(xa + q * CHPX + 16 * cb), make_uint4(gp[0], gp[1], gp[2], gp[3]), acc[q], T());
+                    const uint4 bop = make_uint4(gp[0], gp[1], gp[2], gp[3]);
+#pragma unroll
+                    for (int f = 0; f < NMF; ++f) acc[q][f] = mfma16(read_a(xa[f] + q * CHPX + 16 * cb), bop, acc[q][f], T());
                 }
         }
     }
-    // ---- this band's partial.  Lane (n = (du, dv), row block kr) holds in register r the tap m = 4 kr + r = (a, b) =
-    // (m / 2, m % 2) of its two channels; the taps go through LDS ([tap][channel], 20 floats apart) so that a tap's 16
+    // ---- this band's partial.  Lane (n = (du, dv), row block kr) holds in register r of instruction f the tap block
+    // i = 4 kr + r + 16 f = (a, b) = (i / NB, i % NB) of its two channels; the taps go through LDS ([tap][channel], 20 floats apart) so that a tap's 16
     // channels leave as four 16-byte stores.
     lds_barrier();
     float* const ep = reinterpret_cast<float*>(smem);
@@ -276,11 +306,13 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
 #pragma unroll
     for (int q = 0; q < CPW; ++q)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = 4 * kr + r;
-            const int u = 2 * (m >> 1) + ldu, v = 8 * (m & 1) + ldv;
-            if (u < g.K && v < g.K) ep[(u * g.K + v) * EPP + wv * CPW + q] = acc[q][r];
-        }
+        for (int f = 0; f < NMF; ++f)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * kr + r + 16 * f;
+                const int u = 2 * (i / NB) + ldu, v = 8 * (i % NB) + ldv;
+                if (u < g.K && v < g.K) ep[(u * g.K + v) * EPP + wv * CPW + q] = acc[q][f][r];
+            }
     __syncthreads();
     float* pc = part + (long long)chunk * g.K * g.K * g.C;
     for (int i = tid; i < g.K * g.K * (CS / 4); i += NT) {
@@ -301,14 +333,13 @@ struct WgTzPlan {
     long long nblocks = 0;
 };
 
-// Covered: 16-bit types (the caller checks), C % 8 == 0, K <= 14 (a step's xw operand spans at most 4 row groups:
-// the LDS ring of a larger filter does not fit), 16-byte aligned tensors.
+// Covered: 16-bit types (the caller checks), C % 8 == 0, K <= 17, 16-byte aligned tensors.
 inline WgTzPlan wgrad_tz_plan(int B, int H, int W, int C, int K, int PH, int PW) {
     WgTzPlan p;
     WgTzGeom& g = p.g;
     g.B = B, g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.K = K;
     g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
-    if (K < 1 || K > 14 || C % 8 != 0 || B < 1 || g.OH < 1 || g.OW < 1) return p;
+    if (K < 1 || K > 17 || C % 8 != 0 || B < 1 || g.OH < 1 || g.OW < 1) return p;
     if ((long long)H * W * C > 0x1fffffffLL || (long long)g.OH * g.OW * C > 0x1fffffffLL) return p;
     p.ncb = g.OW <= 32 ? 5 : 8;
     const int twg = 8 * p.ncb - 8, ta = wgrad_tz_nga(K);
@@ -335,10 +366,10 @@ inline size_t wgrad_tz_workspace(int B, int H, int W, int C, int K, int PH, int 
     return p.ok ? (size_t)B * p.g.nbands * p.g.ncolt * K * K * C * sizeof(float) : 0;
 }
 
-template <typename T, int NGA, int NCB>
+template <typename T, int NGA, int NCB, int NB>
 static int launch_wgrad_tz(const WgTzPlan& p, const void* x, const void* gy, void* ws, hipStream_t s) {
-    using Sh = WgTzShape<NGA, NCB>;
-    auto kern = dwconv_wgrad_tz_k<T, NGA, NCB>;
+    using Sh = WgTzShape<NGA, NCB, NB>;
+    auto kern = dwconv_wgrad_tz_k<T, NGA, NCB, NB>;
     static std::once_flag attr_once;
     std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)p.nblocks), dim3(Sh::NT), Sh::lds_bytes, s, (const T*)x, (const T*)gy, (float*)ws, p.g);

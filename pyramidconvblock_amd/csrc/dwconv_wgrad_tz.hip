@@ -1,5 +1,5 @@
 // Depthwise-convolution weight gradient on the dense matrix cores (dwconv_wgrad_tz.h): the instantiations of the
-// kernel template (filter sizes 1..14 by the row groups an operand spans, two tile widths, two 16-bit types), the workspace query
+// kernel template (filter sizes 1..17 by the row groups an operand spans, two tile widths, two 16-bit types), the workspace query
 // and the launcher.
 #include "dwconv_wgrad_tz.h"
 
@@ -15,13 +15,14 @@ size_t dwconv_wgrad_tz_workspace(int B, int H, int W, int C, int K, int PH, int 
 template <typename T>
 static int wgrad_tz_go(const WgTzPlan& p, const void* x, const void* gy, void* ws, hipStream_t s) {
     const int nga = wgrad_tz_nga(p.g.K);
-#define PDW_TZ(NGA_)                                                                  \
-    case NGA_:                                                                        \
-        return p.ncb == 8 ? launch_wgrad_tz<T, NGA_, 8>(p, x, gy, ws, s) : launch_wgrad_tz<T, NGA_, 5>(p, x, gy, ws, s);
+#define PDW_TZ(NGA_, NB_)                                                            \
+    return p.ncb == 8 ? launch_wgrad_tz<T, NGA_, 8, NB_>(p, x, gy, ws, s) : launch_wgrad_tz<T, NGA_, 5, NB_>(p, x, gy, ws, s);
+    if (p.g.K == 17) { PDW_TZ(5, 3) }
     switch (nga) {
-        PDW_TZ(2)
-        PDW_TZ(3)
-        PDW_TZ(4)
+        case 2: PDW_TZ(2, 2)
+        case 3: PDW_TZ(3, 2)
+        case 4: PDW_TZ(4, 2)
+        case 5: PDW_TZ(5, 2)
         default: return -1;
     }
 #undef PDW_TZ

@@ -37,7 +37,7 @@ def _run(oracle, shape, k, dtype, stride=1, padding=None, dilation=1, seed=0, di
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [3, 7, 9, 13, 17])
+@pytest.mark.parametrize("k", [3, 5, 7, 9, 11, 13, 15, 17])
 def test_same_padding_small(oracle, dtype, k):
     _run(oracle, (2, 20, 23, 24), k, dtype)
 
