@@ -65,6 +65,18 @@ int pdw_dwconv_fwd(const void *x, const void *w, void *y, int B, int H, int W, i
 int pdw_dwconv_fwd_pool(const void *x, const void *w, void *y, void *xp, int B, int H, int W, int C, int KH, int KW,
                         int SH, int SW, int PH, int PW, int DH, int DW, int h, int wp, int dtype, void *stream);
 
+/* Inference form of SimpleGate's convolution and gate (conv_block.py:17-19) for stride 1 and a square filter:
+ *   y[b,i,j, ych + c] = conv(x)[b,i,j,c] * conv(x)[b,i,j,C/2 + c] * sqrt(C/2),   c < C/2,
+ * written with a pixel stride of ldy channels (0: C/2), e.g. straight into its slice of the concatenation of
+ * conv_block.py:43, so that the convolution output itself never reaches HBM.  The product is formed from the rounded
+ * convolution outputs in fp32 and rounded once, as pdw_gate_fwd does.  xp (may be NULL): the 2x2 average pool of x,
+ * [B,H/2,W/2,C] (needs even H, W, pad and 2*pad = K-1).  Returns 3 when the fused kernel does not cover the case
+ * (it needs a 16-bit dtype, C % 16 == 0, odd K <= 13, ldy and ych multiples of 8): the caller then runs pdw_dwconv_fwd
+ * (or pdw_dwconv_fwd_pool) and pdw_gate_fwd.  No counterpart in the reference, which keeps the convolution output for
+ * its backward. */
+int pdw_dwconv_fwd_gate(const void *x, const void *w, void *y, void *xp, int B, int H, int W, int C, int K, int pad,
+                        int ldy, int ych, int dtype, void *stream);
+
 /* Input gradient (exact adjoint of pdw_dwconv_fwd in x): gy[B,OH,OW,C] -> dx[B,H,W,C]; H,W are
  * the forward INPUT extents.  Fully overwrites dx (no pre-zeroing needed).
  * Replaces the launch of _depthwise_conv_backward_input_kernel, dwconv_triton.py:358-366
@@ -244,6 +256,13 @@ int pdw_block_mid_bwd(const void *gy, const void *xf, const void *xh, void *gxf,
                       int h, int w, int I, int ldgy, const float *parts, int nparts, const void *m,
                       const void *w_pool, void *gbias, void *gbias2, void *gw_pool, float *dmean, void *workspace,
                       size_t workspace_bytes, int P, int D, int dtype, void *stream);
+/* The middle of the two-scale block at inference: the gated half-resolution scale xh[B,h,w,G] upsampled
+ * (pdw_bilinear_fwd) into y[..., :G] with pixel stride ldy (its slice of the concatenation), together with
+ * pdw_pool_branch_fwd_parts, in one launch where the combination is covered and one after the other otherwise.
+ * conv_block.py:20-21, :46-49. */
+int pdw_block_mid_infer(const void *xh, void *y, int B, int H, int W, int h, int w, int G, int ldy,
+                        const float *parts, int nparts, const void *w_pool, const void *b_pool, const void *b_out,
+                        void *m, float *rowbias, int P, int D, int dtype, void *stream);
 
 /* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 8 == 0;
  * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).
@@ -297,6 +316,18 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
  * when the call's work on `stream` is done.  Results are bitwise those of the separate calls.
  * Replaces the Python-level sequence of ConvBlock.forward, conv_block.py:36-49, and its autograd backward. */
 int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype);
+/* Inference forward of the same block (same coverage): y only.  conv_up, then each scale's convolution with the gate
+ * applied in its store (pdw_dwconv_fwd_gate; the full-resolution one also pools its input for the second scale), the
+ * half-resolution gate upsampled into its slice of the concatenation, conv_out plus the mean branch.  Neither
+ * convolution output is written to HBM, and every intermediate lives in `workspace`
+ * (pdw_convblock_infer_workspace_bytes).  Where the fused convolution does not cover the filter size the call runs
+ * the launches of pdw_convblock_fwd on workspace tensors instead.  Same arithmetic as pdw_convblock_fwd except that
+ * the half-resolution gate is rounded to `dtype` before it is upsampled.  Replaces ConvBlock.forward under
+ * torch.no_grad(), conv_block.py:36-49 with :13-22. */
+size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype);
+int pdw_convblock_infer(const void *x, const void *w_up, const void *w_dw0, const void *w_dw1, const void *w_pool,
+                        const void *b_pool, const void *w_out, const void *b_out, void *y, void *workspace,
+                        size_t workspace_bytes, int B, int H, int W, int D, int I, int K, int dtype, void *stream);
 size_t pdw_convblock_fwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype);
 int pdw_convblock_fwd(const void *x, const void *w_up, const void *w_dw0, const void *w_dw1, const void *w_pool,
                       const void *b_pool, const void *w_out, const void *b_out, void *a, void *c0, void *xp, void *c1,

@@ -27,6 +27,7 @@ _SIGS = {
     "pdw_conv_out_size": (c_int, [c_int] * 5),
     "pdw_dwconv_fwd": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
     "pdw_dwconv_fwd_pool": (c_int, [c_void_p] * 4 + _CONV + [c_int, c_int, c_int, c_void_p]),
+    "pdw_dwconv_fwd_gate": (c_int, [c_void_p] * 4 + [c_int] * 9 + [c_void_p]),
     "pdw_dwconv_dgrad": (c_int, [c_void_p] * 3 + _CONV + [c_int, c_void_p]),
     "pdw_reduce_defer_begin": (c_int, []),
     "pdw_reduce_defer_flush": (c_int, [c_void_p]),
@@ -40,6 +41,8 @@ _SIGS = {
     "pdw_convblock_supported": (c_int, [c_int] * 7),
     "pdw_convblock_fwd_workspace_bytes": (c_size_t, [c_int] * 7),
     "pdw_convblock_fwd": (c_int, [c_void_p] * 16 + [c_size_t] + [c_int] * 7 + [c_void_p]),
+    "pdw_convblock_infer_workspace_bytes": (c_size_t, [c_int] * 7),
+    "pdw_convblock_infer": (c_int, [c_void_p] * 10 + [c_size_t] + [c_int] * 7 + [c_void_p]),
     "pdw_convblock_bwd_workspace_bytes": (c_size_t, [c_int] * 7),
     "pdw_convblock_bwd": (c_int, [c_void_p] * 22 + [c_size_t] + [c_int] * 7 + [c_void_p]),
     "pdw_avgpool_fwd": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p]),
@@ -63,6 +66,8 @@ _SIGS = {
     "pdw_dense_colsum_rows": (c_int, []),
     "pdw_dense_fwd_colsum": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong]
                              + [c_int] * 4 + [c_void_p]),
+    "pdw_block_mid_infer": (c_int, [c_void_p] * 2 + [c_int] * 7 + [c_void_p, c_int] + [c_void_p] * 5 + [c_int] * 3
+                            + [c_void_p]),
     "pdw_block_mid_fwd": (c_int, [c_void_p] * 3 + [c_int] * 7 + [c_void_p, c_int] + [c_void_p] * 5 + [c_int] * 3
                           + [c_void_p]),
     "pdw_block_mid_bwd": (c_int, [c_void_p] * 5 + [c_int] * 7 + [c_void_p, c_int] + [c_void_p] * 7 + [c_size_t]

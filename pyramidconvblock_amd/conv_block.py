@@ -105,6 +105,25 @@ def _block_call_ok(x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, w_dw) ->
     return bool(_lib.lib().pdw_convblock_supported(B, H, W, D, I, K, _lib.dtype_code(dt)))
 
 
+def convblock_infer(x, w_up, w_out, b_out, w_pool, b_pool, w_dw):
+    """Inference forward through pdw_convblock_infer: y only, neither convolution output written to HBM where the
+    fused convolution + gate covers the filter (conv_block.py:36-49 under no_grad).  The caller has checked
+    ``_block_call_ok``."""
+    dev = _lib.require_device(x)
+    B, H, W, D = x.shape
+    I, K = w_up.shape[0], w_dw[0].shape[0]
+    L, code = _lib.lib(), _lib.dtype_code(x.dtype)
+    y = torch.empty((B, H, W, D), device=dev, dtype=x.dtype)
+    ws = torch.empty(L.pdw_convblock_infer_workspace_bytes(B, H, W, D, I, K, code) // 4 + 1, device=dev,
+                     dtype=torch.float32)
+    _lib.check(L.pdw_convblock_infer(x.data_ptr(), w_up.data_ptr(), w_dw[0].data_ptr(), w_dw[1].data_ptr(),
+                                     w_pool.data_ptr(), b_pool.data_ptr() if b_pool is not None else None,
+                                     w_out.data_ptr(), b_out.data_ptr() if b_out is not None else None, y.data_ptr(),
+                                     ws.data_ptr(), ws.numel() * 4, B, H, W, D, I, K, code, _lib.stream_ptr(dev)),
+               "pdw_convblock_infer")
+    return y
+
+
 def _is_pair(scales) -> bool:
     return len(scales) == 2 and scales[0] == 1. and scales[1] != 1.
 
@@ -377,6 +396,16 @@ class ConvBlock(nn.Module):
         if x.dim() != 4 or x.shape[3] != self.conv_up.in_features:
             raise ValueError(f"expected [B,H,W,{self.conv_up.in_features}] input, got {tuple(x.shape)}")
         scales = tuple(float(g.scale_factor) for g in self.gates)
+        if not (torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))):
+            # nothing to save for a backward: the inference form of the block, where the library covers the shape
+            xc = x.detach().contiguous()
+            args = (self.conv_up.weight.detach(), self.conv_up.bias, self.conv_out.weight.detach(),
+                    None if self.conv_out.bias is None else self.conv_out.bias.detach(), self.conv_pool.weight.detach(),
+                    None if self.conv_pool.bias is None else self.conv_pool.bias.detach(),
+                    [g.conv_spatial.weight.detach() for g in self.gates])
+            if _block_call_ok(xc, scales, *args):
+                with _lib.launch_scope(_lib.require_device(xc)):
+                    return convblock_infer(xc, args[0], args[2], args[3], args[4], args[5], args[6])
         return ConvBlockFunction.apply(x, scales, self.conv_up.weight, self.conv_up.bias, self.conv_out.weight,
                                        self.conv_out.bias, self.conv_pool.weight, self.conv_pool.bias,
                                        *[g.conv_spatial.weight for g in self.gates])

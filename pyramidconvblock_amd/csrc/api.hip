@@ -125,6 +125,23 @@ int pdw_dwconv_fwd_pool(const void* x, const void* w, void* y, void* xp, int B, 
     return avgpool_fwd_launch(x, xp, B, H, W, C, h, wp, dtype, (hipStream_t)stream);
 }
 
+int pdw_dwconv_fwd_gate(const void* x, const void* w, void* y, void* xp, int B, int H, int W, int C, int K, int pad,
+                        int ldy, int ych, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_dwconv_fwd_gate: unknown dtype %d", dtype), 1;
+    if (B < 0 || H < 1 || W < 1 || C < 2 || K < 1 || pad < 0)
+        return set_error("pdw_dwconv_fwd_gate: bad extents B=%d H=%d W=%d C=%d K=%d pad=%d", B, H, W, C, K, pad), 1;
+    if (ldy == 0) ldy = C / 2;
+    if ((C & 1) || ych < 0 || ldy < ych + C / 2)
+        return set_error("pdw_dwconv_fwd_gate: need even C and ych + C/2 <= ldy (C=%d ldy=%d ych=%d)", C, ldy, ych), 1;
+    if (B > 0 && (!x || !w || !y)) return set_error("pdw_dwconv_fwd_gate: null pointer"), 1;
+    if (B == 0) return 0;
+    const int r = dwconv_gate_launch(x, w, y, xp, B, H, W, C, K, pad, pad, ldy, ych, dtype, (hipStream_t)stream);
+    if (r == -1)
+        return set_error("pdw_dwconv_fwd_gate: B=%d H=%d W=%d C=%d K=%d pad=%d dtype=%d not covered by the fused kernel", B,
+                         H, W, C, K, pad, dtype), 3;
+    return r;
+}
+
 int pdw_dwconv_dgrad(const void* gy, const void* w, void* dx, int B, int H, int W, int C, int KH, int KW, int SH,
                      int SW, int PH, int PW, int DH, int DW, int dtype, void* stream) {
     if (int e = check_conv("pdw_dwconv_dgrad", gy, w, dx, B, H, W, C, KH, KW, SH, SW, PH, PW, DH, DW, dtype)) return e;
@@ -408,6 +425,23 @@ int pdw_pool_branch_bwd_parts(const float* parts, int nparts, const void* m, con
     if (!workspace || workspace_bytes < pool_branch_workspace(B, P, D))
         return set_error("pdw_pool_branch_bwd_parts: workspace too small"), 1;
     return pool_branch_bwd_launch(nullptr, m, w_pool, gbias, gbias2, gw_pool, dmean, (float*)workspace, B, P, D, dtype,
+                                  (hipStream_t)stream, parts, nparts);
+}
+
+int pdw_block_mid_infer(const void* xh, void* y, int B, int H, int W, int h, int w, int G, int ldy, const float* parts,
+                        int nparts, const void* w_pool, const void* b_pool, const void* b_out, void* m, float* rowbias,
+                        int P, int D, int dtype, void* stream) {
+    if (int e = check_resample("pdw_block_mid_infer", xh, y, B, H, W, G, h, w, dtype)) return e;
+    if (B < 1 || P < 1 || D < 1 || nparts < 1)
+        return set_error("pdw_block_mid_infer: bad extents B=%d P=%d D=%d nparts=%d", B, P, D, nparts), 1;
+    if (!parts || !w_pool || !m || !rowbias) return set_error("pdw_block_mid_infer: null pointer"), 1;
+    if (ldy == 0) ldy = G;
+    if (ldy < G) return set_error("pdw_block_mid_infer: ldy=%d smaller than G=%d", ldy, G), 1;
+    const int r = bilinear_pool_fwd_launch(xh, y, B, h, w, G, H, W, ldy, parts, nparts, w_pool, b_pool, b_out, m, rowbias,
+                                           P, D, dtype, (hipStream_t)stream);
+    if (r != -1) return r;
+    if (int e = bilinear_fwd_launch(xh, y, B, h, w, G, H, W, ldy, dtype, (hipStream_t)stream)) return e;
+    return pool_branch_fwd_launch(nullptr, w_pool, b_pool, b_out, m, rowbias, nullptr, B, P, D, dtype,
                                   (hipStream_t)stream, parts, nparts);
 }
 

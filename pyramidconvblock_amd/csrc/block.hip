@@ -95,6 +95,67 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
     return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
 }
 
+// The fused convolution + gate needs 16 channels per workgroup, which the operand registers allow up to K = 13.
+static bool infer_fused(int K) { return K <= 13; }
+
+size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
+    if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
+    const Shape s = shape_of(B, H, W, D, I, K, dtype);
+    const size_t full = (size_t)s.N * I * s.es, half = (size_t)B * s.h * s.w * I * s.es;
+    size_t b = up256(full) /* a */ + up256(half) /* xp */ + up256(full) /* cat */ + up256((size_t)B * D * s.es) /* m */ +
+               up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4);
+    if (infer_fused(K))
+        b += up256(half / 2);  // the gated half-resolution scale
+    else
+        b += up256(full) + up256(half);  // c0, c1
+    return b;
+}
+
+int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, const void* w_dw1, const void* w_pool,
+                        const void* b_pool, const void* w_out, const void* b_out, void* y, void* workspace,
+                        size_t workspace_bytes, int B, int H, int W, int D, int I, int K, int dtype, void* stream) {
+    if (!pdw_convblock_supported(B, H, W, D, I, K, dtype))
+        return set_error("pdw_convblock_infer: shape not covered (B=%d H=%d W=%d D=%d I=%d K=%d dtype=%d)", B, H, W, D, I,
+                         K, dtype), 1;
+    for (const void* ptr : {x, w_up, w_dw0, w_dw1, w_pool, w_out, (const void*)y, (const void*)workspace})
+        if (!ptr) return set_error("pdw_convblock_infer: null pointer"), 1;
+    const size_t need = pdw_convblock_infer_workspace_bytes(B, H, W, D, I, K, dtype);
+    if (workspace_bytes < need)
+        return set_error("pdw_convblock_infer: workspace of %zu bytes given, %zu needed", workspace_bytes, need), 1;
+    const Shape s = shape_of(B, H, W, D, I, K, dtype);
+    const size_t full = (size_t)s.N * I * s.es, half = (size_t)B * s.h * s.w * I * s.es;
+    Carver ws{(char*)workspace, workspace_bytes};
+    void* a = ws.take(full);
+    void* xp = ws.take(half);
+    void* cat = ws.take(full);
+    void* m = ws.take((size_t)B * D * s.es);
+    float* xparts = (float*)ws.take((size_t)s.nt * D * 4);
+    float* yp = (float*)ws.take((size_t)B * D * 4);
+    const int pad = K / 2, G = I / 2;
+    if (!infer_fused(K)) {
+        void* c0 = ws.take(full);
+        void* c1 = ws.take(half);
+        // the forward's own launches; its workspace is xparts and yp, which lie next to each other
+        return pdw_convblock_fwd(x, w_up, w_dw0, w_dw1, w_pool, b_pool, w_out, b_out, a, c0, xp, c1, cat, m, y, xparts,
+                                 up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4), B, H, W, D, I, K, dtype, stream);
+    }
+    void* g1 = ws.take(half / 2);
+    if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) return e;
+    // scale 1: conv + gate into cat[..., :G], and the pooled input of scale 1/2            (conv_block.py:14-19)
+    // (the convolution's staging threads hold whole pool windows only when the padding is even)
+    const bool pool_fused = (pad & 1) == 0;
+    if (int e = pdw_dwconv_fwd_gate(a, w_dw0, cat, pool_fused ? xp : nullptr, B, H, W, I, K, pad, I, 0, dtype, stream)) return e;
+    if (!pool_fused)
+        if (int e = pdw_avgpool_fwd(a, xp, B, H, W, I, s.h, s.w, dtype, stream)) return e;
+    // scale 1/2: conv + gate, upsampled into cat[..., G:]                                   (conv_block.py:17-21)
+    if (int e = pdw_dwconv_fwd_gate(xp, w_dw1, g1, nullptr, B, s.h, s.w, I, K, pad, G, 0, dtype, stream)) return e;
+    // ... together with mean -> conv_pool (+ both biases) into yp                             (conv_block.py:46-49)
+    if (int e = pdw_block_mid_infer(g1, (char*)cat + (size_t)G * s.es, B, H, W, s.h, s.w, G, I, xparts, (int)(s.nt / B),
+                                    w_pool, b_pool, b_out, m, yp, s.P, D, dtype, stream))
+        return e;
+    return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
+}
+
 size_t pdw_convblock_bwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
     if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
     const Shape s = shape_of(B, H, W, D, I, K, dtype);

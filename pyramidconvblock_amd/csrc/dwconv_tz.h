@@ -26,9 +26,14 @@
 // small double-buffered LDS tile (pixel-major, one dword of padding per 4 pixels keeps the 4-byte scatter free of
 // bank conflicts) and leave as 16-byte stores, one step behind the MFMAs.
 //
-// MODE 1 (input gradient of a tensor that was also average-pooled 2x2): y += add[i/2, j/2] / 4 in the store.
-// MODE 2 (forward): the 2x2 average pool of x is written to `pool` by the staging threads, which hold exactly the
+// MODE is a set of bits.
+// 1 (input gradient of a tensor that was also average-pooled 2x2): y += add[i/2, j/2] / 4 in the store.
+// 2 (forward): the 2x2 average pool of x is written to `pool` by the staging threads, which hold exactly the
 // four pixels of a pool window in registers (needs even padding, so that windows do not straddle threads).
+// 4 (forward, inference): the gate of conv_block.py:18-19 in the store.  A workgroup's 16 channels are 8 of the first
+// half and the matching 8 of the second half of C, and the two store threads of a pixel multiply four channel pairs
+// each (the rounded convolution outputs, as the stand-alone gate kernel does): y[..., c] = conv[c] * conv[C/2 + c] * gs,
+// C/2 channels wide, written with a pixel stride of YC channels from channel `ych` on (into the concatenation).
 //
 // Zero entries of A multiply real pixels of the window (and the window is wider than K+3 where (K+3) % 8 != 0), so a
 // non-finite input value reaches outputs up to 3 + 8 ICB - (K+3) pixels beyond its K x K footprint as NaN.
@@ -93,6 +98,8 @@ struct TzGeom {
     int CHP;           // LDS bytes per channel plane
     int flip;          // 1: 180-degree rotated filter (input gradient)
     int AH, AW;        // extents of the half-resolution addend / pooled output
+    int YC, ych;       // output pixel stride in channels, first output channel
+    float gs;          // gate factor (MODE & 4)
 };
 
 // 8 values of T: a + b / 4, rounded once more (what an accumulating pool gradient does to a stored tensor).
@@ -108,6 +115,19 @@ __device__ __forceinline__ uint4 tz_add_quarter(uint4 a, uint4 b) {
     return uo.u;
 }
 
+// 4 values of T: a * b * s, rounded once (the arithmetic of the stand-alone gate kernel).
+template <typename T>
+__device__ __forceinline__ uint2 tz_gate(uint2 a, uint2 b, float s) {
+    union U {
+        uint2 u;
+        T t[4];
+    } ua, ub, uo;
+    ua.u = a, ub.u = b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) uo.t[i] = from_f32<T>(to_f32(ua.t[i]) * to_f32(ub.t[i]) * s);
+    return uo.u;
+}
+
 template <typename T, int K, int NPC, int CS, int MODE>
 __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, const T* __restrict__ w,
                                                       const T* __restrict__ add, T* __restrict__ pool,
@@ -116,6 +136,8 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     constexpr int NT = Sh::NT, ICB = Sh::ICB, NKG = Sh::NKG, NM = Sh::NM, PER = Sh::PER, RING = Sh::RING;
     constexpr int NI = Sh::NI, TW = Sh::TW, NH = Sh::NH, CPW = Sh::CPW, RP = Sh::RP, OPX = Sh::OPX, OROWP = Sh::OROWP;
     constexpr int OLB = Sh::OLB, WTH = Sh::WTH, WTW = Sh::WTW;
+    constexpr bool ADD = (MODE & 1) != 0, POOL = (MODE & 2) != 0, GATE = (MODE & 4) != 0;
+    static_assert(!GATE || (CS == 16 && !ADD), "the gate pairs the two 8-channel pieces of a 16-channel slice");
     extern __shared__ uint32_t smem[];
     char* const xl = reinterpret_cast<char*>(smem);        // [NI][CS] planes of CHP bytes: [row][column] of T
     char* const r2 = xl + NI * CS * g.CHP;                 // filter table, then the two result tiles
@@ -132,7 +154,9 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     const int nsteps = (rows_valid + 3) >> 2;
     const int NROWS = 4 * (nsteps + PER - 1);              // window rows the steps read
     const int WCP = (4 * ((cols_valid + 3) / 4 - 1) + 8 * ICB) / 2;  // column pairs the used patches read
-    const long long img_in = (long long)g.H * g.W * g.C, img_out = (long long)g.OH * g.OW * g.C;
+    const long long img_in = (long long)g.H * g.W * g.C, img_out = (long long)g.OH * g.OW * g.YC;
+    // first channel of the slice's 8-channel piece h
+    auto chof = [&](int h) { return GATE ? 8 * sl + h * (g.C >> 1) : c0 + 8 * h; };
 
     // ---- filter slice, 8 channels of a tap per load: requested before the window, so that waiting for it leaves
     // the window's loads in flight
@@ -141,7 +165,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
 #pragma unroll
     for (int i = 0; i < NWL; ++i) {
         const int idx = min(tid + i * NT, K * K * NH - 1);
-        wval[i] = *reinterpret_cast<const uint4*>(w + (idx / NH) * g.C + min(c0 + 8 * (idx % NH), g.C - 8));
+        wval[i] = *reinterpret_cast<const uint4*>(w + (idx / NH) * g.C + min(chof(idx % NH), g.C - 8));
     }
 
     // ---- staging.  The window arrives in passes, requested two ahead into two register buffers.  Passes 0 and 1
@@ -176,15 +200,15 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
         const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI, rpw = idx / NH / WCP / NI;
         irpw[l] = rpw;
         const int ic = ocol0 - g.PW + 2 * cp;
-        const bool any = c0 + 8 * h < g.C && rpw < RPMAX;
-        const uint32_t ioff = (uint32_t)img * (uint32_t)img_in + (uint32_t)(c0 + 8 * h);
+        const bool any = chof(h) < g.C && rpw < RPMAX;
+        const uint32_t ioff = (uint32_t)img * (uint32_t)img_in + (uint32_t)chof(h);
         icol[l][0] = any && ic >= 0 && ic < g.W ? (ioff + (uint32_t)(ic * g.C)) * 2u : kNoCol;
         icol[l][1] = any && ic + 1 >= 0 && ic + 1 < g.W ? (ioff + (uint32_t)((ic + 1) * g.C)) * 2u : kNoCol;
         idst[l] = (img * CS + 8 * h) * g.CHP + (2 * min(rpw, RPMAX - 1)) * RP + 4 * cp;
     }
     // the 2x2 average pool of x (MODE 2) leaves through a buffer descriptor as well: a store past its end is dropped
     __amdgpu_buffer_rsrc_t prsrc = xrsrc;
-    if constexpr (MODE == 2)
+    if constexpr (POOL)
         prsrc = __builtin_amdgcn_make_buffer_rsrc(pool + (long long)b0 * g.AH * g.AW * g.C, (short)0,
                                                   (int)((long long)min(NI, g.B - b0) * g.AH * g.AW * g.C * 2), 0x00020000);
     uint4 buf[2][NLD][4];
@@ -223,12 +247,12 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
                     *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
                 }
             }
-            if constexpr (MODE == 2) {
+            if constexpr (POOL) {
                 // the thread holds one window of the 2x2 pool (H, W, PH, PW even): the band that owns these rows writes it
                 const int idx = tid + l * NT;
                 const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI;
                 const int ir = orow0 - g.PH + wr, ic = ocol0 - g.PW + 2 * cp;
-                const bool mine = irpw[l] < nrp && c0 + 8 * h < g.C && ir >= orow0 && ir < orow0 + rows_valid && ic >= ocol0 &&
+                const bool mine = irpw[l] < nrp && chof(h) < g.C && ir >= orow0 && ir < orow0 + rows_valid && ic >= ocol0 &&
                                   ic < ocol0 + cols_valid;
                 union U {
                     uint4 u;
@@ -238,7 +262,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     o.t[e] = from_f32<T>((((to_f32(p0.t[e]) + to_f32(p1.t[e])) + to_f32(p2.t[e])) + to_f32(p3.t[e])) * 0.25f);
-                const uint32_t off = mine ? (uint32_t)(((img * g.AH + (ir >> 1)) * g.AW + (ic >> 1)) * g.C + c0 + 8 * h) * 2u : kNoRow;
+                const uint32_t off = mine ? (uint32_t)(((img * g.AH + (ir >> 1)) * g.AW + (ic >> 1)) * g.C + chof(h)) * 2u : kNoRow;
                 typedef unsigned v4u __attribute__((ext_vector_type(4)));
                 __builtin_amdgcn_raw_buffer_store_b128(v4u{o.u.x, o.u.y, o.u.z, o.u.w}, prsrc, (int)off, 0, 0);
             }
@@ -264,7 +288,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
             const int idx = tid + i * NT;
             const int h = idx % NH, uv = idx / NH;
             const int u = uv / K, v = uv - u * K;
-            if (idx < K * K * NH && c0 + 8 * h < g.C) {
+            if (idx < K * K * NH && chof(h) < g.C) {
                 const uint32_t d[4] = {wval[i].x, wval[i].y, wval[i].z, wval[i].w};
                 const int uu = g.flip ? K - 1 - u : u, vv = g.flip ? K - 1 - v : v;
                 unsigned short* wp = wt + ((8 * h) * WTH + 3 + uu) * WTW + 3 + vv;
@@ -314,18 +338,18 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     // descriptors (an offset past the end: nothing stored / zero loaded), so that no vector memory instruction of the
     // kernel sits behind a branch and the in-flight counts the staging waits rely on stay exact
     const int sh = tid % NH, scol = (tid / NH) % TW, srow = (tid / NH / TW) % 4, simg = tid / NH / TW / 4;
-    const bool s_ok = simg < NI && scol < cols_valid && c0 + 8 * sh < g.C;
+    const bool s_ok = simg < NI && scol < cols_valid && (GATE || c0 + 8 * sh < g.C);
     const char* const olr = r2 + (min(simg, NI - 1) * 4 + srow) * OROWP + scol * OPX + (scol >> 2) * 4 + 16 * sh;
     const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(
         y + (long long)b0 * img_out, (short)0, (int)(min(NI, g.B - b0) * img_out * 2), 0x00020000);
-    const uint32_t ycol = (uint32_t)simg * (uint32_t)img_out + (uint32_t)((ocol0 + scol) * g.C + c0 + 8 * sh);
+    const uint32_t ycol = (uint32_t)simg * (uint32_t)img_out + (uint32_t)((ocol0 + scol) * g.YC + g.ych + (GATE ? 8 * sl + 4 * sh : c0 + 8 * sh));
     __amdgpu_buffer_rsrc_t arsrc = xrsrc;
-    if constexpr (MODE == 1)
+    if constexpr (ADD)
         arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(add + (long long)b0 * g.AH * g.AW * g.C), (short)0,
                                                   (int)((long long)min(NI, g.B - b0) * g.AH * g.AW * g.C * 2), 0x00020000);
     uint4 addv[2] = {make_uint4(0u, 0u, 0u, 0u), make_uint4(0u, 0u, 0u, 0u)};
     auto add_fetch = [&](int f) {   // the addends of step f's two tiles
-        if constexpr (MODE == 1) {
+        if constexpr (ADD) {
 #pragma unroll
             for (int gi = 0; gi < 2; ++gi) {
                 const int row = 4 * (2 * f + gi) + srow;
@@ -342,12 +366,22 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
             uint4 v;
             v.x = *reinterpret_cast<const uint32_t*>(src), v.y = *reinterpret_cast<const uint32_t*>(src + 4);
             v.z = *reinterpret_cast<const uint32_t*>(src + 8), v.w = *reinterpret_cast<const uint32_t*>(src + 12);
-            if constexpr (MODE == 1) v = tz_add_quarter<T>(v, addv[gi]);
+            if constexpr (ADD) v = tz_add_quarter<T>(v, addv[gi]);
             const int row = 4 * (2 * f + gi) + srow;
             const bool ok = s_ok && f >= 0 && row < rows_valid;
-            const uint32_t off = ok ? (ycol + (uint32_t)((orow0 + row) * g.OW * g.C)) * 2u : kNoRow;
-            typedef unsigned v4u __attribute__((ext_vector_type(4)));
-            __builtin_amdgcn_raw_buffer_store_b128(v4u{v.x, v.y, v.z, v.w}, yrsrc, (int)off, 0, 0);
+            const uint32_t off = ok ? (ycol + (uint32_t)((orow0 + row) * g.OW * g.YC)) * 2u : kNoRow;
+            if constexpr (GATE) {
+                // the thread gates 4 of the pixel's 8 channel pairs: values 4 sh .. 4 sh + 3 of both 8-channel pieces
+                const char* sg = src - 8 * sh;   // (src points 16 sh into the pixel)
+                const uint2 a = make_uint2(*reinterpret_cast<const uint32_t*>(sg), *reinterpret_cast<const uint32_t*>(sg + 4));
+                const uint2 b = make_uint2(*reinterpret_cast<const uint32_t*>(sg + 16), *reinterpret_cast<const uint32_t*>(sg + 20));
+                const uint2 o = tz_gate<T>(a, b, g.gs);
+                typedef unsigned v2u __attribute__((ext_vector_type(2)));
+                __builtin_amdgcn_raw_buffer_store_b64(v2u{o.x, o.y}, yrsrc, (int)off, 0, 0);
+            } else {
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                __builtin_amdgcn_raw_buffer_store_b128(v4u{v.x, v.y, v.z, v.w}, yrsrc, (int)off, 0, 0);
+            }
         }
     };
 
@@ -473,13 +507,15 @@ static int tz_pick_band(int B, int OH, int OW, int C) {
 
 template <typename T, int K, int NPC, int CS>
 static int launch_tz(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
-                     int PH, int PW, bool flip, hipStream_t s) {
+                     int PH, int PW, bool flip, const TzGate* gate, hipStream_t s) {
     using Sh = TzShape<K, NPC, CS>;
     TzGeom g;
     g.B = B, g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0;
     g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
     g.AH = add ? g.OH / 2 : H / 2, g.AW = add ? g.OW / 2 : W / 2;
-    if ((long long)H * W * C * Sh::NI > 0x1fffffffLL || (long long)g.OH * g.OW * C > 0x7fffffffLL) return -1;
+    g.YC = gate ? gate->ldy : C, g.ych = gate ? gate->ych : 0, g.gs = gate ? gate->gs : 1.f;
+    if (gate && (CS != 16 || add || flip || C % 16 != 0 || gate->ldy < gate->ych + C / 2 || (gate->ldy | gate->ych) % 8 != 0)) return -1;
+    if ((long long)H * W * C * Sh::NI > 0x1fffffffLL || (long long)g.OH * g.OW * g.YC * Sh::NI > 0x1fffffffLL) return -1;
     g.BR = tz_pick_band<K, NPC, CS>(B, g.OH, g.OW, C);
     if (g.BR < 4) return -1;
     g.nbands = cdiv(g.OH, g.BR), g.ncolt = cdiv(g.OW, Sh::TW), g.nslices = cdiv(C, CS);
@@ -487,9 +523,16 @@ static int launch_tz(const void* x, const void* w, const void* add, void* pool, 
     const long long nblocks = (long long)cdiv(B, Sh::NI) * g.nbands * g.ncolt * g.nslices;
     if (nblocks > 0x7fffffffLL) return -1;
     const size_t lds = Sh::lds_bytes(g.BR);
-    const int mode = add ? 1 : (pool ? 2 : 0);
-    auto kern = mode == 1 ? dwconv_tz_k<T, K, NPC, CS, 1> : (mode == 2 ? dwconv_tz_k<T, K, NPC, CS, 2> : dwconv_tz_k<T, K, NPC, CS, 0>);
-    static std::once_flag attr_once[3];
+    const int mode = (add ? 1 : 0) | (pool ? 2 : 0) | (gate ? 4 : 0);
+    auto kern = dwconv_tz_k<T, K, NPC, CS, 0>;
+    if (mode == 1) kern = dwconv_tz_k<T, K, NPC, CS, 1>;
+    if (mode == 2) kern = dwconv_tz_k<T, K, NPC, CS, 2>;
+    if constexpr (CS == 16) {
+        if (mode == 4) kern = dwconv_tz_k<T, K, NPC, CS, 4>;
+        if (mode == 6) kern = dwconv_tz_k<T, K, NPC, CS, 6>;
+    }
+    if (mode == 3 || mode == 5 || mode == 7) return -1;
+    static std::once_flag attr_once[8];
     std::call_once(attr_once[mode], [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(Sh::NT), lds, s, (const T*)x, (const T*)w, (const T*)add,
                        (T*)pool, (T*)y, g);
@@ -499,7 +542,7 @@ static int launch_tz(const void* x, const void* w, const void* add, void* pool, 
 // -1: not covered (the caller falls back to the other kernels).
 template <typename T, int K>
 static int launch_tz_best(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
-                          int PH, int PW, bool flip, hipStream_t s) {
+                          int PH, int PW, bool flip, const TzGate* gate, hipStream_t s) {
     const int OH = H + 2 * PH - K + 1, OW = W + 2 * PW - K + 1;
     if (OH < 1 || OW < 1 || C % 8 != 0 || B < 1) return -1;
     if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 15) != 0 ||
@@ -513,16 +556,16 @@ static int launch_tz_best(const void* x, const void* w, const void* add, void* p
     const bool wide_tile = pad16 <= pad8;
     // 16 channels per workgroup (two per wavefront) while the operand registers allow it, else 8
     constexpr int CS = (2 * 4 * TzShape<K, 16, 16>::NM + 2 * 4 * TzShape<K, 16, 16>::RING) <= 160 ? 16 : 8;
-    if (wide_tile) return launch_tz<T, K, 16, CS>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
-    return launch_tz<T, K, 8, CS>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+    if (wide_tile) return launch_tz<T, K, 16, CS>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, gate, s);
+    return launch_tz<T, K, 8, CS>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, gate, s);
 }
 
 template <int K>
 static int launch_tz_dtype(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
-                           int PH, int PW, bool flip, int dtype, hipStream_t s) {
+                           int PH, int PW, bool flip, int dtype, const TzGate* gate, hipStream_t s) {
     switch (dtype) {
-        case kF16: return launch_tz_best<f16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
-        case kBF16: return launch_tz_best<bf16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, s);
+        case kF16: return launch_tz_best<f16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, gate, s);
+        case kBF16: return launch_tz_best<bf16_t, K>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, gate, s);
         default: return -1;
     }
 }

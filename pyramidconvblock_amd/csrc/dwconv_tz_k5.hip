@@ -6,8 +6,8 @@
 namespace pdw {
 
 int dwconv_tz_k5(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C, int PH, int PW,
-                   bool flip, int dtype, hipStream_t s) {
-    return launch_tz_dtype<5>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, s);
+                   bool flip, int dtype, const TzGate* gate, hipStream_t s) {
+    return launch_tz_dtype<5>(x, w, add, pool, y, B, H, W, C, PH, PW, flip, dtype, gate, s);
 }
 
 }  // namespace pdw

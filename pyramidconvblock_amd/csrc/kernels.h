@@ -38,6 +38,18 @@ int reduce_defer_flush(hipStream_t s);
 int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH,
                         int PW, bool flip, int dtype, hipStream_t s, const void* add = nullptr, void* pool = nullptr);
 
+// Fused gate of the matrix-core forward kernel (dwconv_tz.h): the output is C/2 channels wide, written with a pixel
+// stride of ldy channels from channel ych on; gs is the gate factor sqrt(C/2).
+struct TzGate {
+    int ldy, ych;
+    float gs;
+};
+// Forward convolution with the gate of conv_block.py:18-19 applied in the store, and optionally the 2x2 average pool
+// of x written to `pool`.  -1: not covered (16-bit types, C % 16 == 0, stride 1, odd square filters that leave room
+// for 16 channels per workgroup).
+int dwconv_gate_launch(const void* x, const void* w, void* y, void* pool, int B, int H, int W, int C, int K, int PH,
+                       int PW, int ldy, int ych, int dtype, hipStream_t s);
+
 // dwconv_wgrad_tiled.hip: LDS-tiled weight gradient for stride 1, dilation 1, odd square filters <= 17.
 size_t dwconv_wgrad_tiled_workspace(int B, int H, int W, int C, int KH, int KW, int PH, int PW, int dtype);
 int dwconv_wgrad_tiled_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int KH,
@@ -59,6 +71,9 @@ int gate_pair_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, 
                          int dtype, hipStream_t s);
 int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
                          int w, int I, int ldg, int dtype, hipStream_t s);
+int bilinear_pool_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int ldy, const float* parts,
+                             int nparts, const void* wp, const void* bp, const void* bo, void* m, float* rowbias, int P,
+                             int D, int dtype, hipStream_t s);
 int block_mid_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
                          const float* parts, int nparts, const void* wp, const void* bp, const void* bo, void* m,
                          float* rowbias, int P, int D, int dtype, hipStream_t s);

@@ -99,11 +99,8 @@ __device__ __forceinline__ void bl_src(int dst, float scale, int in, int& i0, in
 }
 
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
-                                                      int C, int H, int W, int ldy, float sy, float sx,
-                                                      long long total) {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
+__device__ __forceinline__ void bilinear_fwd_item(const T* __restrict__ x, T* __restrict__ y, int h, int w, int C,
+                                                  int H, int W, int ldy, float sy, float sx, long long idx) {
     const int CV = C / VEC;
     const int c = (int)(idx % CV) * VEC;
     long long t = idx / CV;
@@ -125,6 +122,14 @@ __global__ __launch_bounds__(256) void bilinear_fwd_k(const T* __restrict__ x, T
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = hy * (hx * a[v] + lx * bb[v]) + ly * (hx * cc[v] + lx * d[v]);
     store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w,
+                                                      int C, int H, int W, int ldy, float sy, float sx,
+                                                      long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) bilinear_fwd_item<T, VEC>(x, y, h, w, C, H, W, ldy, sy, sx, idx);
 }
 
 // Weight with which destination index `dst` reads source index m along one axis.
@@ -1080,6 +1085,23 @@ __global__ __launch_bounds__(256) void block_mid_fwd_k(const T* __restrict__ xf,
     }
 }
 
+// Inference: the gated half-resolution scale upsampled into its slice of the concatenation, with the mean branch
+// riding in front as above.
+template <typename T>
+__global__ __launch_bounds__(256) void bilinear_pool_fwd_k(const T* __restrict__ x, T* __restrict__ y, int h, int w, int C,
+                                                           int H, int W, int ldy, float sy, float sx, long long total,
+                                                           const PoolFwdJob job) {
+    extern __shared__ float sm[];
+    unsigned bid = blockIdx.x;
+    if (bid < (unsigned)job.B) {
+        pool_branch_fwd_v8_body<T>(job.part, job.nchunks, job.D, job.inv_p, (const T*)job.wp, (const T*)job.bp,
+                                   (const T*)job.bo, (T*)job.m, job.rowbias, bid, sm);
+        return;
+    }
+    const long long idx = (long long)(bid - job.B) * blockDim.x + threadIdx.x;
+    if (idx < total) bilinear_fwd_item<T, 8>(x, y, h, w, C, H, W, ldy, sy, sx, idx);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void block_mid_bwd_k(const T* __restrict__ gy, const T* __restrict__ xf,
                                                        const T* __restrict__ xh, T* __restrict__ gxf,
@@ -1324,6 +1346,29 @@ int block_mid_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, 
         hipLaunchKernelGGL((block_mid_fwd_k<bf16_t>), dim3(bf + bh + B), dim3(256), lds, s, (const bf16_t*)xf,
                            (const bf16_t*)xh, (bf16_t*)y, h, w, I, H, W, ldy, sy, sx, sc, bf, tf, th, job);
     return check_launch("block_mid_fwd");
+}
+
+// Bilinear upsample (x[B,h,w,C] -> y[..., :C] with pixel stride ldy) and the mean branch in one launch; -1 when the
+// combination is not covered.
+int bilinear_pool_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int H, int W, int ldy, const float* parts,
+                             int nparts, const void* wp, const void* bp, const void* bo, void* m, float* rowbias, int P,
+                             int D, int dtype, hipStream_t s) {
+    const void* ptrs[2] = {x, y};
+    if (pick_vec(gcd_int(C, ldy), esize(dtype), ptrs, 2) != 8 || !pool_v8_ok(wp, nullptr, parts, B, D, dtype)) return -1;
+    const long long total = (long long)B * H * W * (C / 8);
+    unsigned blocks;
+    if (total == 0) return -1;
+    if (!grid_for(total, &blocks) || (unsigned long long)blocks + B > 0x7fffffffULL) return 1;
+    const float sy = (float)h / (float)H, sx = (float)w / (float)W;
+    const PoolFwdJob job{parts, nparts, B, D, 1.f / (float)P, wp, bp, bo, m, rowbias};
+    const size_t lds = (size_t)9 * D * sizeof(float);
+    if (dtype == kF16)
+        hipLaunchKernelGGL((bilinear_pool_fwd_k<f16_t>), dim3(blocks + B), dim3(256), lds, s, (const f16_t*)x, (f16_t*)y, h,
+                           w, C, H, W, ldy, sy, sx, total, job);
+    else
+        hipLaunchKernelGGL((bilinear_pool_fwd_k<bf16_t>), dim3(blocks + B), dim3(256), lds, s, (const bf16_t*)x,
+                           (bf16_t*)y, h, w, C, H, W, ldy, sy, sx, total, job);
+    return check_launch("bilinear_pool_fwd");
 }
 
 int block_mid_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
