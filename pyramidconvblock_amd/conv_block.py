@@ -71,21 +71,34 @@ NO_UP_PAIR = False
 
 
 def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
-    """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I], as a batched product over S slabs of N summed in fp32."""
+    """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I].  16-bit operands: a batched product over S slabs of L = N // S rows with
+    fp32 accumulation and output, summed in fp32 (the slabs give the library GEMM enough independent tiles; a single
+    product over N rows runs on a handful of workgroups), plus the N - S*L left-over rows in fp32."""
     N = g2d.shape[0]
-    S = 1
-    while S < 256 and N % (2 * S) == 0 and N // (2 * S) >= 128:
-        S *= 2
-    if S == 1 or g2d.dtype == torch.float32:
-        return g2d.float().t() @ x2d.float() if N else g2d.new_zeros((g2d.shape[1], x2d.shape[1]), dtype=torch.float32)
-    a = g2d.view(S, N // S, -1).transpose(1, 2)
-    b = x2d.view(S, N // S, -1)
+    if N == 0:
+        return g2d.new_zeros((g2d.shape[1], x2d.shape[1]), dtype=torch.float32)
+    if g2d.dtype == torch.float32:
+        return g2d.t() @ x2d
+    # slabs: a divisor of N (no left-over rows) if one gives 32..256 slabs of at least 48 rows, else a power of two
+    S = max((d for d in range(32, 257) if N % d == 0 and N // d >= 48), default=0)
+    if S == 0:
+        S = 1
+        while S < 256 and N // (2 * S) >= 128:
+            S *= 2
+    L = N // S
+    a = g2d[:S * L].view(S, L, -1).transpose(1, 2)
+    b = x2d[:S * L].view(S, L, -1)
+    out = None
     if _BMM_FP32_OUT[0]:
         try:
-            return torch.bmm(a, b, out_dtype=torch.float32).sum(0)
+            out = torch.bmm(a, b, out_dtype=torch.float32).sum(0)
         except (TypeError, RuntimeError):
             _BMM_FP32_OUT[0] = False
-    return torch.bmm(a, b).float().sum(0)
+    if out is None:
+        out = torch.bmm(a, b).float().sum(0) if S > 1 else a[0].float() @ b[0].float()
+    if S * L < N:
+        out = out + g2d[S * L:].float().t() @ x2d[S * L:].float()
+    return out
 
 
 def _block_call_ok(x, scales, w_up, b_up, w_out, b_out, w_pool, b_pool, w_dw) -> bool:
