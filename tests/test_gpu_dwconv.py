@@ -248,3 +248,17 @@ def test_forward_with_pooled_input(oracle, dtype, shape):
     y, xp = dwconv_forward(x.cuda(), w.cuda(), *geo, pool_to=hw)
     assert_close(y, oracle.dwconv_fwd(x.double().numpy(), w.double().numpy(), 1, k // 2, 1), dtype, "y")
     assert_close(xp, oracle.avgpool_fwd(x.double().numpy(), hw), dtype, "pooled input")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_matrix_core_kernels(oracle, seed):
+    """Random extents, batch sizes, channel counts (multiples of 8) and filter sizes through the 16-bit stride-1
+    kernels: ragged bands and column tiles, one or two images per instruction, one to many channel slices."""
+    rng = np.random.default_rng(100 + seed)
+    k = int(rng.choice([3, 5, 7, 9, 11, 13, 15, 17]))
+    B = int(rng.integers(1, 6))
+    H = int(rng.integers(max(4, k // 2 + 1), 75))
+    W = int(rng.integers(max(4, k // 2 + 1), 75))
+    C = 8 * int(rng.integers(1, 10))
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    _run(oracle, (B, H, W, C), k, dtype, seed=seed)
