@@ -300,28 +300,9 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
                 }
             }
         }
-        lds_barrier();
+        // (the table is read after the barrier that also publishes the window's first passes)
     }
-    // ---- this wavefront's A operands: lane = (m = 4 di + dj, k group kg); operand t covers k groups 4t .. 4t+3
     const int ln = lane & 15, kg = lane >> 4;
-    uint4 A[CPW][NM];
-    {
-        const int di = ln >> 2, dj = ln & 3;
-#pragma unroll
-        for (int q = 0; q < CPW; ++q) {
-#pragma unroll
-            for (int t = 0; t < NM; ++t) {
-                const int kap = 4 * t + kg;
-                const int r = kap / ICB, cb = kap - r * ICB;
-                const int v0 = 8 * cb - dj + 3;  // first of the lane's 8 table columns
-                const uint32_t* wp = reinterpret_cast<const uint32_t*>(
-                    wt + (v0 & 1) * WTC + ((wv * CPW + q) * WTH + r - di + 3) * WTW + (v0 & ~1));
-                const bool real = kap < NKG;
-                A[q][t] = make_uint4(real ? wp[0] : 0u, real ? wp[1] : 0u, real ? wp[2] : 0u, real ? wp[3] : 0u);
-            }
-        }
-    }
-
     // ---- per-lane addresses
     // B operands: lane = (patch n = image * NPC + pc, k group kg); operand a = ICB * rowgroup + i covers window rows
     // 4 rowgroup + (4i + kg) / ICB, column block (4i + kg) % ICB
@@ -402,6 +383,25 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     commit(buf[1], 1);
     issue(buf[1], 3);
     lds_barrier();
+    // ---- this wavefront's A operands: lane = (m = 4 di + dj, k group kg); operand t covers k groups 4t .. 4t+3
+    uint4 A[CPW][NM];
+    {
+        const int di = ln >> 2, dj = ln & 3;
+#pragma unroll
+        for (int q = 0; q < CPW; ++q) {
+#pragma unroll
+            for (int t = 0; t < NM; ++t) {
+                const int kap = 4 * t + kg;
+                const int r = kap / ICB, cb = kap - r * ICB;
+                const int v0 = 8 * cb - dj + 3;  // first of the lane's 8 table columns
+                const uint32_t* wp = reinterpret_cast<const uint32_t*>(
+                    wt + (v0 & 1) * WTC + ((wv * CPW + q) * WTH + r - di + 3) * WTW + (v0 & ~1));
+                const bool real = kap < NKG;
+                A[q][t] = make_uint4(real ? wp[0] : 0u, real ? wp[1] : 0u, real ? wp[2] : 0u, real ? wp[3] : 0u);
+            }
+        }
+    }
+
 #pragma unroll
     for (int j = 0; j < PER - 1; ++j) load_group(j, 4 * j * RP);
     // A step is two row groups (8 output rows).  Trips of UNRF steps run without a test between the staging calls: a
@@ -494,6 +494,7 @@ template <int K, int NPC, int CS>
 static int tz_pick_band(int B, int OH, int OW, int C) {
     using Sh = TzShape<K, NPC, CS>;
     const long long per_band = (long long)cdiv(B, Sh::NI) * cdiv(C, CS) * cdiv(OW, Sh::TW);
+    if (const char* e = tune_env("PDW_TZ_BR")) return atoi(e);
     int best = 0;
     double best_cost = 0;
     for (int br = 4; br <= ((OH + 3) / 4) * 4; br += 4) {
