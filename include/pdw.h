@@ -296,10 +296,13 @@ int pdw_dense_wgrad(const void *a, const void *b, void *dw, void *workspace, siz
  * (+ rowbias[n / P], fp32 [ceil(N/P), I], may be NULL; P >= 32) and dw[O,I] = gy^T x (workspace and summation as pdw_dense_wgrad, size pdw_dense_wgrad_workspace_bytes(N, O, I)); with
  * colsum != NULL also the sums of gy over groups of pdw_dense_colsum_rows() rows, as pdw_dense_fwd_colsum.  The two
  * products share the chip instead of following each other (each alone leaves half of it waiting on memory).
- * Covered: 16-bit, (O, I) = (128, 64), (64, 128), (64, 32) or (32, 64) (pdw_dense_bwd_pair_supported): the backward of conv_out and
- * conv_up, conv_block.py:44 and :37, in ConvBlock(128); other shapes take pdw_dense_fwd(w_kmajor) and
- * pdw_dense_wgrad.  Unlike pdw_dense_wgrad it carries no recorded summations along. */
+ * Covered (pdw_dense_bwd_pair_supported): 16-bit types and the widths pdw_dense_fwd and pdw_dense_wgrad both cover
+ * (multiples of 8 up to 128, at most 8 tiles of 32 x 32 in dW); (O, I) = (128, 64), (64, 128), (64, 32), (32, 64) -
+ * the backward of conv_out and conv_up, conv_block.py:44 and :37, in ConvBlock(128) and ConvBlock(64) - run with
+ * the extents as compile-time constants, and only those can also write colsum
+ * (pdw_dense_bwd_pair_colsum_supported); other shapes take pdw_dense_fwd(w_kmajor) and pdw_dense_wgrad.  Unlike pdw_dense_wgrad it carries no recorded summations along. */
 int pdw_dense_bwd_pair_supported(int O, int I, int dtype);
+int pdw_dense_bwd_pair_colsum_supported(int O, int I, int dtype); /* ... with the tile sums (`colsum` != NULL) */
 int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, float *colsum, void *dw, void *workspace,
                        size_t workspace_bytes, const float *rowbias, int P, long long N, int O, int I, int dtype,
                        void *stream);

@@ -81,6 +81,7 @@ _SIGS = {
     "pdw_dense_wgrad_workspace_bytes": (c_size_t, [c_longlong, c_int, c_int]),
     "pdw_dense_wgrad": (c_int, [c_void_p] * 4 + [c_size_t, c_longlong, c_int, c_int, c_int, c_void_p]),
     "pdw_dense_bwd_pair_supported": (c_int, [c_int] * 3),
+    "pdw_dense_bwd_pair_colsum_supported": (c_int, [c_int] * 3),
     "pdw_dense_bwd_pair": (c_int, [c_void_p] * 7 + [c_size_t, c_void_p, c_int, c_longlong, c_int, c_int, c_int,
                                    c_void_p]),
 }

@@ -293,9 +293,10 @@ class ConvBlockFunction(torch.autograd.Function):
         # the four weight gradients end in a small summation kernel each: they are run as one launch at the end
         with _lib.deferred_reductions(gy.device):
             gparts = None
-            if fast_out and N > 0 and cat.dtype == dt and ops.dense_backward_pair_supported(D, G * ns, dt):
+            want = pool_fast and ops.dense_colsum_supported(D, G * ns, dt, H * W)
+            if (fast_out and N > 0 and cat.dtype == dt
+                    and ops.dense_backward_pair_supported(D, G * ns, dt, colsum=bool(want))):
                 # both products that read gy share one launch
-                want = pool_fast and ops.dense_colsum_supported(D, G * ns, dt, H * W)
                 dcat, gparts, grad_w_out = ops.dense_backward_pair(gy, w_out.detach().contiguous(),
                                                                    cat.contiguous(), colsum=want)
             elif fast_out:

@@ -561,6 +561,10 @@ int pdw_dense_bwd_pair_supported(int O, int I, int dtype) {
     return valid_dtype(dtype) ? dense_bwd_pair_supported(O, I, dtype) : 0;
 }
 
+int pdw_dense_bwd_pair_colsum_supported(int O, int I, int dtype) {
+    return valid_dtype(dtype) ? dense_bwd_pair_colsum_supported(O, I, dtype) : 0;
+}
+
 int pdw_dense_bwd_pair(const void* gy, const void* w, const void* x, void* dx, float* colsum, void* dw, void* workspace,
                        size_t workspace_bytes, const float* rowbias, int P, long long N, int O, int I, int dtype,
                        void* stream) {

@@ -54,7 +54,7 @@ int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype)
     if ((long long)B * H * W * (D > I ? D : I) > 0x7fffffffLL) return 0;
     if ((H * W) % pdw_dense_colsum_rows()) return 0;
     return pdw_dense_supported(D, I, dtype) && pdw_dense_supported(I, D, dtype) && pdw_dense_colsum_supported(D, I, dtype) &&
-           pdw_dense_bwd_pair_supported(D, I, dtype) && pdw_dense_bwd_pair_supported(I, D, dtype);
+           pdw_dense_bwd_pair_colsum_supported(D, I, dtype) && pdw_dense_bwd_pair_supported(I, D, dtype);
 }
 
 size_t pdw_convblock_fwd_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {

@@ -593,6 +593,22 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_pair_k(const T* __restrict__
                                                blockIdx.x - nwg, nrows, dsm);
 }
 
+// The same for any widths the two bodies cover (multiples of 8 up to 128 with at most 8 accumulator tiles): extents
+// from the arguments, MT = ceil(O / 32), NT = ceil(I / 32).  No tile sums of gy.
+template <typename T, int MT, int NT>
+__global__ __launch_bounds__(256, 2) void dense_bwd_pair_gen_k(const T* __restrict__ gy, const T* __restrict__ W,
+                                                               const T* __restrict__ xin, T* __restrict__ dx,
+                                                               float* __restrict__ part,
+                                                               const float* __restrict__ rowbias, int P, long long N,
+                                                               int O, int I, int nwg, int nrows) {
+    extern __shared__ uint32_t dsm[];
+    if ((int)blockIdx.x < nwg)
+        dense_wgrad_body<T, MT, NT, false>(gy, xin, part, N, O, I, nwg, dsm);
+    else
+        dense_rows_body<T, true, false>(gy, W, nullptr, rowbias, dx, nullptr, N, O, I, P, (O + 15) / 16, (I + 31) / 32,
+                                        blockIdx.x - nwg, nrows, dsm);
+}
+
 static bool dense_dims_ok(int K, int NO, int dtype) {
     return dtype != kF32 && K >= 8 && K <= 16 * kKT && K % 8 == 0 && NO >= 8 && NO <= 32 * kNT && NO % 8 == 0;
 }
@@ -756,10 +772,20 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
     return dense_wgrad_t<bf16_t>(a, b, dw, ws, N, M, NO, s);
 }
 
+static bool pair_exact(int O, int I) {
+    return (O == 128 && I == 64) || (O == 64 && I == 128) || (O == 64 && I == 32) || (O == 32 && I == 64);
+}
+
 int dense_bwd_pair_supported(int O, int I, int dtype) {
-    return (dtype != kF32 && ((O == 128 && I == 64) || (O == 64 && I == 128) || (O == 64 && I == 32) || (O == 32 && I == 64)))
-               ? 1
-               : 0;
+    if (dtype == kF32) return 0;
+    if (pair_exact(O, I)) return 1;
+    // any widths both bodies cover: the row product with K = O, NO = I and the weight gradient with M = O, NO = I
+    return (dense_dims_ok(O, I, dtype) && dense_wgrad_supported(O, I, dtype)) ? 1 : 0;
+}
+
+// with the 32-row tile sums of gy (the `colsum` argument of the launch): the block's own shapes only
+int dense_bwd_pair_colsum_supported(int O, int I, int dtype) {
+    return (dtype != kF32 && pair_exact(O, I) && O >= 64 && dense_colsum_supported(O, I, dtype)) ? 1 : 0;
 }
 
 // -1: shape not covered.  ws: dense_wgrad_workspace(N, O, I) bytes.
@@ -777,10 +803,11 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
     long long nrows = (ntiles + 3) / 4;
     const int cap = tune_env("PDW_PAIR_ROWS") ? atoi(tune_env("PDW_PAIR_ROWS")) : 256;  // the second slot of every CU
     if (nrows > cap) nrows = cap;
-    if (colsum && (O < 64 || !dense_colsum_supported(O, I, dtype))) return -1;
+    if (colsum && !dense_bwd_pair_colsum_supported(O, I, dtype)) return -1;
     // rows product: K = O, NO = I (inner dimension padded to 64 or 128 in LDS); weight gradient: M = O, NO = I
-    const size_t lds_rows = ((size_t)I * ((O > 64 ? 128 : 64) + 8) + 4 * 32 * ((O > I ? O : I) + 8)) * 2 +
-                            (rowbias ? (size_t)4 * 2 * I * sizeof(float) : 0);
+    const int nnt = cdiv(I, 32);
+    const size_t lds_rows = ((size_t)nnt * 32 * ((O > 64 ? 128 : 64) + 8) + 4 * 32 * ((O > I ? O : I) + 8)) * 2 +
+                            (rowbias ? (size_t)4 * 2 * nnt * 32 * sizeof(float) : 0);
     const size_t lds_wg = (size_t)2 * kWgRows * (O + 8 + I + 8) * 2;
     const size_t lds = lds_rows > lds_wg ? lds_rows : lds_wg;
     const dim3 grid((unsigned)(nwg + nrows));
@@ -797,7 +824,22 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
     } else {                                                    \
         PDW_PAIR(T, false, 32, 64);                             \
     }
-    if (dtype == kF16) { PDW_PAIR_T(f16_t) } else { PDW_PAIR_T(bf16_t) }
+#define PDW_PAIR_GEN(T, MT_, NT_)                                                                                   \
+    if (mt == MT_ && nt == NT_)                                                                                      \
+        hipLaunchKernelGGL((dense_bwd_pair_gen_k<T, MT_, NT_>), grid, dim3(256), lds, s, (const T*)gy, (const T*)w,   \
+                           (const T*)xin, (T*)dx, (float*)ws, rowbias, P > 0 ? P : 1, N, O, I, nwg, (int)nrows);
+#define PDW_PAIR_GEN_T(T)                                                                                           \
+    PDW_PAIR_GEN(T, 1, 1) PDW_PAIR_GEN(T, 1, 2) PDW_PAIR_GEN(T, 2, 1) PDW_PAIR_GEN(T, 2, 2) PDW_PAIR_GEN(T, 1, 3)     \
+    PDW_PAIR_GEN(T, 3, 1) PDW_PAIR_GEN(T, 2, 3) PDW_PAIR_GEN(T, 3, 2) PDW_PAIR_GEN(T, 1, 4) PDW_PAIR_GEN(T, 4, 1)     \
+    PDW_PAIR_GEN(T, 2, 4) PDW_PAIR_GEN(T, 4, 2)
+    if (pair_exact(O, I)) {
+        if (dtype == kF16) { PDW_PAIR_T(f16_t) } else { PDW_PAIR_T(bf16_t) }
+    } else {
+        const int mt = cdiv(O, 32), nt = cdiv(I, 32);
+        if (dtype == kF16) { PDW_PAIR_GEN_T(f16_t) } else { PDW_PAIR_GEN_T(bf16_t) }
+    }
+#undef PDW_PAIR_GEN_T
+#undef PDW_PAIR_GEN
 #undef PDW_PAIR_T
 #undef PDW_PAIR
     if (int e = check_launch("dense_bwd_pair")) return e;

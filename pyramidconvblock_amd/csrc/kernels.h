@@ -112,6 +112,7 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
                        hipStream_t s);
 // input gradient (optionally with the column sums of gy) and weight gradient of a layer W[O][I] in one launch
 int dense_bwd_pair_supported(int O, int I, int dtype);
+int dense_bwd_pair_colsum_supported(int O, int I, int dtype);
 int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* dx, float* colsum, void* dw, void* ws,
                           const float* rowbias, int P, long long N, int O, int I, int dtype, hipStream_t s);
 

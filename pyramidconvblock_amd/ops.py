@@ -297,11 +297,13 @@ def dense_wgrad(a, b):
     return dw
 
 
-def dense_backward_pair_supported(O, I, dtype, rows_per_image=None) -> bool:
+def dense_backward_pair_supported(O, I, dtype, rows_per_image=None, colsum=False) -> bool:
     """Whether dense_backward_pair covers a layer with weight [O, I] (and a per-image term over images of
-    rows_per_image rows)."""
-    return (dtype in _lib._DTYPES and (rows_per_image is None or rows_per_image >= 32)
-            and bool(_lib.lib().pdw_dense_bwd_pair_supported(int(O), int(I), _lib.dtype_code(dtype))))
+    rows_per_image rows; with `colsum`, the tile sums of gy as well)."""
+    if dtype not in _lib._DTYPES or (rows_per_image is not None and rows_per_image < 32):
+        return False
+    fn = _lib.lib().pdw_dense_bwd_pair_colsum_supported if colsum else _lib.lib().pdw_dense_bwd_pair_supported
+    return bool(fn(int(O), int(I), _lib.dtype_code(dtype)))
 
 
 def dense_backward_pair(gy, w, x, colsum=False, rowbias=None, rows_per_image=1):

@@ -301,19 +301,19 @@ def test_block_mid_matches_separate_launches(dtype, B, hw, I, D):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N", [1, 70, 96 * 7, 32 * 56 * 56])
-@pytest.mark.parametrize("widths", [(128, 64), (64, 32)])
+@pytest.mark.parametrize("widths", [(128, 64), (64, 32), (96, 48), (48, 24), (104, 40)])
 def test_dense_backward_pair_matches_separate_launches(dtype, N, widths):
     """Input gradient (with column sums) and weight gradient of an I -> O layer from one launch: the same bits
     as the two launches it replaces, and the same with the summation deferred."""
     from pyramidconvblock_amd import _lib, ops
 
     O, I = widths
-    assert ops.dense_backward_pair_supported(O, I, dtype) and not ops.dense_backward_pair_supported(96, 64, dtype)
+    assert ops.dense_backward_pair_supported(O, I, dtype) and not ops.dense_backward_pair_supported(120, 104, dtype)
     gen = torch.Generator().manual_seed(N)
     gy = randn(gen, N, O).to(dtype).cuda()
     x = randn(gen, N, I).to(dtype).cuda()
     w = (randn(gen, O, I) / 8).to(dtype).cuda()
-    colsum = N % ops.dense_colsum_rows() == 0
+    colsum = N % ops.dense_colsum_rows() == 0 and widths in ((128, 64), (64, 32))   # tile sums: the block's shapes only
     if colsum:
         dx0, parts0 = ops.dense_forward(gy, w, w_kmajor=True, colsum=True)
     else:
