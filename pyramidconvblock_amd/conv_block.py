@@ -71,14 +71,12 @@ NO_UP_PAIR = False
 
 
 def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
-    """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I].  16-bit operands: a batched product over S slabs of L = N // S rows with
-    fp32 accumulation and output, summed in fp32 (the slabs give the library GEMM enough independent tiles; a single
+    """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I]: a batched product over S slabs of L = N // S rows (16-bit operands: with
+    fp32 accumulation and output), summed in fp32 (the slabs give the library GEMM enough independent tiles; a single
     product over N rows runs on a handful of workgroups), plus the N - S*L left-over rows in fp32."""
     N = g2d.shape[0]
     if N == 0:
         return g2d.new_zeros((g2d.shape[1], x2d.shape[1]), dtype=torch.float32)
-    if g2d.dtype == torch.float32:
-        return g2d.t() @ x2d
     # slabs: a divisor of N (no left-over rows) if one gives 32..256 slabs of at least 48 rows, else a power of two
     S = max((d for d in range(32, 257) if N % d == 0 and N // d >= 48), default=0)
     if S == 0:
@@ -89,7 +87,9 @@ def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
     a = g2d[:S * L].view(S, L, -1).transpose(1, 2)
     b = x2d[:S * L].view(S, L, -1)
     out = None
-    if _BMM_FP32_OUT[0]:
+    if g2d.dtype == torch.float32:
+        out = torch.bmm(a, b).sum(0)
+    elif _BMM_FP32_OUT[0]:
         try:
             out = torch.bmm(a, b, out_dtype=torch.float32).sum(0)
         except (TypeError, RuntimeError):

@@ -348,6 +348,10 @@ static TiledPlan plan_tiled(int OH, int OW, int KH, int B, int C) {
     const int slots = 4 * (64 / CS);
     const int slices = cdiv(C, CS);
     TiledPlan best;
+    // tiles that leave room for two workgroups per compute unit; where none fits (wide fp32 filters: the filter
+    // slice alone is KH * KW * 128 bytes), any tile that fits at all
+    for (long long lds_cap : {72LL * 1024, 156LL * 1024}) {
+        if (best.cost >= 0) break;
     for (int nrg = 1; nrg <= 32; ++nrg)
         for (int nst = 1; nst <= 16; ++nst) {
             const int np = nrg * nst;
@@ -356,7 +360,7 @@ static TiledPlan plan_tiled(int OH, int OW, int KH, int B, int C) {
             if ((th >= 2 * OH && nrg > 1) || (tw >= 2 * OW && nst > 1)) continue;
             const int rows_in = th + KH - 1, cpn = (tw + KW - 1 + PK - 1) / PK;
             const long long lds = ((long long)rows_in * cpn + (long long)KH * NP) * CS * 4;
-            if (lds > 72 * 1024) continue;
+            if (lds > lds_cap) continue;
             const long long nt = (long long)B * cdiv(OH, th) * cdiv(OW, tw);
             int occ = (int)((160 * 1024) / (lds + 512));
             occ = occ < 1 ? 1 : (occ > 3 ? 3 : occ);
@@ -370,6 +374,7 @@ static TiledPlan plan_tiled(int OH, int OW, int KH, int B, int C) {
             const double cost = (nt * slices >= 512 ? (double)nt * slices / 512.0 : span) * (compute + stage);
             if (best.cost < 0 || cost < best.cost) best.cost = cost, best.nrg = nrg, best.nst = nst;
         }
+    }
     return best;
 }
 
