@@ -227,8 +227,9 @@ def load_traffic():
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic_by_kernel.txt")) as f:
             for line in f:
-                if "=" in line and not line.lstrip().startswith("#"):
-                    key, _, val = line.partition("=")
+                line = line.split("#", 1)[0]
+                if "=" in line:
+                    key, _, val = line.rpartition("=")   # keys carry "k=13" themselves
                     out[key.strip()] = float(val.split()[0])
     except OSError:
         pass
