@@ -4,6 +4,8 @@
 
 Every csrc/*.hip file is compiled to an object (in parallel) and linked into
 pyramidconvblock_amd/libpdw.so.  hipcc cross-compiles, so no GPU is needed.
+With PDW_TUNE_BUILD=1 in the environment of the build the library is compiled with -DPDW_TUNE, which makes
+its planners honour the PDW_* override variables (for experiments; the product build reads no environment).
 """
 from __future__ import annotations
 
@@ -19,7 +21,7 @@ OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libpdw.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-FLAGS = [
+FLAGS = (["-DPDW_TUNE"] if os.environ.get("PDW_TUNE_BUILD") else []) + [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=fast",
     # keep the compiler from forming packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

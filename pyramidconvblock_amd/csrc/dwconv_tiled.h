@@ -349,9 +349,12 @@ static TiledPlan plan_tiled(int OH, int OW, int KH, int B, int C) {
     const int slices = cdiv(C, CS);
     TiledPlan best;
     // tiles that leave room for two workgroups per compute unit; where none fits (wide fp32 filters: the filter
-    // slice alone is KH * KW * 128 bytes), any tile that fits at all
+    // slice alone is KH * KW * 128 bytes), any tile that fits at all.  fp32 filters from 13 x 13 on choose among all
+    // tiles: the ones that leave room for a second workgroup are the 8-column patches, measured half as fast as a
+    // 14-column patch with the compute unit to itself (253 against 130 us at [32,56,56,128]; at 9 x 9 the other way)
+    const bool fp32_big = sizeof(T) == 4 && (tune_env("PDW_FP32_BIG") ? atoi(tune_env("PDW_FP32_BIG")) != 0 : KH * KW >= 169);
     for (long long lds_cap : {72LL * 1024, 156LL * 1024}) {
-        if (best.cost >= 0) break;
+        if (best.cost >= 0 && !fp32_big) break;
     for (int nrg = 1; nrg <= 32; ++nrg)
         for (int nst = 1; nst <= 16; ++nst) {
             const int np = nrg * nst;
