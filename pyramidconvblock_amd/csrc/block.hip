@@ -95,8 +95,9 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
     return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
 }
 
-// The fused convolution + gate needs 16 channels per workgroup, which the operand registers allow up to K = 13.
-static bool infer_fused(int K) { return K <= 13; }
+// The fused convolution + gate needs 16 channels per workgroup, which the operand registers allow up to K = 13, and
+// images small enough for the kernel's 32-bit offsets (two images side by side).
+static bool infer_fused(int H, int W, int I, int K) { return K <= 13 && (long long)H * W * I * 2 <= 0x1fffffffLL; }
 
 size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
     if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
@@ -104,7 +105,7 @@ size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, in
     const size_t full = (size_t)s.N * I * s.es, half = (size_t)B * s.h * s.w * I * s.es;
     size_t b = up256(full) /* a */ + up256(half) /* xp */ + up256(full) /* cat */ + up256((size_t)B * D * s.es) /* m */ +
                up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4);
-    if (infer_fused(K))
+    if (infer_fused(H, W, I, K))
         b += up256(half / 2);  // the gated half-resolution scale
     else
         b += up256(full) + up256(half);  // c0, c1
@@ -132,7 +133,7 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
     float* xparts = (float*)ws.take((size_t)s.nt * D * 4);
     float* yp = (float*)ws.take((size_t)B * D * 4);
     const int pad = K / 2, G = I / 2;
-    if (!infer_fused(K)) {
+    if (!infer_fused(H, W, I, K)) {
         void* c0 = ws.take(full);
         void* c1 = ws.take(half);
         // the forward's own launches; its workspace is xparts and yp, which lie next to each other
