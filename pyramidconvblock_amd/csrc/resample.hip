@@ -678,7 +678,25 @@ __global__ __launch_bounds__(256) void spatial_sum_final_k(const float* __restri
 // ---------------------------------------------------------------- pooled branch (global mean -> dense layer)
 // Forward, one workgroup per image: m[b,:] = (sum of the chunk partials) / P rounded to T, then
 // rowbias[b,o] = sum_c m[b,c] * Wp[o,c] + bp[o] + bo[o]  (fp32).  The dot products are spread over
-// 8 lanes per output feature (strided over c, combined with wavefront shuffles).
+// Sum of one column of the chunk partials of an image, 8 loads in flight (fixed order: bit-reproducible).
+__device__ __forceinline__ float chunk_column_sum(const float* __restrict__ pp, int nchunks, int D) {
+    float s[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] = 0.f;
+    int q = 0;
+    for (; q + 8 <= nchunks; q += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = pp[(long long)(q + j) * D];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[j] += v[j];
+    }
+    for (; q < nchunks; ++q) s[0] += pp[(long long)q * D];
+    return ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+}
+
+// 8 lanes per output feature (strided over c, combined with wavefront shuffles).  gridDim.y slices of 32 output
+// features each (every slice forms the image's mean again: the partials are a few KB in L2).
 template <typename T>
 __global__ __launch_bounds__(256) void pool_branch_fwd_k(const float* __restrict__ part, int nchunks, int D, float inv_p,
                                                          const T* __restrict__ wp, const T* __restrict__ bp,
@@ -687,24 +705,16 @@ __global__ __launch_bounds__(256) void pool_branch_fwd_k(const float* __restrict
     extern __shared__ float sm[];  // [D]
     const int b = blockIdx.x;
     for (int c = threadIdx.x; c < D; c += 256) {
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-        const float* pp = part + (long long)b * nchunks * D + c;
-        int q = 0;
-        for (; q + 4 <= nchunks; q += 4) {
-            s0 += pp[(long long)q * D], s1 += pp[(long long)(q + 1) * D];
-            s2 += pp[(long long)(q + 2) * D], s3 += pp[(long long)(q + 3) * D];
-        }
-        for (; q < nchunks; ++q) s0 += pp[(long long)q * D];
-        const T mv = from_f32<T>(((s0 + s1) + (s2 + s3)) * inv_p);
-        m[(long long)b * D + c] = mv;
+        const T mv = from_f32<T>(chunk_column_sum(part + (long long)b * nchunks * D + c, nchunks, D) * inv_p);
+        if (blockIdx.y == 0) m[(long long)b * D + c] = mv;
         sm[c] = to_f32(mv);
     }
     __syncthreads();
     const int sub = threadIdx.x & 7;
-    for (int o = threadIdx.x >> 3; o < D; o += 32) {
+    for (int o = blockIdx.y * 32 + (threadIdx.x >> 3); o < D; o += 32 * gridDim.y) {
         const T* wr = wp + (long long)o * D;
         float acc = 0.f;
-#pragma unroll 4
+#pragma unroll 8
         for (int c = sub; c < D; c += 8) acc = fmaf(sm[c], to_f32(wr[c]), acc);
         acc += __shfl_xor(acc, 1);
         acc += __shfl_xor(acc, 2);
@@ -726,15 +736,7 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_a_k(const float* __restri
     extern __shared__ float sm[];  // [D] column sums, then [OL][D] partial products
     const int b = blockIdx.x;
     for (int c = threadIdx.x; c < D; c += 256) {
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-        const float* pp = part + (long long)b * nchunks * D + c;
-        int q = 0;
-        for (; q + 4 <= nchunks; q += 4) {
-            s0 += pp[(long long)q * D], s1 += pp[(long long)(q + 1) * D];
-            s2 += pp[(long long)(q + 2) * D], s3 += pp[(long long)(q + 3) * D];
-        }
-        for (; q < nchunks; ++q) s0 += pp[(long long)q * D];
-        const float s = (s0 + s1) + (s2 + s3);
+        const float s = chunk_column_sum(part + (long long)b * nchunks * D + c, nchunks, D);
         gs[(long long)b * D + c] = s;
         sm[c] = s;
     }
@@ -759,10 +761,17 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_a_k(const float* __restri
         }
     } else {
         for (int c = threadIdx.x; c < D; c += 256) {
-            float acc = 0.f;
-#pragma unroll 4
-            for (int o = 0; o < D; ++o) acc = fmaf(sm[o], to_f32(wp[(long long)o * D + c]), acc);
-            dmean[(long long)b * D + c] = acc * inv_p;
+            float a4[4] = {0.f, 0.f, 0.f, 0.f};   // four independent chains, 16 loads in flight
+            int o = 0;
+            for (; o + 16 <= D; o += 16) {
+                float wv[16];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) wv[j] = to_f32(wp[(long long)(o + j) * D + c]);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) a4[j & 3] = fmaf(sm[o + j], wv[j], a4[j & 3]);
+            }
+            for (; o < D; ++o) a4[0] = fmaf(sm[o], to_f32(wp[(long long)o * D + c]), a4[0]);
+            dmean[(long long)b * D + c] = ((a4[0] + a4[1]) + (a4[2] + a4[3])) * inv_p;
         }
     }
 }
@@ -1529,15 +1538,15 @@ int pool_branch_fwd_launch(const void* x, const void* wp, const void* bp, const 
     }
     switch (dtype) {
         case kF32:
-            hipLaunchKernelGGL((pool_branch_fwd_k<float>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const float*)wp,
+            hipLaunchKernelGGL((pool_branch_fwd_k<float>), dim3(B, (D + 31) / 32), dim3(256), lds, s, ws, n, D, inv_p, (const float*)wp,
                                (const float*)bp, (const float*)bo, (float*)m, rowbias);
             break;
         case kF16:
-            hipLaunchKernelGGL((pool_branch_fwd_k<f16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const f16_t*)wp,
+            hipLaunchKernelGGL((pool_branch_fwd_k<f16_t>), dim3(B, (D + 31) / 32), dim3(256), lds, s, ws, n, D, inv_p, (const f16_t*)wp,
                                (const f16_t*)bp, (const f16_t*)bo, (f16_t*)m, rowbias);
             break;
         default:
-            hipLaunchKernelGGL((pool_branch_fwd_k<bf16_t>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p,
+            hipLaunchKernelGGL((pool_branch_fwd_k<bf16_t>), dim3(B, (D + 31) / 32), dim3(256), lds, s, ws, n, D, inv_p,
                                (const bf16_t*)wp, (const bf16_t*)bp, (const bf16_t*)bo, (bf16_t*)m, rowbias);
     }
     return check_launch("pool_branch_fwd");
