@@ -404,14 +404,14 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
 
 #pragma unroll
     for (int j = 0; j < PER - 1; ++j) load_group(j, 4 * j * RP);
-    // A step is two row groups (8 output rows).  Trips of UNRF steps run without a test between the staging calls: a
-    // trip may run past the band's end, where loads read nothing, stores are dropped and only the products (no memory
-    // request among them) are skipped.  Besides its products a step
+    // A step is two row groups (8 output rows).  Trips of UNRF steps (the ring's period in steps), left after the
+    // band's last step by a uniform exit between steps.  Besides its products a step
     // stores the previous step's tiles and commits the pass the NEXT step needs; the wavefronts 0-3 do the products
     // first and the others last, so that of the two wavefronts a SIMD holds one feeds the matrix pipe while the
     // other moves data (both make the same memory requests in the same order: the in-flight counts stay exact).
     const int nfat = (nsteps + 1) >> 1;
     int fdone = 0;
+    bool left = false;
     auto stage_step = [&](int jf, int f) {
         store(f - 1);
         add_fetch(f);
@@ -474,7 +474,13 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
                 stage_step(jf, f);
                 if (f < nfat) compute_step(jf, f);
             }
+            if (f + 1 >= nfat) {   // the band's last step (uniform): its tiles are stored after the loop
+                left = true;
+                fdone = f + 1;
+                break;
+            }
         }
+        if (left) break;
         fdone = f0 + UNRF;
 #pragma unroll
         for (int q = 0; q < CPW; ++q)

@@ -250,8 +250,8 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
         }
     }
     auto read_a = [&](const char* p) { return *reinterpret_cast<const uint4*>(p); };   // 16-byte aligned
-    // Steps in trips of 4 without a test in between (the band's last trip may run up to 3 steps past its end: their gy
-    // rows read as zero, their loads move nothing).  A step first commits what the NEXT step adds to the windows (an
+    // Steps in trips of 4, left after the band's last step (a uniform exit between steps: the loads of passes past the
+    // band's end, requested on the way, move nothing).  A step first commits what the NEXT step adds to the windows (an
     // 8-row pass of xw or of gy on alternating steps; with 3 gy slots one row group of gy every step, the pass's
     // registers being requested again once both of its groups are in LDS), behind the barrier that ends the previous step's reads of the ring slots it
     // overwrites; no condition depends on data, so the loads keep their exact in-flight counts.
@@ -295,6 +295,10 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
 #pragma unroll
                     for (int f = 0; f < NMF; ++f) acc[q][f] = mfma16(read_a(xa[f] + q * CHPX + 16 * cb), bop, acc[q][f], T());
                 }
+            if (t + 1 >= nsteps) {   // the band's last step (uniform): the rest of the trip would multiply zeros
+                s0 = nsteps;
+                break;
+            }
         }
     }
     // ---- this band's partial.  Lane (n = (du, dv), row block kr) holds in register r of instruction f the tap block
