@@ -294,8 +294,10 @@ class ConvBlockFunction(torch.autograd.Function):
         with _lib.deferred_reductions(gy.device):
             gparts = None
             want = pool_fast and ops.dense_colsum_supported(D, G * ns, dt, H * W)
-            if (fast_out and N > 0 and cat.dtype == dt
-                    and ops.dense_backward_pair_supported(D, G * ns, dt, colsum=bool(want))):
+            pair_out = fast_out and N > 0 and cat.dtype == dt
+            if pair_out and want and not ops.dense_backward_pair_supported(D, G * ns, dt, colsum=True):
+                want = False   # the pair without the tile sums (the mean branch then sums gy itself) beats two launches
+            if pair_out and ops.dense_backward_pair_supported(D, G * ns, dt, colsum=bool(want)):
                 # both products that read gy share one launch
                 dcat, gparts, grad_w_out = ops.dense_backward_pair(gy, w_out.detach().contiguous(),
                                                                    cat.contiguous(), colsum=want)

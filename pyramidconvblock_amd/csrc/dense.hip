@@ -263,7 +263,8 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                             (hb ? to_f32(braw.v[2]) : 0.f) + brow.z, (hb ? to_f32(braw.v[3]) : 0.f) + brow.w);
         }
         float cs[8];
-        if constexpr (COLSUM) {
+        const bool cs_lanes = K == 128 || K == 64;   // a lane keeps its 8 columns over all chunks (64 % (K/8) == 0)
+        if (COLSUM && cs_lanes) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) cs[j] = 0.f;
 #pragma unroll
@@ -283,9 +284,22 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             else
                 xf[kt] = Frag{{0u, 0u, 0u, 0u}};
         }
+        if (COLSUM && !cs_lanes) {
+            // other widths: lane sums one dword column (two features) of the tile in LDS over its 32 rows (rows past
+            // the tensor were written as zeros)
+            float s0 = 0.f, s1 = 0.f;
+            if (2 * lane < K) {
+#pragma unroll 8
+                for (int r = 0; r < 32; ++r) {
+                    const uint32_t v = *reinterpret_cast<const uint32_t*>(tl + r * ldt + 2 * lane);
+                    s0 += half_to_f32<T>(v & 0xffffu), s1 += half_to_f32<T>(v >> 16);
+                }
+                *reinterpret_cast<float2*>(colsum + tile * K + 2 * lane) = make_float2(s0, s1);
+            }
+        }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // fragments are in registers: the buffer may be overwritten
         if (tile + nw < ntiles) load_tile(tile + nw);  // next tile in flight during the MFMAs and the store
-        if constexpr (COLSUM) {
+        if (COLSUM && cs_lanes) {
             float* tf = reinterpret_cast<float*>(tl);  // [512 / K lane groups][K]
             *reinterpret_cast<float4*>(tf + lane * 8) = make_float4(cs[0], cs[1], cs[2], cs[3]);
             *reinterpret_cast<float4*>(tf + lane * 8 + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
@@ -617,9 +631,7 @@ int dense_rows_supported(int K, int NO, int dtype) { return dense_dims_ok(K, NO,
 
 int dense_colsum_rows() { return 32; }
 
-int dense_colsum_supported(int K, int NO, int dtype) {
-    return (dense_dims_ok(K, NO, dtype) && (K == 64 || K == 128)) ? 1 : 0;
-}
+int dense_colsum_supported(int K, int NO, int dtype) { return dense_dims_ok(K, NO, dtype) ? 1 : 0; }
 
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
                       long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum,
