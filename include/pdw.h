@@ -299,8 +299,8 @@ int pdw_dense_wgrad(const void *a, const void *b, void *dw, void *workspace, siz
  * Covered (pdw_dense_bwd_pair_supported): 16-bit types and the widths pdw_dense_fwd and pdw_dense_wgrad both cover
  * (multiples of 8 up to 128, at most 8 tiles of 32 x 32 in dW); (O, I) = (128, 64), (64, 128), (64, 32), (32, 64) -
  * the backward of conv_out and conv_up, conv_block.py:44 and :37, in ConvBlock(128) and ConvBlock(64) - run with
- * the extents as compile-time constants, and only those can also write colsum
- * (pdw_dense_bwd_pair_colsum_supported); other shapes take pdw_dense_fwd(w_kmajor) and pdw_dense_wgrad.  Unlike pdw_dense_wgrad it carries no recorded summations along. */
+ * the extents as compile-time constants; colsum where pdw_dense_bwd_pair_colsum_supported says so (the widths
+ * pdw_dense_fwd_colsum covers); other shapes take pdw_dense_fwd(w_kmajor) and pdw_dense_wgrad.  Unlike pdw_dense_wgrad it carries no recorded summations along. */
 int pdw_dense_bwd_pair_supported(int O, int I, int dtype);
 int pdw_dense_bwd_pair_colsum_supported(int O, int I, int dtype); /* ... with the tile sums (`colsum` != NULL) */
 int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, float *colsum, void *dw, void *workspace,
@@ -311,7 +311,8 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
  * launch sequence of the entry points above (5 launches forward; 6 launches and one summation launch backward)
  * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
  * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense
- * kernels and pdw_dense_bwd_pair cover (D = 128, I = 64 or D = 64, I = 32), odd K.  All tensors channels-last and contiguous, all
+ * kernels and pdw_dense_bwd_pair cover (multiples of 8 up to 128; D = 128, I = 64 and D = 64, I = 32 run the variants with
+ * compile-time extents), odd K.  All tensors channels-last and contiguous, all
  * parameters in `dtype`: x, y[B,H,W,D]; w_up[I,D]; w_dw0, w_dw1[K,K,I]; w_pool[D,D]; w_out[D,I]; b_pool, b_out[D] or
  * NULL.  The forward writes what the backward reads again: a = conv_up(x), c0 = conv(a), xp = pool(a)[B,H/2,W/2,I],
  * c1 = conv(xp), cat[B,H,W,I] (the gated scales), m[B,D] (per-image mean of x).  The backward overwrites dx and the

@@ -608,19 +608,19 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_pair_k(const T* __restrict__
 }
 
 // The same for any widths the two bodies cover (multiples of 8 up to 128 with at most 8 accumulator tiles): extents
-// from the arguments, MT = ceil(O / 32), NT = ceil(I / 32).  No tile sums of gy.
-template <typename T, int MT, int NT>
+// from the arguments, MT = ceil(O / 32), NT = ceil(I / 32).
+template <typename T, int MT, int NT, bool COLSUM>
 __global__ __launch_bounds__(256, 2) void dense_bwd_pair_gen_k(const T* __restrict__ gy, const T* __restrict__ W,
                                                                const T* __restrict__ xin, T* __restrict__ dx,
-                                                               float* __restrict__ part,
+                                                               float* __restrict__ colsum, float* __restrict__ part,
                                                                const float* __restrict__ rowbias, int P, long long N,
                                                                int O, int I, int nwg, int nrows) {
     extern __shared__ uint32_t dsm[];
     if ((int)blockIdx.x < nwg)
         dense_wgrad_body<T, MT, NT, false>(gy, xin, part, N, O, I, nwg, dsm);
     else
-        dense_rows_body<T, true, false>(gy, W, nullptr, rowbias, dx, nullptr, N, O, I, P, (O + 15) / 16, (I + 31) / 32,
-                                        blockIdx.x - nwg, nrows, dsm);
+        dense_rows_body<T, true, COLSUM>(gy, W, nullptr, rowbias, dx, colsum, N, O, I, P, (O + 15) / 16, (I + 31) / 32,
+                                         blockIdx.x - nwg, nrows, dsm);
 }
 
 static bool dense_dims_ok(int K, int NO, int dtype) {
@@ -795,9 +795,11 @@ int dense_bwd_pair_supported(int O, int I, int dtype) {
     return (dense_dims_ok(O, I, dtype) && dense_wgrad_supported(O, I, dtype)) ? 1 : 0;
 }
 
-// with the 32-row tile sums of gy (the `colsum` argument of the launch): the block's own shapes only
+// with the 32-row tile sums of gy (the `colsum` argument of the launch)
 int dense_bwd_pair_colsum_supported(int O, int I, int dtype) {
-    return (dtype != kF32 && pair_exact(O, I) && O >= 64 && dense_colsum_supported(O, I, dtype)) ? 1 : 0;
+    return (dense_bwd_pair_supported(O, I, dtype) && (!pair_exact(O, I) || O >= 64) && dense_colsum_supported(O, I, dtype))
+               ? 1
+               : 0;
 }
 
 // -1: shape not covered.  ws: dense_wgrad_workspace(N, O, I) bytes.
@@ -837,9 +839,16 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
         PDW_PAIR(T, false, 32, 64);                             \
     }
 #define PDW_PAIR_GEN(T, MT_, NT_)                                                                                   \
-    if (mt == MT_ && nt == NT_)                                                                                      \
-        hipLaunchKernelGGL((dense_bwd_pair_gen_k<T, MT_, NT_>), grid, dim3(256), lds, s, (const T*)gy, (const T*)w,   \
-                           (const T*)xin, (T*)dx, (float*)ws, rowbias, P > 0 ? P : 1, N, O, I, nwg, (int)nrows);
+    if (mt == MT_ && nt == NT_) {                                                                                    \
+        if (colsum)                                                                                                  \
+            hipLaunchKernelGGL((dense_bwd_pair_gen_k<T, MT_, NT_, true>), grid, dim3(256), lds, s, (const T*)gy,     \
+                               (const T*)w, (const T*)xin, (T*)dx, colsum, (float*)ws, rowbias, P > 0 ? P : 1, N, O, \
+                               I, nwg, (int)nrows);                                                                  \
+        else                                                                                                         \
+            hipLaunchKernelGGL((dense_bwd_pair_gen_k<T, MT_, NT_, false>), grid, dim3(256), lds, s, (const T*)gy,    \
+                               (const T*)w, (const T*)xin, (T*)dx, colsum, (float*)ws, rowbias, P > 0 ? P : 1, N, O, \
+                               I, nwg, (int)nrows);                                                                  \
+    }
 #define PDW_PAIR_GEN_T(T)                                                                                           \
     PDW_PAIR_GEN(T, 1, 1) PDW_PAIR_GEN(T, 1, 2) PDW_PAIR_GEN(T, 2, 1) PDW_PAIR_GEN(T, 2, 2) PDW_PAIR_GEN(T, 1, 3)     \
     PDW_PAIR_GEN(T, 3, 1) PDW_PAIR_GEN(T, 2, 3) PDW_PAIR_GEN(T, 3, 2) PDW_PAIR_GEN(T, 1, 4) PDW_PAIR_GEN(T, 4, 1)     \
