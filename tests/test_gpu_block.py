@@ -66,6 +66,10 @@ def test_config5_ragged(oracle, dtype, k):
     (128, 11, (2, 16, 16, 128), torch.float32),
     (64, 7, (3, 8, 16, 64), torch.float16),        # narrow block through the single library call per direction
     (128, 17, (2, 24, 32, 128), torch.float16),
+    (32, 7, (3, 8, 8, 32), torch.bfloat16),        # widths 32/16, 96/48, 112/... through the generic-extent dense pair
+    (96, 9, (2, 16, 16, 96), torch.float16),
+    (96, 13, (4, 28, 32, 96), torch.bfloat16),
+    (112, 5, (2, 8, 12, 112), torch.bfloat16),     # inner width 56: not a multiple of 16, the launches one by one
 ])
 def test_small_and_odd_even_extents(oracle, case):
     """Even extents take the fused two-scale path (paired launches, deferred summations); small and unusual
