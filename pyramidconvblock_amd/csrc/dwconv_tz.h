@@ -81,12 +81,15 @@ struct TzShape {
     static_assert(K % 2 == 1 && K >= 3 && K <= 17, "odd filters up to 17");
     static_assert(NPC == 16 || NPC == 8, "patches per image row");
     static_assert(CS == 8 || CS == 16, "channels per workgroup");
-    static constexpr int win_rows(int BR) { return BR + 4 * (PER - 1); }  // BR % 4 == 0
-    static constexpr int chp(int BR) {                                   // bytes per channel plane, = 8 mod 16
-        const int b = win_rows(BR) * RP;
-        return b % 16 == 8 ? b : b + 8;
-    }
-    static constexpr size_t lds_bytes(int BR) { return (size_t)NI * CS * chp(BR) + R2B; }
+    static constexpr int win_rows(int BR) { return BR + 4 * (PER - 1); }  // window rows of a band; BR % 4 == 0
+    // The window lives in LDS as a ring of NR row groups (of 4 rows), window row r at ring row r % NRR: a step reads
+    // the two row groups it adds to the operand registers while the next step's two are being written, and the
+    // first step needs PER + 1 row groups in place before it starts.
+    static constexpr int NR = PER + 1 > 4 ? PER + 1 : 4;
+    static constexpr int NRR = 4 * NR;
+    static constexpr int CHP = NRR * RP % 16 == 8 ? NRR * RP : NRR * RP + 8;  // bytes per channel plane, = 8 mod 16
+    static constexpr size_t lds_bytes = (size_t)NI * CS * CHP + R2B;
+    static_assert(lds_bytes <= 160 * 1024, "LDS");
 };
 
 struct TzGeom {
@@ -95,7 +98,6 @@ struct TzGeom {
     int PH, PW;        // padding
     int BR;            // output rows of a band (multiple of 4)
     int nbands, ncolt, nslices;
-    int CHP;           // LDS bytes per channel plane
     int flip;          // 1: 180-degree rotated filter (input gradient)
     int AH, AW;        // extents of the half-resolution addend / pooled output
     int YC, ych;       // output pixel stride in channels, first output channel
@@ -135,12 +137,12 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     using Sh = TzShape<K, NPC, CS>;
     constexpr int NT = Sh::NT, ICB = Sh::ICB, NKG = Sh::NKG, NM = Sh::NM, PER = Sh::PER, RING = Sh::RING;
     constexpr int NI = Sh::NI, TW = Sh::TW, NH = Sh::NH, CPW = Sh::CPW, RP = Sh::RP, OPX = Sh::OPX, OROWP = Sh::OROWP;
-    constexpr int OLB = Sh::OLB, WTH = Sh::WTH, WTW = Sh::WTW;
+    constexpr int OLB = Sh::OLB, WTH = Sh::WTH, WTW = Sh::WTW, NR = Sh::NR, NRR = Sh::NRR, CHP = Sh::CHP;
     constexpr bool ADD = (MODE & 1) != 0, POOL = (MODE & 2) != 0, GATE = (MODE & 4) != 0;
     static_assert(!GATE || (CS == 16 && !ADD), "the gate pairs the two 8-channel pieces of a 16-channel slice");
     extern __shared__ uint32_t smem[];
-    char* const xl = reinterpret_cast<char*>(smem);        // [NI][CS] planes of CHP bytes: [row][column] of T
-    char* const r2 = xl + NI * CS * g.CHP;                 // filter table, then the two result tiles
+    char* const xl = reinterpret_cast<char*>(smem);        // [NI][CS] planes of CHP bytes: [ring row][column] of T
+    char* const r2 = xl + NI * CS * CHP;                 // filter table, then the two result tiles
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     int bid = xcd_remap(blockIdx.x, gridDim.x);
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     auto xload = [&](uint32_t off) { return xload_from(xrsrc, off); };
     uint32_t icol[NLD][2];  // byte offsets of the item's two columns (image and channel piece included), or kNoCol
     int irpw[NLD];          // row pair within a pass
-    int idst[NLD];          // LDS byte offset of the item in a pass that starts at window row 0
+    int idst[NLD];          // LDS byte offset of the item's plane and column pair
 #pragma unroll
     for (int l = 0; l < NLD; ++l) {
         const int idx = tid + l * NT;
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
         const uint32_t ioff = (uint32_t)img * (uint32_t)img_in + (uint32_t)chof(h);
         icol[l][0] = any && ic >= 0 && ic < g.W ? (ioff + (uint32_t)(ic * g.C)) * 2u : kNoCol;
         icol[l][1] = any && ic + 1 >= 0 && ic + 1 < g.W ? (ioff + (uint32_t)((ic + 1) * g.C)) * 2u : kNoCol;
-        idst[l] = (img * CS + 8 * h) * g.CHP + (2 * min(rpw, RPMAX - 1)) * RP + 4 * cp;
+        idst[l] = (img * CS + 8 * h) * CHP + 4 * cp;
     }
     // the 2x2 average pool of x (MODE 2) leaves through a buffer descriptor as well: a store past its end is dropped
     __amdgpu_buffer_rsrc_t prsrc = xrsrc;
@@ -237,14 +239,16 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
                 const uint32_t a1[4] = {bf[l][1].x, bf[l][1].y, bf[l][1].z, bf[l][1].w};
                 const uint32_t a2[4] = {bf[l][2].x, bf[l][2].y, bf[l][2].z, bf[l][2].w};
                 const uint32_t a3[4] = {bf[l][3].x, bf[l][3].y, bf[l][3].z, bf[l][3].w};
-                char* dst = xl + idst[l] + wr0 * RP;
+                int rr = wr0 % NRR + 2 * irpw[l];   // ring row of the item's first row (a pair never wraps: both even)
+                rr -= rr >= NRR ? NRR : 0;
+                char* dst = xl + idst[l] + rr * RP;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     // column pair of channels 2j and 2j+1, the item's two rows
-                    *reinterpret_cast<uint32_t*>(dst + (2 * j) * g.CHP) = __builtin_amdgcn_perm(a1[j], a0[j], 0x05040100u);
-                    *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * g.CHP) = __builtin_amdgcn_perm(a1[j], a0[j], 0x07060302u);
-                    *reinterpret_cast<uint32_t*>(dst + (2 * j) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x05040100u);
-                    *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * g.CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j) * CHP) = __builtin_amdgcn_perm(a1[j], a0[j], 0x05040100u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * CHP) = __builtin_amdgcn_perm(a1[j], a0[j], 0x07060302u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j) * CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x05040100u);
+                    *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * CHP + RP) = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
                 }
             }
             if constexpr (POOL) {
@@ -312,7 +316,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     for (int q = 0; q < CPW; ++q)
 #pragma unroll
         for (int i = 0; i < ICB; ++i)
-            xb[q][i] = xl + (pimg * CS + wv * CPW + q) * g.CHP + ((4 * i + kg) / ICB) * RP + ((4 * i + kg) % ICB) * 16 + pc * 8;
+            xb[q][i] = xl + (pimg * CS + wv * CPW + q) * CHP + ((4 * i + kg) / ICB) * RP + ((4 * i + kg) % ICB) * 16 + pc * 8;
     // results: register r of a lane is output (row kg, column 4 pc + r) of patch n
     char* const olw = r2 + (pimg * 4 + kg) * OROWP + (4 * pc) * OPX + pc * 4 + 2 * (wv * CPW);
     // store phase: one 16-byte piece (image, row, column, h) of each 4-row result tile per thread, through buffer
@@ -421,12 +425,13 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     auto compute_step = [&](int jf, int f) {
         // the two row groups this step adds to the ring; the second goes to the slot of the step's own first
         // group, which the first tile still reads, so it waits in registers until the products are issued
-        load_group((2 * jf + PER - 1) % PER, 4 * (2 * jf + PER - 1) * RP);
+        load_group((2 * jf + PER - 1) % PER, ((2 * f + PER - 1) % NR) * (4 * RP));
+        const int late_off = ((2 * f + PER) % NR) * (4 * RP);
         uint4 late[CPW][ICB];
 #pragma unroll
         for (int q = 0; q < CPW; ++q)
 #pragma unroll
-            for (int i = 0; i < ICB; ++i) late[q][i] = read16(xb[q][i] + 4 * (2 * jf + PER) * RP);
+            for (int i = 0; i < ICB; ++i) late[q][i] = read16(xb[q][i] + late_off);
         tz_f32x4 acc[2][CPW];
 #pragma unroll
         for (int gi = 0; gi < 2; ++gi)
@@ -482,10 +487,6 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
         }
         if (left) break;
         fdone = f0 + UNRF;
-#pragma unroll
-        for (int q = 0; q < CPW; ++q)
-#pragma unroll
-            for (int i = 0; i < ICB; ++i) xb[q][i] += 4 * (2 * UNRF) * RP;
     }
     lds_barrier();
     store(fdone - 1);
@@ -504,7 +505,6 @@ static int tz_pick_band(int B, int OH, int OW, int C) {
     int best = 0;
     double best_cost = 0;
     for (int br = 4; br <= ((OH + 3) / 4) * 4; br += 4) {
-        if (Sh::lds_bytes(br) > 160 * 1024) break;
         const long long wgs = per_band * cdiv(OH, br);
         const double cost = (double)cdiv(wgs, 256) * (Sh::win_rows(br) + 8);
         if (best == 0 || cost <= best_cost) best = br, best_cost = cost;
@@ -526,10 +526,9 @@ static int launch_tz(const void* x, const void* w, const void* add, void* pool, 
     g.BR = tz_pick_band<K, NPC, CS>(B, g.OH, g.OW, C);
     if (g.BR < 4) return -1;
     g.nbands = cdiv(g.OH, g.BR), g.ncolt = cdiv(g.OW, Sh::TW), g.nslices = cdiv(C, CS);
-    g.CHP = Sh::chp(g.BR);
     const long long nblocks = (long long)cdiv(B, Sh::NI) * g.nbands * g.ncolt * g.nslices;
     if (nblocks > 0x7fffffffLL) return -1;
-    const size_t lds = Sh::lds_bytes(g.BR);
+    const size_t lds = Sh::lds_bytes;
     const int mode = (add ? 1 : 0) | (pool ? 2 : 0) | (gate ? 4 : 0);
     auto kern = dwconv_tz_k<T, K, NPC, CS, 0>;
     if (mode == 1) kern = dwconv_tz_k<T, K, NPC, CS, 1>;
