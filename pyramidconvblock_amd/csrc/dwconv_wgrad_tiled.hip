@@ -87,6 +87,9 @@ int dwconv_wgrad_mfma_pair_k17(const void* xa, const void* gya, void* dwa, void*
 size_t dwconv_wgrad_tz_workspace(int B, int H, int W, int C, int K, int PH, int PW, int dtype);
 int dwconv_wgrad_tz_launch(const void* x, const void* gy, void* dw, void* ws, int B, int H, int W, int C, int K, int PH,
                            int PW, int dtype, hipStream_t s);
+int dwconv_wgrad_tz_pair_launch(const void* x0, const void* gy0, void* dw0, void* ws0, int H0, int W0, const void* x1,
+                                const void* gy1, void* dw1, void* ws1, int H1, int W1, int B, int C, int K, int PH, int PW,
+                                int dtype, hipStream_t s);
 static bool wgrad_tz_enabled() {
     const char* e = tune_env("PDW_WGRAD_TZ");
     return !(e && atoi(e) == 0);
@@ -135,8 +138,12 @@ int dwconv_wgrad_pair_launch(const void* xa, const void* gya, void* dwa, void* w
                              int dtype, hipStream_t s) {
     if (!wgrad_mfma_enabled(dtype) || tune_env("PDW_NO_WGRAD_PAIR")) return -1;
     if (wgrad_tz_enabled() && dwconv_wgrad_tz_workspace(B, Ha, Wa, C, K, PH, PW, dtype) &&
-        dwconv_wgrad_tz_workspace(B, Hb, Wb, C, K, PH, PW, dtype))
-        return -1;  // the dense matrix-core kernel covers both: two launches of it beat the shared launch of this one
+        dwconv_wgrad_tz_workspace(B, Hb, Wb, C, K, PH, PW, dtype)) {
+        // the dense matrix-core kernel covers both: as one launch of it, else as two (which beat the shared launch of
+        // the kernel below)
+        if (tune_env("PDW_NO_TZ_PAIR")) return -1;
+        return dwconv_wgrad_tz_pair_launch(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, K, PH, PW, dtype, s);
+    }
     switch (K) {
         case 3: return dwconv_wgrad_mfma_pair_k3(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);
         case 5: return dwconv_wgrad_mfma_pair_k5(xa, gya, dwa, wsa, Ha, Wa, xb, gyb, dwb, wsb, Hb, Wb, B, C, PH, PW, dtype, s);

@@ -76,9 +76,10 @@ struct WgTzGeom {
     int nbands, ncolt, nslices;
 };
 
+// One workgroup's band: `blk` of the problem's `nblk` workgroups.
 template <typename T, int NGA, int NCB, int NB>
-__global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict__ x, const T* __restrict__ gy,
-                                                            float* __restrict__ part, const WgTzGeom g) {
+__device__ __forceinline__ void dwconv_wgrad_tz_body(const T* __restrict__ x, const T* __restrict__ gy,
+                                                     float* __restrict__ part, const WgTzGeom& g, int blk, int nblk) {
     using Sh = WgTzShape<NGA, NCB, NB>;
     constexpr int NT = Sh::NT, CS = Sh::CS, CPW = Sh::CPW, NH = Sh::NH, TWG = Sh::TWG, RPX = Sh::RPX, RPG = Sh::RPG, NMF = Sh::NMF;
     constexpr int NSX = Sh::NSX, NSG = Sh::NSG, GBX = Sh::GBX, GBG = Sh::GBG, CHPX = Sh::CHPX, CHPG = Sh::CHPG;
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
     char* const gl = xl + Sh::XB;                     // two copies of [CS] planes of CHPG bytes
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    int bid = xcd_remap(blk, nblk);
     const int sl = bid % g.nslices;
     bid /= g.nslices;
     const int ct = bid % g.ncolt;
@@ -325,6 +326,26 @@ __global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict_
     }
 }
 
+template <typename T, int NGA, int NCB, int NB>
+__global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_k(const T* __restrict__ x, const T* __restrict__ gy,
+                                                            float* __restrict__ part, const WgTzGeom g) {
+    dwconv_wgrad_tz_body<T, NGA, NCB, NB>(x, gy, part, g, blockIdx.x, gridDim.x);
+}
+
+// Two problems of the same filter size in one launch (the two scales of a block): the second problem's nblk1
+// workgroups come first in the grid.  With one workgroup per compute unit and two problems that each fill the chip
+// once, a compute unit runs one band of each back to back, without the drain and the launch between two kernels.
+template <typename T, int NGA, int NCB0, int NCB1, int NB>
+__global__ __launch_bounds__(512, 1) void dwconv_wgrad_tz_pair_k(const T* __restrict__ x0, const T* __restrict__ gy0,
+                                                                 float* __restrict__ part0, const WgTzGeom g0,
+                                                                 const T* __restrict__ x1, const T* __restrict__ gy1,
+                                                                 float* __restrict__ part1, const WgTzGeom g1, int nblk1) {
+    if ((int)blockIdx.x < nblk1)
+        dwconv_wgrad_tz_body<T, NGA, NCB1, NB>(x1, gy1, part1, g1, blockIdx.x, nblk1);
+    else
+        dwconv_wgrad_tz_body<T, NGA, NCB0, NB>(x0, gy0, part0, g0, blockIdx.x - nblk1, gridDim.x - nblk1);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Host side
 
@@ -378,6 +399,21 @@ static int launch_wgrad_tz(const WgTzPlan& p, const void* x, const void* gy, voi
     std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)p.nblocks), dim3(Sh::NT), Sh::lds_bytes, s, (const T*)x, (const T*)gy, (float*)ws, p.g);
     return check_launch("dwconv_wgrad_tz");
+}
+
+template <typename T, int NGA, int NCB0, int NCB1, int NB>
+static int launch_wgrad_tz_pair(const WgTzPlan& p0, const void* x0, const void* gy0, void* ws0, const WgTzPlan& p1,
+                                const void* x1, const void* gy1, void* ws1, hipStream_t s) {
+    using Sh0 = WgTzShape<NGA, NCB0, NB>;
+    using Sh1 = WgTzShape<NGA, NCB1, NB>;
+    auto kern = dwconv_wgrad_tz_pair_k<T, NGA, NCB0, NCB1, NB>;
+    static std::once_flag attr_once;
+    std::call_once(attr_once, [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
+    if (p0.nblocks + p1.nblocks > 0x7fffffffLL) return -1;
+    const size_t lds = Sh0::lds_bytes > Sh1::lds_bytes ? Sh0::lds_bytes : Sh1::lds_bytes;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(p0.nblocks + p1.nblocks)), dim3(Sh0::NT), lds, s, (const T*)x0, (const T*)gy0,
+                       (float*)ws0, p0.g, (const T*)x1, (const T*)gy1, (float*)ws1, p1.g, (int)p1.nblocks);
+    return check_launch("dwconv_wgrad_tz_pair");
 }
 
 }  // namespace pdw
