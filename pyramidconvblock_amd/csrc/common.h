@@ -21,6 +21,15 @@ __device__ __forceinline__ T from_f32(float v) {
     return (T)v;  // round-to-nearest-even (v_cvt_f16_f32 / v_cvt_pk_bf16_f32)
 }
 
+// a * b * s as an fp32 value of its own.  Without the barrier the compiler may fuse the second multiplication with
+// a following conversion to a 16-bit type (one rounding instead of two), in some kernels and element positions and
+// not in others: results that differ in the last bit for about one value in 20 000.
+__device__ __forceinline__ float gate_f32(float a, float b, float s) {
+    float q = a * b * s;
+    asm volatile("" : "+v"(q));
+    return q;
+}
+
 // N consecutive channels moved as one naturally aligned access of N*sizeof(T) bytes.
 template <typename T, int N>
 struct alignas(sizeof(T) * N) ChanVec {

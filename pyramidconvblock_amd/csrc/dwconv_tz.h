@@ -126,7 +126,7 @@ __device__ __forceinline__ uint2 tz_gate(uint2 a, uint2 b, float s) {
     } ua, ub, uo;
     ua.u = a, ub.u = b;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) uo.t[i] = from_f32<T>(to_f32(ua.t[i]) * to_f32(ub.t[i]) * s);
+    for (int i = 0; i < 4; ++i) uo.t[i] = from_f32<T>(gate_f32(to_f32(ua.t[i]), to_f32(ub.t[i]), s));
     return uo.u;
 }
 

@@ -98,6 +98,18 @@ __device__ __forceinline__ void bl_src(int dst, float scale, int in, int& i0, in
     lam = src - (float)lo;
 }
 
+// One resized value from its four taps (row y0: g00, g01; row y1: g10, g11) and bl_src's weights.  The order of the
+// operations and the fused multiply-adds are spelled out and the result is an fp32 value of its own (see gate_f32),
+// so that every kernel that resizes produces the same bits whatever the compiler would contract.
+__device__ __forceinline__ float bl_mix(float g00, float g01, float g10, float g11, float ly, float lx) {
+    const float hy = 1.f - ly, hx = 1.f - lx;
+    const float t0 = __fmaf_rn(lx, g01, __fmul_rn(hx, g00));
+    const float t1 = __fmaf_rn(lx, g11, __fmul_rn(hx, g10));
+    float r = __fmaf_rn(ly, t1, __fmul_rn(hy, t0));
+    asm volatile("" : "+v"(r));
+    return r;
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void bilinear_fwd_item(const T* __restrict__ x, T* __restrict__ y, int h, int w, int C,
                                                   int H, int W, int ldy, float sy, float sx, long long idx) {
@@ -118,9 +130,8 @@ __device__ __forceinline__ void bilinear_fwd_item(const T* __restrict__ x, T* __
     load_f32<T, VEC>(xb + ((long long)y0 * w + x1) * C, bb);
     load_f32<T, VEC>(xb + ((long long)y1 * w + x0) * C, cc);
     load_f32<T, VEC>(xb + ((long long)y1 * w + x1) * C, d);
-    const float hy = 1.f - ly, hx = 1.f - lx;
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) o[v] = hy * (hx * a[v] + lx * bb[v]) + ly * (hx * cc[v] + lx * d[v]);
+    for (int v = 0; v < VEC; ++v) o[v] = bl_mix(a[v], bb[v], cc[v], d[v], ly, lx);
     store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
 }
 
@@ -288,7 +299,7 @@ __device__ __forceinline__ void gate_fwd_item(const T* __restrict__ x, T* __rest
     load_f32<T, VEC>(x + m * I + c, a);
     load_f32<T, VEC>(x + m * I + G + c, b);
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) o[v] = a[v] * b[v] * s;
+    for (int v = 0; v < VEC; ++v) o[v] = gate_f32(a[v], b[v], s);
     store_f32<T, VEC>(y + m * ldy + c, o);
 }
 
@@ -311,8 +322,8 @@ __device__ __forceinline__ void gate_bwd_item(const T* __restrict__ x, const T* 
     load_f32<T, VEC>(gy + m * ldg + c, g);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-        ga[v] = g[v] * b[v] * s;
-        gb[v] = g[v] * a[v] * s;
+        ga[v] = gate_f32(g[v], b[v], s);
+        gb[v] = gate_f32(g[v], a[v], s);
     }
     store_f32<T, VEC>(gx + m * I + c, ga);
     store_f32<T, VEC>(gx + m * I + G + c, gb);
@@ -360,7 +371,7 @@ __device__ __forceinline__ void gate_fwd_items(const T* __restrict__ x, T* __res
         if (u + kGateAhead < U) load(u + kGateAhead);
         float o[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) o[v] = to_f32(a[u].v[v]) * to_f32(b[u].v[v]) * s;
+        for (int v = 0; v < VEC; ++v) o[v] = gate_f32(to_f32(a[u].v[v]), to_f32(b[u].v[v]), s);
         if (first + u * step < total) store_f32<T, VEC>(y + m[u] * ldy + c[u], o);
     }
 }
@@ -393,8 +404,8 @@ __device__ __forceinline__ void gate_bwd_items(const T* __restrict__ x, const T*
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
             const float gv = to_f32(g[u].v[v]);
-            ga[v] = gv * to_f32(b[u].v[v]) * s;
-            gb[v] = gv * to_f32(a[u].v[v]) * s;
+            ga[v] = gate_f32(gv, to_f32(b[u].v[v]), s);
+            gb[v] = gate_f32(gv, to_f32(a[u].v[v]), s);
         }
         if (first + u * step < total) {
             store_f32<T, VEC>(gx + m[u] * I + c[u], ga);
@@ -430,14 +441,13 @@ __device__ __forceinline__ void gate_bilinear_fwd_item(const T* __restrict__ x, 
     pa[1] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o01), pb[1] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o01 + G);
     pa[2] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o10), pb[2] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o10 + G);
     pa[3] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o11), pb[3] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + o11 + G);
-    const float hy = 1.f - ly, hx = 1.f - lx;
     float o[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
         float gv[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) gv[k] = to_f32(from_f32<T>(to_f32(pa[k].v[v]) * to_f32(pb[k].v[v]) * s));
-        o[v] = hy * (hx * gv[0] + lx * gv[1]) + ly * (hx * gv[2] + lx * gv[3]);
+        for (int k = 0; k < 4; ++k) gv[k] = to_f32(from_f32<T>(gate_f32(to_f32(pa[k].v[v]), to_f32(pb[k].v[v]), s)));
+        o[v] = bl_mix(gv[0], gv[1], gv[2], gv[3], ly, lx);
     }
     store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
 }
@@ -484,7 +494,7 @@ __device__ __forceinline__ void gate_bilinear_fwd_x2_item(const T* __restrict__ 
         for (int k = 0; k < 3; ++k)
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
-                gv[r][k][v] = to_f32(from_f32<T>(to_f32(pa[r][k].v[v]) * to_f32(pb[r][k].v[v]) * s));
+                gv[r][k][v] = to_f32(from_f32<T>(gate_f32(to_f32(pa[r][k].v[v]), to_f32(pb[r][k].v[v]), s)));
 #pragma unroll
     for (int di = 0; di < 2; ++di) {
         // Output row 2m + di takes source rows m-1+di and m+di; at the image border bl_src moves the pair one
@@ -493,18 +503,15 @@ __device__ __forceinline__ void gate_bilinear_fwd_x2_item(const T* __restrict__ 
         int y0, y1;
         float ly;
         bl_src(2 * m + di, 0.5f, h, y0, y1, ly);
-        const float hy = 1.f - ly;
 #pragma unroll
         for (int dj = 0; dj < 2; ++dj) {
             int x0, x1;
             float lx;
             bl_src(2 * n + dj, 0.5f, w, x0, x1, lx);
-            const float hx = 1.f - lx;
             float o[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
-                o[v] = hy * (hx * gv[di][dj][v] + lx * gv[di][dj + 1][v]) +
-                       ly * (hx * gv[di + 1][dj][v] + lx * gv[di + 1][dj + 1][v]);
+                o[v] = bl_mix(gv[di][dj][v], gv[di][dj + 1][v], gv[di + 1][dj][v], gv[di + 1][dj + 1][v], ly, lx);
             store_f32<T, VEC>(y + ((b * H + 2 * m + di) * W + 2 * n + dj) * ldy + c, o);
         }
     }
@@ -582,8 +589,8 @@ __device__ __forceinline__ void bilinear_gate_bwd_x2_item(const T* __restrict__ 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
         const float g = to_f32(from_f32<T>(acc[v]));  // the resampled gradient as the separate kernel stores it
-        ga[v] = g * to_f32(xb.v[v]) * s;
-        gbv[v] = g * to_f32(xa.v[v]) * s;
+        ga[v] = gate_f32(g, to_f32(xb.v[v]), s);
+        gbv[v] = gate_f32(g, to_f32(xa.v[v]), s);
     }
     T* op = gx + ((b * h + m) * w + n) * I + c;
     store_f32<T, VEC>(op, ga);
