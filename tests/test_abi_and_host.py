@@ -52,10 +52,11 @@ def test_single_call_block_host_logic_without_gpu():
     assert L.pdw_convblock_supported(32, 56, 56, 128, 64, 13, BF16) == 1
     assert L.pdw_convblock_supported(1, 4, 8, 128, 64, 3, F16) == 1
     assert L.pdw_convblock_supported(2, 32, 32, 64, 32, 7, BF16) == 1
+    assert L.pdw_convblock_supported(8, 112, 112, 96, 48, 17, F16) == 1
     for bad in ((32, 56, 56, 128, 64, 13, F32),    # 16-bit types only
                 (32, 57, 56, 128, 64, 13, BF16),   # odd extent: the pooled scale is not an exact half
                 (32, 56, 56, 128, 64, 12, BF16),   # even filter
-                (32, 56, 56, 96, 48, 13, BF16),    # widths without the paired dense backward
+                (32, 56, 56, 160, 80, 13, BF16),   # widths beyond the dense kernels (128)
                 (0, 56, 56, 128, 64, 13, BF16),
                 (2, 6, 6, 128, 64, 3, BF16)):      # 36 rows per image: not whole row tiles
         assert L.pdw_convblock_supported(*bad) == 0, bad
