@@ -105,6 +105,11 @@ int pdw_dwconv_dgrad_addpool(const void *gy, const void *w, const void *gp, void
  * layer's weight and bias (gw_pool, gbias, gbias2) in the same way instead of computing them in its own launch.
  * No counterpart in the reference (its backward launches every kernel separately, dwconv_triton.py:358-385);
  * the ConvBlock backward (conv_block.py:36-49 under autograd) uses it for its weight gradients. */
+/* out[i] = sum over p < nparts of parts[p * n + i], added in fp32 in a fixed order and rounded once to `dtype`: the
+ * last step of every weight gradient here, on its own for callers that make the partial products themselves (the
+ * operator's weight gradient of conv_up / conv_out for widths the dense kernels do not cover is a batched library
+ * product over row slabs; autograd of conv_block.py:37, 44).  Subject to the deferral below like the others. */
+int pdw_sum_parts(const float *parts, void *out, int nparts, long long n, int dtype, void *stream);
 int pdw_reduce_defer_begin(void);
 int pdw_reduce_defer_flush(void *stream);
 /* pdw_dense_fwd that also runs the reductions recorded so far (see above) in spare workgroups of its own launch;

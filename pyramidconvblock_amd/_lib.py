@@ -73,6 +73,7 @@ _SIGS = {
     "pdw_block_mid_bwd": (c_int, [c_void_p] * 5 + [c_int] * 7 + [c_void_p, c_int] + [c_void_p] * 7 + [c_size_t]
                           + [c_int] * 3 + [c_void_p]),
     "pdw_pool_branch_bwd": (c_int, [c_void_p] * 8 + [c_size_t] + [c_int] * 4 + [c_void_p]),
+    "pdw_sum_parts": (c_int, [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p]),
     "pdw_dense_supported": (c_int, [c_int] * 3),
     "pdw_dense_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong] + [c_int] * 4
                       + [c_void_p]),

@@ -70,10 +70,12 @@ FORCE_STEPWISE = False
 NO_UP_PAIR = False
 
 
-def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
-    """g2d[N,O]^T @ x2d[N,I] -> fp32 [O,I]: a batched product over S slabs of L = N // S rows (16-bit operands: with
+def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor, out_dtype=torch.float32) -> torch.Tensor:
+    """g2d[N,O]^T @ x2d[N,I] -> [O,I]: a batched product over S slabs of L = N // S rows (16-bit operands: with
     fp32 accumulation and output), summed in fp32 (the slabs give the library GEMM enough independent tiles; a single
-    product over N rows runs on a handful of workgroups), plus the N - S*L left-over rows in fp32."""
+    product over N rows runs on a handful of workgroups), plus the N - S*L left-over rows in fp32.  Without left-over
+    rows the slabs are summed by the library's own fixed-order summation (ops.sum_parts), straight into `out_dtype`;
+    otherwise the result is fp32."""
     N = g2d.shape[0]
     if N == 0:
         return g2d.new_zeros((g2d.shape[1], x2d.shape[1]), dtype=torch.float32)
@@ -87,13 +89,18 @@ def _weight_grad(g2d: torch.Tensor, x2d: torch.Tensor) -> torch.Tensor:
     a = g2d[:S * L].view(S, L, -1).transpose(1, 2)
     b = x2d[:S * L].view(S, L, -1)
     out = None
+    parts = None
     if g2d.dtype == torch.float32:
-        out = torch.bmm(a, b).sum(0)
+        parts = torch.bmm(a, b)
     elif _BMM_FP32_OUT[0]:
         try:
-            out = torch.bmm(a, b, out_dtype=torch.float32).sum(0)
+            parts = torch.bmm(a, b, out_dtype=torch.float32)
         except (TypeError, RuntimeError):
             _BMM_FP32_OUT[0] = False
+    if parts is not None:
+        if S * L == N and g2d.is_cuda:
+            return ops.sum_parts(parts, out_dtype)
+        out = parts.sum(0)
     if out is None:
         out = torch.bmm(a, b).float().sum(0) if S > 1 else a[0].float() @ b[0].float()
     if S * L < N:
@@ -310,7 +317,7 @@ class ConvBlockFunction(torch.autograd.Function):
                 grad_w_out = ops.dense_wgrad(gy, cat)
             else:
                 dcat = torch.matmul(g2d, w_out).view(B, H, W, G * ns)
-                grad_w_out = _weight_grad(g2d, cat.view(N, G * ns))
+                grad_w_out = _weight_grad(g2d, cat.view(N, G * ns), w_out.dtype)
 
             gcs = None
             if (pool_fast and gparts is not None and _is_pair(scales) and H == 2 * convs[1].shape[1]
@@ -385,7 +392,7 @@ class ConvBlockFunction(torch.autograd.Function):
                     dx = ops.dense_forward(da, w_up.detach().contiguous(), w_kmajor=True, rowbias=dmean,
                                            rows_per_image=H * W, flush_reductions=True)
             else:
-                grad_w_up = _weight_grad(a2d, x.view(N, D))
+                grad_w_up = _weight_grad(a2d, x.view(N, D), w_up.dtype)
                 if ctx.needs_input_grad[0]:
                     dx = ops.add_rowbias_(torch.matmul(a2d, w_up).view(B, H, W, D), dmean)
         grad_w_out = grad_w_out.to(w_out.dtype)

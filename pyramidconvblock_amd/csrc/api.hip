@@ -178,6 +178,18 @@ int pdw_dwconv_dgrad_addpool(const void* gy, const void* w, const void* gp, void
     return avgpool_bwd_launch(gp, dx, B, H, W, C, h, wp, 1, dtype, (hipStream_t)stream);
 }
 
+int pdw_sum_parts(const float* parts, void* out, int nparts, long long n, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_sum_parts: unknown dtype %d", dtype), 1;
+    if (nparts < 1 || n < 0 || n > 0x7fffffffLL) return set_error("pdw_sum_parts: bad extents nparts=%d n=%lld", nparts, n), 1;
+    if (n == 0) return 0;
+    if (!parts || !out) return set_error("pdw_sum_parts: null pointer"), 1;
+    switch (dtype) {
+        case kF32: return wgrad_reduce_launch<float>(parts, out, nparts, (int)n, (hipStream_t)stream);
+        case kF16: return wgrad_reduce_launch<f16_t>(parts, out, nparts, (int)n, (hipStream_t)stream);
+        default: return wgrad_reduce_launch<bf16_t>(parts, out, nparts, (int)n, (hipStream_t)stream);
+    }
+}
+
 int pdw_reduce_defer_begin(void) { return reduce_defer_begin(); }
 
 int pdw_reduce_defer_flush(void* stream) { return reduce_defer_flush((hipStream_t)stream); }

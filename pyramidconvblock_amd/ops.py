@@ -297,6 +297,18 @@ def dense_wgrad(a, b):
     return dw
 
 
+def sum_parts(parts, dtype):
+    """parts[S, ...] (fp32) -> their sum over S, added in fp32 in a fixed order and rounded once to `dtype`
+    (pdw_sum_parts; inside a deferral the summation joins the pass's single reduction launch)."""
+    dev = _lib.require_device(parts)
+    assert parts.dtype == torch.float32 and parts.dim() >= 2
+    parts = parts.contiguous()
+    out = torch.empty(parts.shape[1:], device=dev, dtype=dtype)
+    _launch("pdw_sum_parts", dev, parts.data_ptr(), out.data_ptr(), parts.shape[0], out.numel(), _lib.dtype_code(dtype))
+    _lib.keep_until_flush(parts)
+    return out
+
+
 def dense_backward_pair_supported(O, I, dtype, rows_per_image=None, colsum=False) -> bool:
     """Whether dense_backward_pair covers a layer with weight [O, I] (and a per-image term over images of
     rows_per_image rows; with `colsum`, the tile sums of gy as well)."""

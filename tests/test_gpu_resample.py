@@ -337,3 +337,22 @@ def test_dense_backward_pair_matches_separate_launches(dtype, N, widths):
         dwa = ops.dense_wgrad(x, gy)
         dxb, _, dwb = ops.dense_backward_pair(x, w2, gy, rowbias=rb, rows_per_image=P)
         assert torch.equal(dxb, dxa) and torch.equal(dwb, dwa)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 7), (37, 200, 100), (183, 100, 200), (256, 3, 5), (5, 1)])
+def test_sum_parts_is_the_fp32_sum_rounded_once(shape, dtype):
+    """pdw_sum_parts (the slab summation of the operator's fallback weight gradient): the sum over the leading
+    dimension, against a float64 sum; 16-bit outputs within half an ulp of it plus the fp32 summation error."""
+    from pyramidconvblock_amd import ops
+
+    gen = torch.Generator().manual_seed(11)
+    parts = torch.randn(*shape, generator=gen, dtype=torch.float32)
+    out = ops.sum_parts(parts.cuda(), dtype)
+    torch.cuda.synchronize()
+    assert out.dtype == dtype and tuple(out.shape) == tuple(shape[1:])
+    ref = parts.double().sum(0)
+    eps = {torch.float32: 2.0 ** -24, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    tol = eps * ref.abs() + shape[0] * 2.0 ** -24 * parts.abs().double().sum(0) + 1e-7
+    assert bool(((out.double().cpu() - ref).abs() <= tol).all())
