@@ -328,20 +328,21 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             const int img = min((int)((m < N ? m : N - 1) / P), nimg - 1);
             blr += (img - (int)(tile * 32 / P)) * NOP;
         }
-        for (int nt = 0; nt < nnt; ++nt) {
-            // all LDS reads of the feature tile are issued before its first MFMA
+        // One 32-feature tile: its weight fragments and bias values (all LDS reads issued before the first MFMA), the
+        // product, and the way out (bias added, rounded, into the tile buffer).
+        auto load_w = [&](int nt, Frag (&wf)[kKT], float4 (&r4)[4]) {
             const T* wr = wl + (nt * 32 + l32) * ldw + 8 * half;
-            Frag wf[kKT];
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
             if (nkt > 4) {
 #pragma unroll
                 for (int kt = 4; kt < 8; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
             }
-            float4 r4[4];
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4)
                 r4[g4] = hasb ? *reinterpret_cast<const float4*>(blr + nt * 32 + g4 * 8) : make_float4(0.f, 0.f, 0.f, 0.f);
+        };
+        auto product = [&](const Frag (&wf)[kKT]) {
             f32x16 acc;
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -351,6 +352,9 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
 #pragma unroll
                 for (int kt = 4; kt < 8; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
             }
+            return acc;
+        };
+        auto way_out = [&](int nt, const f32x16& acc, const float4 (&r4)[4]) {
             // lane owns row l32 of the tile and features n0..n0+3 of each accumulator group
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
@@ -361,6 +365,31 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                     o[2] = acc[g4 * 4 + 2] + r4[g4].z, o[3] = acc[g4 * 4 + 3] + r4[g4].w;
                     store_f32<T, 4>(tl + l32 * ldt + n0, o);
                 }
+            }
+        };
+        if constexpr (STATIC) {
+            // Software pipeline over the feature tiles (unrolled): tile nt + 1's LDS reads are issued before tile nt's
+            // MFMAs, and tile nt's way out follows the issue of tile nt + 1's MFMAs, so neither the read latency nor
+            // the MFMA latency of a tile sits between two tiles.
+            constexpr int NNT = SNO / 32;
+            Frag wf[2][kKT];
+            float4 r4[3][4];   // (three tiles' bias values are alive at once: nt - 1 on its way out, nt, nt + 1 read ahead)
+            f32x16 acc[2];
+            load_w(0, wf[0], r4[0]);
+#pragma unroll
+            for (int nt = 0; nt < NNT; ++nt) {
+                if (nt + 1 < NNT) load_w(nt + 1, wf[(nt + 1) % 2], r4[(nt + 1) % 3]);
+                acc[nt % 2] = product(wf[nt % 2]);
+                if (nt > 0) way_out(nt - 1, acc[(nt - 1) % 2], r4[(nt - 1) % 3]);
+            }
+            way_out(NNT - 1, acc[(NNT - 1) % 2], r4[(NNT - 1) % 3]);
+        } else {
+            for (int nt = 0; nt < nnt; ++nt) {
+                Frag wf[kKT];
+                float4 r4[4];
+                load_w(nt, wf, r4);
+                const f32x16 acc = product(wf);
+                way_out(nt, acc, r4);
             }
         }
         // coalesced copy-out of the 32 x NO tile (same wavefront wrote it: no workgroup barrier needed)
