@@ -156,6 +156,18 @@ int pdw_dwconv_wgrad_static(const void *x, const void *gy, void *dw, int B, int 
 int pdw_dwconv_wgrad_pair(const void *x0, const void *gy0, void *dw0, void *workspace0, size_t workspace0_bytes,
                           int H0, int W0, const void *x1, const void *gy1, void *dw1, void *workspace1,
                           size_t workspace1_bytes, int H1, int W1, int B, int C, int K, int dtype, void *stream);
+/* The three convolution launches at the end of a two-scale block's backward pass that do not depend on one another, as
+ * one launch (backward of conv_block.py:14-16, 41 under autograd): dx = the full scale's input gradient from gy0 and w0
+ * plus a quarter of gp per 2x2 block (what pdw_dwconv_dgrad_addpool computes; gp [B,H/2,W/2,C] is the pooled scale's
+ * input gradient), dw0 = the full scale's weight gradient from x0 and gy0, dw1 = the half scale's from x1 and gy1
+ * [B,H/2,W/2,C].  Square odd filter, stride 1, padding K/2, even H and W; workspaces as for the two pdw_dwconv_wgrad
+ * calls.  Status 3 (nothing launched) when the fused kernel does not cover the case (fp32, C % 16, images narrower than
+ * 33 columns...): the caller then makes the three calls.  Results are bitwise those of the separate calls; between
+ * pdw_reduce_defer_begin/flush the two summations are recorded like any other. */
+int pdw_dwconv_bwd3(const void *gy0, const void *w0, const void *gp, void *dx, const void *x0, void *dw0,
+                    void *workspace0, size_t workspace0_bytes, const void *x1, const void *gy1, void *dw1,
+                    void *workspace1, size_t workspace1_bytes, int B, int H, int W, int C, int K, int dtype,
+                    void *stream);
 
 /* Adaptive average pooling x[B,H,W,C] -> y[B,h,w,C]; bin i covers [floor(i*H/h), ceil((i+1)*H/h)).
  * Replaces F.adaptive_avg_pool2d at conv_block.py:16 and the launch at avgpool_triton.py:225-229

@@ -271,6 +271,27 @@ int pdw_dwconv_wgrad_pair(const void* x0, const void* gy0, void* dw0, void* work
                             stream);
 }
 
+int pdw_dwconv_bwd3(const void* gy0, const void* w0, const void* gp, void* dx, const void* x0, void* dw0, void* workspace0,
+                    size_t workspace0_bytes, const void* x1, const void* gy1, void* dw1, void* workspace1,
+                    size_t workspace1_bytes, int B, int H, int W, int C, int K, int dtype, void* stream) {
+    const int P = K / 2;
+    if (!(K & 1)) return set_error("pdw_dwconv_bwd3: odd filter size needed (K=%d)", K), 1;
+    if ((H & 1) || (W & 1)) return set_error("pdw_dwconv_bwd3: even extents needed (H=%d W=%d)", H, W), 1;
+    if (int e = check_conv("pdw_dwconv_bwd3", x0, gy0, dw0, B, H, W, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (int e = check_conv("pdw_dwconv_bwd3", x1, gy1, dw1, B, H / 2, W / 2, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (!w0 || !gp || !dx || !dw0 || !dw1) return set_error("pdw_dwconv_bwd3: null pointer"), 1;
+    const size_t need0 = pdw_dwconv_wgrad_workspace_bytes(B, H, W, C, K, K, 1, 1, P, P, 1, 1, dtype);
+    const size_t need1 = pdw_dwconv_wgrad_workspace_bytes(B, H / 2, W / 2, C, K, K, 1, 1, P, P, 1, 1, dtype);
+    if (!workspace0 || workspace0_bytes < need0 || !workspace1 || workspace1_bytes < need1)
+        return set_error("pdw_dwconv_bwd3: workspaces of %zu and %zu bytes given, %zu and %zu needed", workspace0_bytes,
+                         workspace1_bytes, need0, need1), 1;
+    if (B == 0) return 0;
+    const int r = dwconv_bwd3_launch(gy0, w0, gp, dx, x0, dw0, workspace0, x1, gy1, dw1, workspace1, B, H, W, C, K, dtype,
+                                     (hipStream_t)stream);
+    if (r == -1) return set_error("pdw_dwconv_bwd3: case not covered (B=%d H=%d W=%d C=%d K=%d dtype=%d)", B, H, W, C, K, dtype), 3;
+    return r;
+}
+
 int pdw_avgpool_fwd(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
     if (int e = check_resample("pdw_avgpool_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
     return avgpool_fwd_launch(x, y, B, H, W, C, h, w, dtype, (hipStream_t)stream);

@@ -223,11 +223,25 @@ int pdw_convblock_bwd(const void* gy, const void* x, const void* a, const void* 
                                    gb_out ? gb_out : (void*)gbias, gb_pool ? gb_pool : (void*)(gbias + (size_t)D * s.es),
                                    gw_pool, dmean, ws_pool, up256(b_pool_ws), s.P, D, dtype, stream)))
             break;
-        // depthwise convs: weight gradients of both scales, then the input gradients, pooled scale first
+        // depthwise convs: the pooled scale's input gradient, then the full scale's (which adds it) together with the
+        // weight gradients of both scales in one launch where that is covered
+        {
+            if ((e = pdw_dwconv_dgrad(gch, w_dw1, dxp, B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream))) break;
+            const int r = pdw_dwconv_bwd3(gcf, w_dw0, dxp, da, a, gw_dw0, ws_w0, up256(b_w0), xp, gch, gw_dw1, ws_w1,
+                                          up256(b_w1), B, H, W, I, K, dtype, stream);
+            if (r != 0 && r != 3) {
+                e = r;
+                break;
+            }
+            if (r == 0) {
+                e = pdw_dense_bwd_pair(da, w_up, x, dx, nullptr, gw_up, ws_pu, up256(b_pu), dmean, s.P, s.N, I, D, dtype, stream);
+                break;
+            }
+        }
+        // otherwise: weight gradients of both scales, then the full scale's input gradient
         if ((e = pdw_dwconv_wgrad_pair(a, gcf, gw_dw0, ws_w0, up256(b_w0), H, W, xp, gch, gw_dw1, ws_w1, up256(b_w1), s.h,
                                        s.w, B, I, K, dtype, stream)))
             break;
-        if ((e = pdw_dwconv_dgrad(gch, w_dw1, dxp, B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream))) break;
         if ((e = pdw_dwconv_dgrad_addpool(gcf, w_dw0, dxp, da, B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, s.h, s.w, dtype,
                                           stream)))
             break;

@@ -130,10 +130,11 @@ __device__ __forceinline__ uint2 tz_gate(uint2 a, uint2 b, float s) {
     return uo.u;
 }
 
+// One workgroup's band: `blk` of the problem's `nblk` workgroups.
 template <typename T, int K, int NPC, int CS, int MODE>
-__global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, const T* __restrict__ w,
-                                                      const T* __restrict__ add, T* __restrict__ pool,
-                                                      T* __restrict__ y, const TzGeom g) {
+__device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T* __restrict__ w,
+                                               const T* __restrict__ add, T* __restrict__ pool, T* __restrict__ y,
+                                               const TzGeom& g, int blk, int nblk) {
     using Sh = TzShape<K, NPC, CS>;
     constexpr int NT = Sh::NT, ICB = Sh::ICB, NKG = Sh::NKG, NM = Sh::NM, PER = Sh::PER, RING = Sh::RING;
     constexpr int NI = Sh::NI, TW = Sh::TW, NH = Sh::NH, CPW = Sh::CPW, RP = Sh::RP, OPX = Sh::OPX, OROWP = Sh::OROWP;
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     char* const r2 = xl + NI * CS * CHP;                 // filter table, then the two result tiles
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    int bid = xcd_remap(blockIdx.x, gridDim.x);
+    int bid = xcd_remap(blk, nblk);
     const int sl = bid % g.nslices;
     bid /= g.nslices;
     const int ct = bid % g.ncolt;
@@ -492,6 +493,13 @@ __global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, c
     store(fdone - 1);
 }
 
+template <typename T, int K, int NPC, int CS, int MODE>
+__global__ __launch_bounds__(512, 1) void dwconv_tz_k(const T* __restrict__ x, const T* __restrict__ w,
+                                                      const T* __restrict__ add, T* __restrict__ pool,
+                                                      T* __restrict__ y, const TzGeom g) {
+    dwconv_tz_body<T, K, NPC, CS, MODE>(x, w, add, pool, y, g, blockIdx.x, gridDim.x);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Host side
 
@@ -512,22 +520,31 @@ static int tz_pick_band(int B, int OH, int OW, int C) {
     return best;
 }
 
+// The geometry of a launch (false: not covered) and its number of workgroups.
+template <int K, int NPC, int CS>
+static bool tz_make_geom(TzGeom& g, long long& nblocks, bool add, int B, int H, int W, int C, int PH, int PW, bool flip,
+                         const TzGate* gate) {
+    using Sh = TzShape<K, NPC, CS>;
+    g.B = B, g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0;
+    g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
+    g.AH = add ? g.OH / 2 : H / 2, g.AW = add ? g.OW / 2 : W / 2;
+    g.YC = gate ? gate->ldy : C, g.ych = gate ? gate->ych : 0, g.gs = gate ? gate->gs : 1.f;
+    if (gate && (CS != 16 || add || flip || C % 16 != 0 || gate->ldy < gate->ych + C / 2 || (gate->ldy | gate->ych) % 8 != 0)) return false;
+    if ((long long)H * W * C * Sh::NI > 0x1fffffffLL || (long long)g.OH * g.OW * g.YC * Sh::NI > 0x1fffffffLL) return false;
+    g.BR = tz_pick_band<K, NPC, CS>(B, g.OH, g.OW, C);
+    if (g.BR < 4) return false;
+    g.nbands = cdiv(g.OH, g.BR), g.ncolt = cdiv(g.OW, Sh::TW), g.nslices = cdiv(C, CS);
+    nblocks = (long long)cdiv(B, Sh::NI) * g.nbands * g.ncolt * g.nslices;
+    return nblocks <= 0x7fffffffLL;
+}
+
 template <typename T, int K, int NPC, int CS>
 static int launch_tz(const void* x, const void* w, const void* add, void* pool, void* y, int B, int H, int W, int C,
                      int PH, int PW, bool flip, const TzGate* gate, hipStream_t s) {
     using Sh = TzShape<K, NPC, CS>;
     TzGeom g;
-    g.B = B, g.H = H, g.W = W, g.C = C, g.PH = PH, g.PW = PW, g.flip = flip ? 1 : 0;
-    g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
-    g.AH = add ? g.OH / 2 : H / 2, g.AW = add ? g.OW / 2 : W / 2;
-    g.YC = gate ? gate->ldy : C, g.ych = gate ? gate->ych : 0, g.gs = gate ? gate->gs : 1.f;
-    if (gate && (CS != 16 || add || flip || C % 16 != 0 || gate->ldy < gate->ych + C / 2 || (gate->ldy | gate->ych) % 8 != 0)) return -1;
-    if ((long long)H * W * C * Sh::NI > 0x1fffffffLL || (long long)g.OH * g.OW * g.YC * Sh::NI > 0x1fffffffLL) return -1;
-    g.BR = tz_pick_band<K, NPC, CS>(B, g.OH, g.OW, C);
-    if (g.BR < 4) return -1;
-    g.nbands = cdiv(g.OH, g.BR), g.ncolt = cdiv(g.OW, Sh::TW), g.nslices = cdiv(C, CS);
-    const long long nblocks = (long long)cdiv(B, Sh::NI) * g.nbands * g.ncolt * g.nslices;
-    if (nblocks > 0x7fffffffLL) return -1;
+    long long nblocks;
+    if (!tz_make_geom<K, NPC, CS>(g, nblocks, add != nullptr, B, H, W, C, PH, PW, flip, gate)) return -1;
     const size_t lds = Sh::lds_bytes;
     const int mode = (add ? 1 : 0) | (pool ? 2 : 0) | (gate ? 4 : 0);
     auto kern = dwconv_tz_k<T, K, NPC, CS, 0>;

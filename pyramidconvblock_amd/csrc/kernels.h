@@ -116,4 +116,10 @@ int dense_bwd_pair_colsum_supported(int O, int I, int dtype);
 int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* dx, float* colsum, void* dw, void* ws,
                           const float* rowbias, int P, long long N, int O, int I, int dtype, hipStream_t s);
 
+// dwconv_bwd3.hip: input gradient (+ pooled branch's) of the full scale and the weight gradients of both scales of a
+// two-scale block in one launch; -1 = not covered
+int dwconv_bwd3_launch(const void* gyf, const void* w0, const void* addp, void* dx, const void* x0, void* dw0, void* ws0,
+                       const void* x1, const void* gy1, void* dw1, void* ws1, int B, int H, int W, int C, int K, int dtype,
+                       hipStream_t s);
+
 }  // namespace pdw

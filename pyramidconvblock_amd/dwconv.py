@@ -124,6 +124,40 @@ def dwconv_wgrad_pair(x0, gy0, x1, gy1, w_shape):
     return dws[0], dws[1]
 
 
+def dwconv_bwd3(gy0, w0, gp, x0, x1, gy1):
+    """The end of a two-scale block's backward pass as one call of the library (pdw_dwconv_bwd3): returns
+    (dx, dw0, dw1) = (dwconv_dgrad(gy0, w0, pooled_grad=gp), dwconv_wgrad(x0, gy0), dwconv_wgrad(x1, gy1)) for 'same'
+    convolutions with one odd square filter shape, x1 / gy1 / gp at exactly half the extents of x0 / gy0; None when
+    the fused kernel does not cover the case (the caller then makes the three calls)."""
+    dev = _lib.require_device(gy0, w0, gp, x0, x1, gy1)
+    L = _lib.lib()
+    K, C = int(w0.shape[0]), int(w0.shape[2])
+    B, H, W = x0.shape[0], x0.shape[1], x0.shape[2]
+    if (w0.shape[0] != w0.shape[1] or K % 2 == 0 or x0.shape != gy0.shape or x1.shape != gy1.shape or gp.shape != x1.shape
+            or tuple(x1.shape) != (B, H // 2, W // 2, C) or H % 2 or W % 2 or x0.shape[3] != C
+            or any(t.dtype != x0.dtype for t in (gy0, w0, gp, x1, gy1)) or B == 0):
+        return None
+    code = _lib.dtype_code(x0.dtype)
+    dx = torch.empty_like(x0)
+    dws = [torch.empty(tuple(w0.shape), device=dev, dtype=x0.dtype) for _ in range(2)]
+    wss = []
+    for x in (x0, x1):
+        nbytes = L.pdw_dwconv_wgrad_workspace_bytes(B, x.shape[1], x.shape[2], C, K, K, 1, 1, K // 2, K // 2, 1, 1, code)
+        wss.append(torch.empty(max(nbytes, 4) // 4 + 1, device=dev, dtype=torch.float32))
+    args = [t.contiguous() for t in (gy0, w0, gp, x0, x1, gy1)]
+    with _lib.on_device(dev):
+        st = L.pdw_dwconv_bwd3(args[0].data_ptr(), args[1].data_ptr(), args[2].data_ptr(), dx.data_ptr(), args[3].data_ptr(),
+                               dws[0].data_ptr(), wss[0].data_ptr(), wss[0].numel() * 4, args[4].data_ptr(),
+                               args[5].data_ptr(), dws[1].data_ptr(), wss[1].data_ptr(), wss[1].numel() * 4, B, H, W, C, K,
+                               code, _lib.stream_ptr(dev))
+    if st == 3:
+        return None
+    _lib.check(st, "pdw_dwconv_bwd3")
+    for ws in wss:
+        _lib.keep_until_flush(ws)
+    return dx, dws[0], dws[1]
+
+
 class DepthwiseConv2DFunction(torch.autograd.Function):
     """apply(input[B,H,W,C], weight[k1,k2,C], stride, padding, dilation, dtype) -> output[B,OH,OW,C] of `dtype`.
 

@@ -131,6 +131,36 @@ def test_wgrad_pair_is_the_two_separate_calls(dtype, case):
         assert torch.equal(w, g) and torch.equal(w, l)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("case", [(32, 56, 56, 64, 13), (8, 112, 112, 48, 17), (2, 40, 36, 32, 9), (3, 34, 70, 16, 3),
+                                  (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7)])
+def test_bwd3_is_the_three_separate_calls(dtype, case):
+    """pdw_dwconv_bwd3 (the full scale's input gradient with the pooled branch's added and the weight gradients of
+    both scales in one launch) gives bitwise the results of the three separate calls, immediately and with the
+    summations deferred; where the fused kernel does not cover the case it says so and launches nothing."""
+    from pyramidconvblock_amd import _lib
+    from pyramidconvblock_amd.dwconv import dwconv_bwd3, dwconv_dgrad, dwconv_wgrad
+
+    B, H, W, C, k = case
+    gen = torch.Generator().manual_seed(13)
+    gy0, x0 = (randn(gen, B, H, W, C).to(dtype).cuda() for _ in range(2))
+    gp, x1, gy1 = (randn(gen, B, H // 2, W // 2, C).to(dtype).cuda() for _ in range(3))
+    w0 = (randn(gen, k, k, C) / k).to(dtype).cuda()
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    got = dwconv_bwd3(gy0, w0, gp, x0, x1, gy1)
+    covered = dtype != torch.float32 and C % 16 == 0 and W > 32
+    assert (got is not None) == covered
+    if got is None:
+        return
+    want = [dwconv_dgrad(gy0, w0, x0.shape, *geo, pooled_grad=gp), dwconv_wgrad(x0, gy0, (k, k, C), *geo),
+            dwconv_wgrad(x1, gy1, (k, k, C), *geo)]
+    with _lib.deferred_reductions(gy0.device):
+        later = dwconv_bwd3(gy0, w0, gp, x0, x1, gy1)
+    torch.cuda.synchronize()
+    for w, g, l in zip(want, got, later):
+        assert torch.equal(w, g) and torch.equal(w, l)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_full_size_properties(dtype):
     """Size-independent checks at the benchmark shape: delta kernel = identity, linearity in w,
