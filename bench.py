@@ -262,8 +262,31 @@ def kernel_rooflines(B, H, W, D, k, dtype):
             out.append(dict(kernel=f"{name}[{B}x{h}x{w}x{I},k={k}]", seconds=t, alg_bytes=conv_bytes, flops=flops,
                             issued_flops=2.0 * issued * n_el if issued else None, pipe="mfma"))
         del xs, gs
-    # resampling kernels of the half-resolution gate
+    # the backward's largest launch: full-scale input gradient (adds the pooled branch's) + both weight gradients
     h, w = H // 2, W // 2
+    nF, nH = B * H * W * I, B * h * w * I
+    nbuf = max(2, int(600e6 // (4 * nF * es)) + 1)
+    gf = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    xf = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    gp = [torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    xh = [torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    gh = [torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    wt = (torch.randn(k, k, I, device="cuda") / k).to(dtype)
+    if dwconv.dwconv_bwd3(gf[0], wt, gp[0], xf[0], xh[0], gh[0]) is not None:
+        from pyramidconvblock_amd import _lib
+
+        def four(i):   # as in the block, the summations of the weight-gradient partials are deferred: one small
+            with _lib.deferred_reductions(gf[0].device):   # launch per 4 calls here, one per backward pass there
+                for j in range(4 * i, 4 * i + 4):
+                    dwconv.dwconv_bwd3(gf[j % nbuf], wt, gp[j % nbuf], xf[j % nbuf], xh[j % nbuf], gh[j % nbuf])
+
+        t = time_kernel_events(four, nbuf, iters=6) / 4
+        out.append(dict(kernel=f"dwconv_bwd3[{B}x{H}x{W}x{I},k={k}]", seconds=t,
+                        alg_bytes=es * (3 * nF + 3 * nH + 3 * k * k * I), flops=2.0 * k * k * (2 * nF + nH),
+                        issued_flops=(2.0 * (iss["fwd"] * nF + iss["wgrad"] * (nF + nH)) if iss["wgrad"] else None),
+                        pipe="mfma"))
+    del gf, xf, gp, xh, gh
+    # resampling kernels of the half-resolution gate
     nbuf = 8
     a = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
     p = [torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(nbuf)]
@@ -323,7 +346,8 @@ def conv_rows(B, H, W, C, dtype, ks=(9, 13, 17)):
 
 def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     """Launches one hot kernel `iters` times at its shape inside the headline block (for rocprofv3 runs).
-    name: {fwd,dgrad,wgrad}_{full,half} | conv128 (stand-alone forward at C = D) | avgpool_fwd | avgpool_bwd |
+    name: {fwd,dgrad,wgrad}_{full,half} | bwd3 (full-scale input gradient + both weight gradients, one launch) |
+    conv128 (stand-alone forward at C = D) | avgpool_fwd | avgpool_bwd |
     bilinear_fwd | bilinear_bwd | dense_{fwd,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pair = both
     gradients in one launch) | step (whole forward+backward steps, eager) | copy"""
     from pyramidconvblock_amd import avgpool, dwconv, up
@@ -350,6 +374,11 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         x = torch.randn(B, H, W, D, device="cuda").to(dtype)
         wt = (torch.randn(k, k, D, device="cuda") / k).to(dtype)
         fn = lambda: dwconv.dwconv_forward(x, wt, *geo)
+    elif name == "bwd3":
+        gf, xf = (torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(2))
+        gp, xh, gh = (torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(3))
+        wt = (torch.randn(k, k, I, device="cuda") / k).to(dtype)
+        fn = lambda: dwconv.dwconv_bwd3(gf, wt, gp, xf, xh, gh)
     elif op in ("fwd", "dgrad", "wgrad"):
         hh, ww = (H, W) if res == "full" else (h, w)
         x = torch.randn(B, hh, ww, I, device="cuda").to(dtype)
@@ -450,7 +479,7 @@ def main():
     ap.add_argument("--no-configs", action="store_true", help="skip the rows of the other workloads")
     ap.add_argument("--no-torch-gpu", action="store_true", help="skip the torch-operator comparator on the GPU")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
-                    "{fwd,dgrad,wgrad}_{full,half}, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
+                    "{fwd,dgrad,wgrad}_{full,half}, bwd3, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
                     "dense_{fwd,dgrad,wgrad,pair}, step, copy")
     ap.add_argument("--torch-gpu-only", action="store_true", help="(internal) time the torch-operator comparator and exit")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
