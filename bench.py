@@ -176,6 +176,42 @@ def measure_block(m, shape, dtype, dist, steps, warmup, with_forward=True):
     return out
 
 
+def measure_block_in_one_graph(m, shape, dtype, steps, warmup):
+    """ms per forward+backward step when one HIP graph holds a step on each buffer set (n_sets steps per replay):
+    the block as one of several layers of a captured model, where the idle time between two graph replays is
+    shared by the layers instead of falling on a single block."""
+    B, H, W, D = shape
+    k = m.gates[0].conv_spatial.weight.shape[0]
+    ns = n_sets(B, H, W, D, k, torch.empty((), dtype=dtype).element_size())
+    sets = [make_inputs(shape, dtype, "normal", seed=i) for i in range(ns)]
+    xs = [x.detach().clone().requires_grad_() for x, _ in sets]
+    keep = []
+
+    def steps_once():
+        for x, (_, g) in zip(xs, sets):
+            x.grad = None
+            for p in m.parameters():
+                p.grad = None
+            y = m(x)
+            torch.autograd.backward(y, g)
+            keep.append([y, x.grad] + [p.grad for p in m.parameters()])   # graph-owned results stay referenced
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        steps_once()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    keep.clear()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        steps_once()
+    t = time_gpu(graph.replay, max(1, steps // ns), max(1, warmup // ns)) / ns * 1e3
+    for p in m.parameters():
+        p.grad = None
+    return t, ns
+
+
 def torch_gpu_block(shape, D, k, dtype, steps, warmup):
     """The same block through torch's own GPU operators, as the reference's benchmark times its all-torch twin on
     the same device (pyramid_dwconv/conv_block.py:52-97, :99-158): NCHW, 1x1 and grouped F.conv2d,
@@ -504,6 +540,7 @@ def main():
 
     m = make_block(D, k, dtype)
     head = measure_block(m, (B, H, W, D), dtype, "normal", args.steps, args.warmup)
+    t_chain, n_chain = measure_block_in_one_graph(m, (B, H, W, D), dtype, args.steps, args.warmup)
     # eager launches of the same step (host-bound), for reference
     x0, g0 = make_inputs((B, H, W, D), dtype, "normal", 0)
     x0.requires_grad_()
@@ -544,6 +581,10 @@ def main():
         "warm_fwd_ms": head["fwd_ms_warm"],
         "eager_ms_per_step": t_eager * 1e3,
         "launch": "one HIP graph replay per step (eager launch time in eager_ms_per_step)",
+        "in_graph_ms_per_step": t_chain,
+        "in_graph_note": f"{n_chain} steps (one per buffer set) captured in ONE graph, time per replay / {n_chain}: the "
+                         "block as one of several layers of a captured model; `value` instead pays the idle time "
+                         "between two graph replays once per step",
         "block_hbm_frac_fwd_bwd": bytes_fb / (t_step * HBM_PEAK),
         "block_hbm_frac_fwd_bwd_warm": bytes_fb / (head["fwd_bwd_ms_warm"] * 1e-3 * HBM_PEAK),
         "block_hbm_frac_fwd": bytes_f / (head["fwd_ms"] * 1e-3 * HBM_PEAK),

@@ -1,7 +1,7 @@
 """HIP-graph capture of a forward+backward step.
 
-A ConvBlock step is ~50 short kernels; launched one by one from Python the host is the
-bottleneck.  ``GraphedStep`` captures ``y = module(x); backward(y, grad)`` once into a HIP
+A ConvBlock step is a dozen short kernels (about 150 us of GPU time at [32,56,56,128]); launched
+one by one from Python and the autograd engine the host takes longer than the GPU.  ``GraphedStep`` captures ``y = module(x); backward(y, grad)`` once into a HIP
 graph (through ``torch.cuda.CUDAGraph``) and replays it.  Every kernel of libpdw.so is capture
 safe: no allocation, no synchronisation, no memset nodes.
 """
