@@ -19,7 +19,9 @@
 // twice the rate of narrower ones on this part (measured: 256 against 128 bytes per clock), which is why the
 // column offsets of the xw operand are multiples of 8 elements: it is one ds_read_b128.  The fine offsets (du, dv)
 // shift gy by single elements, so gy is staged twice, the second copy one element to the left, and a lane reads
-// whichever copy makes its run of 8 values dword aligned (two ds_read2_b32).
+// whichever copy makes its run of 8 values dword aligned (two ds_read2_b32).  A gy staging item is 4 consecutive
+// columns of one row (x an 8-channel piece), so that both copies are written as 8-byte stores: the second copy's last
+// pair takes the first column of the item to the right through a lane shift (a window row sits in one wavefront).
 //
 // Staging is the streamed scheme of dwconv_tz.h: both tensors arrive in passes of 8 rows, requested two ahead
 // into two register buffers each and committed to LDS one step before they are read; the LDS windows are rings of
@@ -64,7 +66,12 @@ struct WgTzShape {
     static_assert(NGA >= 2 && NGA <= 5 && (NCB == 8 || NCB == 5) && (NB == 2 || NB == 3), "row groups spanned, column blocks");
     static_assert(RPX % 128 == 32 && RPX >= 2 * WCX && RPG % 128 == 40 && RPG >= 2 * WCG && CHPX % 16 == 0 && GCB % 128 == 24,
                   "operand alignment / bank spread");
-    static_assert(4 * (WCX / 2) * NH <= NT && 4 * (WCG / 2) * NH <= NT, "a pass is at most one item per thread");
+    // gy staging item: 4 consecutive columns of one window row x an 8-channel piece; a window row is GLPR consecutive
+    // lanes of one wavefront (the item to the right is NH lanes up: its first column completes the second copy's
+    // last pair), GRPW whole rows per wavefront
+    static constexpr int GLPR = (WCG / 4) * NH, GRPW = 64 / GLPR;
+    static_assert(4 * (WCX / 2) * NH <= NT && GRPW >= 1 && (8 + GRPW - 1) / GRPW <= NT / 64 && WCG % 4 == 0,
+                  "a pass is at most one item per thread");
     static_assert(lds_bytes <= 160 * 1024, "LDS");
 };
 
@@ -83,7 +90,7 @@ __device__ __forceinline__ void dwconv_wgrad_tz_body(const T* __restrict__ x, co
     using Sh = WgTzShape<NGA, NCB, NB>;
     constexpr int NT = Sh::NT, CS = Sh::CS, CPW = Sh::CPW, NH = Sh::NH, TWG = Sh::TWG, RPX = Sh::RPX, RPG = Sh::RPG, NMF = Sh::NMF;
     constexpr int NSX = Sh::NSX, NSG = Sh::NSG, GBX = Sh::GBX, GBG = Sh::GBG, CHPX = Sh::CHPX, CHPG = Sh::CHPG;
-    constexpr int WCPX = Sh::WCX / 2, WCPG = Sh::WCG / 2;
+    constexpr int WCPX = Sh::WCX / 2;
     extern __shared__ uint32_t smem[];
     char* const xl = reinterpret_cast<char*>(smem);   // [CS] planes of CHPX bytes: [slot][row][column]
     char* const gl = xl + Sh::XB;                     // two copies of [CS] planes of CHPG bytes
@@ -117,8 +124,9 @@ __device__ __forceinline__ void dwconv_wgrad_tz_body(const T* __restrict__ x, co
     // item of a pass: (row pair 0..3, column pair, 8-channel piece h), h fastest
     const int ih = tid % NH;
     const bool chok = c0 + 8 * ih < g.C;
-    uint32_t xcol[2], gcol[2];
-    int xrp, grp, xdst, gdst;
+    uint32_t xcol[2], gcol[4];
+    int xrp, grow, xdst, gdst;
+    bool gact;
     {
         const int cp = (tid / NH) % WCPX, rp = tid / NH / WCPX;
         xrp = rp < 4 ? rp : -1;
@@ -129,13 +137,16 @@ __device__ __forceinline__ void dwconv_wgrad_tz_body(const T* __restrict__ x, co
         xdst = (8 * ih) * CHPX + ih * Sh::XHALF + (2 * min(rp, 3)) * RPX + 4 * cp;
     }
     {
-        const int cp = (tid / NH) % WCPG, rp = tid / NH / WCPG;
-        grp = rp < 4 ? rp : -1;
-        const int jc = 2 * cp - 8;   // column relative to j0: the band's own columns are 0 .. cols_valid-1
-        const bool any = chok && rp < 4;
-        gcol[0] = any && jc >= 0 && jc < cols_valid ? (uint32_t)((j0 + jc) * g.C + c0 + 8 * ih) * 2u : kNoCol;
-        gcol[1] = any && jc + 1 >= 0 && jc + 1 < cols_valid ? (uint32_t)((j0 + jc + 1) * g.C + c0 + 8 * ih) * 2u : kNoCol;
-        gdst = (8 * ih) * CHPG + (2 * (min(rp, 3) & 1)) * RPG + 4 * cp;   // within the row group (rp >> 1) of the pass
+        grow = wv * Sh::GRPW + lane / Sh::GLPR;          // row of the pass
+        const int q = (lane % Sh::GLPR) / NH;            // columns 4 q .. 4 q + 3 of the window
+        gact = chok && lane < Sh::GRPW * Sh::GLPR && grow < 8;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int jc = 4 * q + p - 8;   // column relative to j0: the band's own columns are 0 .. cols_valid-1
+            gcol[p] = gact && jc >= 0 && jc < cols_valid ? (uint32_t)((j0 + jc) * g.C + c0 + 8 * ih) * 2u : kNoCol;
+        }
+        grow = min(grow, 7);
+        gdst = (8 * ih) * CHPG + (grow & 3) * RPG + 8 * q;   // within the row group (grow >> 2) of the pass
     }
     uint4 bx[2][4], bg[2][4];
     auto issue_x = [&](uint4 (&bf)[4], int pass) {   // xw rows 8 pass .. 8 pass + 7 (window row 0 = x row i0 - PH)
@@ -150,13 +161,10 @@ __device__ __forceinline__ void dwconv_wgrad_tz_body(const T* __restrict__ x, co
         bf[3] = bload(xrsrc, r1 + xcol[1]);
     };
     auto issue_g = [&](uint4 (&bf)[4], int pass) {   // gy rows i0 + 8 pass .. + 7, the band's own rows only
-        const int wr = 8 * pass + 2 * max(grp, 0);
+        const int wr = 8 * pass + grow;
         const uint32_t r0 = wr < rows_valid ? (uint32_t)((i0 + wr) * g.OW * g.C) * 2u : kNoRow;
-        const uint32_t r1 = wr + 1 < rows_valid ? (uint32_t)((i0 + wr + 1) * g.OW * g.C) * 2u : kNoRow;
-        bf[0] = bload(grsrc, r0 + gcol[0]);
-        bf[1] = bload(grsrc, r0 + gcol[1]);
-        bf[2] = bload(grsrc, r1 + gcol[0]);
-        bf[3] = bload(grsrc, r1 + gcol[1]);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) bf[p] = bload(grsrc, r0 + gcol[p]);   // lanes without an item read zeros
     };
     auto commit_x = [&](const uint4 (&bf)[4], int pass) {
         if (xrp < 0) return;
@@ -171,35 +179,33 @@ __device__ __forceinline__ void dwconv_wgrad_tz_body(const T* __restrict__ x, co
             *reinterpret_cast<uint32_t*>(dst + (2 * j + 1) * CHPX + RPX) = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
         }
     };
-    const bool gfirst = (tid / NH) % WCPG == 0;  // the item's first column is the window's first: nothing to its left
+    // the value of the lane NH up (the next item of the row; zeros behind the row's last item: no item or no column)
+    auto from_right = [&](uint32_t v) {
+        static_assert(NH == 2, "two single-lane wavefront shifts");
+        v = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x130, 0xf, 0xf, true);   // wave_shl:1: lane i takes lane i + 1
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x130, 0xf, 0xf, true);
+    };
     auto commit_g = [&](const uint4 (&bf)[4], int pass, int half) {   // half 0 / 1: one row group of the pass; -1: both
-        if (grp < 0 || (half >= 0 && (grp >> 1) != half)) return;
         const uint32_t a0[4] = {bf[0].x, bf[0].y, bf[0].z, bf[0].w}, a1[4] = {bf[1].x, bf[1].y, bf[1].z, bf[1].w};
         const uint32_t a2[4] = {bf[2].x, bf[2].y, bf[2].z, bf[2].w}, a3[4] = {bf[3].x, bf[3].y, bf[3].z, bf[3].w};
-        char* dst = gl + gdst + ((2 * pass + (grp >> 1)) % NSG) * GBG;
+        uint32_t a4[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t p00 = __builtin_amdgcn_perm(a1[j], a0[j], 0x05040100u), p01 = __builtin_amdgcn_perm(a1[j], a0[j], 0x07060302u);
-            const uint32_t p10 = __builtin_amdgcn_perm(a3[j], a2[j], 0x05040100u), p11 = __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u);
+        for (int j = 0; j < 4; ++j) a4[j] = from_right(a0[j]);   // every lane takes part in the shift
+        if (!gact || (half >= 0 && (grow >> 2) != half)) return;
+        char* dst = gl + gdst + ((2 * pass + (grow >> 2)) % NSG) * GBG;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {   // channels 2 j (low halves) and 2 j + 1 (high halves) of the piece
             char* d0 = dst + (2 * j) * CHPG;
             char* d1 = dst + (2 * j + 1) * CHPG;
-            *reinterpret_cast<uint32_t*>(d0) = p00;
-            *reinterpret_cast<uint32_t*>(d1) = p01;
-            *reinterpret_cast<uint32_t*>(d0 + RPG) = p10;
-            *reinterpret_cast<uint32_t*>(d1 + RPG) = p11;
-            // second copy, one element to the left: column c goes to index c - 1
-            char* e0 = d0 + Sh::GCB;
-            char* e1 = d1 + Sh::GCB;
-            *reinterpret_cast<unsigned short*>(e0) = (unsigned short)(p00 >> 16);
-            *reinterpret_cast<unsigned short*>(e1) = (unsigned short)(p01 >> 16);
-            *reinterpret_cast<unsigned short*>(e0 + RPG) = (unsigned short)(p10 >> 16);
-            *reinterpret_cast<unsigned short*>(e1 + RPG) = (unsigned short)(p11 >> 16);
-            if (!gfirst) {
-                *reinterpret_cast<unsigned short*>(e0 - 2) = (unsigned short)(p00 & 0xffffu);
-                *reinterpret_cast<unsigned short*>(e1 - 2) = (unsigned short)(p01 & 0xffffu);
-                *reinterpret_cast<unsigned short*>(e0 + RPG - 2) = (unsigned short)(p10 & 0xffffu);
-                *reinterpret_cast<unsigned short*>(e1 + RPG - 2) = (unsigned short)(p11 & 0xffffu);
-            }
+            *reinterpret_cast<uint2*>(d0) = make_uint2(__builtin_amdgcn_perm(a1[j], a0[j], 0x05040100u),
+                                                       __builtin_amdgcn_perm(a3[j], a2[j], 0x05040100u));
+            *reinterpret_cast<uint2*>(d1) = make_uint2(__builtin_amdgcn_perm(a1[j], a0[j], 0x07060302u),
+                                                       __builtin_amdgcn_perm(a3[j], a2[j], 0x07060302u));
+            // second copy, one element to the left: column c goes to index c - 1 (columns 4 q + 1 .. 4 q + 4 here)
+            *reinterpret_cast<uint2*>(d0 + Sh::GCB) = make_uint2(__builtin_amdgcn_perm(a2[j], a1[j], 0x05040100u),
+                                                                 __builtin_amdgcn_perm(a4[j], a3[j], 0x05040100u));
+            *reinterpret_cast<uint2*>(d1 + Sh::GCB) = make_uint2(__builtin_amdgcn_perm(a2[j], a1[j], 0x07060302u),
+                                                                 __builtin_amdgcn_perm(a4[j], a3[j], 0x07060302u));
         }
     };
     issue_x(bx[0], 0);
