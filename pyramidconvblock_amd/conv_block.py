@@ -21,7 +21,8 @@ from torch import nn
 from torch.nn import functional as F
 
 from . import _lib, ops
-from .dwconv import OptimizedDepthwiseConv2d, dwconv_dgrad, dwconv_forward, dwconv_wgrad, dwconv_wgrad_pair
+from .dwconv import (OptimizedDepthwiseConv2d, dwconv_bwd3, dwconv_dgrad, dwconv_forward, dwconv_wgrad,
+                     dwconv_wgrad_pair)
 
 
 class GateFunction(torch.autograd.Function):
@@ -347,8 +348,24 @@ class ConvBlockFunction(torch.autograd.Function):
             srcs = [pooled[i] if scales[i] != 1. else a for i in range(ns)]
             if (gcs is not None and ns == 2 and w_dw[0].shape == w_dw[1].shape and w_dw[0].shape[0] == w_dw[0].shape[1]
                     and w_dw[0].shape[0] % 2 == 1 and all(t.is_contiguous() and t.dtype == dt for t in (*srcs, *gcs))):
-                # the weight gradients of both scales in one launch (the smaller problem fills the larger one's tail)
-                grad_w_dw[0], grad_w_dw[1] = dwconv_wgrad_pair(srcs[0], gcs[0], srcs[1], gcs[1], w_dw[0].shape)
+                k = w_dw[0].shape[0]
+                fused = None
+                if tuple(srcs[1].shape) == (B, H // 2, W // 2, I) and H % 2 == 0 and W % 2 == 0 and scales[0] == 1.:
+                    # the launches of pdw_convblock_bwd: the half scale's input gradient, then the full scale's (which
+                    # adds it) and both weight gradients as one launch
+                    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+                    ws = [w.detach().to(dt).contiguous() for w in w_dw]
+                    dxp = dwconv_dgrad(gcs[1], ws[1], srcs[1].shape, *geo)
+                    fused = dwconv_bwd3(gcs[0], ws[0], dxp, srcs[0], srcs[1], gcs[1])
+                    if fused is None:
+                        waiting.append(dxp)
+                        order = [i for i in order if i != 1]
+                if fused is not None:
+                    da, grad_w_dw[0], grad_w_dw[1] = fused
+                    order = []
+                else:
+                    # the weight gradients of both scales in one launch (the smaller problem fills the larger one's tail)
+                    grad_w_dw[0], grad_w_dw[1] = dwconv_wgrad_pair(srcs[0], gcs[0], srcs[1], gcs[1], w_dw[0].shape)
             for i in order:
                 s = scales[i]
                 w = w_dw[i].detach().to(dt).contiguous()

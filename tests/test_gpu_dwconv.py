@@ -136,8 +136,11 @@ def test_wgrad_pair_is_the_two_separate_calls(dtype, case):
                                   (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7)])
 def test_bwd3_is_the_three_separate_calls(dtype, case):
     """pdw_dwconv_bwd3 (the full scale's input gradient with the pooled branch's added and the weight gradients of
-    both scales in one launch) gives bitwise the results of the three separate calls, immediately and with the
-    summations deferred; where the fused kernel does not cover the case it says so and launches nothing."""
+    both scales in one launch) gives the results of the three separate calls: the input gradient bitwise, the weight
+    gradients up to the order of the fp32 summation (the launch cuts the images into fewer, taller bands, so its
+    partial sums are other ones: a difference of one rounding of the result at most), and bitwise the same whether the
+    summations run at once or deferred; where the fused kernel does not cover the case it says so and launches
+    nothing."""
     from pyramidconvblock_amd import _lib
     from pyramidconvblock_amd.dwconv import dwconv_bwd3, dwconv_dgrad, dwconv_wgrad
 
@@ -157,8 +160,14 @@ def test_bwd3_is_the_three_separate_calls(dtype, case):
     with _lib.deferred_reductions(gy0.device):
         later = dwconv_bwd3(gy0, w0, gp, x0, x1, gy1)
     torch.cuda.synchronize()
+    assert torch.equal(want[0], got[0])
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     for w, g, l in zip(want, got, later):
-        assert torch.equal(w, g) and torch.equal(w, l)
+        assert torch.equal(g, l)
+        w, g = w.float(), g.float()
+        # one unit in the last place of the larger value, plus the fp32 rounding of sums of B * H * W products
+        tol = 2 * ulp * torch.maximum(w.abs(), g.abs()) + 1e-5 * (B * H * W) ** 0.5
+        assert bool(((w - g).abs() <= tol).all()), float((w - g).abs().max())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
