@@ -169,6 +169,17 @@ int pdw_dwconv_bwd3(const void *gy0, const void *w0, const void *gp, void *dx, c
                     void *workspace1, size_t workspace1_bytes, int B, int H, int W, int C, int K, int dtype,
                     void *stream);
 
+/* The forward convolutions of both scales of a two-scale block as one launch (conv_block.py:14-16 at scales 1 and
+ * 1/2): y0 = conv(x0, w0) on [B,H,W,C] and y1 = conv(x1, w1) on [B,H/2,W/2,C], x1 being an input (the caller's 2x2
+ * average pool of x0, pdw_avgpool_fwd).  Square odd filter, stride 1, padding K/2, even H and W.  Status 3 (nothing
+ * launched) when the fused kernel does not cover the case (fp32, C % 8, images narrower than 33 columns;
+ * pdw_dwconv_fwd2_supported says so beforehand, so that a caller can have the full scale's convolution write the pool
+ * instead: pdw_dwconv_fwd_pool): the caller then makes two pdw_dwconv_fwd calls.  Results are bitwise those of the
+ * separate calls. */
+int pdw_dwconv_fwd2_supported(int B, int H, int W, int C, int K, int dtype); /* 1: pdw_dwconv_fwd2 takes the case */
+int pdw_dwconv_fwd2(const void *x0, const void *w0, void *y0, const void *x1, const void *w1, void *y1, int B, int H,
+                    int W, int C, int K, int dtype, void *stream);
+
 /* Adaptive average pooling x[B,H,W,C] -> y[B,h,w,C]; bin i covers [floor(i*H/h), ceil((i+1)*H/h)).
  * Replaces F.adaptive_avg_pool2d at conv_block.py:16 and the launch at avgpool_triton.py:225-229
  * (kernel :14-107; integer bin arithmetic here instead of the fp16 one at :42-47). */
@@ -302,6 +313,15 @@ int pdw_dense_colsum_supported(int K, int NO, int dtype);
 int pdw_dense_colsum_rows(void);
 int pdw_dense_fwd_colsum(const void *x, const void *w, int w_kmajor, const void *bias, const float *rowbias, void *y,
                          float *colsum, long long N, int K, int NO, int P, int dtype, void *stream);
+
+/* pdw_dense_fwd_colsum for the pixels of x[B,H,W,K] (no rowbias) that also writes the 2x2 average pool of y,
+ * pool[B,H/2,W/2,NO] = what pdw_avgpool_fwd makes of y (conv_block.py:37 together with the pooling of conv_block.py:16
+ * for the second scale: the convolutions of both scales can then start together, pdw_dwconv_fwd2).  The kernel's row
+ * tiles are blocks of 4 image rows x 8 columns, so colsum[t] are the sums of x over such blocks (still H*W/32 per
+ * image, image after image).  Status 3 (nothing launched) where not covered: 16-bit types, K = 128, NO = 64, H % 4 == 0,
+ * W % 8 == 0 only. */
+int pdw_dense_fwd_colsum_pool(const void *x, const void *w, const void *bias, void *y, float *colsum, void *pool, int B,
+                              int H, int W, int K, int NO, int dtype, void *stream);
 
 /* Weight gradient of such a layer: dw[m,o] = sum_n a[n,m] * b[n,o]  (a[N,M], b[N,NO] -> dw[M,NO]), fp32
  * accumulation, two deterministic passes through `workspace` (no atomics). */

@@ -21,8 +21,8 @@ from torch import nn
 from torch.nn import functional as F
 
 from . import _lib, ops
-from .dwconv import (OptimizedDepthwiseConv2d, dwconv_bwd3, dwconv_dgrad, dwconv_forward, dwconv_wgrad,
-                     dwconv_wgrad_pair)
+from .dwconv import (OptimizedDepthwiseConv2d, dwconv_bwd3, dwconv_dgrad, dwconv_forward, dwconv_forward2,
+                     dwconv_wgrad, dwconv_wgrad_pair)
 
 
 class GateFunction(torch.autograd.Function):
@@ -199,7 +199,16 @@ class ConvBlockFunction(torch.autograd.Function):
         same_dt = w_pool.dtype == dt and all(b is None or b.dtype == dt for b in (b_pool, b_out))
         # the per-image sums of x that the mean branch needs are taken by conv_up's kernel while it reads x
         xparts = None
-        if fast_up and same_dt and B > 0 and ops.dense_colsum_supported(D, I, dt, H * W):
+        xp_ready = None   # the second scale's input, where conv_up's kernel pools its own result
+        two = (_is_pair(scales) and B > 0 and scales[1] == 0.5 and H % 2 == 0 and W % 2 == 0 and len(w_dw) == 2
+               and w_dw[0].shape == w_dw[1].shape and w_dw[0].shape[0] == w_dw[0].shape[1] and x.is_cuda
+               and dt != torch.float32
+               and bool(_lib.lib().pdw_dwconv_fwd2_supported(B, H, W, I, w_dw[0].shape[0], _lib.dtype_code(dt))))
+        fused_up = ops.dense_forward_pool(x, w_up.detach().contiguous(), bias=b_up) if (
+            two and fast_up and same_dt and b_up is None) else None
+        if fused_up is not None:
+            a, xparts, xp_ready = fused_up
+        elif fast_up and same_dt and B > 0 and ops.dense_colsum_supported(D, I, dt, H * W):
             a, xparts = ops.dense_forward(x, w_up.detach().contiguous(), bias=b_up, colsum=True)
         else:
             a = ops.dense_forward(x, w_up.detach().contiguous(), bias=b_up) if fast_up else F.linear(x, w_up, b_up)
@@ -209,7 +218,17 @@ class ConvBlockFunction(torch.autograd.Function):
         convs, pooled = [], []
         pair = _is_pair(scales)           # scales (1, s): both gates go into cat in one launch
         ready = None                      # pooled input already produced by the full-resolution conv's kernel
-        for i, s in enumerate(scales):
+        both = None
+        if two:
+            # the launches of pdw_convblock_fwd: the second scale's input, then both convolutions as one launch
+            ws = [w.detach().to(dt).contiguous() for w in w_dw]
+            xp = xp_ready if xp_ready is not None else ops.avgpool_forward(a, (H // 2, W // 2))
+            both = dwconv_forward2(a, ws[0], xp, ws[1])
+            if both is not None:
+                convs, pooled = [both[0], both[1]], [None, xp]
+            else:
+                ready = xp
+        for i, s in enumerate(scales if both is None else ()):
             w = w_dw[i].detach().to(dt).contiguous()
             k1, k2 = w.shape[0], w.shape[1]
             geo = ((1, 1), (k1 // 2, k2 // 2), (1, 1))
@@ -222,7 +241,7 @@ class ConvBlockFunction(torch.autograd.Function):
                     ops.gate_bilinear_forward(c, (H, W), out=dst)
             else:
                 p = None
-                if pair and B > 0:   # the conv reads `a` anyway: it also writes the next scale's pooled input
+                if pair and B > 0 and ready is None:   # the conv reads `a` anyway: it also writes the next scale's pooled input
                     c, ready = dwconv_forward(a, w, *geo, pool_to=(int(H * scales[1]), int(W * scales[1])))
                 else:
                     c = dwconv_forward(a, w, *geo)

@@ -292,6 +292,23 @@ int pdw_dwconv_bwd3(const void* gy0, const void* w0, const void* gp, void* dx, c
     return r;
 }
 
+int pdw_dwconv_fwd2_supported(int B, int H, int W, int C, int K, int dtype) {
+    return valid_dtype(dtype) && dwconv_fwd2_covers(B, H, W, C, K, dtype) ? 1 : 0;
+}
+
+int pdw_dwconv_fwd2(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H, int W,
+                    int C, int K, int dtype, void* stream) {
+    const int P = K / 2;
+    if (!(K & 1)) return set_error("pdw_dwconv_fwd2: odd filter size needed (K=%d)", K), 1;
+    if ((H & 1) || (W & 1)) return set_error("pdw_dwconv_fwd2: even extents needed (H=%d W=%d)", H, W), 1;
+    if (int e = check_conv("pdw_dwconv_fwd2", x0, w0, y0, B, H, W, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (int e = check_conv("pdw_dwconv_fwd2", x1, w1, y1, B, H / 2, W / 2, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (B == 0) return 0;
+    const int r = dwconv_fwd2_launch(x0, w0, y0, x1, w1, y1, B, H, W, C, K, dtype, (hipStream_t)stream);
+    if (r == -1) return set_error("pdw_dwconv_fwd2: case not covered (B=%d H=%d W=%d C=%d K=%d dtype=%d)", B, H, W, C, K, dtype), 3;
+    return r;
+}
+
 int pdw_avgpool_fwd(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
     if (int e = check_resample("pdw_avgpool_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
     return avgpool_fwd_launch(x, y, B, H, W, C, h, w, dtype, (hipStream_t)stream);
@@ -537,6 +554,20 @@ int pdw_dense_fwd_colsum(const void* x, const void* w, int w_kmajor, const void*
     if (r == -1)
         return set_error("pdw_dense_fwd_colsum: K=%d NO=%d dtype=%d not supported (see pdw_dense_colsum_supported)", K,
                          NO, dtype), 3;
+    return r;
+}
+
+int pdw_dense_fwd_colsum_pool(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
+                              int H, int W, int K, int NO, int dtype, void* stream) {
+    if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd_colsum_pool: unknown dtype %d", dtype), 1;
+    if (B < 0 || H < 2 || W < 2 || (H & 1) || (W & 1) || K < 1 || NO < 1)
+        return set_error("pdw_dense_fwd_colsum_pool: bad extents B=%d H=%d W=%d K=%d NO=%d", B, H, W, K, NO), 1;
+    if (B > 0 && (!x || !w || !y || !colsum || !pool)) return set_error("pdw_dense_fwd_colsum_pool: null pointer"), 1;
+    if (B == 0) return 0;
+    const int r = dense_rows_pool_launch(x, w, bias, y, colsum, pool, B, H, W, K, NO, dtype, (hipStream_t)stream);
+    if (r == -1)
+        return set_error("pdw_dense_fwd_colsum_pool: case not covered (B=%d H=%d W=%d K=%d NO=%d dtype=%d)", B, H, W, K, NO,
+                         dtype), 3;
     return r;
 }
 

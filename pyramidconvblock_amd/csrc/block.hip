@@ -82,11 +82,30 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
     float* yp = (float*)ws.take((size_t)B * D * 4);         // mean branch: one row per image
     const int pad = K / 2;
     // conv_up, with the tile sums of x for the mean branch                                   (conv_block.py:37, 46)
-    if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) return e;
-    // full-resolution conv, which also pools its input for the second scale                  (conv_block.py:14-16)
-    if (int e = pdw_dwconv_fwd_pool(a, w_dw0, c0, xp, B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, s.h, s.w, dtype, stream))
+    // (where the layer's kernel can also pool its result for the second scale, the convolutions need no pooling launch)
+    const bool two = pdw_dwconv_fwd2_supported(B, H, W, I, K, dtype) != 0;
+    int pooled = 3;
+    if (two) {
+        pooled = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream);
+        if (pooled != 0 && pooled != 3) return pooled;
+    }
+    if (pooled == 3)
+        if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) return e;
+    // the second scale's input, then the convolutions of both scales as one launch; where that launch does not take the
+    // shape, the full-resolution conv also pools its input and the second scale's follows   (conv_block.py:14-16)
+    int both = 3;
+    if (two) {
+        if (pooled == 3)
+            if (int e = pdw_avgpool_fwd(a, xp, B, H, W, I, s.h, s.w, dtype, stream)) return e;
+        both = pdw_dwconv_fwd2(a, w_dw0, c0, xp, w_dw1, c1, B, H, W, I, K, dtype, stream);
+        if (both != 0 && both != 3) return both;
+        if (both == 3)
+            if (int e = pdw_dwconv_fwd(a, w_dw0, c0, B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream)) return e;
+    } else if (int e = pdw_dwconv_fwd_pool(a, w_dw0, c0, xp, B, H, W, I, K, K, 1, 1, pad, pad, 1, 1, s.h, s.w, dtype, stream)) {
         return e;
-    if (int e = pdw_dwconv_fwd(xp, w_dw1, c1, B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream)) return e;
+    }
+    if (both == 3)
+        if (int e = pdw_dwconv_fwd(xp, w_dw1, c1, B, s.h, s.w, I, K, K, 1, 1, pad, pad, 1, 1, dtype, stream)) return e;
     // both gates into cat, mean -> conv_pool (+ both biases) into yp                          (conv_block.py:40-49)
     if (int e = pdw_block_mid_fwd(c0, c1, cat, B, H, W, s.h, s.w, I, I, xparts, (int)(s.nt / B), w_pool, b_pool, b_out, m,
                                   yp, s.P, D, dtype, stream))

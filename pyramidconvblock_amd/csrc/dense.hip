@@ -145,13 +145,28 @@ struct WTransposer {
 // With both fixed (and then K % 16 == 0, NO % 32 == 0) a full tile is whole passes of 64 chunks in and out and
 // whole MFMA steps, and its code has no per-lane predicates and no loop bounds to test: those were a third of the
 // generic kernel's vector-ALU work.
-template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0>
+//
+// POOL (SK = 128, SNO = 64; rows are the pixels of [B, Himg, Wimg] images, Himg % 4 == 0, Wimg % 8 == 0, no rowbias): a
+// tile is a block of 4 image rows x 8 columns instead of 32 consecutive pixels (a load or store instruction still
+// covers 1 KB of consecutive bytes: 4 pixels of K values, 8 pixels of NO), so that it holds 2 x 4 whole windows of
+// the 2x2 average pool of Y, which the kernel writes to `pool` [B, Himg/2, Wimg/2, NO] from the result tile in LDS:
+// (((y00 + y01) + y10) + y11) / 4 in fp32 of the rounded results, as the pooling kernel computes it.
+template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0, bool POOL = false>
 __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T* __restrict__ W,
                                                 const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                 T* __restrict__ Y, float* __restrict__ colsum, long long N, int Kd,
                                                 int NOd, int P, int nktd, int nntd, int bid, int nblocks,
-                                                uint32_t* dsm) {
+                                                uint32_t* dsm, T* __restrict__ pool = nullptr, int Himg = 0,
+                                                int Wimg = 0) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
+    static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
+    // first pixel of tile t (POOL)
+    auto tile_pixel = [&](long long t, int& b, int& rb, int& cb) {
+        const int tw = Wimg >> 3, tpi = (Himg >> 2) * tw;
+        b = (int)(t / tpi);
+        const int r = (int)(t - (long long)b * tpi);
+        rb = r / tw, cb = r - rb * tw;
+    };
     static_assert(!STATIC || (SK % 16 == 0 && SNO % 32 == 0 && SK <= 128 && SNO <= 128), "static dense shape");
     const int K = STATIC ? SK : Kd, NO = STATIC ? SNO : NOd;
     const int nkt = STATIC ? SK / 16 : nktd, nnt = STATIC ? SNO / 32 : nntd;
@@ -186,7 +201,14 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
         const T* base = X + t * 32 * K;
         const long long rows_left = N - t * 32;         // rows of this tile that exist
-        if (STATIC && rows_left >= 32) {
+        if constexpr (POOL) {
+            int b, rb, cb;
+            tile_pixel(t, b, rb, cb);
+            base = X + (((long long)b * Himg + 4 * rb) * Wimg + 8 * cb) * K;
+#pragma unroll
+            for (int i = 0; i < LP; ++i)   // chunks i*64 .. of the tile: its pixels 4 i .. 4 i + 3 = image row i / 2, 4 columns
+                raw[i] = *reinterpret_cast<const Frag*>(base + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * K + lane * 8);
+        } else if (STATIC && rows_left >= 32) {
 #pragma unroll
             for (int i = 0; i < LP; ++i) {
                 if (i * 64 < nin)
@@ -397,7 +419,36 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         {
             const long long rows_left = N - tile * 32;
             T* yb = Y + tile * 32 * NO;
-            if (STATIC && rows_left >= 32) {  // (an array of its own: one array written on both paths ends up in scratch)
+            if constexpr (POOL) {
+                int b, rb, cb;
+                tile_pixel(tile, b, rb, cb);
+                yb = Y + (((long long)b * Himg + 4 * rb) * Wimg + 8 * cb) * NO;
+                Frag of[LO];
+#pragma unroll
+                for (int i = 0; i < LO; ++i)
+                    if (i * 64 < 32 * cpr) of[i] = *reinterpret_cast<const Frag*>(tl + oout[i]);
+                // the lane's window of the pool (2 x 4 per tile) and 8 of its features
+                const int wr = lane >> 5, wc = (lane >> 3) & 3, ch = (lane & 7) * 8;
+                const T* p00 = tl + (16 * wr + 2 * wc) * ldt + ch;
+                const Frag q00 = *reinterpret_cast<const Frag*>(p00), q01 = *reinterpret_cast<const Frag*>(p00 + ldt);
+                const Frag q10 = *reinterpret_cast<const Frag*>(p00 + 8 * ldt), q11 = *reinterpret_cast<const Frag*>(p00 + 9 * ldt);
+#pragma unroll
+                for (int i = 0; i < LO; ++i)   // chunks i*64 .. = image row i of the tile, 8 pixels
+                    if (i * 64 < 32 * cpr) *reinterpret_cast<Frag*>(yb + (long long)i * Wimg * NO + lane * 8) = of[i];
+                Frag o;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float lo = (((half_to_f32<T>(q00.v[j] & 0xffffu) + half_to_f32<T>(q01.v[j] & 0xffffu)) +
+                                       half_to_f32<T>(q10.v[j] & 0xffffu)) + half_to_f32<T>(q11.v[j] & 0xffffu)) * 0.25f;
+                    const float hi = (((half_to_f32<T>(q00.v[j] >> 16) + half_to_f32<T>(q01.v[j] >> 16)) +
+                                       half_to_f32<T>(q10.v[j] >> 16)) + half_to_f32<T>(q11.v[j] >> 16)) * 0.25f;
+                    ChanVec<T, 2> pv;
+                    pv.v[0] = from_f32<T>(lo), pv.v[1] = from_f32<T>(hi);
+                    o.v[j] = *reinterpret_cast<const uint32_t*>(&pv);
+                }
+                T* pb = pool + ((((long long)b * (Himg >> 1) + 2 * rb + wr) * (Wimg >> 1)) + 4 * cb + wc) * NO + ch;
+                *reinterpret_cast<Frag*>(pb) = o;
+            } else if (STATIC && rows_left >= 32) {  // (an array of its own: one array written on both paths ends up in scratch)
                 Frag of[LO];
 #pragma unroll
                 for (int i = 0; i < LO; ++i)
@@ -434,6 +485,18 @@ __global__ __launch_bounds__(256, 2) void dense_rows_k(const T* __restrict__ X, 
     extern __shared__ uint32_t dsm[];
     dense_rows_body<T, KMAJOR, COLSUM, SK, SNO>(X, W, bias, rowbias, Y, colsum, N, K, NO, P, nkt, nnt, blockIdx.x,
                                                 gridDim.x, dsm);
+}
+
+// The 128 -> 64 layer over the pixels of [B, Himg, Wimg] images with the tile sums of X and the 2x2 average pool of Y
+// (dense_rows_body, POOL).
+template <typename T>
+__global__ __launch_bounds__(256, 2) void dense_rows_pool_k(const T* __restrict__ X, const T* __restrict__ W,
+                                                         const T* __restrict__ bias, T* __restrict__ Y,
+                                                         float* __restrict__ colsum, T* __restrict__ pool, long long N,
+                                                         int Himg, int Wimg) {
+    extern __shared__ uint32_t dsm[];
+    dense_rows_body<T, false, true, 128, 64, true>(X, W, bias, nullptr, Y, colsum, N, 128, 64, 1, 8, 2, blockIdx.x,
+                                                   gridDim.x, dsm, pool, Himg, Wimg);
 }
 
 // The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
@@ -747,6 +810,32 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
 #undef PDW_GO_S
 #undef PDW_GO
     return check_launch("dense_rows");
+}
+
+// y = x W^T (+ bias) for the pixels of [B, H, W] images with K = 128 features in and NO = 64 out, the sums of x over
+// each 32-pixel tile (tiles of 4 rows x 8 columns here: still H * W / 32 per image, image after image) and the 2x2
+// average pool of y.  -1: not covered (other widths, extents that are not multiples of 4 x 8, fp32).
+int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
+                           int H, int W, int K, int NO, int dtype, hipStream_t s) {
+    if (dtype == kF32 || K != 128 || NO != 64 || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
+    if (tune_env("PDW_DENSE_GENERIC") || tune_env("PDW_NO_DENSE_POOL")) return -1;
+    const long long N = (long long)B * H * W;
+    if (N > 0x7fffffffLL) return -1;
+    for (const void* p : {x, w, (const void*)y, (const void*)colsum, (const void*)pool})
+        if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
+    if (reinterpret_cast<uintptr_t>(bias) & 7) return -1;
+    const long long ntiles = N / 32;
+    long long blocks = (ntiles + 3) / 4;
+    const int cap = tune_env("PDW_DENSE_BLOCKS") ? atoi(tune_env("PDW_DENSE_BLOCKS")) : 512;
+    if (blocks > cap) blocks = cap;
+    const size_t lds = ((size_t)2 * 32 * (128 + 8) + 4 * 32 * (128 + 8)) * 2 + (bias ? (size_t)4 * 2 * 2 * 32 * sizeof(float) : 0);
+    if (dtype == kF16)
+        hipLaunchKernelGGL(dense_rows_pool_k<f16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const f16_t*)x, (const f16_t*)w,
+                           (const f16_t*)bias, (f16_t*)y, colsum, (f16_t*)pool, N, H, W);
+    else
+        hipLaunchKernelGGL(dense_rows_pool_k<bf16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const bf16_t*)x,
+                           (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, colsum, (bf16_t*)pool, N, H, W);
+    return check_launch("dense_rows_pool");
 }
 
 static void dense_wgrad_plan(long long N, int* blocks, int* stages_per_block) {

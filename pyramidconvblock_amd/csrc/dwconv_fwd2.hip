@@ -1,0 +1,37 @@
+// Dispatch of the block's two forward convolution launches as one (dwconv_fwd2.h) by filter size.
+#include "common.h"
+#include "kernels.h"
+
+namespace pdw {
+
+#define PDW_FWD2_DECL(K)                                                                                              \
+    int dwconv_fwd2_k##K(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H, \
+                         int W, int C, int dtype, hipStream_t s);
+PDW_FWD2_DECL(3) PDW_FWD2_DECL(5) PDW_FWD2_DECL(7) PDW_FWD2_DECL(9) PDW_FWD2_DECL(11) PDW_FWD2_DECL(13) PDW_FWD2_DECL(15)
+PDW_FWD2_DECL(17)
+#undef PDW_FWD2_DECL
+
+// Whether dwconv_fwd2_launch takes the case (aligned tensors assumed): what a caller checks before it pools the
+// input with a launch of its own instead of letting the full scale's convolution write the pool.
+bool dwconv_fwd2_covers(int B, int H, int W, int C, int K, int dtype) {
+    if (tune_env("PDW_NO_FWD2")) return false;
+    if (dtype == kF32 || K < 3 || K > 17 || !(K & 1) || C % 8 != 0 || (H & 1) || (W & 1) || B < 1 || H < 2 || W < 2) return false;
+    const long long pad16 = (long long)cdiv(W, 64) * 64 * B, pad8 = (long long)cdiv(W, 32) * 32 * cdiv(B, 2) * 2;
+    return pad16 <= pad8 && (long long)H * W * C * 2 <= 0x1fffffffLL;
+}
+
+// -1: not covered (the caller makes the two launches).
+int dwconv_fwd2_launch(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
+                       int W, int C, int K, int dtype, hipStream_t s) {
+    if (tune_env("PDW_NO_FWD2")) return -1;
+    switch (K) {
+#define PDW_FWD2_CASE(KK) \
+    case KK: return dwconv_fwd2_k##KK(x0, w0, y0, x1, w1, y1, B, H, W, C, dtype, s);
+        PDW_FWD2_CASE(3) PDW_FWD2_CASE(5) PDW_FWD2_CASE(7) PDW_FWD2_CASE(9) PDW_FWD2_CASE(11) PDW_FWD2_CASE(13)
+        PDW_FWD2_CASE(15) PDW_FWD2_CASE(17)
+#undef PDW_FWD2_CASE
+        default: return -1;
+    }
+}
+
+}  // namespace pdw

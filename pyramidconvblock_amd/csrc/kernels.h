@@ -104,6 +104,10 @@ int dense_rows_supported(int K, int NO, int dtype);
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
                       long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum = nullptr,
                       const struct ReduceJobs* rider = nullptr);
+// the 128 -> 64 layer over the pixels of [B, H, W] images with the tile sums of x (tiles of 4 rows x 8 columns) and the
+// 2x2 average pool of y; -1 = not covered
+int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
+                           int H, int W, int K, int NO, int dtype, hipStream_t s);
 int dense_colsum_supported(int K, int NO, int dtype);
 int dense_colsum_rows();
 int dense_wgrad_supported(int M, int NO, int dtype);
@@ -121,5 +125,11 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
 int dwconv_bwd3_launch(const void* gyf, const void* w0, const void* addp, void* dx, const void* x0, void* dw0, void* ws0,
                        const void* x1, const void* gy1, void* dw1, void* ws1, int B, int H, int W, int C, int K, int dtype,
                        hipStream_t s);
+
+// dwconv_fwd2.hip: the forward convolutions of both scales of a two-scale block (the second at half the extents, its
+// own input) in one launch; -1 = not covered
+bool dwconv_fwd2_covers(int B, int H, int W, int C, int K, int dtype);
+int dwconv_fwd2_launch(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
+                       int W, int C, int K, int dtype, hipStream_t s);
 
 }  // namespace pdw

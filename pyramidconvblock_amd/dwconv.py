@@ -124,6 +124,28 @@ def dwconv_wgrad_pair(x0, gy0, x1, gy1, w_shape):
     return dws[0], dws[1]
 
 
+def dwconv_forward2(x0, w0, x1, w1):
+    """The 'same' convolutions of a two-scale block's two scales as one call of the library (pdw_dwconv_fwd2):
+    (conv(x0, w0), conv(x1, w1)) with one odd square filter shape and x1 at exactly half the extents of x0; None when
+    the fused kernel does not cover the case (the caller then makes the two calls)."""
+    dev = _lib.require_device(x0, w0, x1, w1)
+    L = _lib.lib()
+    K, C = int(w0.shape[0]), int(w0.shape[2])
+    B, H, W = x0.shape[0], x0.shape[1], x0.shape[2]
+    if (w0.shape[0] != w0.shape[1] or K % 2 == 0 or w1.shape != w0.shape or tuple(x1.shape) != (B, H // 2, W // 2, C)
+            or H % 2 or W % 2 or x0.shape[3] != C or any(t.dtype != x0.dtype for t in (w0, x1, w1)) or B == 0):
+        return None
+    args = [t.contiguous() for t in (x0, w0, x1, w1)]
+    y0, y1 = torch.empty_like(args[0]), torch.empty_like(args[2])
+    with _lib.on_device(dev):
+        st = L.pdw_dwconv_fwd2(args[0].data_ptr(), args[1].data_ptr(), y0.data_ptr(), args[2].data_ptr(), args[3].data_ptr(),
+                               y1.data_ptr(), B, H, W, C, K, _lib.dtype_code(x0.dtype), _lib.stream_ptr(dev))
+    if st == 3:
+        return None
+    _lib.check(st, "pdw_dwconv_fwd2")
+    return y0, y1
+
+
 def dwconv_bwd3(gy0, w0, gp, x0, x1, gy1):
     """The end of a two-scale block's backward pass as one call of the library (pdw_dwconv_bwd3): returns
     (dx, dw0, dw1) = (dwconv_dgrad(gy0, w0, pooled_grad=gp), dwconv_wgrad(x0, gy0), dwconv_wgrad(x1, gy1)) for 'same'

@@ -281,6 +281,31 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
     return y
 
 
+def dense_forward_pool(x, w, bias=None):
+    """x[B, H, W, K] -> (y, parts, pool): y = x W^T (+ bias), parts the fp32 sums of x over the kernel's 32-pixel tiles
+    (H * W / 32 per image) and pool the 2x2 average pool of y, in one launch (pdw_dense_fwd_colsum_pool); None where
+    the kernel does not cover the case."""
+    dev = _lib.require_device(x, w)
+    x, w, bias = _aligned(x), _aligned(w), _aligned(bias)
+    if x.dim() != 4 or not x.is_contiguous() or not w.is_contiguous() or w.dtype != x.dtype:
+        return None
+    B, H, W, K = x.shape
+    NO = w.shape[0]
+    if w.shape[1] != K or B == 0 or H % 2 or W % 2 or (bias is not None and bias.dtype != x.dtype):
+        return None
+    y = torch.empty((B, H, W, NO), device=dev, dtype=x.dtype)
+    parts = torch.empty((B * H * W // 32, K), device=dev, dtype=torch.float32)
+    pool = torch.empty((B, H // 2, W // 2, NO), device=dev, dtype=x.dtype)
+    with _lib.on_device(dev):
+        st = _lib.lib().pdw_dense_fwd_colsum_pool(x.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                                  y.data_ptr(), parts.data_ptr(), pool.data_ptr(), B, H, W, K, NO,
+                                                  _lib.dtype_code(x.dtype), _lib.stream_ptr(dev))
+    if st == 3:
+        return None
+    _lib.check(st, "pdw_dense_fwd_colsum_pool")
+    return y, parts, pool
+
+
 def dense_wgrad(a, b):
     """dw[m, o] = sum_n a[n, m] * b[n, o] over all leading dimensions; returns [M, NO] in a's dtype."""
     dev = _lib.require_device(a, b)

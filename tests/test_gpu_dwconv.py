@@ -133,6 +133,37 @@ def test_wgrad_pair_is_the_two_separate_calls(dtype, case):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", [(32, 56, 56, 64, 13), (8, 112, 112, 48, 17), (2, 40, 36, 32, 9), (3, 34, 70, 16, 3),
+                                  (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7), (5, 58, 66, 24, 5),
+                                  (64, 56, 56, 64, 11), (1, 130, 72, 16, 13)])
+def test_fwd2_is_the_two_separate_calls(dtype, case):
+    """pdw_dwconv_fwd2 (the convolutions of a block's two scales in one launch, with band heights of its own) gives
+    bitwise the results of the two separate calls; pdw_dwconv_fwd2_supported says beforehand whether it takes the
+    shape."""
+    from pyramidconvblock_amd import _lib
+    from pyramidconvblock_amd.dwconv import dwconv_forward, dwconv_forward2
+
+    B, H, W, C, k = case
+    gen = torch.Generator().manual_seed(17)
+    x0 = randn(gen, B, H, W, C).to(dtype).cuda()
+    x1 = randn(gen, B, H // 2, W // 2, C).to(dtype).cuda()
+    w0, w1 = ((randn(gen, k, k, C) / k).to(dtype).cuda() for _ in range(2))
+    geo = ((1, 1), (k // 2, k // 2), (1, 1))
+    got = dwconv_forward2(x0, w0, x1, w1)
+    # the full scale must be a shape for which the kernel's 64-column tile wastes no more than its 32-column one
+    wide = -(-W // 64) * 64 * B <= -(-W // 32) * 32 * (-(-B // 2) * 2)
+    covered = dtype != torch.float32 and C % 8 == 0 and wide
+    assert bool(_lib.lib().pdw_dwconv_fwd2_supported(B, H, W, C, k, _lib.dtype_code(dtype))) == covered
+    assert (got is not None) == covered
+    if got is None:
+        return
+    want = [dwconv_forward(x0, w0, *geo), dwconv_forward(x1, w1, *geo)]
+    torch.cuda.synchronize()
+    for w, g in zip(want, got):
+        assert torch.equal(w, g)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("case", [(32, 56, 56, 64, 13), (8, 112, 112, 48, 17), (2, 40, 36, 32, 9), (3, 34, 70, 16, 3),
                                   (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7)])
 def test_bwd3_is_the_three_separate_calls(dtype, case):
     """pdw_dwconv_bwd3 (the full scale's input gradient with the pooled branch's added and the weight gradients of

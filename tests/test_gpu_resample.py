@@ -263,6 +263,35 @@ def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
         assert_close(a, b.double().cpu().numpy(), dtype, what + " from parts")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("case", [(32, 56, 56, 128, 64), (3, 8, 16, 128, 64), (1, 4, 8, 128, 64), (2, 12, 40, 128, 64),
+                                  (2, 10, 16, 128, 64), (2, 8, 12, 128, 64), (2, 8, 16, 64, 32), (5, 36, 24, 128, 64)])
+def test_dense_forward_pool_is_the_layer_then_the_pool(dtype, case):
+    """pdw_dense_fwd_colsum_pool: the layer's result bitwise that of pdw_dense_fwd, its 2x2 average pool bitwise that of
+    pdw_avgpool_fwd on it, and per-image sums of x from the tile sums (tiles of 4 rows x 8 columns) equal to a float64
+    sum; where the kernel does not cover the case (other widths, extents off 4 x 8, fp32) it says so."""
+    from pyramidconvblock_amd import ops
+
+    B, H, W, K, NO = case
+    gen = torch.Generator().manual_seed(H + W)
+    x = randn(gen, B, H, W, K).to(dtype).cuda()
+    w = (randn(gen, NO, K) / 8).to(dtype).cuda()
+    got = ops.dense_forward_pool(x, w)
+    covered = dtype != torch.float32 and (K, NO) == (128, 64) and H % 4 == 0 and W % 8 == 0
+    assert (got is not None) == covered
+    if got is None:
+        return
+    y, parts, pool = got
+    assert torch.equal(y, ops.dense_forward(x, w))
+    assert torch.equal(pool, ops.avgpool_forward(y, (H // 2, W // 2)))
+    assert parts.shape == (B * H * W // 32, K)
+    ref = x.double().view(B, H * W, K).sum(1)
+    mine = parts.double().view(B, H * W // 32, K).sum(1)
+    assert (mine - ref).abs().max().item() <= 1e-5 * max(1.0, ref.abs().max().item())
+    blocks = x.double().view(B, H // 4, 4, W // 8, 8, K).sum((2, 4)).reshape(-1, K)
+    assert (parts.double() - blocks).abs().max().item() <= 1e-5 * max(1.0, blocks.abs().max().item())
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,hw,I,D", [(2, (8, 12), 32, 64), (3, (28, 28), 64, 128), (1, (4, 8), 16, 128)])
 def test_block_mid_matches_separate_launches(dtype, B, hw, I, D):
