@@ -382,7 +382,8 @@ def conv_rows(B, H, W, C, dtype, ks=(9, 13, 17)):
 
 def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     """Launches one hot kernel `iters` times at its shape inside the headline block (for rocprofv3 runs).
-    name: {fwd,dgrad,wgrad}_{full,half} | bwd3 (full-scale input gradient + both weight gradients, one launch) |
+    name: {fwd,dgrad,wgrad}_{full,half} | fwd2 (the forward convolutions of both scales, one launch) |
+    bwd3 (full-scale input gradient + both weight gradients, one launch) |
     conv128 (stand-alone forward at C = D) | avgpool_fwd | avgpool_bwd |
     bilinear_fwd | bilinear_bwd | dense_{fwd,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pair = both
     gradients in one launch) | step (whole forward+backward steps, eager) | copy"""
@@ -410,6 +411,11 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         x = torch.randn(B, H, W, D, device="cuda").to(dtype)
         wt = (torch.randn(k, k, D, device="cuda") / k).to(dtype)
         fn = lambda: dwconv.dwconv_forward(x, wt, *geo)
+    elif name == "fwd2":
+        xf = torch.randn(B, H, W, I, device="cuda").to(dtype)
+        xh = torch.randn(B, h, w, I, device="cuda").to(dtype)
+        wt, wt1 = ((torch.randn(k, k, I, device="cuda") / k).to(dtype) for _ in range(2))
+        fn = lambda: dwconv.dwconv_forward2(xf, wt, xh, wt1)
     elif name == "bwd3":
         gf, xf = (torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(2))
         gp, xh, gh = (torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(3))
@@ -515,7 +521,7 @@ def main():
     ap.add_argument("--no-configs", action="store_true", help="skip the rows of the other workloads")
     ap.add_argument("--no-torch-gpu", action="store_true", help="skip the torch-operator comparator on the GPU")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
-                    "{fwd,dgrad,wgrad}_{full,half}, bwd3, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
+                    "{fwd,dgrad,wgrad}_{full,half}, fwd2, bwd3, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
                     "dense_{fwd,dgrad,wgrad,pair}, step, copy")
     ap.add_argument("--torch-gpu-only", action="store_true", help="(internal) time the torch-operator comparator and exit")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")

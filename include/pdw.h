@@ -180,6 +180,13 @@ int pdw_dwconv_fwd2_supported(int B, int H, int W, int C, int K, int dtype); /* 
 int pdw_dwconv_fwd2(const void *x0, const void *w0, void *y0, const void *x1, const void *w1, void *y1, int B, int H,
                     int W, int C, int K, int dtype, void *stream);
 
+/* pdw_dwconv_fwd2 with the gate of pdw_dwconv_fwd_gate applied in the store of each scale (inference: neither
+ * convolution output reaches HBM): y0[b,i,j, ych0 + c] and y1[b,i,j, ych1 + c], c < C/2, at pixel strides of ldy0 / ldy1
+ * channels (0: C/2).  Covered where pdw_dwconv_fwd2 is and C % 16 == 0, K <= 13, strides and offsets multiples of 8;
+ * status 3 otherwise (the caller then makes two pdw_dwconv_fwd_gate calls).  Results bitwise those calls'. */
+int pdw_dwconv_fwd2_gate(const void *x0, const void *w0, void *y0, int ldy0, int ych0, const void *x1, const void *w1,
+                         void *y1, int ldy1, int ych1, int B, int H, int W, int C, int K, int dtype, void *stream);
+
 /* Adaptive average pooling x[B,H,W,C] -> y[B,h,w,C]; bin i covers [floor(i*H/h), ceil((i+1)*H/h)).
  * Replaces F.adaptive_avg_pool2d at conv_block.py:16 and the launch at avgpool_triton.py:225-229
  * (kernel :14-107; integer bin arithmetic here instead of the fp16 one at :42-47). */

@@ -309,6 +309,25 @@ int pdw_dwconv_fwd2(const void* x0, const void* w0, void* y0, const void* x1, co
     return r;
 }
 
+int pdw_dwconv_fwd2_gate(const void* x0, const void* w0, void* y0, int ldy0, int ych0, const void* x1, const void* w1,
+                         void* y1, int ldy1, int ych1, int B, int H, int W, int C, int K, int dtype, void* stream) {
+    const int P = K / 2;
+    if (!(K & 1)) return set_error("pdw_dwconv_fwd2_gate: odd filter size needed (K=%d)", K), 1;
+    if ((H & 1) || (W & 1)) return set_error("pdw_dwconv_fwd2_gate: even extents needed (H=%d W=%d)", H, W), 1;
+    if (int e = check_conv("pdw_dwconv_fwd2_gate", x0, w0, y0, B, H, W, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (int e = check_conv("pdw_dwconv_fwd2_gate", x1, w1, y1, B, H / 2, W / 2, C, K, K, 1, 1, P, P, 1, 1, dtype)) return e;
+    if (ldy0 == 0) ldy0 = C / 2;
+    if (ldy1 == 0) ldy1 = C / 2;
+    if ((C & 1) || ych0 < 0 || ych1 < 0 || ldy0 < ych0 + C / 2 || ldy1 < ych1 + C / 2)
+        return set_error("pdw_dwconv_fwd2_gate: need even C and ych + C/2 <= ldy (C=%d ldy=%d,%d ych=%d,%d)", C, ldy0, ldy1,
+                         ych0, ych1), 1;
+    if (B == 0) return 0;
+    const int r = dwconv_fwd2_launch(x0, w0, y0, x1, w1, y1, B, H, W, C, K, dtype, (hipStream_t)stream, ldy0, ych0, ldy1, ych1);
+    if (r == -1)
+        return set_error("pdw_dwconv_fwd2_gate: case not covered (B=%d H=%d W=%d C=%d K=%d dtype=%d)", B, H, W, C, K, dtype), 3;
+    return r;
+}
+
 int pdw_avgpool_fwd(const void* x, void* y, int B, int H, int W, int C, int h, int w, int dtype, void* stream) {
     if (int e = check_resample("pdw_avgpool_fwd", x, y, B, H, W, C, h, w, dtype)) return e;
     return avgpool_fwd_launch(x, y, B, H, W, C, h, w, dtype, (hipStream_t)stream);

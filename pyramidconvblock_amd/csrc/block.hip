@@ -160,15 +160,37 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
                                  up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4), B, H, W, D, I, K, dtype, stream);
     }
     void* g1 = ws.take(half / 2);
-    if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) return e;
-    // scale 1: conv + gate into cat[..., :G], and the pooled input of scale 1/2            (conv_block.py:14-19)
-    // (the convolution's staging threads hold whole pool windows only when the padding is even)
-    const bool pool_fused = (pad & 1) == 0;
-    if (int e = pdw_dwconv_fwd_gate(a, w_dw0, cat, pool_fused ? xp : nullptr, B, H, W, I, K, pad, I, 0, dtype, stream)) return e;
-    if (!pool_fused)
-        if (int e = pdw_avgpool_fwd(a, xp, B, H, W, I, s.h, s.w, dtype, stream)) return e;
-    // scale 1/2: conv + gate, upsampled into cat[..., G:]                                   (conv_block.py:17-21)
-    if (int e = pdw_dwconv_fwd_gate(xp, w_dw1, g1, nullptr, B, s.h, s.w, I, K, pad, G, 0, dtype, stream)) return e;
+    // conv_up; where its kernel can also pool its result, the gated convolutions of both scales follow as one launch
+    // (scale 1 into cat[..., :G], scale 1/2 into g1)                                        (conv_block.py:14-19, 37)
+    int both = 3;
+    if (pdw_dwconv_fwd2_supported(B, H, W, I, K, dtype)) {
+        const int pooled = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream);
+        if (pooled != 0 && pooled != 3) return pooled;
+        if (pooled == 0) {
+            both = pdw_dwconv_fwd2_gate(a, w_dw0, cat, I, 0, xp, w_dw1, g1, G, 0, B, H, W, I, K, dtype, stream);
+            if (both != 0 && both != 3) return both;
+        } else if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) {
+            return e;
+        }
+        if (both == 3 && pooled == 0) {   // the pool is there: the two gated convolutions one after the other
+            if (int e = pdw_dwconv_fwd_gate(a, w_dw0, cat, nullptr, B, H, W, I, K, pad, I, 0, dtype, stream)) return e;
+            if (int e = pdw_dwconv_fwd_gate(xp, w_dw1, g1, nullptr, B, s.h, s.w, I, K, pad, G, 0, dtype, stream)) return e;
+            both = 0;
+        }
+    } else if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) {
+        return e;
+    }
+    if (both == 3) {
+        // scale 1: conv + gate into cat[..., :G], and the pooled input of scale 1/2            (conv_block.py:14-19)
+        // (the convolution's staging threads hold whole pool windows only when the padding is even)
+        const bool pool_fused = (pad & 1) == 0;
+        if (int e = pdw_dwconv_fwd_gate(a, w_dw0, cat, pool_fused ? xp : nullptr, B, H, W, I, K, pad, I, 0, dtype, stream))
+            return e;
+        if (!pool_fused)
+            if (int e = pdw_avgpool_fwd(a, xp, B, H, W, I, s.h, s.w, dtype, stream)) return e;
+        // scale 1/2: conv + gate, upsampled into cat[..., G:]                                   (conv_block.py:17-21)
+        if (int e = pdw_dwconv_fwd_gate(xp, w_dw1, g1, nullptr, B, s.h, s.w, I, K, pad, G, 0, dtype, stream)) return e;
+    }
     // ... together with mean -> conv_pool (+ both biases) into yp                             (conv_block.py:46-49)
     if (int e = pdw_block_mid_infer(g1, (char*)cat + (size_t)G * s.es, B, H, W, s.h, s.w, G, I, xparts, (int)(s.nt / B),
                                     w_pool, b_pool, b_out, m, yp, s.P, D, dtype, stream))

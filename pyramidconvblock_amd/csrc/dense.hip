@@ -160,12 +160,14 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                                                 int Wimg = 0) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
     static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
-    // first pixel of tile t (POOL)
-    auto tile_pixel = [&](long long t, int& b, int& rb, int& cb) {
-        const int tw = Wimg >> 3, tpi = (Himg >> 2) * tw;
-        b = (int)(t / tpi);
-        const int r = (int)(t - (long long)b * tpi);
-        rb = r / tw, cb = r - rb * tw;
+    // POOL: first pixel of a tile and first pixel of its part of the pooled tensor (two 32-bit divisions per tile,
+    // taken once, when the tile is requested, and kept for its way out)
+    int px_next = 0, pp_next = 0, px_cur = 0, pp_cur = 0;
+    auto tile_pixel = [&](long long t) {
+        const unsigned tw = (unsigned)Wimg >> 3, tpi = ((unsigned)Himg >> 2) * tw;
+        const unsigned ti = (unsigned)t, b = ti / tpi, r = ti - b * tpi, rb = r / tw, cb = r - rb * tw;
+        px_next = (int)((b * (unsigned)Himg + 4 * rb) * (unsigned)Wimg + 8 * cb);
+        pp_next = (int)((b * ((unsigned)Himg >> 1) + 2 * rb) * ((unsigned)Wimg >> 1) + 4 * cb);
     };
     static_assert(!STATIC || (SK % 16 == 0 && SNO % 32 == 0 && SK <= 128 && SNO <= 128), "static dense shape");
     const int K = STATIC ? SK : Kd, NO = STATIC ? SNO : NOd;
@@ -202,9 +204,8 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         const T* base = X + t * 32 * K;
         const long long rows_left = N - t * 32;         // rows of this tile that exist
         if constexpr (POOL) {
-            int b, rb, cb;
-            tile_pixel(t, b, rb, cb);
-            base = X + (((long long)b * Himg + 4 * rb) * Wimg + 8 * cb) * K;
+            tile_pixel(t);
+            base = X + (long long)px_next * K;
 #pragma unroll
             for (int i = 0; i < LP; ++i)   // chunks i*64 .. of the tile: its pixels 4 i .. 4 i + 3 = image row i / 2, 4 columns
                 raw[i] = *reinterpret_cast<const Frag*>(base + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * K + lane * 8);
@@ -274,6 +275,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     __syncthreads();
     for (long long tile = gw; tile < ntiles; tile += nw) {
         [[maybe_unused]] const bool first = tile == gw;
+        px_cur = px_next, pp_cur = pp_next;   // (POOL) set when this tile was requested
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
 #pragma unroll
         for (int i = 0; i < LP; ++i)
@@ -420,9 +422,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             const long long rows_left = N - tile * 32;
             T* yb = Y + tile * 32 * NO;
             if constexpr (POOL) {
-                int b, rb, cb;
-                tile_pixel(tile, b, rb, cb);
-                yb = Y + (((long long)b * Himg + 4 * rb) * Wimg + 8 * cb) * NO;
+                yb = Y + (long long)px_cur * NO;
                 Frag of[LO];
 #pragma unroll
                 for (int i = 0; i < LO; ++i)
@@ -446,7 +446,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                     pv.v[0] = from_f32<T>(lo), pv.v[1] = from_f32<T>(hi);
                     o.v[j] = *reinterpret_cast<const uint32_t*>(&pv);
                 }
-                T* pb = pool + ((((long long)b * (Himg >> 1) + 2 * rb + wr) * (Wimg >> 1)) + 4 * cb + wc) * NO + ch;
+                T* pb = pool + ((long long)pp_cur + wr * (Wimg >> 1) + wc) * NO + ch;
                 *reinterpret_cast<Frag*>(pb) = o;
             } else if (STATIC && rows_left >= 32) {  // (an array of its own: one array written on both paths ends up in scratch)
                 Frag of[LO];

@@ -23,14 +23,16 @@ struct Fwd2Args {
     int s0, n0, s1, n1;   // first workgroup and number of workgroups of each problem
 };
 
-template <typename T, int K, int CS, int NPC1>
+// MODE 0: the convolutions; 4: each with the gate applied in its store (dwconv_tz.h), 16 channels per workgroup only.
+template <typename T, int K, int CS, int NPC1, int MODE>
 __global__ __launch_bounds__(512, 1) void dwconv_fwd2_k(const Fwd2Args a) {
     const unsigned blk = blockIdx.x;
     if (blk - (unsigned)a.s0 < (unsigned)a.n0)
-        dwconv_tz_body<T, K, 16, CS, 0>((const T*)a.x0, (const T*)a.w0, nullptr, nullptr, (T*)a.y0, a.g0, (int)blk - a.s0, a.n0);
+        dwconv_tz_body<T, K, 16, CS, MODE>((const T*)a.x0, (const T*)a.w0, nullptr, nullptr, (T*)a.y0, a.g0, (int)blk - a.s0,
+                                           a.n0);
     else
-        dwconv_tz_body<T, K, NPC1, CS, 0>((const T*)a.x1, (const T*)a.w1, nullptr, nullptr, (T*)a.y1, a.g1, (int)blk - a.s1,
-                                          a.n1);
+        dwconv_tz_body<T, K, NPC1, CS, MODE>((const T*)a.x1, (const T*)a.w1, nullptr, nullptr, (T*)a.y1, a.g1,
+                                             (int)blk - a.s1, a.n1);
 }
 
 // Workgroups dealt in grid order to the earliest free of 256 compute units: the time the last one ends.
@@ -106,11 +108,15 @@ static Fwd2Plan fwd2_plan(int B, const TzGeom& g0, const TzGeom& g1) {
 
 // -1: not covered (the caller makes the two launches).  16-bit types, C % 8 == 0, padding K / 2, the second scale
 // exactly half the first, the full scale in the wide tile.
+// gate0, gate1 (both or neither): the gate in the store of each scale, y0 / y1 then being the gated tensors with the
+// strides and channel offsets the gates name (16-channel slices only: filters up to 13).
 template <int K>
 static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
-                       int W, int C, int dtype, hipStream_t s) {
+                       int W, int C, int dtype, hipStream_t s, const TzGate* gate0 = nullptr,
+                       const TzGate* gate1 = nullptr) {
     constexpr int CS = (2 * 4 * TzShape<K, 16, 16>::NM + 2 * 4 * TzShape<K, 16, 16>::RING) <= 160 ? 16 : 8;
     if (dtype == kF32 || C % 8 != 0 || (H & 1) || (W & 1) || B < 1 || H < 2 || W < 2) return -1;
+    if ((gate0 != nullptr) != (gate1 != nullptr) || (gate0 && CS != 16)) return -1;
     const int P = K / 2, h = H / 2, wd = W / 2;
     for (const void* p : {x0, w0, (const void*)y0, x1, w1, (const void*)y1})
         if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
@@ -122,11 +128,16 @@ static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1,
     const bool wide1 = wide(wd);
     Fwd2Args a;
     long long n0, n1;
-    if (!tz_make_geom<K, 16, CS>(a.g0, n0, false, B, H, W, C, P, P, false, nullptr)) return -1;
-    if (!(wide1 ? tz_make_geom<K, 16, CS>(a.g1, n1, false, B, h, wd, C, P, P, false, nullptr)
-                : tz_make_geom<K, 8, CS>(a.g1, n1, false, B, h, wd, C, P, P, false, nullptr)))
+    if (!tz_make_geom<K, 16, CS>(a.g0, n0, false, B, H, W, C, P, P, false, gate0)) return -1;
+    if (!(wide1 ? tz_make_geom<K, 16, CS>(a.g1, n1, false, B, h, wd, C, P, P, false, gate1)
+                : tz_make_geom<K, 8, CS>(a.g1, n1, false, B, h, wd, C, P, P, false, gate1)))
         return -1;
-    const Fwd2Plan plan = wide1 ? fwd2_plan<K, CS, 16>(B, a.g0, a.g1) : fwd2_plan<K, CS, 8>(B, a.g0, a.g1);
+    Fwd2Plan plan = wide1 ? fwd2_plan<K, CS, 16>(B, a.g0, a.g1) : fwd2_plan<K, CS, 8>(B, a.g0, a.g1);
+    if (const char* e = tune_env("PDW_FWD2_BANDS")) {   // "bands of the full scale, of the half scale, first problem"
+        if (sscanf(e, "%d,%d,%d", &plan.nb[0], &plan.nb[1], &plan.first) != 3) return -1;
+    }
+    if (tune_env("PDW_FWD2_PRINT"))
+        fprintf(stderr, "fwd2 plan B=%d H=%d W=%d C=%d K=%d: bands %d %d first %d\n", B, H, W, C, K, plan.nb[0], plan.nb[1], plan.first);
     auto rows_of = [](int oh, int nb) { return (cdiv(oh, nb) + 3) / 4 * 4; };
     a.g0.BR = rows_of(a.g0.OH, plan.nb[0]), a.g0.nbands = cdiv(a.g0.OH, a.g0.BR);
     a.g1.BR = rows_of(a.g1.OH, plan.nb[1]), a.g1.nbands = cdiv(a.g1.OH, a.g1.BR);
@@ -139,19 +150,27 @@ static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1,
     size_t lds = TzShape<K, 16, CS>::lds_bytes;
     if (!wide1 && TzShape<K, 8, CS>::lds_bytes > lds) lds = TzShape<K, 8, CS>::lds_bytes;
     const unsigned grid = (unsigned)(n0 + n1);
-    static std::once_flag once[4];
-#define PDW_FWD2_GO(T, NPC1, SLOT)                                                                                    \
+    static std::once_flag once[8];
+#define PDW_FWD2_GO(T, NPC1, MODE, SLOT)                                                                              \
     {                                                                                                                 \
-        auto kern = dwconv_fwd2_k<T, K, CS, NPC1>;                                                                    \
+        auto kern = dwconv_fwd2_k<T, K, CS, NPC1, MODE>;                                                              \
         std::call_once(once[SLOT], [&] {                                                                              \
             (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);     \
         });                                                                                                           \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, s, a);                                                   \
     }
-    if (dtype == kF16) {
-        if (wide1) PDW_FWD2_GO(f16_t, 16, 0) else PDW_FWD2_GO(f16_t, 8, 1)
+    if (gate0) {
+        if constexpr (CS == 16) {
+            if (dtype == kF16) {
+                if (wide1) PDW_FWD2_GO(f16_t, 16, 4, 4) else PDW_FWD2_GO(f16_t, 8, 4, 5)
+            } else {
+                if (wide1) PDW_FWD2_GO(bf16_t, 16, 4, 6) else PDW_FWD2_GO(bf16_t, 8, 4, 7)
+            }
+        }
+    } else if (dtype == kF16) {
+        if (wide1) PDW_FWD2_GO(f16_t, 16, 0, 0) else PDW_FWD2_GO(f16_t, 8, 0, 1)
     } else {
-        if (wide1) PDW_FWD2_GO(bf16_t, 16, 2) else PDW_FWD2_GO(bf16_t, 8, 3)
+        if (wide1) PDW_FWD2_GO(bf16_t, 16, 0, 2) else PDW_FWD2_GO(bf16_t, 8, 0, 3)
     }
 #undef PDW_FWD2_GO
     return check_launch("dwconv_fwd2");

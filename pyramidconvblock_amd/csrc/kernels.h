@@ -129,7 +129,10 @@ int dwconv_bwd3_launch(const void* gyf, const void* w0, const void* addp, void* 
 // dwconv_fwd2.hip: the forward convolutions of both scales of a two-scale block (the second at half the extents, its
 // own input) in one launch; -1 = not covered
 bool dwconv_fwd2_covers(int B, int H, int W, int C, int K, int dtype);
+// (ldy0 > 0: each convolution with the gate applied in its store, written at pixel strides ldy0 / ldy1 from channels
+// ych0 / ych1)
 int dwconv_fwd2_launch(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
-                       int W, int C, int K, int dtype, hipStream_t s);
+                       int W, int C, int K, int dtype, hipStream_t s, int ldy0 = 0, int ych0 = 0, int ldy1 = 0,
+                       int ych1 = 0);
 
 }  // namespace pdw

@@ -74,6 +74,38 @@ def test_conv_gate_equals_separate_kernels_bitwise():
     assert torch.equal(y, ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,k", [((32, 56, 56, 64), 13), ((2, 40, 36, 32), 9), ((3, 34, 70, 16), 3),
+                                     ((1, 36, 40, 48), 5), ((2, 40, 48, 32), 15), ((2, 20, 24, 32), 9)])
+def test_two_scale_conv_gate_is_the_two_calls(shape, k, dtype):
+    """pdw_dwconv_fwd2_gate (the gated convolutions of both scales in one launch, into strided outputs) gives bitwise
+    the results of two pdw_dwconv_fwd_gate calls, and status 3 where it does not cover the case."""
+    from pyramidconvblock_amd import _lib
+
+    L = _lib.lib()
+    B, H, W, C = shape
+    G = C // 2
+    gen = torch.Generator().manual_seed(k + H)
+    x0 = randn(gen, B, H, W, C).to(dtype).cuda()
+    x1 = randn(gen, B, H // 2, W // 2, C).to(dtype).cuda()
+    w0, w1 = ((randn(gen, k, k, C) / k).to(dtype).cuda() for _ in range(2))
+    y0 = torch.full((B, H, W, C), 7.0, device="cuda", dtype=dtype)           # the gate's G channels from channel G on
+    y1 = torch.full((B, H // 2, W // 2, G), 7.0, device="cuda", dtype=dtype)
+    rc = L.pdw_dwconv_fwd2_gate(x0.data_ptr(), w0.data_ptr(), y0.data_ptr(), C, G, x1.data_ptr(), w1.data_ptr(),
+                                y1.data_ptr(), G, 0, B, H, W, C, k, DT[dtype],
+                                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    wide = -(-W // 64) * 64 * B <= -(-W // 32) * 32 * (-(-B // 2) * 2)
+    covered = dtype != torch.float32 and C % 16 == 0 and k <= 13 and wide
+    assert rc == (0 if covered else 3)
+    if not covered:
+        return
+    r0, want0, _ = _gate_conv(x0, w0, C, G, False, dtype)
+    r1, want1, _ = _gate_conv(x1, w1, G, 0, False, dtype)
+    assert r0 == 0 and r1 == 0
+    assert torch.equal(y0, want0) and torch.equal(y1, want1)
+
+
 def test_conv_gate_not_covered_returns_3():
     x = torch.zeros(1, 8, 8, 32, device="cuda")
     w = torch.zeros(5, 5, 32, device="cuda")
