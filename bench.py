@@ -298,9 +298,19 @@ def kernel_rooflines(B, H, W, D, k, dtype):
             out.append(dict(kernel=f"{name}[{B}x{h}x{w}x{I},k={k}]", seconds=t, alg_bytes=conv_bytes, flops=flops,
                             issued_flops=2.0 * issued * n_el if issued else None, pipe="mfma"))
         del xs, gs
-    # the backward's largest launch: full-scale input gradient (adds the pooled branch's) + both weight gradients
     h, w = H // 2, W // 2
     nF, nH = B * H * W * I, B * h * w * I
+    # the forward convolutions of both scales as one launch
+    nbuf = max(2, int(600e6 // (2.5 * nF * es)) + 1)
+    xf = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    xh = [torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(nbuf)]
+    wt, wt1 = ((torch.randn(k, k, I, device="cuda") / k).to(dtype) for _ in range(2))
+    if dwconv.dwconv_forward2(xf[0], wt, xh[0], wt1) is not None:
+        t = time_kernel_events(lambda i: dwconv.dwconv_forward2(xf[i], wt, xh[i], wt1), nbuf)
+        out.append(dict(kernel=f"dwconv_fwd2[{B}x{H}x{W}x{I},k={k}]", seconds=t, alg_bytes=es * (2 * nF + 2 * nH + 2 * k * k * I),
+                        flops=2.0 * k * k * (nF + nH), issued_flops=2.0 * iss["fwd"] * (nF + nH), pipe="mfma"))
+    del xf, xh
+    # the backward's largest launch: full-scale input gradient (adds the pooled branch's) + both weight gradients
     nbuf = max(2, int(600e6 // (4 * nF * es)) + 1)
     gf = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
     xf = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
@@ -345,6 +355,9 @@ def kernel_rooflines(B, H, W, D, k, dtype):
         ("gate_fwd", lambda i: ops.gate_forward(c[i]), nbuf, es * 1.5 * N * I, 0.0, "valu"),
         ("gate_bwd", lambda i: ops.gate_backward(c[i], gbig[i]), nbuf, es * 2.5 * N * I, 0.0, "valu"),
         ("dense_fwd", lambda i: ops.dense_forward(xin[i], wup), 4, es * (N * D + N * I + D * I), 2.0 * N * D * I, "mfma"),
+        # conv_up as the block runs it: with the tile sums of x and the 2x2 average pool of its result
+        ("dense_fwd_pool", lambda i: ops.dense_forward_pool(xin[i], wup), 4, es * (N * D + N * I + N * I // 4 + D * I),
+         2.0 * N * D * I, "mfma"),
         ("dense_dgrad", lambda i: ops.dense_forward(a[i], wup, w_kmajor=True), 4, es * (N * D + N * I + D * I),
          2.0 * N * D * I, "mfma"),
         ("dense_wgrad", lambda i: ops.dense_wgrad(a[i % 4], xin[i % 4]), 4, es * (N * D + N * I + D * I),
@@ -385,7 +398,8 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
     name: {fwd,dgrad,wgrad}_{full,half} | fwd2 (the forward convolutions of both scales, one launch) |
     bwd3 (full-scale input gradient + both weight gradients, one launch) |
     conv128 (stand-alone forward at C = D) | avgpool_fwd | avgpool_bwd |
-    bilinear_fwd | bilinear_bwd | dense_{fwd,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pair = both
+    bilinear_fwd | bilinear_bwd | dense_{fwd,pool,dgrad,wgrad,pair} (the conv_up layer: [N,D] <-> [N,D/2]; pool = forward with tile sums and the
+    2x2 pool of the result; pair = both
     gradients in one launch) | step (whole forward+backward steps, eager) | copy"""
     from pyramidconvblock_amd import avgpool, dwconv, up
 
@@ -437,6 +451,7 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         wup = (torch.randn(I, D, device="cuda") / D ** 0.5).to(dtype)
         rb = torch.randn(B, D, device="cuda")
         fn = {"fwd": lambda: ops.dense_forward(xin, wup),
+              "pool": lambda: ops.dense_forward_pool(xin, wup),
               "dgrad": lambda: ops.dense_forward(ain, wup, w_kmajor=True, rowbias=rb, rows_per_image=H * W),
               "wgrad": lambda: ops.dense_wgrad(ain, xin),
               "pair": lambda: ops.dense_backward_pair(ain, wup, xin, rowbias=rb, rows_per_image=H * W)}[res]
@@ -522,7 +537,7 @@ def main():
     ap.add_argument("--no-torch-gpu", action="store_true", help="skip the torch-operator comparator on the GPU")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
                     "{fwd,dgrad,wgrad}_{full,half}, fwd2, bwd3, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
-                    "dense_{fwd,dgrad,wgrad,pair}, step, copy")
+                    "dense_{fwd,pool,dgrad,wgrad,pair}, step, copy")
     ap.add_argument("--torch-gpu-only", action="store_true", help="(internal) time the torch-operator comparator and exit")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
     args = ap.parse_args()
