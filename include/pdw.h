@@ -162,8 +162,10 @@ int pdw_dwconv_wgrad_pair(const void *x0, const void *gy0, void *dw0, void *work
  * input gradient), dw0 = the full scale's weight gradient from x0 and gy0, dw1 = the half scale's from x1 and gy1
  * [B,H/2,W/2,C].  Square odd filter, stride 1, padding K/2, even H and W; workspaces as for the two pdw_dwconv_wgrad
  * calls.  Status 3 (nothing launched) when the fused kernel does not cover the case (fp32, C % 16, images narrower than
- * 33 columns...): the caller then makes the three calls.  Results are bitwise those of the separate calls; between
- * pdw_reduce_defer_begin/flush the two summations are recorded like any other. */
+ * 33 columns...): the caller then makes the three calls.  dx is bitwise that of the separate call; the weight gradients
+ * are the same sums taken over other bands of the images (the launch chooses its own band heights: as few bands as fill
+ * the chip together with the other two problems), so they can differ from pdw_dwconv_wgrad's in the last bit, and are
+ * the same from call to call.  Between pdw_reduce_defer_begin/flush the two summations are recorded like any other. */
 int pdw_dwconv_bwd3(const void *gy0, const void *w0, const void *gp, void *dx, const void *x0, void *dw0,
                     void *workspace0, size_t workspace0_bytes, const void *x1, const void *gy1, void *dw1,
                     void *workspace1, size_t workspace1_bytes, int B, int H, int W, int C, int K, int dtype,
@@ -352,7 +354,8 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
                        void *stream);
 
 /* The whole block of conv_block.py:25-49 (scales (1, 1/2), conv_up without bias) as one host call each way: the
- * launch sequence of the entry points above (5 launches forward; 6 launches and one summation launch backward)
+ * launch sequence of the entry points above (4 launches forward: conv_up with the pool of its result, the convolutions
+ * of both scales, gates and mean branch, conv_out; 5 launches and one summation launch backward)
  * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
  * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense
  * kernels and pdw_dense_bwd_pair cover (multiples of 8 up to 128; D = 128, I = 64 and D = 64, I = 32 run the variants with
@@ -361,11 +364,13 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
  * NULL.  The forward writes what the backward reads again: a = conv_up(x), c0 = conv(a), xp = pool(a)[B,H/2,W/2,I],
  * c1 = conv(xp), cat[B,H,W,I] (the gated scales), m[B,D] (per-image mean of x).  The backward overwrites dx and the
  * parameter gradients (gb_pool, gb_out may be NULL).  Workspaces: device scratch of the stated size, free for reuse
- * when the call's work on `stream` is done.  Results are bitwise those of the separate calls.
+ * when the call's work on `stream` is done.  Results are bitwise those of the calls listed above made one by one.
  * Replaces the Python-level sequence of ConvBlock.forward, conv_block.py:36-49, and its autograd backward. */
 int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype);
-/* Inference forward of the same block (same coverage): y only.  conv_up, then each scale's convolution with the gate
- * applied in its store (pdw_dwconv_fwd_gate; the full-resolution one also pools its input for the second scale), the
+/* Inference forward of the same block (same coverage): y only.  conv_up (which also pools its result for the second
+ * scale where its kernel can, pdw_dense_fwd_colsum_pool), then each scale's convolution with the gate applied in its
+ * store (both as one launch, pdw_dwconv_fwd2_gate, or pdw_dwconv_fwd_gate twice, the full-resolution one then pooling
+ * its input), the
  * half-resolution gate upsampled into its slice of the concatenation, conv_out plus the mean branch.  Neither
  * convolution output is written to HBM, and every intermediate lives in `workspace`
  * (pdw_convblock_infer_workspace_bytes).  Where the fused convolution does not cover the filter size the call runs
