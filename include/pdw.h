@@ -19,8 +19,11 @@
  *     message available from pdw_last_error() (thread-local).
  *   - Callable from several host threads at once.  The library keeps three pieces of state: the per-thread
  *     error text, the per-thread list of summations recorded between pdw_reduce_defer_begin() and
- *     pdw_reduce_defer_flush(), and a once-per-process set-up of each large kernel's LDS limit (guarded by
- *     std::call_once).  It reads no environment variables: every launch plan is a function of the arguments.
+ *     pdw_reduce_defer_flush(), a once-per-process set-up of each large kernel's LDS limit (guarded by
+ *     std::call_once), and a cache of launch plans per shape for the launches that hold several problems (behind a
+ *     mutex; a plan is a function of the shape alone, so the cache changes no result).  The no-allocation entry point
+ *     has a device buffer of its own, described there.  The library reads no environment variables: every launch plan
+ *     is a function of the arguments.
  *   - Non-finite inputs: the matrix-core convolution kernels multiply a window of input pixels somewhat larger
  *     than the filter by zero-padded filter operands, so an Inf or NaN input pixel can turn outputs up to
  *     PDW_NONFINITE_REACH pixels beyond the filter's own footprint into NaN (0 * Inf).  Outputs further away, and

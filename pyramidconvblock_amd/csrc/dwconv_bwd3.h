@@ -42,7 +42,7 @@ __global__ __launch_bounds__(512, 1) void dwconv_bwd3_k(const Bwd3Args a) {
 // Band heights and grid order of the three problems.  A compute unit holds one workgroup of this launch at a time, and a
 // band costs a start-up (first windows, operand set-up) that does not depend on its height, so unlike a launch of its
 // own, which has to fill the chip, a problem here is best cut into as few bands as the other problems leave room for:
-// each candidate (1, 2, 3, 4 or the stand-alone planner's number of bands per problem) is priced by dealing its
+// each candidate (1, 2, 4 or the stand-alone planner's number of bands per problem) is priced by dealing its
 // workgroups, longest problem first (the grid order), to the earliest free of 256 compute units.  Band costs in
 // microseconds, fitted to traces of this launch at [32,56,56,64] (whole-image bands for all three: 28.7 us against
 // 37.4 us with the bands of the separate launches at K = 13, 30.3 against 38.5 at K = 9, 50.0 against 60.2 at K = 17).
@@ -91,11 +91,11 @@ static Bwd3Plan bwd3_plan(int B, const TzGeom& gd, const WgTzPlan& p0, const WgT
     Bwd3Plan best{};
     double best_t = 0;
     // with many times more whole-image bands than compute units the chip is full whatever the cut: fewest start-ups
-    const bool plenty = per_band[0] + per_band[1] + per_band[2] > 2048;
-    const int cand[5] = {1, 2, 3, 4, 0};   // 0: the stand-alone planner's count
-    for (int a = 0; a < 5; ++a)
-        for (int b = 0; b < 5; ++b)
-            for (int c = 0; c < 5; ++c) {
+    const bool plenty = per_band[0] + per_band[1] + per_band[2] > 1536;
+    const int cand[4] = {1, 2, 4, 0};   // 0: the stand-alone planner's count
+    for (int a = 0; a < 4; ++a)
+        for (int b = 0; b < 4; ++b)
+            for (int c = 0; c < 4; ++c) {
                 const int pick[3] = {cand[a], cand[b], cand[c]};
                 if (plenty && (a | b | c) != 0) continue;
                 int nb[3];

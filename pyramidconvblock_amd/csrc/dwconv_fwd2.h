@@ -80,10 +80,10 @@ static Fwd2Plan fwd2_plan(int B, const TzGeom& g0, const TzGeom& g1) {
     };
     Fwd2Plan best{{standalone[0], standalone[1]}, 0};
     double best_t = 0;
-    const bool plenty = per_band[0] + per_band[1] > 2048;   // the chip is full whatever the cut: fewest start-ups
-    const int cand[5] = {1, 2, 3, 4, 0};                    // 0: the stand-alone planner's count
-    for (int a = 0; a < 5; ++a)
-        for (int b = 0; b < 5; ++b) {
+    const bool plenty = per_band[0] + per_band[1] > 1536;   // the chip is full whatever the cut: fewest start-ups
+    const int cand[4] = {1, 2, 4, 0};                       // 0: the stand-alone planner's count
+    for (int a = 0; a < 4; ++a)
+        for (int b = 0; b < 4; ++b) {
             if (plenty && (a | b) != 0) continue;
             const int pick[2] = {cand[a], cand[b]};
             int nb[2];
