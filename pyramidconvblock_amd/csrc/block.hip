@@ -1,5 +1,5 @@
 // The pyramid block of conv_block.py:25-49 as one host call each way: the launch sequence that the Python operator
-// makes through the single entry points (5 launches forward, 7 backward), for callers that cannot afford an
+// makes through the single entry points (4 launches forward, 6 backward), for callers that cannot afford an
 // interpreter between launches.  Host code only: every step is one of the library's own entry points, in the order
 // and with the arguments of pyramidconvblock_amd/conv_block.py, so the results are bitwise the same.
 #include <stdint.h>
