@@ -672,6 +672,9 @@ def main():
             "flops_per_byte": ai, "machine_flops_per_byte": MFMA_PEAK / HBM_PEAK,
             "mfma_issue_frac": (dom["issued_flops"] / dom["seconds"] / MFMA_PEAK) if dom["issued_flops"] else None,
             "limiter": "not the roofline: LDS operand reads and exposed load latency (profiles/)",
+            "timed": "HIP events around graph replays of the call over rotating buffers; a weight-gradient call includes "
+                     "its summation launches (dwconv_bwd3: one deferred summation launch per 4 calls, about 3 us per "
+                     "call on top of the kernel; the kernel trace under profiles/ has the kernel alone)",
         }
         result["kernels"] = []
         for r in ks:
