@@ -326,8 +326,30 @@ def kernel_rooflines(B, H, W, D, k, dtype):
                 for j in range(4 * i, 4 * i + 4):
                     dwconv.dwconv_bwd3(gf[j % nbuf], wt, gp[j % nbuf], xf[j % nbuf], xh[j % nbuf], gh[j % nbuf])
 
-        t = time_kernel_events(four, nbuf, iters=6) / 4
-        out.append(dict(kernel=f"dwconv_bwd3[{B}x{H}x{W}x{I},k={k}]", seconds=t,
+        t_call = time_kernel_events(four, nbuf, iters=6) / 4
+        # the launch alone: a graph of `group` calls whose summations are recorded inside the capture and run after
+        # it (the deferral is closed outside the graph), replayed between two HIP events
+        group = min(nbuf, 4)
+        four(0)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        ctx = _lib.deferred_reductions(gf[0].device)
+        with torch.cuda.graph(graph):
+            ctx.__enter__()
+            for j in range(group):
+                dwconv.dwconv_bwd3(gf[j], wt, gp[j], xf[j], xh[j], gh[j])
+        ctx.__exit__(None, None, None)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(24):
+            graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        t = start.elapsed_time(stop) * 1e-3 / (24 * group)
+        del graph
+        out.append(dict(kernel=f"dwconv_bwd3[{B}x{H}x{W}x{I},k={k}]", seconds=t, call_seconds=t_call,
                         alg_bytes=es * (3 * nF + 3 * nH + 3 * k * k * I), flops=2.0 * k * k * (2 * nF + nH),
                         issued_flops=(2.0 * (iss["fwd"] * nF + iss["wgrad"] * (nF + nH)) if iss["wgrad"] else None),
                         pipe="mfma"))
@@ -672,9 +694,9 @@ def main():
             "flops_per_byte": ai, "machine_flops_per_byte": MFMA_PEAK / HBM_PEAK,
             "mfma_issue_frac": (dom["issued_flops"] / dom["seconds"] / MFMA_PEAK) if dom["issued_flops"] else None,
             "limiter": "not the roofline: LDS operand reads and exposed load latency (profiles/)",
-            "timed": "HIP events around graph replays of the call over rotating buffers; a weight-gradient call includes "
-                     "its summation launches (dwconv_bwd3: one deferred summation launch per 4 calls, about 3 us per "
-                     "call on top of the kernel; the kernel trace under profiles/ has the kernel alone)",
+            "timed": "HIP events around graph replays over rotating buffers; for dwconv_bwd3 the graph holds the launch "
+                     "alone (its summations are recorded during the capture and run outside the graph; `call_us` in the "
+                     "kernels row includes them), graph launch gaps included",
         }
         result["kernels"] = []
         for r in ks:
@@ -684,6 +706,8 @@ def main():
                 row["mfma_issue_frac"] = round(r["issued_flops"] / r["seconds"] / MFMA_PEAK, 4)
             if r["kernel"] in traffic:
                 row["traffic"] = traffic[r["kernel"]]
+            if "call_seconds" in r:   # the call with its share of the deferred summation launches
+                row["call_us"] = round(r["call_seconds"] * 1e6, 2)
             result["kernels"].append(row)
 
     if not args.no_torch_gpu:
