@@ -17,11 +17,12 @@
  *     call.  Arithmetic is fp32 (bf16/fp16 products are exact in fp32), one rounding on store.
  *   - Return value: 0 on success; non-zero on invalid arguments or a failed launch, with a
  *     message available from pdw_last_error() (thread-local).
- *   - Callable from several host threads at once.  The library keeps three pieces of state: the per-thread
+ *   - Callable from several host threads at once.  The library keeps four pieces of state: the per-thread
  *     error text, the per-thread list of summations recorded between pdw_reduce_defer_begin() and
  *     pdw_reduce_defer_flush(), a once-per-process set-up of each large kernel's LDS limit (guarded by
- *     std::call_once), and a cache of launch plans per shape for the launches that hold several problems (behind a
- *     mutex; a plan is a function of the shape alone, so the cache changes no result).  The no-allocation entry point
+ *     std::call_once), and a bounded cache of launch plans per shape for the launches that hold several problems (behind a
+ *     mutex, emptied when it reaches 256 shapes; a plan is a function of the shape alone, so the cache changes no
+ *     result).  The no-allocation entry point
  *     has a device buffer of its own, described there.  The library reads no environment variables: every launch plan
  *     is a function of the arguments.
  *   - Non-finite inputs: the matrix-core convolution kernels multiply a window of input pixels somewhat larger
@@ -173,6 +174,11 @@ int pdw_dwconv_bwd3(const void *gy0, const void *w0, const void *gp, void *dx, c
                     void *workspace0, size_t workspace0_bytes, const void *x1, const void *gy1, void *dw1,
                     void *workspace1, size_t workspace1_bytes, int B, int H, int W, int C, int K, int dtype,
                     void *stream);
+/* Host only: the cut pdw_dwconv_bwd3 would choose for these extents (launch planning of the same call sites; no
+ * reference counterpart, the Triton grid is fixed at dwconv_triton.py:318-333).  bands[0..2] receive the number of row
+ * bands per image of the input gradient, the full scale's and the half scale's weight gradient (each >= 1).  Returns 0,
+ * 3 when pdw_dwconv_bwd3 does not cover the case, 1 on invalid arguments.  Touches no device. */
+int pdw_dwconv_bwd3_plan(int B, int H, int W, int C, int K, int dtype, int *bands);
 
 /* The forward convolutions of both scales of a two-scale block as one launch (conv_block.py:14-16 at scales 1 and
  * 1/2): y0 = conv(x0, w0) on [B,H,W,C] and y1 = conv(x1, w1) on [B,H/2,W/2,C], x1 being an input (the caller's 2x2

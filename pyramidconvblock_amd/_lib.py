@@ -78,6 +78,7 @@ _SIGS = {
     "pdw_dwconv_fwd2_supported": (c_int, [c_int] * 6),
     "pdw_dwconv_fwd2": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "pdw_dwconv_fwd2_gate": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_void_p] * 3 + [c_int] * 2 + [c_int] * 6 + [c_void_p]),
+    "pdw_dwconv_bwd3_plan": (c_int, [c_int] * 6 + [c_void_p]),
     "pdw_dwconv_bwd3": (c_int, [c_void_p] * 7 + [c_size_t] + [c_void_p] * 4 + [c_size_t] + [c_int] * 6 + [c_void_p]),
     "pdw_dense_supported": (c_int, [c_int] * 3),
     "pdw_dense_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong] + [c_int] * 4

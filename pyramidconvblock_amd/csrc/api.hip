@@ -1,7 +1,9 @@
 // C ABI of libpdw.so (declared in include/pdw.h): argument validation and dispatch to
 // the kernel launchers.  No allocation, no synchronisation; the only state is the per-thread
-// error text here, the per-thread list of deferred summations (dwconv_direct.hip) and the
-// once-per-process LDS-limit set-up next to each large kernel's launcher.
+// error text here, the per-thread list of deferred summations (dwconv_direct.hip), the
+// once-per-process LDS-limit set-up next to each large kernel's launcher, the bounded per-shape
+// launch-plan caches of the shared conv launches (dwconv_fwd2.h, dwconv_bwd3.h: a std::map behind a
+// mutex each, emptied at kPlanCacheMax entries) and the per-device address of the static scratch array.
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -289,6 +291,15 @@ int pdw_dwconv_bwd3(const void* gy0, const void* w0, const void* gp, void* dx, c
     const int r = dwconv_bwd3_launch(gy0, w0, gp, dx, x0, dw0, workspace0, x1, gy1, dw1, workspace1, B, H, W, C, K, dtype,
                                      (hipStream_t)stream);
     if (r == -1) return set_error("pdw_dwconv_bwd3: case not covered (B=%d H=%d W=%d C=%d K=%d dtype=%d)", B, H, W, C, K, dtype), 3;
+    return r;
+}
+
+int pdw_dwconv_bwd3_plan(int B, int H, int W, int C, int K, int dtype, int* bands) {
+    if (!bands || !valid_dtype(dtype) || B < 1 || H < 2 || W < 2 || C < 1 || K < 1 || !(K & 1) || (H & 1) || (W & 1))
+        return set_error("pdw_dwconv_bwd3_plan: bad arguments (B=%d H=%d W=%d C=%d K=%d dtype=%d)", B, H, W, C, K, dtype), 1;
+    const int r = dwconv_bwd3_launch(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                     nullptr, nullptr, B, H, W, C, K, dtype, nullptr, bands);
+    if (r == -1) return set_error("pdw_dwconv_bwd3_plan: case not covered"), 3;
     return r;
 }
 

@@ -67,6 +67,9 @@ inline int pick_vec(int C, size_t elem, const void* const* ptrs, int nptrs) {
 
 inline int cdiv(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+// Entries a per-shape launch-plan cache may hold before it is emptied (a plan costs microseconds to redo).
+constexpr size_t kPlanCacheMax = 256;
+
 // Planner overrides for experiments (PDW_* environment variables): read only in a build with -DPDW_TUNE.
 // The shipped library never looks at the environment; every planner then takes its own choice.
 #ifdef PDW_TUNE

@@ -88,7 +88,8 @@ static Bwd3Plan bwd3_plan(int B, const TzGeom& gd, const WgTzPlan& p0, const WgT
         const int ncb = i == 1 ? p0.ncb : p1.ncb;
         return 3.0 + 1.5 * nmf * (ncb == 8 ? 1.0 : 0.9) * ((br + 4) / 4);
     };
-    Bwd3Plan best{};
+    // the fallback when no candidate survives: every problem cut as its stand-alone launch cuts it
+    Bwd3Plan best{{std::max(1, standalone[0]), std::max(1, standalone[1]), std::max(1, standalone[2])}, "DFH"};
     double best_t = 0;
     // with many times more whole-image bands than compute units the chip is full whatever the cut: fewest start-ups
     const bool plenty = per_band[0] + per_band[1] + per_band[2] > 1536;
@@ -105,7 +106,7 @@ static Bwd3Plan bwd3_plan(int B, const TzGeom& gd, const WgTzPlan& p0, const WgT
                 for (int i = 0; i < 3; ++i) {
                     nb[i] = pick[i] ? pick[i] : standalone[i];
                     // a weight gradient's partials must fit the workspace sized for the stand-alone plan
-                    if (pick[i] && (nb[i] > oh[i] / 4 || (i > 0 && nb[i] > standalone[i]))) ok = false;
+                    if (pick[i] && (nb[i] > std::max(1, oh[i] / 4) || (i > 0 && nb[i] > standalone[i]))) ok = false;
                     const int br = band_rows(i, nb[i]);
                     nb[i] = cdiv(oh[i], br);
                     cost[i] = band_cost(i, br), count[i] = per_band[i] * nb[i];
@@ -123,6 +124,7 @@ static Bwd3Plan bwd3_plan(int B, const TzGeom& gd, const WgTzPlan& p0, const WgT
                     best.order[3] = 0;
                 }
             }
+    if (cache.size() >= kPlanCacheMax) cache.clear();   // callers with ever-changing shapes: a plan is cheap to redo
     cache[key] = best;
     return best;
 }
@@ -132,13 +134,14 @@ static Bwd3Plan bwd3_plan(int B, const TzGeom& gd, const WgTzPlan& p0, const WgT
 template <int K>
 static int launch_bwd3(const void* gyf, const void* w0, const void* addp, void* dx, const void* x0, void* dw0, void* ws0,
                        const void* x1, const void* gy1, void* dw1, void* ws1, int B, int H, int W, int C, int dtype,
-                       hipStream_t s) {
+                       hipStream_t s, int* plan_out) {
     constexpr int CS = (2 * 4 * TzShape<K, 16, 16>::NM + 2 * 4 * TzShape<K, 16, 16>::RING) <= 160 ? 16 : 8;
     constexpr int NGA0 = (4 + 2 * ((K - 1) / 2) + 3) / 4, NGA = NGA0 < 2 ? 2 : NGA0, NB = K == 17 ? 3 : 2;
     if (dtype == kF32 || C % 16 != 0 || (H & 1) || (W & 1) || B < 1) return -1;
     const int P = K / 2, h = H / 2, wd = W / 2;
-    for (const void* p : {gyf, w0, addp, (const void*)dx, x0, (const void*)ws0, x1, gy1, (const void*)ws1})
-        if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
+    if (!plan_out)
+        for (const void* p : {gyf, w0, addp, (const void*)dx, x0, (const void*)ws0, x1, gy1, (const void*)ws1})
+            if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
     const long long pad16 = (long long)cdiv(W, 64) * 64 * B, pad8 = (long long)cdiv(W, 32) * 32 * cdiv(B, 2) * 2;
     if (pad16 > pad8) return -1;   // the input gradient's wide tile only
     Bwd3Args a;
@@ -153,6 +156,7 @@ static int launch_bwd3(const void* gyf, const void* w0, const void* addp, void* 
     if (tune_env("PDW_BWD3_PRINT"))
         fprintf(stderr, "bwd3 plan B=%d H=%d W=%d C=%d K=%d: bands D %d F %d H %d order %s\n", B, H, W, C, K, plan.nb[0],
                 plan.nb[1], plan.nb[2], plan.order);
+    if (plan.nb[0] < 1 || plan.nb[1] < 1 || plan.nb[2] < 1) return -1;
     auto rows_of = [](int oh, int nb) { return (cdiv(oh, nb) + 3) / 4 * 4; };
     a.gd.BR = rows_of(a.gd.OH, plan.nb[0]), a.gd.nbands = cdiv(a.gd.OH, a.gd.BR);
     nd = (long long)cdiv(B, TzShape<K, 16, CS>::NI) * a.gd.nbands * a.gd.ncolt * a.gd.nslices;
@@ -162,6 +166,10 @@ static int launch_bwd3(const void* gyf, const void* w0, const void* addp, void* 
     p1.nblocks = (long long)B * p1.g.nslices * p1.g.ncolt * p1.g.nbands;
     if (!p0.ok || !p1.ok || p0.ncb != 8 || wgrad_tz_nga(K) != NGA) return -1;
     if (nd + p0.nblocks + p1.nblocks > 0x7fffffffLL) return -1;
+    if (plan_out) {
+        plan_out[0] = a.gd.nbands, plan_out[1] = p0.g.nbands, plan_out[2] = p1.g.nbands;
+        return 0;
+    }
     a.gy = gyf, a.w = w0, a.add = addp, a.dx = dx;
     a.x0 = x0, a.gy0 = gyf, a.x1 = x1, a.gy1 = gy1, a.part0 = (float*)ws0, a.part1 = (float*)ws1;
     a.g0 = p0.g, a.g1 = p1.g, a.nd = (int)nd, a.n1 = (int)p1.nblocks, a.n0 = (int)p0.nblocks;

@@ -102,6 +102,7 @@ static Fwd2Plan fwd2_plan(int B, const TzGeom& g0, const TzGeom& g1) {
             const double t = plenty ? 1.0 : tz_makespan(2, cost, count, ord);
             if (best_t == 0 || t < best_t - 1e-9) best_t = t, best = Fwd2Plan{{nb[0], nb[1]}, ord[0]};
         }
+    if (cache.size() >= kPlanCacheMax) cache.clear();   // callers with ever-changing shapes: a plan is cheap to redo
     cache[key] = best;
     return best;
 }

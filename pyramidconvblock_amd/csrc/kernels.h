@@ -124,7 +124,7 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
 // two-scale block in one launch; -1 = not covered
 int dwconv_bwd3_launch(const void* gyf, const void* w0, const void* addp, void* dx, const void* x0, void* dw0, void* ws0,
                        const void* x1, const void* gy1, void* dw1, void* ws1, int B, int H, int W, int C, int K, int dtype,
-                       hipStream_t s);
+                       hipStream_t s, int* plan_out = nullptr);
 
 // dwconv_fwd2.hip: the forward convolutions of both scales of a two-scale block (the second at half the extents, its
 // own input) in one launch; -1 = not covered

@@ -73,6 +73,28 @@ def test_single_call_block_host_logic_without_gpu():
     assert b"not covered" in L.pdw_last_error()
 
 
+@pytest.mark.parametrize("shape", [(128, 2, 64, 64, 3), (128, 4, 64, 64, 3), (128, 6, 64, 64, 13), (96, 2, 34, 16, 5),
+                                   (512, 6, 40, 128, 17), (32, 56, 56, 64, 13), (8, 56, 56, 64, 13), (1, 8, 36, 16, 9),
+                                   (8, 112, 112, 48, 17), (128, 56, 56, 64, 13)])
+def test_bwd3_planner_strip_shaped_inputs(shape):
+    """The planner of the backward's three-problem launch (host code, no device touched): images of fewer than four
+    rows at the half scale, with batch x channels large enough that only whole-image bands are tried, must still get
+    a plan with at least one band per problem (a plan of zero bands is a division by zero in the launcher)."""
+    from pyramidconvblock_amd import _lib
+
+    L = _lib.lib()
+    bands = (ctypes.c_int * 3)(-1, -1, -1)
+    rc = L.pdw_dwconv_bwd3_plan(*shape, _lib.dtype_code(torch.bfloat16), ctypes.addressof(bands))
+    assert rc == 0, L.pdw_last_error()
+    B, H, W, C, K = shape
+    assert 1 <= bands[0] <= H and 1 <= bands[1] <= H and 1 <= bands[2] <= max(1, H // 2), list(bands)
+    # not covered: fp32, odd extents, narrow images
+    assert L.pdw_dwconv_bwd3_plan(*shape, _lib.dtype_code(torch.float32), ctypes.addressof(bands)) == 3
+    assert L.pdw_dwconv_bwd3_plan(B, H, 16, C, K, 2, ctypes.addressof(bands)) == 3
+    assert L.pdw_dwconv_bwd3_plan(B, H + 1, W, C, K, 2, ctypes.addressof(bands)) == 1
+    assert L.pdw_dwconv_bwd3_plan(B, H, W, C, K, 2, None) == 1
+
+
 def test_module_structure_and_seeded_init_match_reference_recipe():
     import pyramid_dwconv
     from oracle import torch_path

@@ -46,6 +46,18 @@ def test_metric_sweep_bf16(oracle, k):
     _block_case(oracle, 128, k, (8, 56, 56, 128), torch.bfloat16)
 
 
+@pytest.mark.parametrize("k", [9, 17])
+def test_metric_sweep_bf16_full_batch(oracle, k):
+    """The k = 9 / 17 rows of the metric at the shape they are timed on (the shared conv launches choose their band
+    heights and grid order from the shape)."""
+    _block_case(oracle, 128, k, (32, 56, 56, 128), torch.bfloat16)
+
+
+def test_batch_sweep_b64_bf16(oracle):
+    """A larger batch than the headline's: the launch plans with more whole-image bands than compute units."""
+    _block_case(oracle, 128, 13, (64, 56, 56, 128), torch.bfloat16)
+
+
 def test_config4_fp16(oracle):
     _block_case(oracle, 96, 17, (8, 112, 112, 96), torch.float16)
 

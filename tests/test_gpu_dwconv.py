@@ -134,7 +134,8 @@ def test_wgrad_pair_is_the_two_separate_calls(dtype, case):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", [(32, 56, 56, 64, 13), (8, 112, 112, 48, 17), (2, 40, 36, 32, 9), (3, 34, 70, 16, 3),
                                   (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7), (5, 58, 66, 24, 5),
-                                  (64, 56, 56, 64, 11), (1, 130, 72, 16, 13)])
+                                  (64, 56, 56, 64, 11), (1, 130, 72, 16, 13), (32, 56, 56, 64, 9),
+                                  (32, 56, 56, 64, 17), (64, 56, 56, 64, 13), (128, 56, 56, 64, 13)])
 def test_fwd2_is_the_two_separate_calls(dtype, case):
     """pdw_dwconv_fwd2 (the convolutions of a block's two scales in one launch, with band heights of its own) gives
     bitwise the results of the two separate calls; pdw_dwconv_fwd2_supported says beforehand whether it takes the
@@ -164,7 +165,9 @@ def test_fwd2_is_the_two_separate_calls(dtype, case):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", [(32, 56, 56, 64, 13), (8, 112, 112, 48, 17), (2, 40, 36, 32, 9), (3, 34, 70, 16, 3),
-                                  (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7)])
+                                  (1, 36, 40, 48, 15), (2, 20, 24, 40, 9), (4, 56, 56, 64, 7), (32, 56, 56, 64, 9),
+                                  (32, 56, 56, 64, 17), (64, 56, 56, 64, 13), (128, 56, 56, 64, 13),
+                                  (128, 4, 64, 64, 3), (128, 6, 64, 64, 13), (96, 2, 34, 16, 5)])
 def test_bwd3_is_the_three_separate_calls(dtype, case):
     """pdw_dwconv_bwd3 (the full scale's input gradient with the pooled branch's added and the weight gradients of
     both scales in one launch) gives the results of the three separate calls: the input gradient bitwise, the weight

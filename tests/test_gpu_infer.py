@@ -76,7 +76,9 @@ def test_conv_gate_equals_separate_kernels_bitwise():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("shape,k", [((32, 56, 56, 64), 13), ((2, 40, 36, 32), 9), ((3, 34, 70, 16), 3),
-                                     ((1, 36, 40, 48), 5), ((2, 40, 48, 32), 15), ((2, 20, 24, 32), 9)])
+                                     ((1, 36, 40, 48), 5), ((2, 40, 48, 32), 15), ((2, 20, 24, 32), 9),
+                                     ((32, 56, 56, 64), 9), ((32, 56, 56, 64), 17), ((64, 56, 56, 64), 13),
+                                     ((128, 56, 56, 64), 13)])
 def test_two_scale_conv_gate_is_the_two_calls(shape, k, dtype):
     """pdw_dwconv_fwd2_gate (the gated convolutions of both scales in one launch, into strided outputs) gives bitwise
     the results of two pdw_dwconv_fwd_gate calls, and status 3 where it does not cover the case."""
@@ -156,16 +158,26 @@ def test_block_inference_forward(oracle, dim, k, shape, dtype):
     assert (y.float() - yt.detach().float()).abs().max().item() <= TOL[dtype] * scale
 
 
-def test_block_inference_other_shapes_use_the_stepwise_path(oracle):
-    """Shapes the library's single call does not cover (D = 96) still give the right forward under no_grad."""
+@pytest.mark.parametrize("dim,kw", [(112, {}), (128, {"bias": True}), (64, {"scales": (1., 0.5, 0.25)})])
+def test_block_inference_other_shapes_use_the_stepwise_path(oracle, dim, kw):
+    """What the library's single call does not cover (an inner width of 56, a bias on conv_up, three scales) still
+    gives the right forward under no_grad, through the operator's launches one by one."""
     import pyramid_dwconv
+    from pyramidconvblock_amd import conv_block
 
     torch.manual_seed(2)
-    m = pyramid_dwconv.ConvBlock(dim=96, kernel_size=9).to(torch.float16)
+    m = pyramid_dwconv.ConvBlock(dim=dim, kernel_size=9, **kw).to(torch.float16)
     gen = torch.Generator().manual_seed(2)
-    x = randn(gen, 2, 24, 20, 96).to(torch.float16)
+    x = randn(gen, 2, 24, 20, dim).to(torch.float16)
     params = {n: p.detach().double().numpy() for n, p in m.state_dict().items()}
-    yo, _ = oracle.convblock_fwd(x.double().numpy(), params)
-    with torch.no_grad():
-        y = m.cuda()(x.cuda())
+    yo, _ = oracle.convblock_fwd(x.double().numpy(), params, scales=tuple(kw.get("scales", (1., 0.5))))
+    calls = []
+    orig = conv_block.convblock_infer
+    conv_block.convblock_infer = lambda *a, **k: (calls.append(1), orig(*a, **k))[1]
+    try:
+        with torch.no_grad():
+            y = m.cuda()(x.cuda())
+    finally:
+        conv_block.convblock_infer = orig
+    assert not calls, "the single-call inference entry point was taken for a configuration it does not cover"
     assert_close(y, yo, torch.float16, "y")

@@ -13,16 +13,16 @@ def _np(P):
     return {k: v.double().numpy() for k, v in P.items()}
 
 
-def _check_block(oracle, dim, k, shape, seed, dist="normal", bias=False):
+def _check_block(oracle, dim, k, shape, seed, dist="normal", bias=False, scales=(1.0, 0.5), inter_ratio=0.5):
     torch.manual_seed(seed)
-    P = torch_path.default_params(dim, k, bias=bias)
+    P = torch_path.default_params(dim, k, bias=bias, scales=scales, inter_ratio=inter_ratio)
     x = torch.randn(*shape) if dist == "normal" else torch.rand(*shape) * 4 - 2
     g = torch.randn(*shape)
     Pd = {k_: v.double().requires_grad_() for k_, v in P.items()}
     xd = x.double().requires_grad_()
-    yt = torch_path.convblock(xd, Pd)
+    yt = torch_path.convblock(xd, Pd, scales=scales)
     grads = torch.autograd.grad(yt, [xd] + list(Pd.values()), g.double())
-    y, cache = oracle.convblock_fwd(x.numpy(), _np(P))
+    y, cache = oracle.convblock_fwd(x.numpy(), _np(P), scales=scales)
     np.testing.assert_allclose(y, yt.detach().numpy(), atol=1e-11)
     dx, gr = oracle.convblock_bwd(cache, g.numpy())
     np.testing.assert_allclose(dx, grads[0].numpy(), atol=1e-10)
@@ -46,6 +46,20 @@ def test_config1_cpu_plumbing(oracle):
 def test_ragged_config5_small_batch(oracle, k):
     """Config 5 geometry (57x61, C=200 -> 100 conv channels, odd pool bins) at B=1."""
     _check_block(oracle, 200, k, (1, 57, 61, 200), 0, dist="uniform")
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 16, 64), (2, 13, 19, 64)])
+@pytest.mark.parametrize("scales", [(1.,), (0.5,), (1., 0.5, 0.25), (0.5, 1.), (1., 1.), (1., 0.75)])
+def test_block_scales(oracle, scales, shape):
+    """The oracle's block with every non-default ``scales`` tuple the GPU tests use it for as their checker,
+    against autograd through torch's library operators in float64 (pooled extents int(H * s), conv_block.py:16;
+    one gate per scale, concatenated in order, conv_block.py:41-44)."""
+    _check_block(oracle, 64, 7, shape, 11, scales=scales)
+
+
+@pytest.mark.parametrize("inter_ratio", [0.25, 0.75, 1.0])
+def test_block_inter_ratio(oracle, inter_ratio):
+    _check_block(oracle, 64, 5, (2, 10, 12, 64), 12, inter_ratio=inter_ratio)
 
 
 def test_block_with_up_bias(oracle):

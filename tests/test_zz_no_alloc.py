@@ -26,11 +26,15 @@ def _both(shape, k, dtype, seed):
     _lib.check(L.pdw_dwconv_wgrad(x.data_ptr(), gy.data_ptr(), ref.data_ptr(), ws.data_ptr(), ws.numel() * 4, *geo,
                                   code, stream), "pdw_dwconv_wgrad")
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # the device's own free-byte count (hipMemGetInfo): torch's allocator statistics would not see a hipMalloc or
+    # hipFree made inside the library
+    before, reserved = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
     _lib.check(L.pdw_dwconv_wgrad_static(x.data_ptr(), gy.data_ptr(), got.data_ptr(), *geo, code, stream),
                "pdw_dwconv_wgrad_static")
+    during = torch.cuda.mem_get_info()[0]
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_reserved() == reserved
+    assert during == before and torch.cuda.mem_get_info()[0] == before
     assert torch.isfinite(got.float()).all()
     assert torch.equal(got, ref), f"{shape} k={k} {dtype}: max diff {(got.float() - ref.float()).abs().max().item()}"
 
