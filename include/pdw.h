@@ -190,6 +190,17 @@ int pdw_dwconv_bwd3_plan(int B, int H, int W, int C, int K, int dtype, int *band
 int pdw_dwconv_fwd2_supported(int B, int H, int W, int C, int K, int dtype); /* 1: pdw_dwconv_fwd2 takes the case */
 int pdw_dwconv_fwd2(const void *x0, const void *w0, void *y0, const void *x1, const void *w1, void *y1, int B, int H,
                     int W, int C, int K, int dtype, void *stream);
+/* pdw_dwconv_fwd2 with the block's mean branch in B more workgroups of the same launch (conv_block.py:46-49:
+ * m[b] = mean of x over the positions, rounded; rowbias[b] = m[b] w_pool^T + b_pool + b_out in fp32, the row that
+ * pdw_dense_fwd adds to every output row of image b), from the sums of x over groups of positions that conv_up's
+ * kernel left in parts [B][nparts][D] (pdw_dense_fwd_colsum): what pdw_pool_branch_fwd_parts computes, bitwise.  The
+ * branch is three dependent trips to memory and a few kilobytes; in a launch of its own, or in one that saturates the
+ * memory system, it costs microseconds, here it runs beside the convolutions.  Status 3 (nothing launched) where
+ * pdw_dwconv_fwd2 does not take the case or the branch is not covered (D % 8, D > 128). */
+int pdw_dwconv_fwd2_mean(const void *x0, const void *w0, void *y0, const void *x1, const void *w1, void *y1, int B,
+                         int H, int W, int C, int K, const float *parts, int nparts, const void *w_pool,
+                         const void *b_pool, const void *b_out, void *m, float *rowbias, int P, int D, int dtype,
+                         void *stream);
 
 /* pdw_dwconv_fwd2 with the gate of pdw_dwconv_fwd_gate applied in the store of each scale (inference: neither
  * convolution output reaches HBM): y0[b,i,j, ych0 + c] and y1[b,i,j, ych1 + c], c < C/2, at pixel strides of ldy0 / ldy1
@@ -340,6 +351,16 @@ int pdw_dense_fwd_colsum(const void *x, const void *w, int w_kmajor, const void 
  * W % 8 == 0 only. */
 int pdw_dense_fwd_colsum_pool(const void *x, const void *w, const void *bias, void *y, float *colsum, void *pool, int B,
                               int H, int W, int K, int NO, int dtype, void *stream);
+
+/* The output layer of a two-scale block on rows made where they are multiplied (conv_block.py:18-21, 41-44 and :44
+ * as one launch): y[b,i,j,:] = [ gate(cf[b,i,j]) | bilinear resize to H x W of gate(ch[b]) at (i,j) ] w^T + bias +
+ * rowbias[b], with cf[B,H,W,I] and ch[B,H/2,W/2,I] the convolution outputs of the two scales, gate(v) = v[:I/2] *
+ * v[I/2:] * sqrt(I/2) rounded to `dtype`, w[D][I], bias[D] or NULL, rowbias fp32 [B][D] or NULL.  cat[B,H,W,I] (or
+ * NULL) receives the rows, which the backward pass reads again.  Bitwise what pdw_gate_pair_fwd (or pdw_block_mid_fwd)
+ * followed by pdw_dense_fwd produce; the gated tensor is not read back from memory.  Status 3 (nothing launched)
+ * where not covered: 16-bit types, I = 64, D = 128, H % 4 == 0, W % 8 == 0 only. */
+int pdw_dense_fwd_gated(const void *cf, const void *ch, void *cat, const void *w, const void *bias,
+                        const float *rowbias, void *y, int B, int H, int W, int I, int D, int dtype, void *stream);
 
 /* Weight gradient of such a layer: dw[m,o] = sum_n a[n,m] * b[n,o]  (a[N,M], b[N,NO] -> dw[M,NO]), fp32
  * accumulation, two deterministic passes through `workspace` (no atomics). */

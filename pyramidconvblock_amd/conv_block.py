@@ -22,6 +22,7 @@ from torch.nn import functional as F
 
 from . import _lib, ops
 from .dwconv import (OptimizedDepthwiseConv2d, dwconv_bwd3, dwconv_dgrad, dwconv_forward, dwconv_forward2,
+                     dwconv_forward2_mean,
                      dwconv_wgrad, dwconv_wgrad_pair)
 
 
@@ -219,11 +220,19 @@ class ConvBlockFunction(torch.autograd.Function):
         pair = _is_pair(scales)           # scales (1, s): both gates go into cat in one launch
         ready = None                      # pooled input already produced by the full-resolution conv's kernel
         both = None
+        mean_done = None                  # (m, yp) where the mean branch ran in the convolutions' launch
         if two:
             # the launches of pdw_convblock_fwd: the second scale's input, then both convolutions as one launch
             ws = [w.detach().to(dt).contiguous() for w in w_dw]
             xp = xp_ready if xp_ready is not None else ops.avgpool_forward(a, (H // 2, W // 2))
-            both = dwconv_forward2(a, ws[0], xp, ws[1])
+            # where conv_up left the tile sums of x, the mean branch rides in the convolutions' launch
+            if xparts is not None and same_dt:
+                both = dwconv_forward2_mean(a, ws[0], xp, ws[1], xparts, H * W, w_pool.detach().contiguous(), b_pool,
+                                            b_out)
+                if both is not None:
+                    mean_done, both = both[2:], both[:2]
+            if both is None:
+                both = dwconv_forward2(a, ws[0], xp, ws[1])
             if both is not None:
                 convs, pooled = [both[0], both[1]], [None, xp]
             else:
@@ -249,14 +258,23 @@ class ConvBlockFunction(torch.autograd.Function):
                     ops.gate_forward(c, out=dst)
             convs.append(c)
             pooled.append(p)
-        if pair and xparts is not None:
+        y = None
+        if mean_done is not None:
+            # the mean branch is done: conv_out makes its rows (both gates, the resize) where it multiplies them and
+            # writes them to cat for the backward pass; where that kernel does not cover the widths, the gates' launch
+            m, yp = mean_done
+            if w_out.dtype == dt:
+                y = ops.dense_forward_gated(convs[0], convs[1], w_out.detach().contiguous(), rowbias=yp, cat=cat)
+            if y is None:
+                ops.gate_pair_forward(convs[0], convs[1], cat)
+        elif pair and xparts is not None:
             # both gates and the mean branch (mean -> conv_pool, plus conv_out's bias: one fp32 row per image) in
             # one launch
             m, yp = ops.block_mid_forward(convs[0], convs[1], cat, xparts, H * W, w_pool.detach().contiguous(),
                                           b_pool, b_out)
         elif pair:
             ops.gate_pair_forward(convs[0], convs[1], cat)
-        if pair and xparts is not None:
+        if mean_done is not None or (pair and xparts is not None):
             pass
         elif same_dt and B > 0:
             # mean over positions -> conv_pool, plus conv_out's bias: one fp32 row per image
@@ -268,7 +286,9 @@ class ConvBlockFunction(torch.autograd.Function):
                 yp = yp + b_out.float()
             yp = yp.contiguous()
         fast_out = ops.dense_supported(G * ns, D, dt) and ops.dense_supported(D, G * ns, dt) and w_out.dtype == dt
-        if fast_out:
+        if y is not None:
+            pass
+        elif fast_out:
             y = ops.dense_forward(cat, w_out.detach().contiguous(), rowbias=yp, rows_per_image=H * W)
         else:
             y = ops.add_rowbias_(F.linear(cat, w_out), yp)

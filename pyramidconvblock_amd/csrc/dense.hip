@@ -14,8 +14,10 @@
 //          Every wavefront accumulates all (m,o) tiles in registers, the wavefronts of a workgroup
 //          are summed through LDS and the per-workgroup fp32 partials are reduced in a fixed order by
 //          wgrad_reduce_parts (no atomics).
+#include <math.h>
 #include <stdlib.h>
 
+#include "bilinear.h"
 #include "common.h"
 #include "kernels.h"
 #include "reduce_parts.h"
@@ -151,23 +153,78 @@ struct WTransposer {
 // covers 1 KB of consecutive bytes: 4 pixels of K values, 8 pixels of NO), so that it holds 2 x 4 whole windows of
 // the 2x2 average pool of Y, which the kernel writes to `pool` [B, Himg/2, Wimg/2, NO] from the result tile in LDS:
 // (((y00 + y01) + y10) + y11) / 4 in fp32 of the rounded results, as the pooling kernel computes it.
-template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0, bool POOL = false>
+//
+// MID (SK = 64, SNO = 128, rows = the pixels of [B, Himg, Wimg] images in the 4 x 8 tiles of POOL): the rows are not
+// loaded but made, from the convolution outputs of a two-scale block (conv_block.py:18-21, 41-44): row (b, i, j) =
+// [ gate(cf[b, i, j]) | bilinear resize to Himg x Wimg of gate(ch[b]) at (i, j) ], cf [B, Himg, Wimg, 64] the full
+// scale, ch [B, Himg/2, Wimg/2, 64] the half scale, gate(v) = v[:32] * v[32:] * gs rounded to T.  A tile's resized
+// half needs the 4 x 6 patch of the half scale around it: the patch is gated once into the tile buffer's spare columns
+// and the tile's 32 pixels take their four taps from there (gated per output pixel it would be 4 gates per value
+// instead of 0.75).  The rows are also written to mid->cat ([B, Himg, Wimg, 64], when not null): the arithmetic, and
+// therefore every bit, is that of the gate kernels followed by this layer on their output.
+struct MidRows {
+    const void *cf, *ch;
+    void* cat;
+    float gs;
+};
+
+// `x` rounded to T, as its 16-bit pattern in the low half of a register.
+template <typename T>
+__device__ __forceinline__ uint32_t f32_to_half(float x) {
+    return (uint32_t)__builtin_bit_cast(unsigned short, from_f32<T>(x));
+}
+
+// 8 gate values a * b * s, each rounded to T (the arithmetic of the stand-alone gate kernels).
+template <typename T>
+__device__ __forceinline__ Frag gate8(const Frag& a, const Frag& b, float s) {
+    Frag o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = gate_f32(half_to_f32<T>(a.v[j] & 0xffffu), half_to_f32<T>(b.v[j] & 0xffffu), s);
+        const float hi = gate_f32(half_to_f32<T>(a.v[j] >> 16), half_to_f32<T>(b.v[j] >> 16), s);
+        o.v[j] = f32_to_half<T>(lo) | (f32_to_half<T>(hi) << 16);
+    }
+    return o;
+}
+
+// 8 bilinear values of four taps (row y0: g00, g01; row y1: g10, g11), rounded to T (the arithmetic of the
+// stand-alone resize kernels).
+template <typename T>
+__device__ __forceinline__ Frag bilinear8(const Frag& g00, const Frag& g01, const Frag& g10, const Frag& g11, float ly,
+                                          float lx) {
+    Frag o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = bl_mix(half_to_f32<T>(g00.v[j] & 0xffffu), half_to_f32<T>(g01.v[j] & 0xffffu),
+                                half_to_f32<T>(g10.v[j] & 0xffffu), half_to_f32<T>(g11.v[j] & 0xffffu), ly, lx);
+        const float hi = bl_mix(half_to_f32<T>(g00.v[j] >> 16), half_to_f32<T>(g01.v[j] >> 16),
+                                half_to_f32<T>(g10.v[j] >> 16), half_to_f32<T>(g11.v[j] >> 16), ly, lx);
+        o.v[j] = f32_to_half<T>(lo) | (f32_to_half<T>(hi) << 16);
+    }
+    return o;
+}
+
+template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0, bool POOL = false, bool MID = false>
 __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T* __restrict__ W,
                                                 const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                 T* __restrict__ Y, float* __restrict__ colsum, long long N, int Kd,
                                                 int NOd, int P, int nktd, int nntd, int bid, int nblocks,
                                                 uint32_t* dsm, T* __restrict__ pool = nullptr, int Himg = 0,
-                                                int Wimg = 0) {
+                                                int Wimg = 0, const MidRows* mid = nullptr) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
     static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
+    static_assert(!MID || (SK == 64 && SNO == 128 && !KMAJOR && !COLSUM && !POOL), "made rows: the 64 -> 128 layer");
     // POOL: first pixel of a tile and first pixel of its part of the pooled tensor (two 32-bit divisions per tile,
     // taken once, when the tile is requested, and kept for its way out)
     int px_next = 0, pp_next = 0, px_cur = 0, pp_cur = 0;
+    [[maybe_unused]] int rb_next = 0, cb_next = 0, rb_cur = 0, cb_cur = 0;   // MID: the tile's block row and column
     auto tile_pixel = [&](long long t) {
         const unsigned tw = (unsigned)Wimg >> 3, tpi = ((unsigned)Himg >> 2) * tw;
         const unsigned ti = (unsigned)t, b = ti / tpi, r = ti - b * tpi, rb = r / tw, cb = r - rb * tw;
         px_next = (int)((b * (unsigned)Himg + 4 * rb) * (unsigned)Wimg + 8 * cb);
         pp_next = (int)((b * ((unsigned)Himg >> 1) + 2 * rb) * ((unsigned)Wimg >> 1) + 4 * cb);
+        rb_next = (int)rb, cb_next = (int)cb;
+        return (int)b;
     };
     static_assert(!STATIC || (SK % 16 == 0 && SNO % 32 == 0 && SK <= 128 && SNO <= 128), "static dense shape");
     const int K = STATIC ? SK : Kd, NO = STATIC ? SNO : NOd;
@@ -200,10 +257,34 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     constexpr int LP = 8;                               // chunk loads per lane (K <= 128)
     Frag raw[LP];
     float4 brow = make_float4(0.f, 0.f, 0.f, 0.f);
+    // MID: a lane makes the 8-value chunks (pixel idx / 4, values 8 (idx % 4) ..) of both halves of the rows for
+    // idx = lane, lane + 64, and gates the chunks (patch pixel idx / 4 < 24, 8 (idx % 4) ..) of the half-scale patch
+    [[maybe_unused]] Frag fa[2], fb[2], ha[2], hb[2];
+    [[maybe_unused]] auto mid_load = [&](long long t) {
+        const int b = tile_pixel(t);
+        const int hh = Himg >> 1, hw = Wimg >> 1;
+        const T* cf = static_cast<const T*>(mid->cf) + (long long)px_next * 64;
+        const T* chb = static_cast<const T*>(mid->ch) + (long long)b * hh * hw * 64;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
+            const T* f = cf + (long long)((pix >> 3) * Wimg + (pix & 7)) * 64 + 8 * cc;
+            fa[p] = *reinterpret_cast<const Frag*>(f);
+            fb[p] = *reinterpret_cast<const Frag*>(f + 32);
+            // (patch entries past the image are never used as taps: clamped, they are readable)
+            const int q = min(pix, 23), qr = q / 6, qc = q - 6 * qr;
+            const int hy = min(max(2 * rb_next - 1 + qr, 0), hh - 1), hx = min(max(4 * cb_next - 1 + qc, 0), hw - 1);
+            const T* hp = chb + (long long)(hy * hw + hx) * 64 + 8 * cc;
+            ha[p] = *reinterpret_cast<const Frag*>(hp);
+            hb[p] = *reinterpret_cast<const Frag*>(hp + 32);
+        }
+    };
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
         const T* base = X + t * 32 * K;
         const long long rows_left = N - t * 32;         // rows of this tile that exist
-        if constexpr (POOL) {
+        if constexpr (MID) {
+            mid_load(t);
+        } else if constexpr (POOL) {
             tile_pixel(t);
             base = X + (long long)px_next * K;
 #pragma unroll
@@ -275,11 +356,53 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     __syncthreads();
     for (long long tile = gw; tile < ntiles; tile += nw) {
         [[maybe_unused]] const bool first = tile == gw;
-        px_cur = px_next, pp_cur = pp_next;   // (POOL) set when this tile was requested
+        px_cur = px_next, pp_cur = pp_next;   // (POOL, MID) set when this tile was requested
+        if constexpr (MID) {
+            rb_cur = rb_next, cb_cur = cb_next;
+            const int hh = Himg >> 1, hw = Wimg >> 1;
+            T* cat = static_cast<T*>(mid->cat);
+            // the gated patch of the half scale: [24 pixels][32] in columns 64.. of the tile buffer's rows
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int idx = p * 64 + lane, q = idx >> 2, cc = idx & 3;
+                const Frag hg = gate8<T>(ha[p], hb[p], mid->gs);
+                if (q < 24) *reinterpret_cast<Frag*>(tl + q * ldt + 64 + 8 * cc) = hg;
+            }
+            // the full scale's half of the rows
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
+                const Frag full = gate8<T>(fa[p], fb[p], mid->gs);
+                *reinterpret_cast<Frag*>(tl + pix * ldt + 8 * cc) = full;
+                if (cat)
+                    *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * 64 + 8 * cc) = full;
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the patch is in LDS (written by other lanes of this wavefront)
+            // the resized half: four taps of the patch per pixel, bl_src's rows, columns and weights
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
+                int y0, y1, x0, x1;
+                float ly, lx;
+                bl_src(4 * rb_cur + (pix >> 3), 0.5f, hh, y0, y1, ly);
+                bl_src(8 * cb_cur + (pix & 7), 0.5f, hw, x0, x1, lx);
+                const int oy = 2 * rb_cur - 1, ox = 4 * cb_cur - 1;   // source row / column of patch entry (0, 0)
+                const T* pt = tl + 64 + 8 * cc;
+                const Frag g00 = *reinterpret_cast<const Frag*>(pt + ((y0 - oy) * 6 + (x0 - ox)) * ldt);
+                const Frag g01 = *reinterpret_cast<const Frag*>(pt + ((y0 - oy) * 6 + (x1 - ox)) * ldt);
+                const Frag g10 = *reinterpret_cast<const Frag*>(pt + ((y1 - oy) * 6 + (x0 - ox)) * ldt);
+                const Frag g11 = *reinterpret_cast<const Frag*>(pt + ((y1 - oy) * 6 + (x1 - ox)) * ldt);
+                const Frag up = bilinear8<T>(g00, g01, g10, g11, ly, lx);
+                *reinterpret_cast<Frag*>(tl + pix * ldt + 32 + 8 * cc) = up;
+                if (cat)
+                    *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * 64 + 32 + 8 * cc) = up;
+            }
+        } else {
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
 #pragma unroll
         for (int i = 0; i < LP; ++i)
             if (STATIC ? i * 64 < nin : oin[i] >= 0) *reinterpret_cast<Frag*>(tl + oin[i]) = raw[i];
+        }
         if (hasb && bcol < NOP) {
             const bool hb = bias != nullptr && bcol < NO;
             *reinterpret_cast<float4*>(bl + half * NOP + bcol) =
@@ -322,7 +445,13 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // fragments are in registers: the buffer may be overwritten
-        if (tile + nw < ntiles) load_tile(tile + nw);  // next tile in flight during the MFMAs and the store
+        if constexpr (MID) {
+            // unconditionally (the last tile asks for itself again, from the caches): behind a branch the loaded
+            // registers are copied into the loop's own at the end of the branch, which waits for the data there
+            load_tile(tile + nw < ntiles ? tile + nw : tile);
+        } else {
+            if (tile + nw < ntiles) load_tile(tile + nw);  // next tile in flight during the MFMAs and the store
+        }
         if (COLSUM && cs_lanes) {
             float* tf = reinterpret_cast<float*>(tl);  // [512 / K lane groups][K]
             *reinterpret_cast<float4*>(tf + lane * 8) = make_float4(cs[0], cs[1], cs[2], cs[3]);
@@ -448,6 +577,14 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 }
                 T* pb = pool + ((long long)pp_cur + wr * (Wimg >> 1) + wc) * NO + ch;
                 *reinterpret_cast<Frag*>(pb) = o;
+            } else if constexpr (MID) {
+                yb = Y + (long long)px_cur * NO;
+                Frag of[LO];
+#pragma unroll
+                for (int i = 0; i < LO; ++i) of[i] = *reinterpret_cast<const Frag*>(tl + oout[i]);
+#pragma unroll
+                for (int i = 0; i < LO; ++i)   // chunks i*64 .. = pixels 4 i .. 4 i + 3 of the tile: image row i / 2, 4 columns
+                    *reinterpret_cast<Frag*>(yb + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * NO + lane * 8) = of[i];
             } else if (STATIC && rows_left >= 32) {  // (an array of its own: one array written on both paths ends up in scratch)
                 Frag of[LO];
 #pragma unroll
@@ -497,6 +634,17 @@ __global__ __launch_bounds__(256, 2) void dense_rows_pool_k(const T* __restrict_
     extern __shared__ uint32_t dsm[];
     dense_rows_body<T, false, true, 128, 64, true>(X, W, bias, nullptr, Y, colsum, N, 128, 64, 1, 8, 2, blockIdx.x,
                                                    gridDim.x, dsm, pool, Himg, Wimg);
+}
+
+// The 64 -> 128 layer on rows made from the two scales of a pyramid block (dense_rows_body, MID).
+template <typename T>
+__global__ __launch_bounds__(256, 2) void dense_mid_rows_k(const T* __restrict__ W, const T* __restrict__ bias,
+                                                        const float* __restrict__ rowbias, T* __restrict__ Y,
+                                                        long long N, int Himg, int Wimg, const MidRows mid) {
+    extern __shared__ uint32_t dsm[];
+    dense_rows_body<T, false, false, 64, 128, false, true>(nullptr, W, bias, rowbias, Y, nullptr, N, 64, 128,
+                                                            Himg * Wimg, 4, 4, blockIdx.x, gridDim.x, dsm, nullptr, Himg,
+                                                            Wimg, &mid);
 }
 
 // The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
@@ -836,6 +984,36 @@ int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void*
         hipLaunchKernelGGL(dense_rows_pool_k<bf16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const bf16_t*)x,
                            (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, colsum, (bf16_t*)pool, N, H, W);
     return check_launch("dense_rows_pool");
+}
+
+// y[N][128] = rows w^T + bias + rowbias[image] for the rows made from a pyramid block's two convolution outputs
+// (dense_rows_body, MID): cf [B,H,W,64], ch [B,H/2,W/2,64]; cat (optional) receives the rows.  -1: not covered (other
+// widths, extents that are not multiples of 4 x 8, fp32).
+int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void* w, const void* bias,
+                          const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s) {
+    if (dtype == kF32 || I != 64 || D != 128 || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
+    if (tune_env("PDW_NO_DENSE_MID")) return -1;
+    const long long N = (long long)B * H * W;
+    if (N > 0x7fffffffLL / 128) return -1;
+    for (const void* p : {cf, ch, w, (const void*)y})
+        if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
+    if ((reinterpret_cast<uintptr_t>(cat) & 15) || (reinterpret_cast<uintptr_t>(rowbias) & 15) ||
+        (reinterpret_cast<uintptr_t>(bias) & 7))
+        return -1;
+    const long long ntiles = N / 32;
+    long long blocks = (ntiles + 3) / 4;
+    const int cap = tune_env("PDW_DENSE_BLOCKS") ? atoi(tune_env("PDW_DENSE_BLOCKS")) : 512;
+    if (blocks > cap) blocks = cap;
+    const size_t lds = ((size_t)4 * 32 * (64 + 8) + 4 * 32 * (128 + 8)) * 2 +
+                       ((bias || rowbias) ? (size_t)4 * 2 * 4 * 32 * sizeof(float) : 0);
+    const MidRows mid{cf, ch, cat, sqrtf((float)(I / 2))};
+    if (dtype == kF16)
+        hipLaunchKernelGGL(dense_mid_rows_k<f16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const f16_t*)w,
+                           (const f16_t*)bias, rowbias, (f16_t*)y, N, H, W, mid);
+    else
+        hipLaunchKernelGGL(dense_mid_rows_k<bf16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const bf16_t*)w,
+                           (const bf16_t*)bias, rowbias, (bf16_t*)y, N, H, W, mid);
+    return check_launch("dense_mid_rows");
 }
 
 static void dense_wgrad_plan(long long N, int* blocks, int* stages_per_block) {

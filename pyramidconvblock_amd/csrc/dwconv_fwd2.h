@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "dwconv_tz.h"
+#include "pool_branch.h"
 
 namespace pdw {
 
@@ -21,6 +22,7 @@ struct Fwd2Args {
     void *y0, *y1;
     TzGeom g0, g1;
     int s0, n0, s1, n1;   // first workgroup and number of workgroups of each problem
+    PoolFwdJob mean;      // workgroups behind both problems (one per image, mean.B of them): the block's mean branch
 };
 
 // MODE 0: the convolutions; 4: each with the gate applied in its store (dwconv_tz.h), 16 channels per workgroup only.
@@ -30,9 +32,18 @@ __global__ __launch_bounds__(512, 1) void dwconv_fwd2_k(const Fwd2Args a) {
     if (blk - (unsigned)a.s0 < (unsigned)a.n0)
         dwconv_tz_body<T, K, 16, CS, MODE>((const T*)a.x0, (const T*)a.w0, nullptr, nullptr, (T*)a.y0, a.g0, (int)blk - a.s0,
                                            a.n0);
-    else
+    else if (blk - (unsigned)a.s1 < (unsigned)a.n1)
         dwconv_tz_body<T, K, NPC1, CS, MODE>((const T*)a.x1, (const T*)a.w1, nullptr, nullptr, (T*)a.y1, a.g1,
                                              (int)blk - a.s1, a.n1);
+    else {
+        // The mean branch (per-image mean -> conv_pool -> the row added to every output row of the image) needs a
+        // launch whose memory system is not saturated, and its inputs are ready when this one starts: last in the
+        // grid, its short workgroups go to compute units the convolutions leave free or have finished with.
+        extern __shared__ uint32_t smem[];
+        pool_branch_fwd_v8_body<T>(a.mean.part, a.mean.nchunks, a.mean.D, a.mean.inv_p, (const T*)a.mean.wp,
+                                   (const T*)a.mean.bp, (const T*)a.mean.bo, (T*)a.mean.m, a.mean.rowbias,
+                                   (int)blk - a.n0 - a.n1, reinterpret_cast<float*>(smem));
+    }
 }
 
 // Workgroups dealt in grid order to the earliest free of 256 compute units: the time the last one ends.
@@ -114,7 +125,7 @@ static Fwd2Plan fwd2_plan(int B, const TzGeom& g0, const TzGeom& g1) {
 template <int K>
 static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
                        int W, int C, int dtype, hipStream_t s, const TzGate* gate0 = nullptr,
-                       const TzGate* gate1 = nullptr) {
+                       const TzGate* gate1 = nullptr, const PoolFwdJob* mean = nullptr) {
     constexpr int CS = (2 * 4 * TzShape<K, 16, 16>::NM + 2 * 4 * TzShape<K, 16, 16>::RING) <= 160 ? 16 : 8;
     if (dtype == kF32 || C % 8 != 0 || (H & 1) || (W & 1) || B < 1 || H < 2 || W < 2) return -1;
     if ((gate0 != nullptr) != (gate1 != nullptr) || (gate0 && CS != 16)) return -1;
@@ -144,13 +155,16 @@ static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1,
     a.g1.BR = rows_of(a.g1.OH, plan.nb[1]), a.g1.nbands = cdiv(a.g1.OH, a.g1.BR);
     n0 = (long long)cdiv(B, TzShape<K, 16, CS>::NI) * a.g0.nbands * a.g0.ncolt * a.g0.nslices;
     n1 = (long long)cdiv(B, wide1 ? TzShape<K, 16, CS>::NI : TzShape<K, 8, CS>::NI) * a.g1.nbands * a.g1.ncolt * a.g1.nslices;
-    if (n0 + n1 > 0x7fffffffLL) return -1;
+    const int nmean = mean ? mean->B : 0;
+    if (n0 + n1 + nmean > 0x7fffffffLL) return -1;
+    a.mean = mean ? *mean : PoolFwdJob{};
     a.x0 = x0, a.w0 = w0, a.y0 = y0, a.x1 = x1, a.w1 = w1, a.y1 = y1;
     a.n0 = (int)n0, a.n1 = (int)n1;
     a.s0 = plan.first == 0 ? 0 : a.n1, a.s1 = plan.first == 0 ? a.n0 : 0;
     size_t lds = TzShape<K, 16, CS>::lds_bytes;
     if (!wide1 && TzShape<K, 8, CS>::lds_bytes > lds) lds = TzShape<K, 8, CS>::lds_bytes;
-    const unsigned grid = (unsigned)(n0 + n1);
+    if (nmean > 0 && lds < (size_t)9 * mean->D * sizeof(float)) lds = (size_t)9 * mean->D * sizeof(float);
+    const unsigned grid = (unsigned)(n0 + n1 + nmean);
     static std::once_flag once[8];
 #define PDW_FWD2_GO(T, NPC1, MODE, SLOT)                                                                              \
     {                                                                                                                 \

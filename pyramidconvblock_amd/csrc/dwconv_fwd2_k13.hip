@@ -5,8 +5,9 @@
 namespace pdw {
 
 int dwconv_fwd2_k13(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H, int W,
-                    int C, int dtype, hipStream_t s, const TzGate* gate0, const TzGate* gate1) {
-    return launch_fwd2<13>(x0, w0, y0, x1, w1, y1, B, H, W, C, dtype, s, gate0, gate1);
+                    int C, int dtype, hipStream_t s, const TzGate* gate0, const TzGate* gate1,
+                    const PoolFwdJob* mean) {
+    return launch_fwd2<13>(x0, w0, y0, x1, w1, y1, B, H, W, C, dtype, s, gate0, gate1, mean);
 }
 
 }  // namespace pdw

@@ -108,6 +108,10 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
 // 2x2 average pool of y; -1 = not covered
 int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
                            int H, int W, int K, int NO, int dtype, hipStream_t s);
+// the 64 -> 128 layer on rows made from the two convolution outputs of a pyramid block (gates and resize where the
+// tile is staged); cat (optional) receives the rows; -1 = not covered
+int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void* w, const void* bias,
+                          const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s);
 int dense_colsum_supported(int K, int NO, int dtype);
 int dense_colsum_rows();
 int dense_wgrad_supported(int M, int NO, int dtype);
@@ -133,6 +137,6 @@ bool dwconv_fwd2_covers(int B, int H, int W, int C, int K, int dtype);
 // ych0 / ych1)
 int dwconv_fwd2_launch(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
                        int W, int C, int K, int dtype, hipStream_t s, int ldy0 = 0, int ych0 = 0, int ldy1 = 0,
-                       int ych1 = 0);
+                       int ych1 = 0, const struct PoolFwdJob* mean = nullptr);
 
 }  // namespace pdw

@@ -6,6 +6,8 @@
 // no atomics and results are bit-reproducible.
 #include "common.h"
 #include "kernels.h"
+#include "bilinear.h"
+#include "pool_branch.h"
 
 namespace pdw {
 
@@ -85,31 +87,7 @@ __global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T
     store_f32<T, VEC>(dst, acc);
 }
 
-// ---------------------------------------------------------------- bilinear, align_corners=False
-// src = max(scale*(dst+0.5)-0.5, 0), i0 = floor(src), i1 = min(i0+1, in-1), lam = src - i0 (fp32, as ATen does
-// for every element type up to float).
-__device__ __forceinline__ void bl_src(int dst, float scale, int in, int& i0, int& i1, float& lam) {
-    float src = scale * ((float)dst + 0.5f) - 0.5f;
-    src = src < 0.f ? 0.f : src;
-    int lo = (int)src;
-    lo = lo > in - 1 ? in - 1 : lo;
-    i0 = lo;
-    i1 = lo + (lo < in - 1 ? 1 : 0);
-    lam = src - (float)lo;
-}
-
-// One resized value from its four taps (row y0: g00, g01; row y1: g10, g11) and bl_src's weights.  The order of the
-// operations and the fused multiply-adds are spelled out and the result is an fp32 value of its own (see gate_f32),
-// so that every kernel that resizes produces the same bits whatever the compiler would contract.
-__device__ __forceinline__ float bl_mix(float g00, float g01, float g10, float g11, float ly, float lx) {
-    const float hy = 1.f - ly, hx = 1.f - lx;
-    const float t0 = __fmaf_rn(lx, g01, __fmul_rn(hx, g00));
-    const float t1 = __fmaf_rn(lx, g11, __fmul_rn(hx, g10));
-    float r = __fmaf_rn(ly, t1, __fmul_rn(hy, t0));
-    asm volatile("" : "+v"(r));
-    return r;
-}
-
+// ---------------------------------------------------------------- bilinear, align_corners=False (bilinear.h)
 template <typename T, int VEC>
 __device__ __forceinline__ void bilinear_fwd_item(const T* __restrict__ x, T* __restrict__ y, int h, int w, int C,
                                                   int H, int W, int ldy, float sy, float sx, long long idx) {
@@ -827,98 +805,6 @@ __device__ __forceinline__ float colsum_parts(const float* __restrict__ pp, int 
     return (s0 + s1) + (s2 + s3);
 }
 
-// sm[c] = sum over q < nchunks of pp[q * D + c] for c < D, by the whole workgroup of 256: thread = (4-column vector
-// tid % 32, chunk lane tid / 32), up to 8 loads of a thread in flight, the 8 chunk lanes combined through
-// red[8][D].  D % 4 == 0, D <= 128.  Ends with a barrier; the order of the additions is fixed.
-__device__ __forceinline__ void colsum_coop(const float* __restrict__ pp, int nchunks, int D, float* sm, float* red) {
-    const int tid = threadIdx.x, cv = tid & 31, ql = tid >> 5;
-    float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0;
-    if (cv * 4 < D) {
-        const float* p = pp + cv * 4;
-        int q = ql;
-        for (; q + 56 < nchunks; q += 64) {
-            float4 v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(p + (long long)(q + 8 * u) * D);
-#pragma unroll
-            for (int u = 0; u < 8; u += 2) {
-                a0.x += v[u].x, a0.y += v[u].y, a0.z += v[u].z, a0.w += v[u].w;
-                a1.x += v[u + 1].x, a1.y += v[u + 1].y, a1.z += v[u + 1].z, a1.w += v[u + 1].w;
-            }
-        }
-        for (; q < nchunks; q += 8) {
-            const float4 v = *reinterpret_cast<const float4*>(p + (long long)q * D);
-            a0.x += v.x, a0.y += v.y, a0.z += v.z, a0.w += v.w;
-        }
-        *reinterpret_cast<float4*>(red + ql * D + cv * 4) =
-            make_float4(a0.x + a1.x, a0.y + a1.y, a0.z + a1.z, a0.w + a1.w);
-    }
-    __syncthreads();
-    if (tid < D) {
-        float t = 0.f;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) t += red[k * D + tid];
-        sm[tid] = t;
-    }
-    __syncthreads();
-}
-
-template <typename T>
-__device__ __forceinline__ void pool_branch_fwd_v8_body(const float* __restrict__ part, int nchunks, int D,
-                                                        float inv_p, const T* __restrict__ wp,
-                                                        const T* __restrict__ bp, const T* __restrict__ bo,
-                                                        T* __restrict__ m, float* __restrict__ rowbias, int b,
-                                                        float* sm) {  // sm: [D] means, [8][D] partial column sums
-    const int tid = threadIdx.x;
-    // weight rows of this thread: outputs o = tid/8 + 32*pass, channel vectors sub + 8*i  (requested first)
-    const int sub = tid & 7, ol = tid >> 3;
-    ChanVec<T, 8> wv[4][2];
-#pragma unroll
-    for (int pass = 0; pass < 4; ++pass)
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int o = ol + 32 * pass, v = sub + 8 * i;
-            const bool ok = o < D && v * 8 < D;
-            wv[pass][i] = *reinterpret_cast<const ChanVec<T, 8>*>(wp + (ok ? (long long)o * D + v * 8 : 0));
-        }
-    // the biases of this thread's outputs, requested here as well: read where they are added, after the last
-    // barrier, they would be eight dependent trips to memory at the end of the workgroup
-    // (unconditional loads from a readable address, converted where they are used: no branch, no early wait)
-    const T* bpp = bp ? bp : wp;
-    const T* bop = bo ? bo : wp;
-    T braw[4][2];
-#pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const int oc = min(ol + 32 * pass, D - 1);
-        braw[pass][0] = bpp[oc], braw[pass][1] = bop[oc];
-    }
-    colsum_coop(part + (long long)b * nchunks * D, nchunks, D, sm, sm + D);
-    if (tid < D) {
-        const T mv = from_f32<T>(sm[tid] * inv_p);
-        m[(long long)b * D + tid] = mv;
-        sm[tid] = to_f32(mv);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const int o = ol + 32 * pass;
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int v = sub + 8 * i;
-            if (o < D && v * 8 < D) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) acc = fmaf(sm[v * 8 + j], to_f32(wv[pass][i].v[j]), acc);
-            }
-        }
-        acc += __shfl_xor(acc, 1);
-        acc += __shfl_xor(acc, 2);
-        acc += __shfl_xor(acc, 4);
-        acc += (bp ? to_f32(braw[pass][0]) : 0.f) + (bo ? to_f32(braw[pass][1]) : 0.f);
-        if (sub == 0 && o < D) rowbias[(long long)b * D + o] = acc;
-    }
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void pool_branch_fwd_v8_k(const float* __restrict__ part, int nchunks, int D,
                                                             float inv_p, const T* __restrict__ wp,
@@ -1055,14 +941,6 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_v8_k(const float* __restr
 
 // ---- the middle of a two-scale block in one launch each way: the (tiny, latency-bound) mean branch rides on the
 // gate kernels.  Its workgroups come first in the grid, the gate workgroups after them.
-struct PoolFwdJob {
-    const float* part;
-    int nchunks, B, D;
-    float inv_p;
-    const void *wp, *bp, *bo;
-    void* m;
-    float* rowbias;
-};
 struct PoolBwdJob {
     const float* part;
     int nchunks, B, D;
@@ -1333,17 +1211,12 @@ int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* g
 
 // The gate pair and the mean branch (from per-chunk sums `parts`) of a two-scale block in one launch; -1 when the
 // combination is not covered (the caller launches the two separately).
-static bool pool_v8_ok(const void* wp, const void* m_or_null, const float* parts, int B, int D, int dtype) {
-    return dtype != kF32 && D % 8 == 0 && D <= 128 && (reinterpret_cast<uintptr_t>(wp) & 15) == 0 &&
-           (reinterpret_cast<uintptr_t>(m_or_null) & 15) == 0 && (reinterpret_cast<uintptr_t>(parts) & 15) == 0 &&
-           (size_t)(B + 16 * D) * sizeof(float) <= 64 * 1024;
-}
 
 int block_mid_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, int W, int h, int w, int I, int ldy,
                          const float* parts, int nparts, const void* wp, const void* bp, const void* bo, void* m,
                          float* rowbias, int P, int D, int dtype, hipStream_t s) {
     const void* ptrs[3] = {xf, xh, y};
-    if (pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 3) != 8 || !pool_v8_ok(wp, nullptr, parts, B, D, dtype))
+    if (pick_vec(gcd_int(I / 2, ldy), esize(dtype), ptrs, 3) != 8 || !pool_branch_v8_ok(wp, nullptr, parts, B, D, dtype))
         return -1;
     const long long tf = (long long)B * H * W * (I / 2 / 8);
     const long long th = (H == 2 * h && W == 2 * w) ? (long long)B * h * w * (I / 2 / 8) : tf;
@@ -1370,7 +1243,7 @@ int bilinear_pool_fwd_launch(const void* x, void* y, int B, int h, int w, int C,
                              int nparts, const void* wp, const void* bp, const void* bo, void* m, float* rowbias, int P,
                              int D, int dtype, hipStream_t s) {
     const void* ptrs[2] = {x, y};
-    if (pick_vec(gcd_int(C, ldy), esize(dtype), ptrs, 2) != 8 || !pool_v8_ok(wp, nullptr, parts, B, D, dtype)) return -1;
+    if (pick_vec(gcd_int(C, ldy), esize(dtype), ptrs, 2) != 8 || !pool_branch_v8_ok(wp, nullptr, parts, B, D, dtype)) return -1;
     const long long total = (long long)B * H * W * (C / 8);
     unsigned blocks;
     if (total == 0) return -1;
@@ -1393,7 +1266,7 @@ int block_mid_bwd_launch(const void* gy, const void* xf, const void* xh, void* g
                          hipStream_t s) {
     if (H != 2 * h || W != 2 * w || h < 2 || w < 2) return -1;
     const void* ptrs[5] = {gy, xf, xh, gxf, gxh};
-    if (pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 5) != 8 || !pool_v8_ok(wp, m, parts, B, D, dtype)) return -1;
+    if (pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 5) != 8 || !pool_branch_v8_ok(wp, m, parts, B, D, dtype)) return -1;
     const long long tf = (long long)B * H * W * (I / 2 / 8), th = (long long)B * h * w * (I / 2 / 8);
     unsigned bf, bh;
     if (tf == 0) return -1;

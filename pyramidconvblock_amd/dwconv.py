@@ -146,6 +146,39 @@ def dwconv_forward2(x0, w0, x1, w1):
     return y0, y1
 
 
+def dwconv_forward2_mean(x0, w0, x1, w1, parts, P, w_pool, b_pool=None, b_out=None):
+    """dwconv_forward2 with the block's mean branch in the same launch (pdw_dwconv_fwd2_mean): returns
+    (conv(x0, w0), conv(x1, w1), m, rowbias) with m [B, D] the per-image mean of the block's input (from the fp32
+    sums `parts` [B * nparts, D] over groups of positions, P positions per image) and rowbias fp32 [B, D] =
+    m w_pool^T + b_pool + b_out; None when the launch does not cover the case."""
+    dev = _lib.require_device(x0, w0, x1, w1, parts, w_pool)
+    L = _lib.lib()
+    K, C = int(w0.shape[0]), int(w0.shape[2])
+    B, H, W = x0.shape[0], x0.shape[1], x0.shape[2]
+    D = int(w_pool.shape[0])
+    dt = x0.dtype
+    if (w0.shape[0] != w0.shape[1] or K % 2 == 0 or w1.shape != w0.shape or tuple(x1.shape) != (B, H // 2, W // 2, C)
+            or H % 2 or W % 2 or x0.shape[3] != C or B == 0 or parts.dtype != torch.float32 or parts.shape[0] % B
+            or tuple(w_pool.shape) != (D, D) or parts.shape[1] != D
+            or any(t is not None and t.dtype != dt for t in (w0, x1, w1, w_pool, b_pool, b_out))):
+        return None
+    args = [t.contiguous() for t in (x0, w0, x1, w1, parts, w_pool)]
+    y0, y1 = torch.empty_like(args[0]), torch.empty_like(args[2])
+    m = torch.empty((B, D), device=dev, dtype=dt)
+    rowbias = torch.empty((B, D), device=dev, dtype=torch.float32)
+    with _lib.on_device(dev):
+        st = L.pdw_dwconv_fwd2_mean(args[0].data_ptr(), args[1].data_ptr(), y0.data_ptr(), args[2].data_ptr(),
+                                    args[3].data_ptr(), y1.data_ptr(), B, H, W, C, K, args[4].data_ptr(),
+                                    parts.shape[0] // B, args[5].data_ptr(),
+                                    b_pool.data_ptr() if b_pool is not None else None,
+                                    b_out.data_ptr() if b_out is not None else None, m.data_ptr(), rowbias.data_ptr(),
+                                    int(P), D, _lib.dtype_code(dt), _lib.stream_ptr(dev))
+    if st == 3:
+        return None
+    _lib.check(st, "pdw_dwconv_fwd2_mean")
+    return y0, y1, m, rowbias
+
+
 def dwconv_bwd3(gy0, w0, gp, x0, x1, gy1):
     """The end of a two-scale block's backward pass as one call of the library (pdw_dwconv_bwd3): returns
     (dx, dw0, dw1) = (dwconv_dgrad(gy0, w0, pooled_grad=gp), dwconv_wgrad(x0, gy0), dwconv_wgrad(x1, gy1)) for 'same'

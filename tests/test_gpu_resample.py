@@ -385,3 +385,77 @@ def test_sum_parts_is_the_fp32_sum_rounded_once(shape, dtype):
     eps = {torch.float32: 2.0 ** -24, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
     tol = eps * ref.abs() + shape[0] * 2.0 ** -24 * parts.abs().double().sum(0) + 1e-7
     assert bool(((out.double().cpu() - ref).abs() <= tol).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_cat", [True, False])
+@pytest.mark.parametrize("case", [(32, 56, 56, 64, 128), (1, 4, 8, 64, 128), (3, 8, 16, 64, 128), (2, 12, 40, 64, 128),
+                                  (2, 64, 8, 64, 128), (5, 36, 24, 64, 128), (2, 10, 16, 64, 128), (2, 8, 16, 32, 64),
+                                  (70, 8, 8, 64, 128)])
+def test_dense_forward_gated_is_the_gates_then_the_layer(oracle, dtype, with_cat, case):
+    """pdw_dense_fwd_gated (the block's output layer on rows it makes from the two convolution outputs: both gates and
+    the resize where the tile is staged) gives bitwise what the gate launch followed by the plain layer gives, with
+    and without writing the rows out, and the oracle's values; where the kernel does not cover the case (other widths,
+    extents off 4 x 8, fp32) it says so and launches nothing."""
+    from pyramidconvblock_amd import ops
+
+    B, H, W, I, D = case
+    gen = torch.Generator().manual_seed(H * W + B)
+    cf = randn(gen, B, H, W, I).to(dtype).cuda()
+    ch = randn(gen, B, H // 2, W // 2, I).to(dtype).cuda()
+    w = (randn(gen, D, I) / 8).to(dtype).cuda()
+    rowbias = randn(gen, B, D).cuda()
+    cat = torch.full((B, H, W, I), 5.0, device="cuda", dtype=dtype) if with_cat else None
+    y = ops.dense_forward_gated(cf, ch, w, rowbias=rowbias, cat=cat)
+    covered = dtype != torch.float32 and (I, D) == (64, 128) and H % 4 == 0 and W % 8 == 0
+    assert (y is not None) == covered
+    if y is None:
+        return
+    want_cat = torch.empty((B, H, W, I), device="cuda", dtype=dtype)
+    ops.gate_pair_forward(cf, ch, want_cat)
+    want = ops.dense_forward(want_cat, w, rowbias=rowbias, rows_per_image=H * W)
+    torch.cuda.synchronize()
+    if with_cat:
+        assert torch.equal(cat, want_cat)
+    assert torch.equal(y, want)
+    if B * H * W <= 4096:   # and against the oracle, directly
+        g0 = oracle.gate_fwd(cf.double().cpu().numpy())
+        g1 = oracle.bilinear_fwd(oracle.gate_fwd(ch.double().cpu().numpy()), (H, W))
+        rows = torch.cat([torch.from_numpy(g0), torch.from_numpy(g1)], -1)
+        yo = rows @ w.double().cpu().t() + rowbias.double().cpu()[:, None, None, :]
+        assert_close(y, yo.numpy(), dtype, "y")
+    y2 = ops.dense_forward_gated(cf, ch, w)   # no per-image rows
+    assert torch.equal(y2, ops.dense_forward(want_cat, w))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("case", [(32, 56, 56, 64, 13, 128), (2, 40, 36, 32, 9, 64), (64, 56, 56, 64, 11, 128),
+                                  (3, 34, 70, 16, 3, 24), (1, 36, 40, 48, 15, 96), (2, 20, 24, 40, 9, 80),
+                                  (4, 56, 56, 64, 7, 136)])
+@pytest.mark.parametrize("biases", [(True, True), (False, False)])
+def test_fwd2_mean_is_the_convolutions_and_the_mean_branch(dtype, case, biases):
+    """pdw_dwconv_fwd2_mean (both convolutions and the block's mean branch in one launch) gives bitwise the results of
+    pdw_dwconv_fwd2 and pdw_pool_branch_fwd_parts; status 3 where either part is not covered."""
+    from pyramidconvblock_amd import ops
+    from pyramidconvblock_amd.dwconv import dwconv_forward2, dwconv_forward2_mean
+
+    B, H, W, C, k, D = case
+    gen = torch.Generator().manual_seed(B + k)
+    x0 = randn(gen, B, H, W, C).to(dtype).cuda()
+    x1 = randn(gen, B, H // 2, W // 2, C).to(dtype).cuda()
+    w0, w1 = ((randn(gen, k, k, C) / k).to(dtype).cuda() for _ in range(2))
+    nparts = 5
+    parts = randn(gen, B * nparts, D).cuda()
+    wp = (randn(gen, D, D) / 8).to(dtype).cuda()
+    bp, bo = ((randn(gen, D).to(dtype).cuda() if b else None) for b in biases)
+    got = dwconv_forward2_mean(x0, w0, x1, w1, parts, H * W, wp, bp, bo)
+    convs = dwconv_forward2(x0, w0, x1, w1)
+    covered = convs is not None and D % 8 == 0 and D <= 128
+    assert (got is not None) == covered
+    if got is None:
+        return
+    x = torch.empty(B, H * W, D, device="cuda", dtype=dtype)   # (only its shape is used when parts are given)
+    m, rowbias = ops.pool_branch_forward(x, wp, bp, bo, parts=parts)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0], convs[0]) and torch.equal(got[1], convs[1])
+    assert torch.equal(got[2], m) and torch.equal(got[3], rowbias)
