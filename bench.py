@@ -25,7 +25,14 @@ import os
 import sys
 import time
 
-import torch
+# How the HIP runtime submits a graph replay (a host-side setting of ROCm's runtime, read when it loads; it changes no
+# kernel and no result): with this image's default, every replay of a captured step costs about 4 us more on the GPU
+# than with the kernels submitted as ordinary dispatches.  Set before torch loads the runtime; a value given in the
+# environment wins.  The line reports the setting, and the step's time under the runtime's default beside `value`.
+GRAPH_SUBMIT_ENV = "DEBUG_CLR_GRAPH_PACKET_CAPTURE"
+os.environ.setdefault(GRAPH_SUBMIT_ENV, "0")
+
+import torch  # noqa: E402
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
@@ -561,6 +568,7 @@ def main():
                     "{fwd,dgrad,wgrad}_{full,half}, fwd2, bwd3, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
                     "dense_{fwd,pool,dgrad,wgrad,pair}, step, copy")
     ap.add_argument("--torch-gpu-only", action="store_true", help="(internal) time the torch-operator comparator and exit")
+    ap.add_argument("--headline-only", action="store_true", help="(internal) time the headline step only and exit")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -582,6 +590,10 @@ def main():
         return
 
     m = make_block(D, k, dtype)
+    if args.headline_only:
+        head = measure_block(m, (B, H, W, D), dtype, "normal", args.steps, args.warmup, with_forward=False)
+        print(json.dumps({"fwd_bwd_ms": head["fwd_bwd_ms"], "fwd_bwd_ms_warm": head["fwd_bwd_ms_warm"]}))
+        return
     head = measure_block(m, (B, H, W, D), dtype, "normal", args.steps, args.warmup)
     t_chain, n_chain = measure_block_in_one_graph(m, (B, H, W, D), dtype, args.steps, args.warmup)
     # eager launches of the same step (host-bound), for reference
@@ -624,6 +636,7 @@ def main():
         "warm_fwd_ms": head["fwd_ms_warm"],
         "eager_ms_per_step": t_eager * 1e3,
         "launch": "one HIP graph replay per step (eager launch time in eager_ms_per_step)",
+        "runtime_settings": {GRAPH_SUBMIT_ENV: os.environ.get(GRAPH_SUBMIT_ENV)},
         "in_graph_ms_per_step": t_chain,
         "in_graph_note": f"{n_chain} steps (one per buffer set) captured in ONE graph, time per replay / {n_chain}: the "
                          "block as one of several layers of a captured model; `value` instead pays the idle time "
@@ -709,6 +722,24 @@ def main():
             if "call_seconds" in r:   # the call with its share of the deferred summation launches
                 row["call_us"] = round(r["call_seconds"] * 1e6, 2)
             result["kernels"].append(row)
+
+    if os.environ.get(GRAPH_SUBMIT_ENV) == "0":
+        # the same step under the runtime's default graph submission, in a child process (the setting is read once)
+        import subprocess
+
+        try:
+            env = dict(os.environ)
+            env[GRAPH_SUBMIT_ENV] = "1"
+            cp = subprocess.run([sys.executable, os.path.abspath(__file__), "--headline-only", "--steps", str(args.steps),
+                                 "--warmup", str(args.warmup)], capture_output=True, text=True, timeout=240, env=env)
+            d = json.loads(cp.stdout.strip().splitlines()[-1])
+            result["default_runtime_ms_per_step"] = d["fwd_bwd_ms"]
+            result["default_runtime_warm_ms_per_step"] = d["fwd_bwd_ms_warm"]
+            result["default_runtime_note"] = (f"the rotated / warm step with {GRAPH_SUBMIT_ENV}=1, this image's default: the "
+                                              "runtime replays pre-built dispatch packets, which costs more per replay here")
+        except Exception as e:  # noqa: BLE001
+            result["default_runtime_ms_per_step"] = None
+            result["default_runtime_note"] = f"{type(e).__name__}: {e}"[:300]
 
     if not args.no_torch_gpu:
         # in a child process with a time limit: the library may build its kernels on first use

@@ -75,7 +75,8 @@ int pdw_dwconv_fwd_pool(const void *x, const void *w, void *y, void *xp, int B, 
  * conv_block.py:43, so that the convolution output itself never reaches HBM.  The product is formed from the rounded
  * convolution outputs in fp32 and rounded once, as pdw_gate_fwd does.  xp (may be NULL): the 2x2 average pool of x,
  * [B,H/2,W/2,C] (needs even H, W, pad and 2*pad = K-1).  Returns 3 when the fused kernel does not cover the case
- * (it needs a 16-bit dtype, C % 16 == 0, odd K <= 13, ldy and ych multiples of 8): the caller then runs pdw_dwconv_fwd
+ * (it needs a 16-bit dtype, C % 16 == 0, odd K <= 17, ldy and ych multiples of 8, and K <= 13 when xp is asked for): the
+ * caller then runs pdw_dwconv_fwd
  * (or pdw_dwconv_fwd_pool) and pdw_gate_fwd.  No counterpart in the reference, which keeps the convolution output for
  * its backward. */
 int pdw_dwconv_fwd_gate(const void *x, const void *w, void *y, void *xp, int B, int H, int W, int C, int K, int pad,
@@ -196,15 +197,17 @@ int pdw_dwconv_fwd2(const void *x0, const void *w0, void *y0, const void *x1, co
  * kernel left in parts [B][nparts][D] (pdw_dense_fwd_colsum): what pdw_pool_branch_fwd_parts computes, bitwise.  The
  * branch is three dependent trips to memory and a few kilobytes; in a launch of its own, or in one that saturates the
  * memory system, it costs microseconds, here it runs beside the convolutions.  Status 3 (nothing launched) where
- * pdw_dwconv_fwd2 does not take the case or the branch is not covered (D % 8, D > 128). */
-int pdw_dwconv_fwd2_mean(const void *x0, const void *w0, void *y0, const void *x1, const void *w1, void *y1, int B,
-                         int H, int W, int C, int K, const float *parts, int nparts, const void *w_pool,
-                         const void *b_pool, const void *b_out, void *m, float *rowbias, int P, int D, int dtype,
-                         void *stream);
+ * pdw_dwconv_fwd2 does not take the case or the branch is not covered (D % 8, D > 128).  ldy0 = ldy1 = 0: the
+ * convolution outputs y0, y1 as pdw_dwconv_fwd2 writes them; both > 0: the gated outputs of pdw_dwconv_fwd2_gate at these
+ * pixel strides and channel offsets (inference). */
+int pdw_dwconv_fwd2_mean(const void *x0, const void *w0, void *y0, int ldy0, int ych0, const void *x1, const void *w1,
+                         void *y1, int ldy1, int ych1, int B, int H, int W, int C, int K, const float *parts,
+                         int nparts, const void *w_pool, const void *b_pool, const void *b_out, void *m,
+                         float *rowbias, int P, int D, int dtype, void *stream);
 
 /* pdw_dwconv_fwd2 with the gate of pdw_dwconv_fwd_gate applied in the store of each scale (inference: neither
  * convolution output reaches HBM): y0[b,i,j, ych0 + c] and y1[b,i,j, ych1 + c], c < C/2, at pixel strides of ldy0 / ldy1
- * channels (0: C/2).  Covered where pdw_dwconv_fwd2 is and C % 16 == 0, K <= 13, strides and offsets multiples of 8;
+ * channels (0: C/2).  Covered where pdw_dwconv_fwd2 is and C % 16 == 0, strides and offsets multiples of 8;
  * status 3 otherwise (the caller then makes two pdw_dwconv_fwd_gate calls).  Results bitwise those calls'. */
 int pdw_dwconv_fwd2_gate(const void *x0, const void *w0, void *y0, int ldy0, int ych0, const void *x1, const void *w1,
                          void *y1, int ldy1, int ych1, int B, int H, int W, int C, int K, int dtype, void *stream);
@@ -357,10 +360,13 @@ int pdw_dense_fwd_colsum_pool(const void *x, const void *w, const void *bias, vo
  * rowbias[b], with cf[B,H,W,I] and ch[B,H/2,W/2,I] the convolution outputs of the two scales, gate(v) = v[:I/2] *
  * v[I/2:] * sqrt(I/2) rounded to `dtype`, w[D][I], bias[D] or NULL, rowbias fp32 [B][D] or NULL.  cat[B,H,W,I] (or
  * NULL) receives the rows, which the backward pass reads again.  Bitwise what pdw_gate_pair_fwd (or pdw_block_mid_fwd)
- * followed by pdw_dense_fwd produce; the gated tensor is not read back from memory.  Status 3 (nothing launched)
- * where not covered: 16-bit types, I = 64, D = 128, H % 4 == 0, W % 8 == 0 only. */
+ * followed by pdw_dense_fwd produce; the gated tensor is not read back from memory.  ldf > 0 (inference, after
+ * pdw_dwconv_fwd2_gate): both scales arrive gated, cf[B,H,W,I/2] at a pixel stride of ldf values and ch[B,H/2,W/2,I/2],
+ * only the resize is left to do and cat must be NULL.  Status 3 (nothing launched) where not covered: 16-bit types,
+ * I = 64, D = 128, H % 4 == 0, W % 8 == 0 only. */
 int pdw_dense_fwd_gated(const void *cf, const void *ch, void *cat, const void *w, const void *bias,
-                        const float *rowbias, void *y, int B, int H, int W, int I, int D, int dtype, void *stream);
+                        const float *rowbias, void *y, int B, int H, int W, int I, int D, int ldf, int dtype,
+                        void *stream);
 
 /* Weight gradient of such a layer: dw[m,o] = sum_n a[n,m] * b[n,o]  (a[N,M], b[N,NO] -> dw[M,NO]), fp32
  * accumulation, two deterministic passes through `workspace` (no atomics). */

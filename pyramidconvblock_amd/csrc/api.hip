@@ -321,9 +321,10 @@ int pdw_dwconv_fwd2(const void* x0, const void* w0, void* y0, const void* x1, co
     return r;
 }
 
-int pdw_dwconv_fwd2_mean(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
-                         int W, int C, int K, const float* parts, int nparts, const void* w_pool, const void* b_pool,
-                         const void* b_out, void* m, float* rowbias, int P, int D, int dtype, void* stream) {
+int pdw_dwconv_fwd2_mean(const void* x0, const void* w0, void* y0, int ldy0, int ych0, const void* x1, const void* w1,
+                         void* y1, int ldy1, int ych1, int B, int H, int W, int C, int K, const float* parts, int nparts,
+                         const void* w_pool, const void* b_pool, const void* b_out, void* m, float* rowbias, int P, int D,
+                         int dtype, void* stream) {
     const int Pd = K / 2;
     if (!(K & 1)) return set_error("pdw_dwconv_fwd2_mean: odd filter size needed (K=%d)", K), 1;
     if ((H & 1) || (W & 1)) return set_error("pdw_dwconv_fwd2_mean: even extents needed (H=%d W=%d)", H, W), 1;
@@ -332,10 +333,15 @@ int pdw_dwconv_fwd2_mean(const void* x0, const void* w0, void* y0, const void* x
     if (B < 1 || P < 1 || D < 1 || nparts < 1)
         return set_error("pdw_dwconv_fwd2_mean: bad extents B=%d P=%d D=%d nparts=%d", B, P, D, nparts), 1;
     if (!parts || !w_pool || !m || !rowbias) return set_error("pdw_dwconv_fwd2_mean: null pointer"), 1;
+    if ((ldy0 > 0) != (ldy1 > 0) || ldy0 < 0 || ldy1 < 0 || ych0 < 0 || ych1 < 0 ||
+        (ldy0 > 0 && ((C & 1) || ldy0 < ych0 + C / 2 || ldy1 < ych1 + C / 2)))
+        return set_error("pdw_dwconv_fwd2_mean: gated stores need even C and ych + C/2 <= ldy for both scales (C=%d ldy=%d,%d "
+                         "ych=%d,%d)", C, ldy0, ldy1, ych0, ych1), 1;
     int r = -1;
     if (pool_branch_v8_ok(w_pool, m, parts, B, D, dtype) && !(reinterpret_cast<uintptr_t>(rowbias) & 15)) {
         const PoolFwdJob job{parts, nparts, B, D, 1.f / (float)P, w_pool, b_pool, b_out, m, rowbias};
-        r = dwconv_fwd2_launch(x0, w0, y0, x1, w1, y1, B, H, W, C, K, dtype, (hipStream_t)stream, 0, 0, 0, 0, &job);
+        r = dwconv_fwd2_launch(x0, w0, y0, x1, w1, y1, B, H, W, C, K, dtype, (hipStream_t)stream, ldy0, ych0, ldy1, ych1,
+                               &job);
     }
     if (r == -1)
         return set_error("pdw_dwconv_fwd2_mean: case not covered (B=%d H=%d W=%d C=%d K=%d D=%d dtype=%d)", B, H, W, C, K, D,
@@ -625,13 +631,15 @@ int pdw_dense_fwd_colsum_pool(const void* x, const void* w, const void* bias, vo
 }
 
 int pdw_dense_fwd_gated(const void* cf, const void* ch, void* cat, const void* w, const void* bias, const float* rowbias,
-                        void* y, int B, int H, int W, int I, int D, int dtype, void* stream) {
+                        void* y, int B, int H, int W, int I, int D, int ldf, int dtype, void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd_gated: unknown dtype %d", dtype), 1;
     if (B < 0 || H < 2 || W < 2 || (H & 1) || (W & 1) || I < 2 || (I & 1) || D < 1)
         return set_error("pdw_dense_fwd_gated: bad extents B=%d H=%d W=%d I=%d D=%d", B, H, W, I, D), 1;
     if (B > 0 && (!cf || !ch || !w || !y)) return set_error("pdw_dense_fwd_gated: null pointer"), 1;
+    if (ldf < 0 || (ldf > 0 && (ldf < I / 2 || cat)))
+        return set_error("pdw_dense_fwd_gated: gated inputs need ldf >= I/2 and no cat (ldf=%d I=%d)", ldf, I), 1;
     if (B == 0) return 0;
-    const int r = dense_mid_rows_launch(cf, ch, cat, w, bias, rowbias, y, B, H, W, I, D, dtype, (hipStream_t)stream);
+    const int r = dense_mid_rows_launch(cf, ch, cat, w, bias, rowbias, y, B, H, W, I, D, dtype, (hipStream_t)stream, ldf);
     if (r == -1)
         return set_error("pdw_dense_fwd_gated: case not covered (B=%d H=%d W=%d I=%d D=%d dtype=%d)", B, H, W, I, D, dtype), 3;
     return r;

@@ -99,8 +99,8 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
         if (pooled == 3)
             if (int e = pdw_avgpool_fwd(a, xp, B, H, W, I, s.h, s.w, dtype, stream)) return e;
         // (with the mean branch in the same launch where that is covered: mean -> conv_pool (+ both biases) into yp)
-        both = pdw_dwconv_fwd2_mean(a, w_dw0, c0, xp, w_dw1, c1, B, H, W, I, K, xparts, (int)(s.nt / B), w_pool, b_pool,
-                                    b_out, m, yp, s.P, D, dtype, stream);
+        both = pdw_dwconv_fwd2_mean(a, w_dw0, c0, 0, 0, xp, w_dw1, c1, 0, 0, B, H, W, I, K, xparts, (int)(s.nt / B), w_pool,
+                                    b_pool, b_out, m, yp, s.P, D, dtype, stream);
         if (both != 0 && both != 3) return both;
         mean_done = both == 0;
         if (both == 3) both = pdw_dwconv_fwd2(a, w_dw0, c0, xp, w_dw1, c1, B, H, W, I, K, dtype, stream);
@@ -115,7 +115,7 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
     if (mean_done) {
         // conv_out on rows it makes itself (both gates, the resize), written to cat for the backward; where its kernel
         // does not cover the widths, the gates' launch and the plain layer                   (conv_block.py:40-44, 49)
-        const int r = pdw_dense_fwd_gated(c0, c1, cat, w_out, nullptr, yp, y, B, H, W, I, D, dtype, stream);
+        const int r = pdw_dense_fwd_gated(c0, c1, cat, w_out, nullptr, yp, y, B, H, W, I, D, 0, dtype, stream);
         if (r != 3) return r;
         if (int e = pdw_gate_pair_fwd(c0, c1, cat, B, H, W, s.h, s.w, I, I, dtype, stream)) return e;
         return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
@@ -128,9 +128,8 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
     return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
 }
 
-// The fused convolution + gate needs 16 channels per workgroup, which the operand registers allow up to K = 13, and
-// images small enough for the kernel's 32-bit offsets (two images side by side).
-static bool infer_fused(int H, int W, int I, int K) { return K <= 13 && (long long)H * W * I * 2 <= 0x1fffffffLL; }
+// The fused convolution + gate needs images small enough for the kernel's 32-bit offsets (two images side by side).
+static bool infer_fused(int H, int W, int I, int K) { return K <= 17 && (long long)H * W * I * 2 <= 0x1fffffffLL; }
 
 size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
     if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
@@ -181,6 +180,15 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
         const int pooled = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream);
         if (pooled != 0 && pooled != 3) return pooled;
         if (pooled == 0) {
+            // with the mean branch in the same launch, and then conv_out on rows it puts together itself (the full scale's
+            // gate, written G wide, and the resized half scale's), where its kernel covers the widths and extents: three
+            // launches                                                                        (conv_block.py:41-49)
+            if (I == 64 && D == 128 && H % 4 == 0 && W % 8 == 0 && !(reinterpret_cast<uintptr_t>(w_out) & 15)) {
+                both = pdw_dwconv_fwd2_mean(a, w_dw0, cat, G, 0, xp, w_dw1, g1, G, 0, B, H, W, I, K, xparts, (int)(s.nt / B),
+                                            w_pool, b_pool, b_out, m, yp, s.P, D, dtype, stream);
+                if (both == 0) return pdw_dense_fwd_gated(cat, g1, nullptr, w_out, nullptr, yp, y, B, H, W, I, D, G, dtype, stream);
+                if (both != 3) return both;
+            }
             both = pdw_dwconv_fwd2_gate(a, w_dw0, cat, I, 0, xp, w_dw1, g1, G, 0, B, H, W, I, K, dtype, stream);
             if (both != 0 && both != 3) return both;
         } else if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) {
@@ -197,7 +205,7 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
     if (both == 3) {
         // scale 1: conv + gate into cat[..., :G], and the pooled input of scale 1/2            (conv_block.py:14-19)
         // (the convolution's staging threads hold whole pool windows only when the padding is even)
-        const bool pool_fused = (pad & 1) == 0;
+        const bool pool_fused = (pad & 1) == 0 && K <= 13;   // (with 16 channels per workgroup only)
         if (int e = pdw_dwconv_fwd_gate(a, w_dw0, cat, pool_fused ? xp : nullptr, B, H, W, I, K, pad, I, 0, dtype, stream))
             return e;
         if (!pool_fused)

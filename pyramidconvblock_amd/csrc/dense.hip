@@ -162,9 +162,12 @@ struct WTransposer {
 // and the tile's 32 pixels take their four taps from there (gated per output pixel it would be 4 gates per value
 // instead of 0.75).  The rows are also written to mid->cat ([B, Himg, Wimg, 64], when not null): the arithmetic, and
 // therefore every bit, is that of the gate kernels followed by this layer on their output.
+// MID = 2: both scales arrive gated (cf [B, Himg, Wimg, 32] at a pixel stride of ldf values, ch [B, Himg/2, Wimg/2, 32]):
+// the inference forward, whose convolutions gate in their stores; nothing but y is written.
 struct MidRows {
     const void *cf, *ch;
     void* cat;
+    int ldf;
     float gs;
 };
 
@@ -204,7 +207,7 @@ __device__ __forceinline__ Frag bilinear8(const Frag& g00, const Frag& g01, cons
     return o;
 }
 
-template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0, bool POOL = false, bool MID = false>
+template <typename T, bool KMAJOR, bool COLSUM, int SK = 0, int SNO = 0, bool POOL = false, int MID = 0>
 __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T* __restrict__ W,
                                                 const T* __restrict__ bias, const float* __restrict__ rowbias,
                                                 T* __restrict__ Y, float* __restrict__ colsum, long long N, int Kd,
@@ -213,7 +216,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                                                 int Wimg = 0, const MidRows* mid = nullptr) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
     static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
-    static_assert(!MID || (SK == 64 && SNO == 128 && !KMAJOR && !COLSUM && !POOL), "made rows: the 64 -> 128 layer");
+    static_assert(MID == 0 || (SK == 64 && SNO == 128 && !KMAJOR && !COLSUM && !POOL), "made rows: the 64 -> 128 layer");
     // POOL: first pixel of a tile and first pixel of its part of the pooled tensor (two 32-bit divisions per tile,
     // taken once, when the tile is requested, and kept for its way out)
     int px_next = 0, pp_next = 0, px_cur = 0, pp_cur = 0;
@@ -263,26 +266,27 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     [[maybe_unused]] auto mid_load = [&](long long t) {
         const int b = tile_pixel(t);
         const int hh = Himg >> 1, hw = Wimg >> 1;
-        const T* cf = static_cast<const T*>(mid->cf) + (long long)px_next * 64;
-        const T* chb = static_cast<const T*>(mid->ch) + (long long)b * hh * hw * 64;
+        const int ldf = MID == 1 ? 64 : mid->ldf, ldh = MID == 1 ? 64 : 32;
+        const T* cf = static_cast<const T*>(mid->cf) + (long long)px_next * ldf;
+        const T* chb = static_cast<const T*>(mid->ch) + (long long)b * hh * hw * ldh;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
-            const T* f = cf + (long long)((pix >> 3) * Wimg + (pix & 7)) * 64 + 8 * cc;
+            const T* f = cf + (long long)((pix >> 3) * Wimg + (pix & 7)) * ldf + 8 * cc;
             fa[p] = *reinterpret_cast<const Frag*>(f);
-            fb[p] = *reinterpret_cast<const Frag*>(f + 32);
+            if constexpr (MID == 1) fb[p] = *reinterpret_cast<const Frag*>(f + 32);
             // (patch entries past the image are never used as taps: clamped, they are readable)
             const int q = min(pix, 23), qr = q / 6, qc = q - 6 * qr;
             const int hy = min(max(2 * rb_next - 1 + qr, 0), hh - 1), hx = min(max(4 * cb_next - 1 + qc, 0), hw - 1);
-            const T* hp = chb + (long long)(hy * hw + hx) * 64 + 8 * cc;
+            const T* hp = chb + (long long)(hy * hw + hx) * ldh + 8 * cc;
             ha[p] = *reinterpret_cast<const Frag*>(hp);
-            hb[p] = *reinterpret_cast<const Frag*>(hp + 32);
+            if constexpr (MID == 1) hb[p] = *reinterpret_cast<const Frag*>(hp + 32);
         }
     };
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
         const T* base = X + t * 32 * K;
         const long long rows_left = N - t * 32;         // rows of this tile that exist
-        if constexpr (MID) {
+        if constexpr (MID != 0) {
             mid_load(t);
         } else if constexpr (POOL) {
             tile_pixel(t);
@@ -357,22 +361,24 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     for (long long tile = gw; tile < ntiles; tile += nw) {
         [[maybe_unused]] const bool first = tile == gw;
         px_cur = px_next, pp_cur = pp_next;   // (POOL, MID) set when this tile was requested
-        if constexpr (MID) {
+        if constexpr (MID != 0) {
             rb_cur = rb_next, cb_cur = cb_next;
             const int hh = Himg >> 1, hw = Wimg >> 1;
-            T* cat = static_cast<T*>(mid->cat);
+            T* cat = MID == 1 ? static_cast<T*>(mid->cat) : nullptr;
             // the gated patch of the half scale: [24 pixels][32] in columns 64.. of the tile buffer's rows
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
                 const int idx = p * 64 + lane, q = idx >> 2, cc = idx & 3;
-                const Frag hg = gate8<T>(ha[p], hb[p], mid->gs);
+                Frag hg = ha[p];
+                if constexpr (MID == 1) hg = gate8<T>(ha[p], hb[p], mid->gs);
                 if (q < 24) *reinterpret_cast<Frag*>(tl + q * ldt + 64 + 8 * cc) = hg;
             }
             // the full scale's half of the rows
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
                 const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
-                const Frag full = gate8<T>(fa[p], fb[p], mid->gs);
+                Frag full = fa[p];
+                if constexpr (MID == 1) full = gate8<T>(fa[p], fb[p], mid->gs);
                 *reinterpret_cast<Frag*>(tl + pix * ldt + 8 * cc) = full;
                 if (cat)
                     *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * 64 + 8 * cc) = full;
@@ -445,7 +451,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // fragments are in registers: the buffer may be overwritten
-        if constexpr (MID) {
+        if constexpr (MID != 0) {
             // unconditionally (the last tile asks for itself again, from the caches): behind a branch the loaded
             // registers are copied into the loop's own at the end of the branch, which waits for the data there
             load_tile(tile + nw < ntiles ? tile + nw : tile);
@@ -577,7 +583,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 }
                 T* pb = pool + ((long long)pp_cur + wr * (Wimg >> 1) + wc) * NO + ch;
                 *reinterpret_cast<Frag*>(pb) = o;
-            } else if constexpr (MID) {
+            } else if constexpr (MID != 0) {
                 yb = Y + (long long)px_cur * NO;
                 Frag of[LO];
 #pragma unroll
@@ -637,14 +643,14 @@ __global__ __launch_bounds__(256, 2) void dense_rows_pool_k(const T* __restrict_
 }
 
 // The 64 -> 128 layer on rows made from the two scales of a pyramid block (dense_rows_body, MID).
-template <typename T>
+template <typename T, int MID>
 __global__ __launch_bounds__(256, 2) void dense_mid_rows_k(const T* __restrict__ W, const T* __restrict__ bias,
                                                         const float* __restrict__ rowbias, T* __restrict__ Y,
                                                         long long N, int Himg, int Wimg, const MidRows mid) {
     extern __shared__ uint32_t dsm[];
-    dense_rows_body<T, false, false, 64, 128, false, true>(nullptr, W, bias, rowbias, Y, nullptr, N, 64, 128,
-                                                            Himg * Wimg, 4, 4, blockIdx.x, gridDim.x, dsm, nullptr, Himg,
-                                                            Wimg, &mid);
+    dense_rows_body<T, false, false, 64, 128, false, MID>(nullptr, W, bias, rowbias, Y, nullptr, N, 64, 128,
+                                                           Himg * Wimg, 4, 4, blockIdx.x, gridDim.x, dsm, nullptr, Himg,
+                                                           Wimg, &mid);
 }
 
 // The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
@@ -987,11 +993,14 @@ int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void*
 }
 
 // y[N][128] = rows w^T + bias + rowbias[image] for the rows made from a pyramid block's two convolution outputs
-// (dense_rows_body, MID): cf [B,H,W,64], ch [B,H/2,W/2,64]; cat (optional) receives the rows.  -1: not covered (other
+// (dense_rows_body, MID): cf [B,H,W,64], ch [B,H/2,W/2,64]; cat (optional) receives the rows.  ldf > 0: both scales
+// arrive gated, cf [B,H,W,32] at a pixel stride of ldf values, ch [B,H/2,W/2,32], no cat.  -1: not covered (other
 // widths, extents that are not multiples of 4 x 8, fp32).
 int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void* w, const void* bias,
-                          const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s) {
+                          const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s,
+                          int ldf) {
     if (dtype == kF32 || I != 64 || D != 128 || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
+    if (ldf != 0 && (ldf < 32 || ldf % 8 != 0 || cat)) return -1;
     if (tune_env("PDW_NO_DENSE_MID")) return -1;
     const long long N = (long long)B * H * W;
     if (N > 0x7fffffffLL / 128) return -1;
@@ -1006,13 +1015,16 @@ int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void*
     if (blocks > cap) blocks = cap;
     const size_t lds = ((size_t)4 * 32 * (64 + 8) + 4 * 32 * (128 + 8)) * 2 +
                        ((bias || rowbias) ? (size_t)4 * 2 * 4 * 32 * sizeof(float) : 0);
-    const MidRows mid{cf, ch, cat, sqrtf((float)(I / 2))};
-    if (dtype == kF16)
-        hipLaunchKernelGGL(dense_mid_rows_k<f16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const f16_t*)w,
-                           (const f16_t*)bias, rowbias, (f16_t*)y, N, H, W, mid);
-    else
-        hipLaunchKernelGGL(dense_mid_rows_k<bf16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const bf16_t*)w,
-                           (const bf16_t*)bias, rowbias, (bf16_t*)y, N, H, W, mid);
+    const MidRows mid{cf, ch, cat, ldf, sqrtf((float)(I / 2))};
+#define PDW_MID(T, M)                                                                                                   \
+    hipLaunchKernelGGL((dense_mid_rows_k<T, M>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)w, (const T*)bias, \
+                       rowbias, (T*)y, N, H, W, mid)
+    if (dtype == kF16) {
+        if (ldf) PDW_MID(f16_t, 2); else PDW_MID(f16_t, 1);
+    } else {
+        if (ldf) PDW_MID(bf16_t, 2); else PDW_MID(bf16_t, 1);
+    }
+#undef PDW_MID
     return check_launch("dense_mid_rows");
 }
 

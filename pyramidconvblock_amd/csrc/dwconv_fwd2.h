@@ -25,7 +25,7 @@ struct Fwd2Args {
     PoolFwdJob mean;      // workgroups behind both problems (one per image, mean.B of them): the block's mean branch
 };
 
-// MODE 0: the convolutions; 4: each with the gate applied in its store (dwconv_tz.h), 16 channels per workgroup only.
+// MODE 0: the convolutions; 4: each with the gate applied in its store (dwconv_tz.h).
 template <typename T, int K, int CS, int NPC1, int MODE>
 __global__ __launch_bounds__(512, 1) void dwconv_fwd2_k(const Fwd2Args a) {
     const unsigned blk = blockIdx.x;
@@ -121,14 +121,14 @@ static Fwd2Plan fwd2_plan(int B, const TzGeom& g0, const TzGeom& g1) {
 // -1: not covered (the caller makes the two launches).  16-bit types, C % 8 == 0, padding K / 2, the second scale
 // exactly half the first, the full scale in the wide tile.
 // gate0, gate1 (both or neither): the gate in the store of each scale, y0 / y1 then being the gated tensors with the
-// strides and channel offsets the gates name (16-channel slices only: filters up to 13).
+// strides and channel offsets the gates name.
 template <int K>
 static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
                        int W, int C, int dtype, hipStream_t s, const TzGate* gate0 = nullptr,
                        const TzGate* gate1 = nullptr, const PoolFwdJob* mean = nullptr) {
     constexpr int CS = (2 * 4 * TzShape<K, 16, 16>::NM + 2 * 4 * TzShape<K, 16, 16>::RING) <= 160 ? 16 : 8;
     if (dtype == kF32 || C % 8 != 0 || (H & 1) || (W & 1) || B < 1 || H < 2 || W < 2) return -1;
-    if ((gate0 != nullptr) != (gate1 != nullptr) || (gate0 && CS != 16)) return -1;
+    if ((gate0 != nullptr) != (gate1 != nullptr)) return -1;
     const int P = K / 2, h = H / 2, wd = W / 2;
     for (const void* p : {x0, w0, (const void*)y0, x1, w1, (const void*)y1})
         if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
@@ -175,12 +175,10 @@ static int launch_fwd2(const void* x0, const void* w0, void* y0, const void* x1,
         hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, s, a);                                                   \
     }
     if (gate0) {
-        if constexpr (CS == 16) {
-            if (dtype == kF16) {
-                if (wide1) PDW_FWD2_GO(f16_t, 16, 4, 4) else PDW_FWD2_GO(f16_t, 8, 4, 5)
-            } else {
-                if (wide1) PDW_FWD2_GO(bf16_t, 16, 4, 6) else PDW_FWD2_GO(bf16_t, 8, 4, 7)
-            }
+        if (dtype == kF16) {
+            if (wide1) PDW_FWD2_GO(f16_t, 16, 4, 4) else PDW_FWD2_GO(f16_t, 8, 4, 5)
+        } else {
+            if (wide1) PDW_FWD2_GO(bf16_t, 16, 4, 6) else PDW_FWD2_GO(bf16_t, 8, 4, 7)
         }
     } else if (dtype == kF16) {
         if (wide1) PDW_FWD2_GO(f16_t, 16, 0, 0) else PDW_FWD2_GO(f16_t, 8, 0, 1)

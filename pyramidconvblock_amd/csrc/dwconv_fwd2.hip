@@ -25,14 +25,14 @@ bool dwconv_fwd2_covers(int B, int H, int W, int C, int K, int dtype) {
 }
 
 // -1: not covered (the caller makes the two launches).  ldy0 > 0: both convolutions with the gate applied in the store
-// (y[..., ych + c] = conv[..., c] * conv[..., C/2 + c] * sqrt(C/2) at a pixel stride of ldy channels); filters up to 13.
+// (y[..., ych + c] = conv[..., c] * conv[..., C/2 + c] * sqrt(C/2) at a pixel stride of ldy channels).
 // mean (optional): the block's mean branch in mean->B more workgroups of the same launch.
 int dwconv_fwd2_launch(const void* x0, const void* w0, void* y0, const void* x1, const void* w1, void* y1, int B, int H,
                        int W, int C, int K, int dtype, hipStream_t s, int ldy0, int ych0, int ldy1, int ych1,
                        const PoolFwdJob* mean) {
     if (tune_env("PDW_NO_FWD2")) return -1;
     const bool gated = ldy0 > 0;
-    if (gated && (C % 16 != 0 || K > 13)) return -1;
+    if (gated && C % 16 != 0) return -1;
     const TzGate g0{ldy0, ych0, sqrtf((float)(C / 2))}, g1{ldy1, ych1, sqrtf((float)(C / 2))};
     const TzGate *gate0 = gated ? &g0 : nullptr, *gate1 = gated ? &g1 : nullptr;
     switch (K) {

@@ -34,6 +34,9 @@
 // half and the matching 8 of the second half of C, and the two store threads of a pixel multiply four channel pairs
 // each (the rounded convolution outputs, as the stand-alone gate kernel does): y[..., c] = conv[c] * conv[C/2 + c] * gs,
 // C/2 channels wide, written with a pixel stride of YC channels from channel `ych` on (into the concatenation).
+// With 8 channels per workgroup (filters from 15 on) the slice is 4 channels of each half: every 16-byte load of the
+// staging and of the filter becomes two 8-byte loads C bytes apart, and a pixel's one store thread gates the two
+// halves of its piece.
 //
 // Zero entries of A multiply real pixels of the window (and the window is wider than K+3 where (K+3) % 8 != 0), so a
 // non-finite input value reaches outputs up to 3 + 8 ICB - (K+3) pixels beyond its K x K footprint as NaN.
@@ -140,7 +143,11 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
     constexpr int NI = Sh::NI, TW = Sh::TW, NH = Sh::NH, CPW = Sh::CPW, RP = Sh::RP, OPX = Sh::OPX, OROWP = Sh::OROWP;
     constexpr int OLB = Sh::OLB, WTH = Sh::WTH, WTW = Sh::WTW, NR = Sh::NR, NRR = Sh::NRR, CHP = Sh::CHP;
     constexpr bool ADD = (MODE & 1) != 0, POOL = (MODE & 2) != 0, GATE = (MODE & 4) != 0;
-    static_assert(!GATE || (CS == 16 && !ADD), "the gate pairs the two 8-channel pieces of a 16-channel slice");
+    static_assert(!GATE || !ADD, "the gate is a forward mode");
+    // the gate pairs channel c with channel C/2 + c: a 16-channel slice is 8 channels of each half of C (its two
+    // 8-channel pieces), an 8-channel slice 4 of each (the halves of its one piece, moved as two 8-byte accesses)
+    constexpr bool G8 = GATE && CS == 8;
+    static_assert(!(G8 && POOL), "the pool's stores assume 8 contiguous channels");
     extern __shared__ uint32_t smem[];
     char* const xl = reinterpret_cast<char*>(smem);        // [NI][CS] planes of CHP bytes: [ring row][column] of T
     char* const r2 = xl + NI * CS * CHP;                 // filter table, then the two result tiles
@@ -159,7 +166,7 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
     const int WCP = (4 * ((cols_valid + 3) / 4 - 1) + 8 * ICB) / 2;  // column pairs the used patches read
     const long long img_in = (long long)g.H * g.W * g.C, img_out = (long long)g.OH * g.OW * g.YC;
     // first channel of the slice's 8-channel piece h
-    auto chof = [&](int h) { return GATE ? 8 * sl + h * (g.C >> 1) : c0 + 8 * h; };
+    auto chof = [&](int h) { return G8 ? 4 * sl : GATE ? 8 * sl + h * (g.C >> 1) : c0 + 8 * h; };
 
     // ---- filter slice, 8 channels of a tap per load: requested before the window, so that waiting for it leaves
     // the window's loads in flight
@@ -168,7 +175,13 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
 #pragma unroll
     for (int i = 0; i < NWL; ++i) {
         const int idx = min(tid + i * NT, K * K * NH - 1);
-        wval[i] = *reinterpret_cast<const uint4*>(w + (idx / NH) * g.C + min(chof(idx % NH), g.C - 8));
+        if constexpr (G8) {
+            const T* wp = w + idx * g.C + 4 * sl;
+            const uint2 lo = *reinterpret_cast<const uint2*>(wp), hi = *reinterpret_cast<const uint2*>(wp + (g.C >> 1));
+            wval[i] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        } else {
+            wval[i] = *reinterpret_cast<const uint4*>(w + (idx / NH) * g.C + min(chof(idx % NH), g.C - 8));
+        }
     }
 
     // ---- staging.  The window arrives in passes, requested two ahead into two register buffers.  Passes 0 and 1
@@ -193,7 +206,16 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
         const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
         return make_uint4(v.x, v.y, v.z, v.w);
     };
-    auto xload = [&](uint32_t off) { return xload_from(xrsrc, off); };
+    auto xload = [&](uint32_t off) {
+        if constexpr (G8) {   // 4 channels of each half of C (C bytes apart); a marker offset stays past the end
+            typedef unsigned v2u __attribute__((ext_vector_type(2)));
+            const v2u lo = __builtin_amdgcn_raw_buffer_load_b64(xrsrc, (int)off, 0, 0);
+            const v2u hi = __builtin_amdgcn_raw_buffer_load_b64(xrsrc, (int)(off + (uint32_t)g.C), 0, 0);
+            return make_uint4(lo.x, lo.y, hi.x, hi.y);
+        } else {
+            return xload_from(xrsrc, off);
+        }
+    };
     uint32_t icol[NLD][2];  // byte offsets of the item's two columns (image and channel piece included), or kNoCol
     int irpw[NLD];          // row pair within a pass
     int idst[NLD];          // LDS byte offset of the item's plane and column pair
@@ -203,7 +225,7 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
         const int h = idx % NH, cp = (idx / NH) % WCP, img = (idx / NH / WCP) % NI, rpw = idx / NH / WCP / NI;
         irpw[l] = rpw;
         const int ic = ocol0 - g.PW + 2 * cp;
-        const bool any = chof(h) < g.C && rpw < RPMAX;
+        const bool any = (G8 || chof(h) < g.C) && rpw < RPMAX;
         const uint32_t ioff = (uint32_t)img * (uint32_t)img_in + (uint32_t)chof(h);
         icol[l][0] = any && ic >= 0 && ic < g.W ? (ioff + (uint32_t)(ic * g.C)) * 2u : kNoCol;
         icol[l][1] = any && ic + 1 >= 0 && ic + 1 < g.W ? (ioff + (uint32_t)((ic + 1) * g.C)) * 2u : kNoCol;
@@ -293,7 +315,7 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
             const int idx = tid + i * NT;
             const int h = idx % NH, uv = idx / NH;
             const int u = uv / K, v = uv - u * K;
-            if (idx < K * K * NH && chof(h) < g.C) {
+            if (idx < K * K * NH && (G8 || chof(h) < g.C)) {
                 const uint32_t d[4] = {wval[i].x, wval[i].y, wval[i].z, wval[i].w};
                 const int uu = g.flip ? K - 1 - u : u, vv = g.flip ? K - 1 - v : v;
                 unsigned short* wp = wt + ((8 * h) * WTH + 3 + uu) * WTW + 3 + vv;
@@ -328,7 +350,8 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
     const char* const olr = r2 + (min(simg, NI - 1) * 4 + srow) * OROWP + scol * OPX + (scol >> 2) * 4 + 16 * sh;
     const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(
         y + (long long)b0 * img_out, (short)0, (int)(min(NI, g.B - b0) * img_out * 2), 0x00020000);
-    const uint32_t ycol = (uint32_t)simg * (uint32_t)img_out + (uint32_t)((ocol0 + scol) * g.YC + g.ych + (GATE ? 8 * sl + 4 * sh : c0 + 8 * sh));
+    const uint32_t ycol = (uint32_t)simg * (uint32_t)img_out +
+                          (uint32_t)((ocol0 + scol) * g.YC + g.ych + (G8 ? 4 * sl : GATE ? 8 * sl + 4 * sh : c0 + 8 * sh));
     __amdgpu_buffer_rsrc_t arsrc = xrsrc;
     if constexpr (ADD)
         arsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(add + (long long)b0 * g.AH * g.AW * g.C), (short)0,
@@ -357,10 +380,12 @@ __device__ __forceinline__ void dwconv_tz_body(const T* __restrict__ x, const T*
             const bool ok = s_ok && f >= 0 && row < rows_valid;
             const uint32_t off = ok ? (ycol + (uint32_t)((orow0 + row) * g.OW * g.YC)) * 2u : kNoRow;
             if constexpr (GATE) {
-                // the thread gates 4 of the pixel's 8 channel pairs: values 4 sh .. 4 sh + 3 of both 8-channel pieces
-                const char* sg = src - 8 * sh;   // (src points 16 sh into the pixel)
+                // the thread gates 4 channel pairs of the pixel: values 4 sh .. 4 sh + 3 of both 8-channel pieces, or
+                // the two halves of an 8-channel slice's one piece
+                const char* sg = G8 ? src : src - 8 * sh;   // (src points 16 sh into the pixel)
+                constexpr int PB = G8 ? 8 : 16;             // bytes between a pair's two values
                 const uint2 a = make_uint2(*reinterpret_cast<const uint32_t*>(sg), *reinterpret_cast<const uint32_t*>(sg + 4));
-                const uint2 b = make_uint2(*reinterpret_cast<const uint32_t*>(sg + 16), *reinterpret_cast<const uint32_t*>(sg + 20));
+                const uint2 b = make_uint2(*reinterpret_cast<const uint32_t*>(sg + PB), *reinterpret_cast<const uint32_t*>(sg + PB + 4));
                 const uint2 o = tz_gate<T>(a, b, g.gs);
                 typedef unsigned v2u __attribute__((ext_vector_type(2)));
                 __builtin_amdgcn_raw_buffer_store_b64(v2u{o.x, o.y}, yrsrc, (int)off, 0, 0);
@@ -529,7 +554,7 @@ static bool tz_make_geom(TzGeom& g, long long& nblocks, bool add, int B, int H, 
     g.OH = H + 2 * PH - K + 1, g.OW = W + 2 * PW - K + 1;
     g.AH = add ? g.OH / 2 : H / 2, g.AW = add ? g.OW / 2 : W / 2;
     g.YC = gate ? gate->ldy : C, g.ych = gate ? gate->ych : 0, g.gs = gate ? gate->gs : 1.f;
-    if (gate && (CS != 16 || add || flip || C % 16 != 0 || gate->ldy < gate->ych + C / 2 || (gate->ldy | gate->ych) % 8 != 0)) return false;
+    if (gate && (add || flip || C % 16 != 0 || gate->ldy < gate->ych + C / 2 || (gate->ldy | gate->ych) % 8 != 0)) return false;
     if ((long long)H * W * C * Sh::NI > 0x1fffffffLL || (long long)g.OH * g.OW * g.YC * Sh::NI > 0x1fffffffLL) return false;
     g.BR = tz_pick_band<K, NPC, CS>(B, g.OH, g.OW, C);
     if (g.BR < 4) return false;
@@ -550,11 +575,11 @@ static int launch_tz(const void* x, const void* w, const void* add, void* pool, 
     auto kern = dwconv_tz_k<T, K, NPC, CS, 0>;
     if (mode == 1) kern = dwconv_tz_k<T, K, NPC, CS, 1>;
     if (mode == 2) kern = dwconv_tz_k<T, K, NPC, CS, 2>;
+    if (mode == 4) kern = dwconv_tz_k<T, K, NPC, CS, 4>;
     if constexpr (CS == 16) {
-        if (mode == 4) kern = dwconv_tz_k<T, K, NPC, CS, 4>;
         if (mode == 6) kern = dwconv_tz_k<T, K, NPC, CS, 6>;
     }
-    if (mode == 3 || mode == 5 || mode == 7) return -1;
+    if (mode == 3 || mode == 5 || mode == 7 || (mode == 6 && CS != 16)) return -1;
     static std::once_flag attr_once[8];
     std::call_once(attr_once[mode], [&] { (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(Sh::NT), lds, s, (const T*)x, (const T*)w, (const T*)add,

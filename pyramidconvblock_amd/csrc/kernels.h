@@ -109,9 +109,11 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
 int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
                            int H, int W, int K, int NO, int dtype, hipStream_t s);
 // the 64 -> 128 layer on rows made from the two convolution outputs of a pyramid block (gates and resize where the
-// tile is staged); cat (optional) receives the rows; -1 = not covered
+// tile is staged); cat (optional) receives the rows; ldf > 0: the scales arrive gated, I / 2 wide, the full one at a pixel
+// stride of ldf values; -1 = not covered
 int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void* w, const void* bias,
-                          const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s);
+                          const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s,
+                          int ldf = 0);
 int dense_colsum_supported(int K, int NO, int dtype);
 int dense_colsum_rows();
 int dense_wgrad_supported(int M, int NO, int dtype);

@@ -167,8 +167,8 @@ def dwconv_forward2_mean(x0, w0, x1, w1, parts, P, w_pool, b_pool=None, b_out=No
     m = torch.empty((B, D), device=dev, dtype=dt)
     rowbias = torch.empty((B, D), device=dev, dtype=torch.float32)
     with _lib.on_device(dev):
-        st = L.pdw_dwconv_fwd2_mean(args[0].data_ptr(), args[1].data_ptr(), y0.data_ptr(), args[2].data_ptr(),
-                                    args[3].data_ptr(), y1.data_ptr(), B, H, W, C, K, args[4].data_ptr(),
+        st = L.pdw_dwconv_fwd2_mean(args[0].data_ptr(), args[1].data_ptr(), y0.data_ptr(), 0, 0, args[2].data_ptr(),
+                                    args[3].data_ptr(), y1.data_ptr(), 0, 0, B, H, W, C, K, args[4].data_ptr(),
                                     parts.shape[0] // B, args[5].data_ptr(),
                                     b_pool.data_ptr() if b_pool is not None else None,
                                     b_out.data_ptr() if b_out is not None else None, m.data_ptr(), rowbias.data_ptr(),

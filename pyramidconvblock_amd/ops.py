@@ -281,28 +281,34 @@ def dense_forward(x, w, w_kmajor=False, bias=None, rowbias=None, rows_per_image=
     return y
 
 
-def dense_forward_gated(cf, ch, w, rowbias=None, bias=None, cat=None):
+def dense_forward_gated(cf, ch, w, rowbias=None, bias=None, cat=None, gated=False):
     """The output layer of a two-scale block on rows made in the kernel (pdw_dense_fwd_gated): y = [gate(cf) |
     resize(gate(ch))] W^T + bias + rowbias[image] for the convolution outputs cf [B,H,W,I], ch [B,H/2,W/2,I] of the
-    two scales; `cat` ([B,H,W,I], optional) receives the rows.  None where the kernel does not cover the case."""
+    two scales; `cat` ([B,H,W,I], optional) receives the rows.  With `gated` the scales arrive gated (cf [B,H,W,I/2],
+    possibly a channel slice of a wider tensor, ch [B,H/2,W/2,I/2]) and only the resize is left to do.  None where the
+    kernel does not cover the case."""
     dev = _lib.require_device(cf, ch, w)
-    if cf.dim() != 4 or not (cf.is_contiguous() and ch.is_contiguous() and w.is_contiguous()):
+    if cf.dim() != 4 or not (ch.is_contiguous() and w.is_contiguous()):
         return None
-    B, H, W, I = cf.shape
+    B, H, W, C = cf.shape
+    I = 2 * C if gated else C
     D = w.shape[0]
     dt = cf.dtype
-    if (B == 0 or H % 2 or W % 2 or tuple(ch.shape) != (B, H // 2, W // 2, I) or w.shape[1] != I
+    ldf = _pixel_stride(cf) if gated else 0
+    if not gated and not cf.is_contiguous():
+        return None
+    if (B == 0 or H % 2 or W % 2 or tuple(ch.shape) != (B, H // 2, W // 2, C) or w.shape[1] != I
             or any(t is not None and t.dtype != dt for t in (ch, w, bias, cat))
             or (rowbias is not None and (rowbias.dtype != torch.float32 or tuple(rowbias.shape) != (B, D)
                                          or not rowbias.is_contiguous()))
-            or (cat is not None and (tuple(cat.shape) != (B, H, W, I) or not cat.is_contiguous()))):
+            or (cat is not None and (gated or tuple(cat.shape) != (B, H, W, I) or not cat.is_contiguous()))):
         return None
     y = torch.empty((B, H, W, D), device=dev, dtype=dt)
     with _lib.on_device(dev):
         st = _lib.lib().pdw_dense_fwd_gated(cf.data_ptr(), ch.data_ptr(), cat.data_ptr() if cat is not None else None,
                                             w.data_ptr(), bias.data_ptr() if bias is not None else None,
                                             rowbias.data_ptr() if rowbias is not None else None, y.data_ptr(), B, H, W,
-                                            I, D, _lib.dtype_code(dt), _lib.stream_ptr(dev))
+                                            I, D, ldf, _lib.dtype_code(dt), _lib.stream_ptr(dev))
     if st == 3:
         return None
     _lib.check(st, "pdw_dense_fwd_gated")

@@ -39,6 +39,10 @@ def _gate_conv(x, w, ldy, ych, pool, dtype):
     ((1, 8, 8, 16), 5, 8, 0, True),
     ((2, 30, 26, 96), 11, 104, 56, False),
     ((2, 16, 16, 32), 3, 16, 0, False),
+    ((2, 24, 28, 32), 17, 16, 0, False),     # 8 channels per workgroup: 4 of each half of C
+    ((3, 40, 36, 64), 15, 64, 32, False),
+    ((8, 56, 56, 48), 17, 24, 0, False),     # (C = 48: three 16-channel gate groups over six slices)
+    ((1, 57, 33, 96), 15, 48, 0, False),
 ])
 def test_conv_gate_matches_oracle(oracle, shape, k, ldy, ych, pool, dtype):
     B, H, W, C = shape
@@ -98,7 +102,7 @@ def test_two_scale_conv_gate_is_the_two_calls(shape, k, dtype):
                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     wide = -(-W // 64) * 64 * B <= -(-W // 32) * 32 * (-(-B // 2) * 2)
-    covered = dtype != torch.float32 and C % 16 == 0 and k <= 13 and wide
+    covered = dtype != torch.float32 and C % 16 == 0 and wide
     assert rc == (0 if covered else 3)
     if not covered:
         return
@@ -114,7 +118,7 @@ def test_conv_gate_not_covered_returns_3():
     rc, _, _ = _gate_conv(x, w, 16, 0, False, torch.float32)       # fp32
     assert rc == 3
     xb, wb = x.bfloat16(), torch.zeros(17, 17, 32, device="cuda", dtype=torch.bfloat16)
-    rc, _, _ = _gate_conv(xb, wb, 16, 0, False, torch.bfloat16)     # filter too large for 16 channels per workgroup
+    rc, _, _ = _gate_conv(xb, wb, 16, 0, True, torch.bfloat16)      # pooled output from 8 channels per workgroup
     assert rc == 3
     x24 = torch.zeros(1, 8, 8, 24, device="cuda", dtype=torch.bfloat16)
     rc, _, _ = _gate_conv(x24, torch.zeros(5, 5, 24, device="cuda", dtype=torch.bfloat16), 12, 0, False, torch.bfloat16)
@@ -127,7 +131,8 @@ def test_conv_gate_not_covered_returns_3():
 @pytest.mark.parametrize("dim,k,shape,dtype", [
     (128, 13, (32, 56, 56, 128), torch.bfloat16),    # headline workload
     (128, 9, (4, 56, 56, 128), torch.float16),
-    (128, 17, (4, 56, 56, 128), torch.bfloat16),     # filter beyond the fused kernel: the forward's own launches
+    (128, 17, (4, 56, 56, 128), torch.bfloat16),     # 8 channels per convolution workgroup
+    (128, 15, (2, 24, 40, 128), torch.float16),
     (64, 7, (3, 16, 24, 64), torch.bfloat16),
     (128, 13, (1, 8, 8, 128), torch.bfloat16),
 ])

@@ -426,6 +426,15 @@ def test_dense_forward_gated_is_the_gates_then_the_layer(oracle, dtype, with_cat
         assert_close(y, yo.numpy(), dtype, "y")
     y2 = ops.dense_forward_gated(cf, ch, w)   # no per-image rows
     assert torch.equal(y2, ops.dense_forward(want_cat, w))
+    # both scales arriving gated (the inference forward): the full scale compact or as a slice of a wider tensor
+    G = I // 2
+    g1 = torch.empty((B, H // 2, W // 2, G), device="cuda", dtype=dtype)
+    ops.gate_forward(ch, out=g1)
+    wide = torch.full((B, H, W, I + 8), 3.0, device="cuda", dtype=dtype)
+    wide[..., 8:8 + G] = want_cat[..., :G]
+    for g0 in (want_cat[..., :G].contiguous(), wide[..., 8:8 + G]):
+        y3 = ops.dense_forward_gated(g0, g1, w, rowbias=rowbias, gated=True)
+        assert y3 is not None and torch.equal(y3, want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -459,3 +468,24 @@ def test_fwd2_mean_is_the_convolutions_and_the_mean_branch(dtype, case, biases):
     torch.cuda.synchronize()
     assert torch.equal(got[0], convs[0]) and torch.equal(got[1], convs[1])
     assert torch.equal(got[2], m) and torch.equal(got[3], rowbias)
+    # the same with the gates in the convolutions' stores (the inference forward's launch)
+    import ctypes
+
+    from pyramidconvblock_amd import _lib
+
+    L, G = _lib.lib(), C // 2
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ya, yb = (torch.full((B, H, W, G), 7.0, device="cuda", dtype=dtype) for _ in range(2))
+    za, zb = (torch.full((B, H // 2, W // 2, G), 7.0, device="cuda", dtype=dtype) for _ in range(2))
+    m2, rb2 = torch.zeros_like(m), torch.zeros_like(rowbias)
+    rc = L.pdw_dwconv_fwd2_mean(x0.data_ptr(), w0.data_ptr(), ya.data_ptr(), G, 0, x1.data_ptr(), w1.data_ptr(), za.data_ptr(),
+                                G, 0, B, H, W, C, k, parts.data_ptr(), nparts, wp.data_ptr(),
+                                bp.data_ptr() if bp is not None else None, bo.data_ptr() if bo is not None else None,
+                                m2.data_ptr(), rb2.data_ptr(), H * W, D, _lib.dtype_code(dtype), st)
+    rg = L.pdw_dwconv_fwd2_gate(x0.data_ptr(), w0.data_ptr(), yb.data_ptr(), G, 0, x1.data_ptr(), w1.data_ptr(), zb.data_ptr(),
+                                G, 0, B, H, W, C, k, _lib.dtype_code(dtype), st)
+    torch.cuda.synchronize()
+    assert rc == rg and rc == (0 if C % 16 == 0 else 3)
+    if rc == 0:
+        assert torch.equal(ya, yb) and torch.equal(za, zb) and torch.equal(m2, m) and torch.equal(rb2, rowbias)
+        assert torch.equal(ya, ops.gate_forward(convs[0])) and torch.equal(za, ops.gate_forward(convs[1]))
