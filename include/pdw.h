@@ -390,8 +390,10 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
                        void *stream);
 
 /* The whole block of conv_block.py:25-49 (scales (1, 1/2), conv_up without bias) as one host call each way: the
- * launch sequence of the entry points above (4 launches forward: conv_up with the pool of its result, the convolutions
- * of both scales, gates and mean branch, conv_out; 5 launches and one summation launch backward)
+ * launch sequence of the entry points above (forward: conv_up with the pool of its result, the convolutions of both
+ * scales with the mean branch, conv_out on rows it makes from their outputs, writing cat: 3 launches for D = 128,
+ * I = 64, H % 4 == 0, W % 8 == 0, else 4 with the gates and the mean branch as one launch of their own; backward: 5
+ * launches and one summation launch)
  * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
  * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense
  * kernels and pdw_dense_bwd_pair cover (multiples of 8 up to 128; D = 128, I = 64 and D = 64, I = 32 run the variants with
@@ -404,15 +406,14 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
  * Replaces the Python-level sequence of ConvBlock.forward, conv_block.py:36-49, and its autograd backward. */
 int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype);
 /* Inference forward of the same block (same coverage): y only.  conv_up (which also pools its result for the second
- * scale where its kernel can, pdw_dense_fwd_colsum_pool), then each scale's convolution with the gate applied in its
- * store (both as one launch, pdw_dwconv_fwd2_gate, or pdw_dwconv_fwd_gate twice, the full-resolution one then pooling
- * its input), the
- * half-resolution gate upsampled into its slice of the concatenation, conv_out plus the mean branch.  Neither
- * convolution output is written to HBM, and every intermediate lives in `workspace`
- * (pdw_convblock_infer_workspace_bytes).  Where the fused convolution does not cover the filter size the call runs
- * the launches of pdw_convblock_fwd on workspace tensors instead.  Same arithmetic as pdw_convblock_fwd except that
- * the half-resolution gate is rounded to `dtype` before it is upsampled.  Replaces ConvBlock.forward under
- * torch.no_grad(), conv_block.py:36-49 with :13-22. */
+ * scale where its kernel can, pdw_dense_fwd_colsum_pool); then, where pdw_dense_fwd_gated covers the widths and
+ * extents, the convolutions of both scales with the mean branch in their launch (pdw_dwconv_fwd2_mean) and conv_out on
+ * rows it makes itself from their outputs: three launches, no gated or concatenated tensor in memory.  Elsewhere each
+ * scale's convolution with the gate applied in its store (both as one launch, pdw_dwconv_fwd2_gate, or
+ * pdw_dwconv_fwd_gate twice, the full-resolution one then pooling its input), the half-resolution gate upsampled into
+ * its slice of the concatenation with the mean branch (pdw_block_mid_infer), conv_out: neither convolution output is
+ * written to HBM.  Every intermediate lives in `workspace` (pdw_convblock_infer_workspace_bytes).  Same arithmetic as
+ * pdw_convblock_fwd.  Replaces ConvBlock.forward under torch.no_grad(), conv_block.py:36-49 with :13-22. */
 size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype);
 int pdw_convblock_infer(const void *x, const void *w_up, const void *w_dw0, const void *w_dw1, const void *w_pool,
                         const void *b_pool, const void *w_out, const void *b_out, void *y, void *workspace,

@@ -138,7 +138,7 @@ size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, in
     size_t b = up256(full) /* a */ + up256(half) /* xp */ + up256(full) /* cat */ + up256((size_t)B * D * s.es) /* m */ +
                up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4);
     if (infer_fused(H, W, I, K))
-        b += up256(half / 2);  // the gated half-resolution scale
+        b += up256(half);  // the gated half-resolution scale, or the half scale's convolution output
     else
         b += up256(full) + up256(half);  // c0, c1
     return b;
@@ -172,7 +172,7 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
         return pdw_convblock_fwd(x, w_up, w_dw0, w_dw1, w_pool, b_pool, w_out, b_out, a, c0, xp, c1, cat, m, y, xparts,
                                  up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4), B, H, W, D, I, K, dtype, stream);
     }
-    void* g1 = ws.take(half / 2);
+    void* g1 = ws.take(half);
     // conv_up; where its kernel can also pool its result, the gated convolutions of both scales follow as one launch
     // (scale 1 into cat[..., :G], scale 1/2 into g1)                                        (conv_block.py:14-19, 37)
     int both = 3;
@@ -180,13 +180,14 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
         const int pooled = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream);
         if (pooled != 0 && pooled != 3) return pooled;
         if (pooled == 0) {
-            // with the mean branch in the same launch, and then conv_out on rows it puts together itself (the full scale's
-            // gate, written G wide, and the resized half scale's), where its kernel covers the widths and extents: three
-            // launches                                                                        (conv_block.py:41-49)
+            // where conv_out's kernel can make its rows itself (both gates and the resize where it stages a tile): the
+            // convolutions with the mean branch in their launch, then that layer: three launches.  The convolution
+            // outputs pass through the workspace (measured: as fast as gating them in the convolutions' stores at
+            // K <= 13, 2 us faster at K = 17).                                                (conv_block.py:41-49)
             if (I == 64 && D == 128 && H % 4 == 0 && W % 8 == 0 && !(reinterpret_cast<uintptr_t>(w_out) & 15)) {
-                both = pdw_dwconv_fwd2_mean(a, w_dw0, cat, G, 0, xp, w_dw1, g1, G, 0, B, H, W, I, K, xparts, (int)(s.nt / B),
+                both = pdw_dwconv_fwd2_mean(a, w_dw0, cat, 0, 0, xp, w_dw1, g1, 0, 0, B, H, W, I, K, xparts, (int)(s.nt / B),
                                             w_pool, b_pool, b_out, m, yp, s.P, D, dtype, stream);
-                if (both == 0) return pdw_dense_fwd_gated(cat, g1, nullptr, w_out, nullptr, yp, y, B, H, W, I, D, G, dtype, stream);
+                if (both == 0) return pdw_dense_fwd_gated(cat, g1, nullptr, w_out, nullptr, yp, y, B, H, W, I, D, 0, dtype, stream);
                 if (both != 3) return both;
             }
             both = pdw_dwconv_fwd2_gate(a, w_dw0, cat, I, 0, xp, w_dw1, g1, G, 0, B, H, W, I, K, dtype, stream);
