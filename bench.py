@@ -375,6 +375,22 @@ def kernel_rooflines(B, H, W, D, k, dtype):
     ):
         t = time_kernel_events(fn, nbuf)
         out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=0.0, issued_flops=None, pipe="valu"))
+    # the same four at four times the batch: at the block's own size their tensors are 8-16 MB, which at 8 TB/s is
+    # 1-2 us of traffic under the ~2.8 us that any launch costs here, so the fraction there measures the launch
+    B4, nb4 = 4 * B, 4
+    a4 = [torch.randn(B4, H, W, I, device="cuda").to(dtype) for _ in range(nb4)]
+    p4 = [torch.randn(B4, h, w, I, device="cuda").to(dtype) for _ in range(nb4)]
+    gsm4 = [t_[..., :G].contiguous() for t_ in p4]
+    gbig4 = [t_[..., :G].contiguous() for t_ in a4]
+    for name, fn, nbytes in (
+        (f"avgpool_fwd[{B4}x{H}x{W}x{I}]", lambda i: avgpool.avgpool_forward(a4[i], (h, w)), es * B4 * (H * W + h * w) * I),
+        (f"avgpool_bwd[{B4}x{H}x{W}x{I}]", lambda i: avgpool.avgpool_backward(p4[i], (H, W)), es * B4 * (H * W + h * w) * I),
+        (f"bilinear_fwd[{B4}x{H}x{W}x{G}]", lambda i: up.bilinear_forward(gsm4[i], (H, W)), es * B4 * (H * W + h * w) * G),
+        (f"bilinear_bwd[{B4}x{H}x{W}x{G}]", lambda i: up.bilinear_backward(gbig4[i], (h, w)), es * B4 * (H * W + h * w) * G),
+    ):
+        t = time_kernel_events(fn, nb4, iters=12)
+        out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=0.0, issued_flops=None, pipe="valu"))
+    del a4, p4, gsm4, gbig4
     # gate and the dense conv_up layer ([N,D] <-> [N,I])
     c = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
     xin = [torch.randn(B, H, W, D, device="cuda").to(dtype) for _ in range(4)]

@@ -11,6 +11,33 @@
 
 namespace pdw {
 
+// idx = ((q * n2 + r2) * n1 + r1) * n0 + r0 taken apart.  A thread's flat item index almost always fits 31 bits, and
+// three 32-bit divisions cost a fifth of three 64-bit ones: in these kernels the index arithmetic, not the memory
+// system, was what a wavefront spent most of its instructions on.
+__device__ __forceinline__ void split_idx(long long idx, int n0, int n1, int n2, int& r0, int& r1, int& r2, long long& q) {
+    if ((unsigned long long)idx < 0x80000000ull) {
+        const unsigned u = (unsigned)idx, t0 = u / (unsigned)n0, t1 = t0 / (unsigned)n1, t2 = t1 / (unsigned)n2;
+        r0 = (int)(u - t0 * (unsigned)n0), r1 = (int)(t0 - t1 * (unsigned)n1), r2 = (int)(t1 - t2 * (unsigned)n2);
+        q = (long long)t2;
+    } else {
+        long long t = idx / n0;
+        r0 = (int)(idx - t * n0);
+        const long long t1 = t / n1;
+        r1 = (int)(t - t1 * n1);
+        q = t1 / n2;
+        r2 = (int)(t1 - q * n2);
+    }
+}
+// idx = q * n0 + r0
+__device__ __forceinline__ void split_idx(long long idx, int n0, int& r0, long long& q) {
+    if ((unsigned long long)idx < 0x80000000ull) {
+        const unsigned u = (unsigned)idx, t0 = u / (unsigned)n0;
+        r0 = (int)(u - t0 * (unsigned)n0), q = (long long)t0;
+    } else {
+        q = idx / n0, r0 = (int)(idx - q * n0);
+    }
+}
+
 // ---------------------------------------------------------------- adaptive average pool
 // Host side guarantees in * out < 2^31 (checked in the launchers), so 32-bit arithmetic is exact.
 __device__ __forceinline__ int bin_start(int i, int in, int out) { return (int)((unsigned)(i * in) / (unsigned)out); }
@@ -24,12 +51,20 @@ __global__ __launch_bounds__(256) void avgpool_fwd_k(const T* __restrict__ x, T*
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
-    const int c = (int)(idx % CV) * VEC;
-    long long t = idx / CV;
-    const int j = (int)(t % w);
-    t /= w;
-    const int i = (int)(t % h);
-    const long long b = t / h;
+    int cq, j, i;
+    long long b;
+    split_idx(idx, CV, w, h, cq, j, i, b);
+    const int c = cq * VEC;
+    if (H == 2 * h && W == 2 * w) {   // (uniform) exact halves: the four loads of the 2 x 2 bin in flight together
+        const T* p = x + ((b * H + 2 * i) * W + 2 * j) * C + c;
+        float x00[VEC], x01[VEC], x10[VEC], x11[VEC], o[VEC];
+        load_f32<T, VEC>(p, x00), load_f32<T, VEC>(p + C, x01);
+        load_f32<T, VEC>(p + (long long)W * C, x10), load_f32<T, VEC>(p + (long long)W * C + C, x11);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) o[v] = (((x00[v] + x01[v]) + x10[v]) + x11[v]) * 0.25f;   // the loop's order
+        store_f32<T, VEC>(y + ((b * h + i) * w + j) * C + c, o);
+        return;
+    }
     const int hs = bin_start(i, H, h), he = bin_end(i, H, h);
     const int ws = bin_start(j, W, w), we = bin_end(j, W, w);
     float acc[VEC];
@@ -55,12 +90,10 @@ __global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
-    const int c = (int)(idx % CV) * VEC;
-    long long t = idx / CV;
-    const int iw = (int)(t % W);
-    t /= W;
-    const int ih = (int)(t % H);
-    const long long b = t / H;
+    int cq, iw, ih;
+    long long b;
+    split_idx(idx, CV, W, H, cq, iw, ih, b);
+    const int c = cq * VEC;
     const int i0 = (int)((unsigned)(ih * h) / (unsigned)H), i1 = (int)((unsigned)((ih + 1) * h + H - 1) / (unsigned)H) - 1;
     const int j0 = (int)((unsigned)(iw * w) / (unsigned)W), j1 = (int)((unsigned)((iw + 1) * w + W - 1) / (unsigned)W) - 1;
     float acc[VEC];
@@ -87,17 +120,46 @@ __global__ __launch_bounds__(256) void avgpool_bwd_k(const T* __restrict__ gy, T
     store_f32<T, VEC>(dst, acc);
 }
 
+// Exact halves (H = 2h, W = 2w): a thread takes one pooled pixel's gradient and writes the four input pixels of its
+// bin (one load, four stores; the values are those of the general kernel: gy * 0.25, plus the old value when
+// accumulating).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void avgpool_bwd_x2_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w, int C,
+                                                        int accumulate, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC, W = 2 * w;
+    int cq, j, i;
+    long long b;
+    split_idx(idx, CV, w, h, cq, j, i, b);
+    const int c = cq * VEC;
+    float gv[VEC];
+    load_f32<T, VEC>(gy + ((b * h + i) * w + j) * C + c, gv);
+    T* dst = gx + ((b * 2 * h + 2 * i) * W + 2 * j) * C + c;
+    const long long off[4] = {0, C, (long long)W * C, (long long)W * C + C};
+    float old[4][VEC];
+    if (accumulate) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) load_f32<T, VEC>(dst + off[k], old[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float o[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) o[v] = fmaf(gv[v], 0.25f, 0.f) + (accumulate ? old[k][v] : 0.f);
+        store_f32<T, VEC>(dst + off[k], o);
+    }
+}
+
 // ---------------------------------------------------------------- bilinear, align_corners=False (bilinear.h)
 template <typename T, int VEC>
 __device__ __forceinline__ void bilinear_fwd_item(const T* __restrict__ x, T* __restrict__ y, int h, int w, int C,
                                                   int H, int W, int ldy, float sy, float sx, long long idx) {
     const int CV = C / VEC;
-    const int c = (int)(idx % CV) * VEC;
-    long long t = idx / CV;
-    const int j = (int)(t % W);
-    t /= W;
-    const int i = (int)(t % H);
-    const long long b = t / H;
+    int cq, j, i;
+    long long b;
+    split_idx(idx, CV, W, H, cq, j, i, b);
+    const int c = cq * VEC;
     int y0, y1, x0, x1;
     float ly, lx;
     bl_src(i, sy, h, y0, y1, ly);
@@ -111,6 +173,51 @@ __device__ __forceinline__ void bilinear_fwd_item(const T* __restrict__ x, T* __
 #pragma unroll
     for (int v = 0; v < VEC; ++v) o[v] = bl_mix(a[v], bb[v], cc[v], d[v], ly, lx);
     store_f32<T, VEC>(y + ((b * H + i) * W + j) * ldy + c, o);
+}
+
+// Exactly doubled extents, a 2 x 2 block of outputs per thread: their 16 taps fall on a 3 x 3 neighbourhood of the
+// source (rows m-1 .. m+1, columns n-1 .. n+1, clamped to the image), so 9 loads serve 4 outputs instead of 16.  Same
+// weights (bl_src), same values: at the image border bl_src moves the tap pair one row inwards, but the clamped
+// neighbourhood then holds that row twice, so the static entries (di, di+1) give the same sums.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_fwd_x2_k(const T* __restrict__ x, T* __restrict__ y, int h, int w, int C,
+                                                         int ldy, long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int H = 2 * h, W = 2 * w, CV = C / VEC;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, CV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
+    const T* xb = x + b * h * w * C + c;
+    ChanVec<T, VEC> p[3][3];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        const int rr = min(max(m - 1 + r, 0), h - 1);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int cc = min(max(n - 1 + k, 0), w - 1);
+            p[r][k] = *reinterpret_cast<const ChanVec<T, VEC>*>(xb + ((long long)rr * w + cc) * C);
+        }
+    }
+#pragma unroll
+    for (int di = 0; di < 2; ++di) {
+        int y0, y1;
+        float ly;
+        bl_src(2 * m + di, 0.5f, h, y0, y1, ly);
+#pragma unroll
+        for (int dj = 0; dj < 2; ++dj) {
+            int x0, x1;
+            float lx;
+            bl_src(2 * n + dj, 0.5f, w, x0, x1, lx);
+            float o[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                o[v] = bl_mix(to_f32(p[di][dj].v[v]), to_f32(p[di][dj + 1].v[v]), to_f32(p[di + 1][dj].v[v]),
+                              to_f32(p[di + 1][dj + 1].v[v]), ly, lx);
+            store_f32<T, VEC>(y + ((b * H + 2 * m + di) * W + 2 * n + dj) * ldy + c, o);
+        }
+    }
 }
 
 template <typename T, int VEC>
@@ -148,12 +255,10 @@ __global__ __launch_bounds__(256) void bilinear_bwd_x2_k(const T* __restrict__ g
     if (idx >= total) return;
     const int H = 2 * h, W = 2 * w;
     const int CV = C / VEC;
-    const int c = (int)(idx % CV) * VEC;
-    long long t = idx / CV;
-    const int n = (int)(t % w);
-    t /= w;
-    const int m = (int)(t % h);
-    const long long b = t / h;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, CV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
     float wy[4], wx[4];
     int iy[4], ix[4];
 #pragma unroll
@@ -195,12 +300,10 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
-    const int c = (int)(idx % CV) * VEC;
-    long long t = idx / CV;
-    const int n = (int)(t % w);
-    t /= w;
-    const int m = (int)(t % h);
-    const long long b = t / h;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, CV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
     int ilo, ihi, jlo, jhi;
     bl_dst_range(m, sy, H, ilo, ihi);
     bl_dst_range(n, sx, W, jlo, jhi);
@@ -271,8 +374,10 @@ template <typename T, int VEC>
 __device__ __forceinline__ void gate_fwd_item(const T* __restrict__ x, T* __restrict__ y, int I, int ldy, float s,
                                               long long idx) {
     const int G = I / 2, GV = G / VEC;
-    const int c = (int)(idx % GV) * VEC;
-    const long long m = idx / GV;
+    int cq;
+    long long m;
+    split_idx(idx, GV, cq, m);
+    const int c = cq * VEC;
     float a[VEC], b[VEC], o[VEC];
     load_f32<T, VEC>(x + m * I + c, a);
     load_f32<T, VEC>(x + m * I + G + c, b);
@@ -292,8 +397,10 @@ template <typename T, int VEC>
 __device__ __forceinline__ void gate_bwd_item(const T* __restrict__ x, const T* __restrict__ gy, T* __restrict__ gx,
                                               int I, int ldg, float s, long long idx) {
     const int G = I / 2, GV = G / VEC;
-    const int c = (int)(idx % GV) * VEC;
-    const long long m = idx / GV;
+    int cq;
+    long long m;
+    split_idx(idx, GV, cq, m);
+    const int c = cq * VEC;
     float a[VEC], b[VEC], g[VEC], ga[VEC], gb[VEC];
     load_f32<T, VEC>(x + m * I + c, a);
     load_f32<T, VEC>(x + m * I + G + c, b);
@@ -337,8 +444,10 @@ __device__ __forceinline__ void gate_fwd_items(const T* __restrict__ x, T* __res
         const long long idx = min(first + u * step, total - 1);
         if (sh >= 0)
             c[u] = ((int)idx & (GV - 1)) * VEC, m[u] = idx >> sh;
-        else
-            c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
+        else {
+            split_idx(idx, GV, c[u], m[u]);
+            c[u] *= VEC;
+        }
         a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
         b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
     };
@@ -367,8 +476,10 @@ __device__ __forceinline__ void gate_bwd_items(const T* __restrict__ x, const T*
         const long long idx = min(first + u * step, total - 1);
         if (sh >= 0)
             c[u] = ((int)idx & (GV - 1)) * VEC, m[u] = idx >> sh;
-        else
-            c[u] = (int)(idx % GV) * VEC, m[u] = idx / GV;
+        else {
+            split_idx(idx, GV, c[u], m[u]);
+            c[u] *= VEC;
+        }
         a[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + c[u]);
         b[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(x + m[u] * I + G + c[u]);
         g[u] = *reinterpret_cast<const ChanVec<T, VEC>*>(gy + m[u] * ldg + c[u]);
@@ -401,12 +512,10 @@ __device__ __forceinline__ void gate_bilinear_fwd_item(const T* __restrict__ x, 
                                                        int H, int W, int ldy, float sy, float sx, float s,
                                                        long long idx) {
     const int G = I / 2, GV = G / VEC;
-    const int c = (int)(idx % GV) * VEC;
-    long long t = idx / GV;
-    const int j = (int)(t % W);
-    t /= W;
-    const int i = (int)(t % H);
-    const long long b = t / H;
+    int cq, j, i;
+    long long b;
+    split_idx(idx, GV, W, H, cq, j, i, b);
+    const int c = cq * VEC;
     int y0, y1, x0, x1;
     float ly, lx;
     bl_src(i, sy, h, y0, y1, ly);
@@ -446,12 +555,10 @@ __device__ __forceinline__ void gate_bilinear_fwd_x2_item(const T* __restrict__ 
                                                           int I, int ldy, float s, long long idx) {
     const int H = 2 * h, W = 2 * w;
     const int G = I / 2, GV = G / VEC;
-    const int c = (int)(idx % GV) * VEC;
-    long long t = idx / GV;
-    const int n = (int)(t % w);
-    t /= w;
-    const int m = (int)(t % h);
-    const long long b = t / h;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, GV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
     const T* xb = x + b * h * w * I + c;
     ChanVec<T, VEC> pa[3][3], pb[3][3];
 #pragma unroll
@@ -524,12 +631,10 @@ __device__ __forceinline__ void bilinear_gate_bwd_x2_item(const T* __restrict__ 
                                                           long long idx) {
     const int H = 2 * h, W = 2 * w;
     const int G = I / 2, GV = G / VEC;
-    const int c = (int)(idx % GV) * VEC;
-    long long t = idx / GV;
-    const int n = (int)(t % w);
-    t /= w;
-    const int m = (int)(t % h);
-    const long long b = t / h;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, GV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
     float wy[4], wx[4];
     int iy[4], ix[4];
 #pragma unroll
@@ -1032,8 +1137,10 @@ __global__ __launch_bounds__(256) void add_rowbias_k(T* __restrict__ y, const fl
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int CV = C / VEC;
-    const int c = (int)(idx % CV) * VEC;
-    const long long bp = idx / CV;
+    int cq;
+    long long bp;
+    split_idx(idx, CV, cq, bp);
+    const int c = cq * VEC;
     const int b = (int)(bp / P);
     float a[VEC];
     load_f32<T, VEC>(y + bp * C + c, a);
@@ -1094,8 +1201,17 @@ int avgpool_bwd_launch(const void* gy, void* gx, int B, int H, int W, int C, int
                        hipStream_t s) {
     const void* ptrs[2] = {gy, gx};
     const int vec = pick_vec(C, esize(dtype), ptrs, 2);
-    const long long total = (long long)B * H * W * (C / vec);
     unsigned blocks;
+    if (H == 2 * h && W == 2 * w) {
+        const long long items = (long long)B * h * w * (C / vec);
+        if (items == 0) return 0;
+        if (!grid_for(items, &blocks)) return 1;
+#define CALL(T, V) hipLaunchKernelGGL((avgpool_bwd_x2_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, h, w, C, accumulate, items);
+        PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+        return check_launch("avgpool_bwd");
+    }
+    const long long total = (long long)B * H * W * (C / vec);
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
 #define CALL(T, V) hipLaunchKernelGGL((avgpool_bwd_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)gy, (T*)gx, H, W, C, h, w, accumulate, total);
@@ -1108,8 +1224,17 @@ int bilinear_fwd_launch(const void* x, void* y, int B, int h, int w, int C, int 
                         hipStream_t s) {
     const void* ptrs[2] = {x, y};
     const int vec = pick_vec(gcd_int(C, ldy), esize(dtype), ptrs, 2);
-    const long long total = (long long)B * H * W * (C / vec);
     unsigned blocks;
+    if (H == 2 * h && W == 2 * w) {
+        const long long items = (long long)B * h * w * (C / vec);
+        if (items == 0) return 0;
+        if (!grid_for(items, &blocks)) return 1;
+#define CALL(T, V) hipLaunchKernelGGL((bilinear_fwd_x2_k<T, V>), dim3(blocks), dim3(256), 0, s, (const T*)x, (T*)y, h, w, C, ldy, items);
+        PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+        return check_launch("bilinear_fwd");
+    }
+    const long long total = (long long)B * H * W * (C / vec);
     if (total == 0) return 0;
     if (!grid_for(total, &blocks)) return 1;
     const float sy = (float)h / (float)H, sx = (float)w / (float)W;

@@ -9,9 +9,10 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 
 POOL = [((8, 10), (4, 5), 16), ((57, 61), (28, 30), 100), ((9, 7), (4, 3), 3), ((5, 5), (5, 5), 8), ((7, 9), (1, 1), 6),
-        ((6, 6), (4, 4), 2), ((56, 56), (28, 28), 64), ((4, 5), (9, 11), 4)]
+        ((6, 6), (4, 4), 2), ((56, 56), (28, 28), 64), ((4, 5), (9, 11), 4), ((2, 2), (1, 1), 8), ((2, 6), (1, 3), 5)]
 UP = [((4, 5), (8, 10), 16), ((28, 30), (57, 61), 50), ((3, 4), (7, 9), 3), ((5, 5), (5, 5), 8), ((1, 1), (4, 3), 6),
-      ((8, 8), (5, 6), 2), ((28, 28), (56, 56), 32), ((56, 56), (112, 112), 24)]
+      ((8, 8), (5, 6), 2), ((28, 28), (56, 56), 32), ((56, 56), (112, 112), 24), ((1, 1), (2, 2), 8), ((1, 3), (2, 6), 5),
+      ((2, 1), (4, 2), 16)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
