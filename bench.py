@@ -395,6 +395,9 @@ def kernel_rooflines(B, H, W, D, k, dtype):
     c = [torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(nbuf)]
     xin = [torch.randn(B, H, W, D, device="cuda").to(dtype) for _ in range(4)]
     wup = (torch.randn(I, D, device="cuda") / D ** 0.5).to(dtype)
+    wout = (torch.randn(D, I, device="cuda") / I ** 0.5).to(dtype)
+    rbias = torch.randn(B, D, device="cuda")
+    cats = [torch.empty(B, H, W, I, device="cuda", dtype=dtype) for _ in range(4)]
     N = B * H * W
     for name, fn, nb_, nbytes, fl, pipe in (
         ("gate_fwd", lambda i: ops.gate_forward(c[i]), nbuf, es * 1.5 * N * I, 0.0, "valu"),
@@ -410,6 +413,10 @@ def kernel_rooflines(B, H, W, D, k, dtype):
         # both gradients of conv_up as the block's backward runs them: one launch, gy read once
         ("dense_bwd_pair", lambda i: ops.dense_backward_pair(a[i % 4], wup, xin[i % 4]), 4,
          es * (2 * N * D + N * I + 2 * D * I), 4.0 * N * D * I, "mfma"),
+        # conv_out as the block's forward runs it: on rows it makes from the convolution outputs of both scales (gates,
+        # resize), which it also writes out for the backward
+        ("dense_mid", lambda i: ops.dense_forward_gated(c[i % 4], p[i % 4], wout, rowbias=rbias, cat=cats[i % 4]), 4,
+         es * (N * I + N * I // 4 + N * I + N * D + D * I), 2.0 * N * D * I, "mfma"),
     ):
         t = time_kernel_events(fn, nb_)
         out.append(dict(kernel=name, seconds=t, alg_bytes=nbytes, flops=fl, issued_flops=fl if pipe == "mfma" else None,
@@ -475,6 +482,15 @@ def run_single_kernel(name, iters, B, H, W, D, k, dtype):
         xh = torch.randn(B, h, w, I, device="cuda").to(dtype)
         wt, wt1 = ((torch.randn(k, k, I, device="cuda") / k).to(dtype) for _ in range(2))
         fn = lambda: dwconv.dwconv_forward2(xf, wt, xh, wt1)
+    elif name == "dense_mid":   # conv_out on rows made from the two scales' convolution outputs, writing them to cat
+        from pyramidconvblock_amd import ops
+
+        cf = torch.randn(B, H, W, I, device="cuda").to(dtype)
+        chh = torch.randn(B, h, w, I, device="cuda").to(dtype)
+        cat = torch.empty_like(cf)
+        wout = (torch.randn(D, I, device="cuda") / I ** 0.5).to(dtype)
+        rb = torch.randn(B, D, device="cuda")
+        fn = lambda: ops.dense_forward_gated(cf, chh, wout, rowbias=rb, cat=cat)
     elif name == "bwd3":
         gf, xf = (torch.randn(B, H, W, I, device="cuda").to(dtype) for _ in range(2))
         gp, xh, gh = (torch.randn(B, h, w, I, device="cuda").to(dtype) for _ in range(3))
@@ -582,10 +598,11 @@ def main():
     ap.add_argument("--no-torch-gpu", action="store_true", help="skip the torch-operator comparator on the GPU")
     ap.add_argument("--kernel", default=None, help="only launch this kernel --steps times and exit (for rocprofv3): "
                     "{fwd,dgrad,wgrad}_{full,half}, fwd2, bwd3, conv128, avgpool_{fwd,bwd}, bilinear_{fwd,bwd}, "
-                    "dense_{fwd,pool,dgrad,wgrad,pair}, step, copy")
+                    "dense_{fwd,pool,dgrad,wgrad,pair,mid}, step, copy")
     ap.add_argument("--torch-gpu-only", action="store_true", help="(internal) time the torch-operator comparator and exit")
     ap.add_argument("--headline-only", action="store_true", help="(internal) time the headline step only and exit")
     ap.add_argument("--k", type=int, default=WORKLOAD["k"], help="kernel size for --kernel runs")
+    ap.add_argument("--dtype", default="bf16", choices=sorted(DTYPES), help="element type for --kernel runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (pure data parallel over B; "
@@ -599,7 +616,7 @@ def main():
     dtype = torch.bfloat16
     B, H, W, D, k = (WORKLOAD[n] for n in ("B", "H", "W", "D", "k"))
     if args.kernel:
-        run_single_kernel(args.kernel, args.steps, B, H, W, D, args.k, dtype)
+        run_single_kernel(args.kernel, args.steps, B, H, W, D, args.k, DTYPES[args.dtype])
         return
     if args.torch_gpu_only:
         print(json.dumps({"fwd_bwd_ms": torch_gpu_block((B, H, W, D), D, k, dtype, steps=10, warmup=3)}))

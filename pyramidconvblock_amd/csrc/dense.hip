@@ -21,6 +21,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "reduce_parts.h"
+#include "tile_common.h"
 
 namespace pdw {
 
@@ -648,9 +649,11 @@ __global__ __launch_bounds__(256, 2) void dense_mid_rows_k(const T* __restrict__
                                                         const float* __restrict__ rowbias, T* __restrict__ Y,
                                                         long long N, int Himg, int Wimg, const MidRows mid) {
     extern __shared__ uint32_t dsm[];
+    // (workgroup ids go to the 8 XCDs round-robin: each XCD gets a contiguous range of tiles, so that the half-scale
+    // patches of neighbouring tiles, which overlap, meet in one L2)
     dense_rows_body<T, false, false, 64, 128, false, MID>(nullptr, W, bias, rowbias, Y, nullptr, N, 64, 128,
-                                                           Himg * Wimg, 4, 4, blockIdx.x, gridDim.x, dsm, nullptr, Himg,
-                                                           Wimg, &mid);
+                                                           Himg * Wimg, 4, 4, xcd_remap(blockIdx.x, gridDim.x), gridDim.x,
+                                                           dsm, nullptr, Himg, Wimg, &mid);
 }
 
 // The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
