@@ -408,11 +408,14 @@ int pdw_convblock_supported(int B, int H, int W, int D, int I, int K, int dtype)
 /* Inference forward of the same block (same coverage): y only.  conv_up (which also pools its result for the second
  * scale where its kernel can, pdw_dense_fwd_colsum_pool); then, where pdw_dense_fwd_gated covers the widths and
  * extents, the convolutions of both scales with the mean branch in their launch (pdw_dwconv_fwd2_mean) and conv_out on
- * rows it makes itself from their outputs: three launches, no gated or concatenated tensor in memory.  Elsewhere each
+ * rows it makes itself from their outputs: three launches, no gated or concatenated tensor in memory.  Elsewhere, for
+ * filters up to 13, each
  * scale's convolution with the gate applied in its store (both as one launch, pdw_dwconv_fwd2_gate, or
  * pdw_dwconv_fwd_gate twice, the full-resolution one then pooling its input), the half-resolution gate upsampled into
  * its slice of the concatenation with the mean branch (pdw_block_mid_infer), conv_out: neither convolution output is
- * written to HBM.  Every intermediate lives in `workspace` (pdw_convblock_infer_workspace_bytes).  Same arithmetic as
+ * written to HBM; larger filters at those widths run the launches of pdw_convblock_fwd on workspace tensors (measured
+ * faster than the gated store of their 8-channel slices).  Every intermediate lives in `workspace`
+ * (pdw_convblock_infer_workspace_bytes).  Same arithmetic as
  * pdw_convblock_fwd.  Replaces ConvBlock.forward under torch.no_grad(), conv_block.py:36-49 with :13-22. */
 size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype);
 int pdw_convblock_infer(const void *x, const void *w_up, const void *w_dw0, const void *w_dw1, const void *w_pool,

@@ -93,7 +93,7 @@ using namespace pdw;
 
 extern "C" {
 
-int pdw_version(void) { return 4; }
+int pdw_version(void) { return 5; }
 
 const char* pdw_last_error(void) { return g_err; }
 

@@ -128,8 +128,16 @@ int pdw_convblock_fwd(const void* x, const void* w_up, const void* w_dw0, const 
     return pdw_dense_fwd(cat, w_out, 0, nullptr, yp, y, s.N, I, D, s.P, dtype, stream);
 }
 
-// The fused convolution + gate needs images small enough for the kernel's 32-bit offsets (two images side by side).
-static bool infer_fused(int H, int W, int I, int K) { return K <= 17 && (long long)H * W * I * 2 <= 0x1fffffffLL; }
+// The convolution with the gate in its store, for the widths conv_out's made-rows kernel does not cover: images small
+// enough for the kernel's 32-bit offsets (two images side by side), and filters up to 13 (with the 8-channel slices of
+// larger filters the gated store's 8-byte loads cost more than they save: 62.6 against 54.7 us for the forward at
+// [8,112,112,96], K = 17, so those run the training forward's launches on workspace tensors).
+static bool infer_fused(int H, int W, int I, int K) { return K <= 13 && (long long)H * W * I * 2 <= 0x1fffffffLL; }
+// conv_out on rows it makes itself from the convolution outputs (pdw_dense_fwd_gated), after the convolutions of both
+// scales as one launch: every odd K.
+static bool infer_made_rows(int B, int H, int W, int D, int I, int K, int dtype) {
+    return I == 64 && D == 128 && H % 4 == 0 && W % 8 == 0 && pdw_dwconv_fwd2_supported(B, H, W, I, K, dtype) != 0;
+}
 
 size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
     if (!pdw_convblock_supported(B, H, W, D, I, K, dtype)) return 0;
@@ -137,7 +145,7 @@ size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, in
     const size_t full = (size_t)s.N * I * s.es, half = (size_t)B * s.h * s.w * I * s.es;
     size_t b = up256(full) /* a */ + up256(half) /* xp */ + up256(full) /* cat */ + up256((size_t)B * D * s.es) /* m */ +
                up256((size_t)s.nt * D * 4) + up256((size_t)B * D * 4);
-    if (infer_fused(H, W, I, K))
+    if (infer_made_rows(B, H, W, D, I, K, dtype) || infer_fused(H, W, I, K))
         b += up256(half);  // the gated half-resolution scale, or the half scale's convolution output
     else
         b += up256(full) + up256(half);  // c0, c1
@@ -165,6 +173,22 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
     float* xparts = (float*)ws.take((size_t)s.nt * D * 4);
     float* yp = (float*)ws.take((size_t)B * D * 4);
     const int pad = K / 2, G = I / 2;
+    if (infer_made_rows(B, H, W, D, I, K, dtype) && !(reinterpret_cast<uintptr_t>(w_out) & 15)) {
+        // three launches: conv_up (with the tile sums of x and the pool of its result), the convolutions of both scales
+        // with the mean branch, conv_out on rows made from their outputs, which pass through the workspace (measured:
+        // as fast as gating them in the convolutions' stores at K <= 13, 2 us faster at K = 17)   (conv_block.py:36-49)
+        void* c0 = cat;
+        void* c1 = ws.take(half);
+        if (int e = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream)) return e;
+        int r = pdw_dwconv_fwd2_mean(a, w_dw0, c0, 0, 0, xp, w_dw1, c1, 0, 0, B, H, W, I, K, xparts, (int)(s.nt / B), w_pool,
+                                     b_pool, b_out, m, yp, s.P, D, dtype, stream);
+        if (r == 3) {   // (a mean branch the riding form does not cover, e.g. an unaligned conv_pool weight)
+            if ((r = pdw_dwconv_fwd2(a, w_dw0, c0, xp, w_dw1, c1, B, H, W, I, K, dtype, stream))) return r;
+            r = pdw_pool_branch_fwd_parts(xparts, (int)(s.nt / B), w_pool, b_pool, b_out, m, yp, B, s.P, D, dtype, stream);
+        }
+        if (r) return r;
+        return pdw_dense_fwd_gated(c0, c1, nullptr, w_out, nullptr, yp, y, B, H, W, I, D, 0, dtype, stream);
+    }
     if (!infer_fused(H, W, I, K)) {
         void* c0 = ws.take(full);
         void* c1 = ws.take(half);
@@ -180,16 +204,6 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
         const int pooled = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream);
         if (pooled != 0 && pooled != 3) return pooled;
         if (pooled == 0) {
-            // where conv_out's kernel can make its rows itself (both gates and the resize where it stages a tile): the
-            // convolutions with the mean branch in their launch, then that layer: three launches.  The convolution
-            // outputs pass through the workspace (measured: as fast as gating them in the convolutions' stores at
-            // K <= 13, 2 us faster at K = 17).                                                (conv_block.py:41-49)
-            if (I == 64 && D == 128 && H % 4 == 0 && W % 8 == 0 && !(reinterpret_cast<uintptr_t>(w_out) & 15)) {
-                both = pdw_dwconv_fwd2_mean(a, w_dw0, cat, 0, 0, xp, w_dw1, g1, 0, 0, B, H, W, I, K, xparts, (int)(s.nt / B),
-                                            w_pool, b_pool, b_out, m, yp, s.P, D, dtype, stream);
-                if (both == 0) return pdw_dense_fwd_gated(cat, g1, nullptr, w_out, nullptr, yp, y, B, H, W, I, D, 0, dtype, stream);
-                if (both != 3) return both;
-            }
             both = pdw_dwconv_fwd2_gate(a, w_dw0, cat, I, 0, xp, w_dw1, g1, G, 0, B, H, W, I, K, dtype, stream);
             if (both != 0 && both != 3) return both;
         } else if (int e = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream)) {
