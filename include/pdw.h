@@ -362,8 +362,10 @@ int pdw_dense_fwd_colsum_pool(const void *x, const void *w, const void *bias, vo
  * NULL) receives the rows, which the backward pass reads again.  Bitwise what pdw_gate_pair_fwd (or pdw_block_mid_fwd)
  * followed by pdw_dense_fwd produce; the gated tensor is not read back from memory.  ldf > 0 (inference, after
  * pdw_dwconv_fwd2_gate): both scales arrive gated, cf[B,H,W,I/2] at a pixel stride of ldf values and ch[B,H/2,W/2,I/2],
- * only the resize is left to do and cat must be NULL.  Status 3 (nothing launched) where not covered: 16-bit types,
- * I = 64, D = 128, H % 4 == 0, W % 8 == 0 only. */
+ * only the resize is left to do and cat must be NULL.  Status 3 (nothing launched) where not covered
+ * (pdw_dense_fwd_gated_supported says so beforehand): 16-bit types, H % 4 == 0, W % 8 == 0, I a multiple of 16 up to 64,
+ * D a multiple of 8 up to 128 with D + 8 >= 1.5 I (I = 64, D = 128 runs the variant with compile-time extents). */
+int pdw_dense_fwd_gated_supported(int H, int W, int I, int D, int dtype);
 int pdw_dense_fwd_gated(const void *cf, const void *ch, void *cat, const void *w, const void *bias,
                         const float *rowbias, void *y, int B, int H, int W, int I, int D, int ldf, int dtype,
                         void *stream);
@@ -392,7 +394,8 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
 /* The whole block of conv_block.py:25-49 (scales (1, 1/2), conv_up without bias) as one host call each way: the
  * launch sequence of the entry points above (forward: conv_up with the pool of its result, the convolutions of both
  * scales with the mean branch, conv_out on rows it makes from their outputs, writing cat: 3 launches for D = 128,
- * I = 64, H % 4 == 0, W % 8 == 0, else 4 with the gates and the mean branch as one launch of their own; backward: 5
+ * I = 64, H % 4 == 0, W % 8 == 0; other widths that pdw_dense_fwd_gated covers pool in a launch of their own; else the
+ * gates and the mean branch are one launch before conv_out; backward: 5
  * launches and one summation launch)
  * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
  * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense

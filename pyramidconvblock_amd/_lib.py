@@ -79,6 +79,7 @@ _SIGS = {
     "pdw_dwconv_fwd2": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "pdw_dwconv_fwd2_mean": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_void_p] * 3 + [c_int] * 7 + [c_void_p, c_int]
                              + [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),
+    "pdw_dense_fwd_gated_supported": (c_int, [c_int] * 5),
     "pdw_dense_fwd_gated": (c_int, [c_void_p] * 7 + [c_int] * 7 + [c_void_p]),
     "pdw_dwconv_fwd2_gate": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_void_p] * 3 + [c_int] * 2 + [c_int] * 6 + [c_void_p]),
     "pdw_dwconv_bwd3_plan": (c_int, [c_int] * 6 + [c_void_p]),

@@ -630,6 +630,10 @@ int pdw_dense_fwd_colsum_pool(const void* x, const void* w, const void* bias, vo
     return r;
 }
 
+int pdw_dense_fwd_gated_supported(int H, int W, int I, int D, int dtype) {
+    return valid_dtype(dtype) && H > 0 && W > 0 && I > 0 && D > 0 ? dense_mid_rows_supported(H, W, I, D, dtype) : 0;
+}
+
 int pdw_dense_fwd_gated(const void* cf, const void* ch, void* cat, const void* w, const void* bias, const float* rowbias,
                         void* y, int B, int H, int W, int I, int D, int ldf, int dtype, void* stream) {
     if (!valid_dtype(dtype)) return set_error("pdw_dense_fwd_gated: unknown dtype %d", dtype), 1;

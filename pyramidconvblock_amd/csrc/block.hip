@@ -136,7 +136,7 @@ static bool infer_fused(int H, int W, int I, int K) { return K <= 13 && (long lo
 // conv_out on rows it makes itself from the convolution outputs (pdw_dense_fwd_gated), after the convolutions of both
 // scales as one launch: every odd K.
 static bool infer_made_rows(int B, int H, int W, int D, int I, int K, int dtype) {
-    return I == 64 && D == 128 && H % 4 == 0 && W % 8 == 0 && pdw_dwconv_fwd2_supported(B, H, W, I, K, dtype) != 0;
+    return pdw_dense_fwd_gated_supported(H, W, I, D, dtype) != 0 && pdw_dwconv_fwd2_supported(B, H, W, I, K, dtype) != 0;
 }
 
 size_t pdw_convblock_infer_workspace_bytes(int B, int H, int W, int D, int I, int K, int dtype) {
@@ -174,13 +174,18 @@ int pdw_convblock_infer(const void* x, const void* w_up, const void* w_dw0, cons
     float* yp = (float*)ws.take((size_t)B * D * 4);
     const int pad = K / 2, G = I / 2;
     if (infer_made_rows(B, H, W, D, I, K, dtype) && !(reinterpret_cast<uintptr_t>(w_out) & 15)) {
-        // three launches: conv_up (with the tile sums of x and the pool of its result), the convolutions of both scales
+        // three launches (four where conv_up's kernel does not pool): conv_up (with the tile sums of x and the pool of its result), the convolutions of both scales
         // with the mean branch, conv_out on rows made from their outputs, which pass through the workspace (measured:
         // as fast as gating them in the convolutions' stores at K <= 13, 2 us faster at K = 17)   (conv_block.py:36-49)
         void* c0 = cat;
         void* c1 = ws.take(half);
-        if (int e = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream)) return e;
-        int r = pdw_dwconv_fwd2_mean(a, w_dw0, c0, 0, 0, xp, w_dw1, c1, 0, 0, B, H, W, I, K, xparts, (int)(s.nt / B), w_pool,
+        int r = pdw_dense_fwd_colsum_pool(x, w_up, nullptr, a, xparts, xp, B, H, W, D, I, dtype, stream);
+        if (r == 3) {   // (widths whose conv_up kernel does not pool: the layer with its tile sums, then the pool)
+            if ((r = pdw_dense_fwd_colsum(x, w_up, 0, nullptr, nullptr, a, xparts, s.N, D, I, s.P, dtype, stream))) return r;
+            r = pdw_avgpool_fwd(a, xp, B, H, W, I, s.h, s.w, dtype, stream);
+        }
+        if (r) return r;
+        r = pdw_dwconv_fwd2_mean(a, w_dw0, c0, 0, 0, xp, w_dw1, c1, 0, 0, B, H, W, I, K, xparts, (int)(s.nt / B), w_pool,
                                      b_pool, b_out, m, yp, s.P, D, dtype, stream);
         if (r == 3) {   // (a mean branch the riding form does not cover, e.g. an unaligned conv_pool weight)
             if ((r = pdw_dwconv_fwd2(a, w_dw0, c0, xp, w_dw1, c1, B, H, W, I, K, dtype, stream))) return r;

@@ -217,7 +217,8 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                                                 int Wimg = 0, const MidRows* mid = nullptr) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
     static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
-    static_assert(MID == 0 || (SK == 64 && SNO == 128 && !KMAJOR && !COLSUM && !POOL), "made rows: the 64 -> 128 layer");
+    static_assert(MID == 0 || (((SK == 64 && SNO == 128) || (SK == 0 && SNO == 0)) && !KMAJOR && !COLSUM && !POOL),
+                  "made rows: the 64 -> 128 layer with its extents as constants, or any covered widths");
     // POOL: first pixel of a tile and first pixel of its part of the pooled tensor (two 32-bit divisions per tile,
     // taken once, when the tile is requested, and kept for its way out)
     int px_next = 0, pp_next = 0, px_cur = 0, pp_cur = 0;
@@ -261,27 +262,46 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
     constexpr int LP = 8;                               // chunk loads per lane (K <= 128)
     Frag raw[LP];
     float4 brow = make_float4(0.f, 0.f, 0.f, 0.f);
-    // MID: a lane makes the 8-value chunks (pixel idx / 4, values 8 (idx % 4) ..) of both halves of the rows for
-    // idx = lane, lane + 64, and gates the chunks (patch pixel idx / 4 < 24, 8 (idx % 4) ..) of the half-scale patch
+    // MID: with G = K / 2 gated values per scale and ncc = G / 8 chunks of 8, a lane makes the chunks (pixel idx / ncc,
+    // values 8 (idx % ncc) ..) of both halves of the rows for idx = lane, lane + 64 (idx < 32 ncc: K <= 64), and gates
+    // the chunks (patch pixel idx / ncc < 24, same values) of the half-scale patch.  Lane constants, the same for every
+    // tile: the item's pixel and chunk (clamped for the loads, which then read valid addresses) and whether it exists.
+    const int MG = K >> 1;
+    [[maybe_unused]] int mpix[2] = {0, 0}, mcc[2] = {0, 0};
+    [[maybe_unused]] bool mok[2] = {false, false};
+    if constexpr (MID != 0) {
+        const int ncc = MG >> 3;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int idx = p * 64 + lane;
+            if constexpr (STATIC) {
+                mpix[p] = idx >> 2, mcc[p] = idx & 3, mok[p] = true;
+            } else {
+                const int pix = idx / ncc;
+                mok[p] = pix < 32;
+                mpix[p] = min(pix, 31), mcc[p] = idx - pix * ncc;
+            }
+        }
+    }
     [[maybe_unused]] Frag fa[2], fb[2], ha[2], hb[2];
     [[maybe_unused]] auto mid_load = [&](long long t) {
         const int b = tile_pixel(t);
         const int hh = Himg >> 1, hw = Wimg >> 1;
-        const int ldf = MID == 1 ? 64 : mid->ldf, ldh = MID == 1 ? 64 : 32;
+        const int ldf = MID == 1 ? K : mid->ldf, ldh = MID == 1 ? K : MG;
         const T* cf = static_cast<const T*>(mid->cf) + (long long)px_next * ldf;
         const T* chb = static_cast<const T*>(mid->ch) + (long long)b * hh * hw * ldh;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
+            const int pix = mpix[p], cc = mcc[p];
             const T* f = cf + (long long)((pix >> 3) * Wimg + (pix & 7)) * ldf + 8 * cc;
             fa[p] = *reinterpret_cast<const Frag*>(f);
-            if constexpr (MID == 1) fb[p] = *reinterpret_cast<const Frag*>(f + 32);
+            if constexpr (MID == 1) fb[p] = *reinterpret_cast<const Frag*>(f + MG);
             // (patch entries past the image are never used as taps: clamped, they are readable)
             const int q = min(pix, 23), qr = q / 6, qc = q - 6 * qr;
             const int hy = min(max(2 * rb_next - 1 + qr, 0), hh - 1), hx = min(max(4 * cb_next - 1 + qc, 0), hw - 1);
             const T* hp = chb + (long long)(hy * hw + hx) * ldh + 8 * cc;
             ha[p] = *reinterpret_cast<const Frag*>(hp);
-            if constexpr (MID == 1) hb[p] = *reinterpret_cast<const Frag*>(hp + 32);
+            if constexpr (MID == 1) hb[p] = *reinterpret_cast<const Frag*>(hp + MG);
         }
     };
     auto load_tile = [&](long long t) {                 // coalesced: chunk i*64+lane of the tile's byte range
@@ -366,43 +386,49 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             rb_cur = rb_next, cb_cur = cb_next;
             const int hh = Himg >> 1, hw = Wimg >> 1;
             T* cat = MID == 1 ? static_cast<T*>(mid->cat) : nullptr;
-            // the gated patch of the half scale: [24 pixels][32] in columns 64.. of the tile buffer's rows
+            // the gated patch of the half scale: [24 pixels][G] in columns K.. of the tile buffer's rows
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
-                const int idx = p * 64 + lane, q = idx >> 2, cc = idx & 3;
-                Frag hg = ha[p];
+                const int q = mpix[p], cc = mcc[p];
+                Frag hg;
                 if constexpr (MID == 1) hg = gate8<T>(ha[p], hb[p], mid->gs);
-                if (q < 24) *reinterpret_cast<Frag*>(tl + q * ldt + 64 + 8 * cc) = hg;
+                else hg = Frag{{ha[p].v[0], ha[p].v[1], ha[p].v[2], ha[p].v[3]}};
+                if (mok[p] && q < 24) *reinterpret_cast<Frag*>(tl + q * ldt + K + 8 * cc) = hg;
             }
             // the full scale's half of the rows
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
-                const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
-                Frag full = fa[p];
+                const int pix = mpix[p], cc = mcc[p];
+                Frag full;
                 if constexpr (MID == 1) full = gate8<T>(fa[p], fb[p], mid->gs);
-                *reinterpret_cast<Frag*>(tl + pix * ldt + 8 * cc) = full;
-                if (cat)
-                    *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * 64 + 8 * cc) = full;
+                else full = Frag{{fa[p].v[0], fa[p].v[1], fa[p].v[2], fa[p].v[3]}};
+                if (mok[p]) {
+                    *reinterpret_cast<Frag*>(tl + pix * ldt + 8 * cc) = full;
+                    if (cat)
+                        *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * K + 8 * cc) = full;
+                }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the patch is in LDS (written by other lanes of this wavefront)
             // the resized half: four taps of the patch per pixel, bl_src's rows, columns and weights
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
-                const int idx = p * 64 + lane, pix = idx >> 2, cc = idx & 3;
+                const int pix = mpix[p], cc = mcc[p];
                 int y0, y1, x0, x1;
                 float ly, lx;
                 bl_src(4 * rb_cur + (pix >> 3), 0.5f, hh, y0, y1, ly);
                 bl_src(8 * cb_cur + (pix & 7), 0.5f, hw, x0, x1, lx);
                 const int oy = 2 * rb_cur - 1, ox = 4 * cb_cur - 1;   // source row / column of patch entry (0, 0)
-                const T* pt = tl + 64 + 8 * cc;
+                const T* pt = tl + K + 8 * cc;
                 const Frag g00 = *reinterpret_cast<const Frag*>(pt + ((y0 - oy) * 6 + (x0 - ox)) * ldt);
                 const Frag g01 = *reinterpret_cast<const Frag*>(pt + ((y0 - oy) * 6 + (x1 - ox)) * ldt);
                 const Frag g10 = *reinterpret_cast<const Frag*>(pt + ((y1 - oy) * 6 + (x0 - ox)) * ldt);
                 const Frag g11 = *reinterpret_cast<const Frag*>(pt + ((y1 - oy) * 6 + (x1 - ox)) * ldt);
                 const Frag up = bilinear8<T>(g00, g01, g10, g11, ly, lx);
-                *reinterpret_cast<Frag*>(tl + pix * ldt + 32 + 8 * cc) = up;
-                if (cat)
-                    *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * 64 + 32 + 8 * cc) = up;
+                if (mok[p]) {
+                    *reinterpret_cast<Frag*>(tl + pix * ldt + MG + 8 * cc) = up;
+                    if (cat)
+                        *reinterpret_cast<Frag*>(cat + ((long long)px_cur + (pix >> 3) * Wimg + (pix & 7)) * K + MG + 8 * cc) = up;
+                }
             }
         } else {
         // raw chunks -> LDS [row][k] -> MFMA fragments (row l32, k = kt*16 + 8*half ..)
@@ -588,10 +614,22 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 yb = Y + (long long)px_cur * NO;
                 Frag of[LO];
 #pragma unroll
-                for (int i = 0; i < LO; ++i) of[i] = *reinterpret_cast<const Frag*>(tl + oout[i]);
+                for (int i = 0; i < LO; ++i) of[i] = *reinterpret_cast<const Frag*>(tl + (oout[i] >= 0 ? oout[i] : 0));
+                if constexpr (STATIC) {
 #pragma unroll
-                for (int i = 0; i < LO; ++i)   // chunks i*64 .. = pixels 4 i .. 4 i + 3 of the tile: image row i / 2, 4 columns
-                    *reinterpret_cast<Frag*>(yb + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * NO + lane * 8) = of[i];
+                    for (int i = 0; i < LO; ++i)   // chunks i*64 .. = pixels 4 i .. 4 i + 3 of the tile: image row i / 2, 4 columns
+                        *reinterpret_cast<Frag*>(yb + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * NO + lane * 8) = of[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < LO; ++i)
+                        asm volatile("" : "+v"(of[i].v[0]), "+v"(of[i].v[1]), "+v"(of[i].v[2]), "+v"(of[i].v[3]));
+#pragma unroll
+                    for (int i = 0; i < LO; ++i) {   // chunk i*64 + lane = (pixel, 8 features) of the tile
+                        const int cidx = i * 64 + lane, pix = cidx / cpr, cc = cidx - pix * cpr;
+                        if (pix < 32)
+                            *reinterpret_cast<Frag*>(yb + (long long)((pix >> 3) * Wimg + (pix & 7)) * NO + 8 * cc) = of[i];
+                    }
+                }
             } else if (STATIC && rows_left >= 32) {  // (an array of its own: one array written on both paths ends up in scratch)
                 Frag of[LO];
 #pragma unroll
@@ -644,16 +682,17 @@ __global__ __launch_bounds__(256, 2) void dense_rows_pool_k(const T* __restrict_
 }
 
 // The 64 -> 128 layer on rows made from the two scales of a pyramid block (dense_rows_body, MID).
-template <typename T, int MID>
+template <typename T, int MID, int SK, int SNO>
 __global__ __launch_bounds__(256, 2) void dense_mid_rows_k(const T* __restrict__ W, const T* __restrict__ bias,
                                                         const float* __restrict__ rowbias, T* __restrict__ Y,
-                                                        long long N, int Himg, int Wimg, const MidRows mid) {
+                                                        long long N, int Himg, int Wimg, int K, int NO,
+                                                        const MidRows mid) {
     extern __shared__ uint32_t dsm[];
     // (workgroup ids go to the 8 XCDs round-robin: each XCD gets a contiguous range of tiles, so that the half-scale
     // patches of neighbouring tiles, which overlap, meet in one L2)
-    dense_rows_body<T, false, false, 64, 128, false, MID>(nullptr, W, bias, rowbias, Y, nullptr, N, 64, 128,
-                                                           Himg * Wimg, 4, 4, xcd_remap(blockIdx.x, gridDim.x), gridDim.x,
-                                                           dsm, nullptr, Himg, Wimg, &mid);
+    dense_rows_body<T, false, false, SK, SNO, false, MID>(nullptr, W, bias, rowbias, Y, nullptr, N, K, NO, Himg * Wimg,
+                                                           (K + 15) / 16, (NO + 31) / 32, xcd_remap(blockIdx.x, gridDim.x),
+                                                           gridDim.x, dsm, nullptr, Himg, Wimg, &mid);
 }
 
 // The same with the deferred partial-sum reductions of a backward pass in the first gridDim.x - nblocks
@@ -999,14 +1038,24 @@ int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void*
 // (dense_rows_body, MID): cf [B,H,W,64], ch [B,H/2,W/2,64]; cat (optional) receives the rows.  ldf > 0: both scales
 // arrive gated, cf [B,H,W,32] at a pixel stride of ldf values, ch [B,H/2,W/2,32], no cat.  -1: not covered (other
 // widths, extents that are not multiples of 4 x 8, fp32).
+// Whether dense_mid_rows_launch covers the widths and extents (aligned tensors assumed).
+int dense_mid_rows_supported(int H, int W, int I, int D, int dtype) {
+    if (dtype == kF32 || I < 16 || I > 64 || I % 16 != 0 || !dense_dims_ok(I, D, dtype) || I + I / 2 > (I > D ? I : D) + 8)
+        return 0;
+    return (H % 4 == 0 && W % 8 == 0 && H >= 4 && W >= 8 && !tune_env("PDW_NO_DENSE_MID")) ? 1 : 0;
+}
+
 int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void* w, const void* bias,
                           const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s,
                           int ldf) {
-    if (dtype == kF32 || I != 64 || D != 128 || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
-    if (ldf != 0 && (ldf < 32 || ldf % 8 != 0 || cat)) return -1;
-    if (tune_env("PDW_NO_DENSE_MID")) return -1;
+    // widths: the inner one a multiple of 16 up to 64 (two items per lane make a tile's rows), the outer one whatever the
+    // row kernel covers, wide enough that the half scale's patch fits beside a tile's rows in the tile buffer
+    if (!dense_mid_rows_supported(H, W, I, D, dtype) || B < 1) return -1;
+    if (ldf != 0 && (ldf < I / 2 || ldf % 8 != 0 || cat)) return -1;
     const long long N = (long long)B * H * W;
     if (N > 0x7fffffffLL / 128) return -1;
+    const bool exact = I == 64 && D == 128 && !tune_env("PDW_DENSE_GENERIC");
+    const int nnt = cdiv(D, 32);
     for (const void* p : {cf, ch, w, (const void*)y})
         if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
     if ((reinterpret_cast<uintptr_t>(cat) & 15) || (reinterpret_cast<uintptr_t>(rowbias) & 15) ||
@@ -1016,17 +1065,23 @@ int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void*
     long long blocks = (ntiles + 3) / 4;
     const int cap = tune_env("PDW_DENSE_BLOCKS") ? atoi(tune_env("PDW_DENSE_BLOCKS")) : 512;
     if (blocks > cap) blocks = cap;
-    const size_t lds = ((size_t)4 * 32 * (64 + 8) + 4 * 32 * (128 + 8)) * 2 +
-                       ((bias || rowbias) ? (size_t)4 * 2 * 4 * 32 * sizeof(float) : 0);
+    const size_t lds = ((size_t)nnt * 32 * (64 + 8) + 4 * 32 * ((I > D ? I : D) + 8)) * 2 +
+                       ((bias || rowbias) ? (size_t)4 * 2 * nnt * 32 * sizeof(float) : 0);
     const MidRows mid{cf, ch, cat, ldf, sqrtf((float)(I / 2))};
-#define PDW_MID(T, M)                                                                                                   \
-    hipLaunchKernelGGL((dense_mid_rows_k<T, M>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)w, (const T*)bias, \
-                       rowbias, (T*)y, N, H, W, mid)
+#define PDW_MID(T, M, SK, SNO)                                                                                   \
+    hipLaunchKernelGGL((dense_mid_rows_k<T, M, SK, SNO>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)w, \
+                       (const T*)bias, rowbias, (T*)y, N, H, W, I, D, mid)
+#define PDW_MID_S(T, M)            \
+    if (exact)                     \
+        PDW_MID(T, M, 64, 128);    \
+    else                           \
+        PDW_MID(T, M, 0, 0)
     if (dtype == kF16) {
-        if (ldf) PDW_MID(f16_t, 2); else PDW_MID(f16_t, 1);
+        if (ldf) { PDW_MID_S(f16_t, 2); } else { PDW_MID_S(f16_t, 1); }
     } else {
-        if (ldf) PDW_MID(bf16_t, 2); else PDW_MID(bf16_t, 1);
+        if (ldf) { PDW_MID_S(bf16_t, 2); } else { PDW_MID_S(bf16_t, 1); }
     }
+#undef PDW_MID_S
 #undef PDW_MID
     return check_launch("dense_mid_rows");
 }

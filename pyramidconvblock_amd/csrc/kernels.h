@@ -111,6 +111,7 @@ int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void*
 // the 64 -> 128 layer on rows made from the two convolution outputs of a pyramid block (gates and resize where the
 // tile is staged); cat (optional) receives the rows; ldf > 0: the scales arrive gated, I / 2 wide, the full one at a pixel
 // stride of ldf values; -1 = not covered
+int dense_mid_rows_supported(int H, int W, int I, int D, int dtype);
 int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void* w, const void* bias,
                           const float* rowbias, void* y, int B, int H, int W, int I, int D, int dtype, hipStream_t s,
                           int ldf = 0);

@@ -392,7 +392,8 @@ def test_sum_parts_is_the_fp32_sum_rounded_once(shape, dtype):
 @pytest.mark.parametrize("with_cat", [True, False])
 @pytest.mark.parametrize("case", [(32, 56, 56, 64, 128), (1, 4, 8, 64, 128), (3, 8, 16, 64, 128), (2, 12, 40, 64, 128),
                                   (2, 64, 8, 64, 128), (5, 36, 24, 64, 128), (2, 10, 16, 64, 128), (2, 8, 16, 32, 64),
-                                  (70, 8, 8, 64, 128)])
+                                  (70, 8, 8, 64, 128), (8, 112, 112, 48, 96), (3, 8, 24, 16, 32), (2, 12, 16, 64, 96),
+                                  (2, 8, 8, 32, 128), (2, 8, 8, 48, 56), (2, 8, 8, 96, 128), (2, 8, 8, 24, 48)])
 def test_dense_forward_gated_is_the_gates_then_the_layer(oracle, dtype, with_cat, case):
     """pdw_dense_fwd_gated (the block's output layer on rows it makes from the two convolution outputs: both gates and
     the resize where the tile is staged) gives bitwise what the gate launch followed by the plain layer gives, with
@@ -408,8 +409,13 @@ def test_dense_forward_gated_is_the_gates_then_the_layer(oracle, dtype, with_cat
     rowbias = randn(gen, B, D).cuda()
     cat = torch.full((B, H, W, I), 5.0, device="cuda", dtype=dtype) if with_cat else None
     y = ops.dense_forward_gated(cf, ch, w, rowbias=rowbias, cat=cat)
-    covered = dtype != torch.float32 and (I, D) == (64, 128) and H % 4 == 0 and W % 8 == 0
+    # the inner width a multiple of 16 up to 64, the outer one a multiple of 8 up to 128 and wide enough for the half
+    # scale's patch beside a tile's rows (D + 8 >= 1.5 I)
+    covered = (dtype != torch.float32 and I % 16 == 0 and I <= 64 and D % 8 == 0 and D <= 128 and 3 * I // 2 <= max(I, D) + 8
+               and H % 4 == 0 and W % 8 == 0)
     assert (y is not None) == covered
+    from pyramidconvblock_amd import _lib
+    assert bool(_lib.lib().pdw_dense_fwd_gated_supported(H, W, I, D, _lib.dtype_code(dtype))) == covered
     if y is None:
         return
     want_cat = torch.empty((B, H, W, I), device="cuda", dtype=dtype)
@@ -419,7 +425,7 @@ def test_dense_forward_gated_is_the_gates_then_the_layer(oracle, dtype, with_cat
     if with_cat:
         assert torch.equal(cat, want_cat)
     assert torch.equal(y, want)
-    if B * H * W <= 4096:   # and against the oracle, directly
+    if B * H * W <= 4096 or (I, D) == (48, 96):   # and against the oracle, directly
         g0 = oracle.gate_fwd(cf.double().cpu().numpy())
         g1 = oracle.bilinear_fwd(oracle.gate_fwd(ch.double().cpu().numpy()), (H, W))
         rows = torch.cat([torch.from_numpy(g0), torch.from_numpy(g1)], -1)
