@@ -153,3 +153,20 @@ def test_single_call_block_is_the_stepwise_block(case, out_bias, monkeypatch):
     assert len(single) == len(stepwise)
     for i, (s, t) in enumerate(zip(single, stepwise)):
         assert s is not None and torch.equal(s, t), f"result {i} differs"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_two_scale_blocks(oracle, seed):
+    """Seeded random blocks over the widths, extents and filter sizes of the fused forward (conv_up with or without its
+    pooling variant, the convolutions with the mean branch in their launch, conv_out on rows it makes itself with the
+    extents as constants or as arguments) and its fallbacks (extents off the 4 x 8 tiles, inner widths beyond 64)."""
+    import random
+
+    rng = random.Random(1000 + seed)
+    dim = rng.choice([32, 64, 96, 128, 128, 160, 192])
+    k = rng.choice([3, 5, 7, 9, 11, 13, 15, 17])
+    B = rng.choice([1, 2, 3, 5, 9])
+    H = rng.choice([4, 8, 12, 16, 20, 28, 6, 10])
+    W = rng.choice([8, 16, 24, 40, 56, 12, 36])
+    dtype = rng.choice([torch.float16, torch.bfloat16])
+    _block_case(oracle, dim, k, (B, H, W, dim), dtype, seed=seed)
