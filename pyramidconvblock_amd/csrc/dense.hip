@@ -217,8 +217,8 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                                                 int Wimg = 0, const MidRows* mid = nullptr) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
     static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
-    static_assert(MID == 0 || (((SK == 64 && SNO == 128) || (SK == 0 && SNO == 0)) && !KMAJOR && !COLSUM && !POOL),
-                  "made rows: the 64 -> 128 layer with its extents as constants, or any covered widths");
+    static_assert(MID == 0 || (((STATIC && SK <= 64) || (SK == 0 && SNO == 0)) && !KMAJOR && !COLSUM && !POOL),
+                  "made rows: a layer with its extents as constants (inner width up to 64), or any covered widths");
     // POOL: first pixel of a tile and first pixel of its part of the pooled tensor (two 32-bit divisions per tile,
     // taken once, when the tile is requested, and kept for its way out)
     int px_next = 0, pp_next = 0, px_cur = 0, pp_cur = 0;
@@ -231,9 +231,9 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         rb_next = (int)rb, cb_next = (int)cb;
         return (int)b;
     };
-    static_assert(!STATIC || (SK % 16 == 0 && SNO % 32 == 0 && SK <= 128 && SNO <= 128), "static dense shape");
+    static_assert(!STATIC || (SK % 16 == 0 && SNO % 16 == 0 && SK <= 128 && SNO <= 128), "static dense shape");
     const int K = STATIC ? SK : Kd, NO = STATIC ? SNO : NOd;
-    const int nkt = STATIC ? SK / 16 : nktd, nnt = STATIC ? SNO / 32 : nntd;
+    const int nkt = STATIC ? SK / 16 : nktd, nnt = STATIC ? (SNO + 31) / 32 : nntd;
     T* wl = reinterpret_cast<T*>(dsm);
     // The weights are multiplied as NOP x KP (whole feature tiles, 4 or 8 steps of the inner dimension) with zeros
     // in the padding, so that the multiplication below is straight-line code without predicates.
@@ -274,7 +274,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int idx = p * 64 + lane;
-            if constexpr (STATIC) {
+            if constexpr (STATIC && SK == 64) {
                 mpix[p] = idx >> 2, mcc[p] = idx & 3, mok[p] = true;
             } else {
                 const int pix = idx / ncc;
@@ -518,11 +518,16 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         // product, and the way out (bias added, rounded, into the tile buffer).
         auto load_w = [&](int nt, Frag (&wf)[kKT], float4 (&r4)[4]) {
             const T* wr = wl + (nt * 32 + l32) * ldw + 8 * half;
+            if constexpr (STATIC) {
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
-            if (nkt > 4) {
+                for (int kt = 0; kt < SK / 16; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
+            } else {
 #pragma unroll
-                for (int kt = 4; kt < 8; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
+                for (int kt = 0; kt < 4; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
+                if (nkt > 4) {
+#pragma unroll
+                    for (int kt = 4; kt < 8; ++kt) wf[kt] = *reinterpret_cast<const Frag*>(wr + kt * 16);
+                }
             }
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4)
@@ -532,11 +537,16 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             f32x16 acc;
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+            if constexpr (STATIC) {
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
-            if (nkt > 4) {
+                for (int kt = 0; kt < SK / 16; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
+            } else {
 #pragma unroll
-                for (int kt = 4; kt < 8; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
+                for (int kt = 0; kt < 4; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
+                if (nkt > 4) {
+#pragma unroll
+                    for (int kt = 4; kt < 8; ++kt) acc = mfma32(wf[kt], xf[kt], acc, T());
+                }
             }
             return acc;
         };
@@ -545,7 +555,8 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int n0 = nt * 32 + g4 * 8 + half * 4;
-                if (STATIC || n0 < NO) {
+                // (static widths are multiples of 16: both halves of a group of 8 features exist or neither does)
+                if (STATIC ? nt * 32 + g4 * 8 < NO : n0 < NO) {
                     float o[4];
                     o[0] = acc[g4 * 4] + r4[g4].x, o[1] = acc[g4 * 4 + 1] + r4[g4].y;
                     o[2] = acc[g4 * 4 + 2] + r4[g4].z, o[3] = acc[g4 * 4 + 3] + r4[g4].w;
@@ -557,7 +568,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             // Software pipeline over the feature tiles (unrolled): tile nt + 1's LDS reads are issued before tile nt's
             // MFMAs, and tile nt's way out follows the issue of tile nt + 1's MFMAs, so neither the read latency nor
             // the MFMA latency of a tile sits between two tiles.
-            constexpr int NNT = SNO / 32;
+            constexpr int NNT = (SNO + 31) / 32;
             Frag wf[2][kKT];
             float4 r4[3][4];   // (three tiles' bias values are alive at once: nt - 1 on its way out, nt, nt + 1 read ahead)
             f32x16 acc[2];
@@ -615,10 +626,18 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 Frag of[LO];
 #pragma unroll
                 for (int i = 0; i < LO; ++i) of[i] = *reinterpret_cast<const Frag*>(tl + (oout[i] >= 0 ? oout[i] : 0));
-                if constexpr (STATIC) {
+                if constexpr (STATIC && SNO == 128) {
 #pragma unroll
                     for (int i = 0; i < LO; ++i)   // chunks i*64 .. = pixels 4 i .. 4 i + 3 of the tile: image row i / 2, 4 columns
                         *reinterpret_cast<Frag*>(yb + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * NO + lane * 8) = of[i];
+                } else if constexpr (STATIC) {
+#pragma unroll
+                    for (int i = 0; i < LO; ++i) {   // whole passes (NO % 16 == 0), divisions by constants
+                        if (i * 64 < 32 * (SNO / 8)) {
+                            const int cidx = i * 64 + lane, pix = cidx / (SNO / 8), cc = cidx - pix * (SNO / 8);
+                            *reinterpret_cast<Frag*>(yb + (long long)((pix >> 3) * Wimg + (pix & 7)) * NO + 8 * cc) = of[i];
+                        }
+                    }
                 } else {
 #pragma unroll
                     for (int i = 0; i < LO; ++i)
@@ -722,11 +741,16 @@ constexpr int kWgRows = 64;
 
 // EXACT: M = 32 MT and NO = 32 NT, as compile-time facts: the staging map is shifts and masks, every pass is a
 // whole one and no fragment needs a clamp or a zero (the generic form spends a quarter of its time on those).
-template <typename T, int MT, int NT, bool EXACT>
+// SM, SN > 0 (without EXACT): other extents as compile-time facts (multiples of 8): the staging map divides by
+// constants, a whole stage is read as one contiguous range, and only the last, partial tiles clamp their fragments.
+template <typename T, int MT, int NT, bool EXACT, int SM = 0, int SN = 0>
 __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const T* __restrict__ Bm,
                                                  float* __restrict__ part, long long N, int Md, int NOd, int nblocks,
                                                  uint32_t* dsm) {
-    const int M = EXACT ? 32 * MT : Md, NO = EXACT ? 32 * NT : NOd;
+    constexpr bool SDIM = !EXACT && SM > 0 && SN > 0;
+    static_assert(!SDIM || (SM % 8 == 0 && SN % 8 == 0 && SM <= 32 * MT && SN <= 32 * NT && SM > 32 * (MT - 1) &&
+                            SN > 32 * (NT - 1)), "static extents of the weight gradient");
+    const int M = EXACT ? 32 * MT : SDIM ? SM : Md, NO = EXACT ? 32 * NT : SDIM ? SN : NOd;
     const int lda = M + 8, ldb = NO + 8;  // LDS row pitches (elements)
     const int buf_elems = kWgRows * (lda + ldb);
     T* lds = reinterpret_cast<T*>(dsm);
@@ -760,6 +784,17 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
             for (int p = 0; p < PA; ++p) pa[p] = *reinterpret_cast<const Frag*>(ab + p * 2048);
 #pragma unroll
             for (int p = 0; p < PB; ++p) pb[p] = *reinterpret_cast<const Frag*>(bb + p * 2048);
+            return;
+        }
+        if (SDIM && r0 + kWgRows <= N) {   // a whole stage: contiguous; the last pass may be a partial one
+            const T* ab = A + r0 * M + tid * 8;
+            const T* bb = Bm + r0 * NO + tid * 8;
+#pragma unroll
+            for (int p = 0; p < PA; ++p)
+                pa[p] = tid + p * 256 < nva ? *reinterpret_cast<const Frag*>(ab + p * 2048) : Frag{{0u, 0u, 0u, 0u}};
+#pragma unroll
+            for (int p = 0; p < PB; ++p)
+                pb[p] = tid + p * 256 < nvb ? *reinterpret_cast<const Frag*>(bb + p * 2048) : Frag{{0u, 0u, 0u, 0u}};
             return;
         }
 #pragma unroll
@@ -805,8 +840,9 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
         Frag af[MT], bf[NT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-            const int m = EXACT ? t * 32 + l32 : min(t * 32 + l32, M - 1);
-            const bool ok = EXACT || t * 32 + l32 < M;
+            const bool whole = EXACT || (SDIM && (t + 1) * 32 <= SM);   // (t is a constant once unrolled)
+            const int m = whole ? t * 32 + l32 : min(t * 32 + l32, M - 1);
+            const bool ok = whole || t * 32 + l32 < M;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t lo = ld16(la + (2 * j) * lda + m), hi = ld16(la + (2 * j + 1) * lda + m);
@@ -815,8 +851,9 @@ __device__ __forceinline__ void dense_wgrad_body(const T* __restrict__ A, const 
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const int n = EXACT ? t * 32 + l32 : min(t * 32 + l32, NO - 1);
-            const bool ok = EXACT || t * 32 + l32 < NO;
+            const bool whole = EXACT || (SDIM && (t + 1) * 32 <= SN);
+            const int n = whole ? t * 32 + l32 : min(t * 32 + l32, NO - 1);
+            const bool ok = whole || t * 32 + l32 < NO;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t lo = ld16(lb + (2 * j) * ldb + n), hi = ld16(lb + (2 * j + 1) * ldb + n);
@@ -876,8 +913,8 @@ __global__ __launch_bounds__(256, 2) void dense_wgrad_rider_k(const T* __restric
     dense_wgrad_body<T, MT, NT, EXACT>(A, Bm, part, N, M, NO, nblocks, dsm);
 }
 
-// Input gradient and weight gradient of one dense layer (y = x W^T, W[O][I]) in one launch, for the block's
-// two layer shapes (O, I) = (128, 64) and (64, 128): dx[N][I] = gy W (dense_rows_body, W as W[k][o]) and the
+// Input gradient and weight gradient of one dense layer (y = x W^T, W[O][I]) in one launch, for the layer shapes of
+// pyramid blocks of 128, 96 and 64 features, (O, I) = (128, 64), (64, 128), (96, 48), (48, 96), (64, 32), (32, 64): dx[N][I] = gy W (dense_rows_body, W as W[k][o]) and the
 // partials of dW[O][I] = gy^T x (dense_wgrad_body).  Both read gy and neither fills the chip alone (the weight gradient is one
 // workgroup per compute unit, the row product waits on memory in lockstep): the weight gradient's workgroups come
 // first in the grid, one per compute unit, and the row product's persistent workgroups take the second slot.
@@ -888,10 +925,11 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_pair_k(const T* __restrict__
                                                            const float* __restrict__ rowbias, int P, long long N,
                                                            int nwg, int nrows) {
     extern __shared__ uint32_t dsm[];
+    constexpr bool EX = O % 32 == 0 && I % 32 == 0;   // else: the extents as constants, partial last tiles
     if ((int)blockIdx.x < nwg)
-        dense_wgrad_body<T, O / 32, I / 32, true>(gy, xin, part, N, O, I, nwg, dsm);
+        dense_wgrad_body<T, (O + 31) / 32, (I + 31) / 32, EX, EX ? 0 : O, EX ? 0 : I>(gy, xin, part, N, O, I, nwg, dsm);
     else
-        dense_rows_body<T, true, COLSUM, O, I>(gy, W, nullptr, rowbias, dx, colsum, N, O, I, P, O / 16, I / 32,
+        dense_rows_body<T, true, COLSUM, O, I>(gy, W, nullptr, rowbias, dx, colsum, N, O, I, P, O / 16, (I + 31) / 32,
                                                blockIdx.x - nwg, nrows, dsm);
 }
 
@@ -997,6 +1035,10 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     } else {                              \
         PDW_GO_S(T, KM, false);           \
     }
+    // conv_up of a 96-feature pyramid block (with the tile sums): its extents as constants, too
+    if (K == 96 && NO == 48 && colsum && !w_kmajor && !tune_env("PDW_DENSE_GENERIC")) {
+        if (dtype == kF16) PDW_GO(f16_t, false, true, 96, 48); else PDW_GO(bf16_t, false, true, 96, 48);
+    } else
     if (dtype == kF16) {
         if (w_kmajor) { PDW_GO2(f16_t, true) } else { PDW_GO2(f16_t, false) }
     } else {
@@ -1055,6 +1097,7 @@ int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void*
     const long long N = (long long)B * H * W;
     if (N > 0x7fffffffLL / 128) return -1;
     const bool exact = I == 64 && D == 128 && !tune_env("PDW_DENSE_GENERIC");
+    const bool exact96 = I == 48 && D == 96 && !tune_env("PDW_DENSE_GENERIC");
     const int nnt = cdiv(D, 32);
     for (const void* p : {cf, ch, w, (const void*)y})
         if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
@@ -1074,6 +1117,8 @@ int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void*
 #define PDW_MID_S(T, M)            \
     if (exact)                     \
         PDW_MID(T, M, 64, 128);    \
+    else if (exact96)              \
+        PDW_MID(T, M, 48, 96);     \
     else                           \
         PDW_MID(T, M, 0, 0)
     if (dtype == kF16) {
@@ -1151,7 +1196,8 @@ int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long lo
 }
 
 static bool pair_exact(int O, int I) {
-    return (O == 128 && I == 64) || (O == 64 && I == 128) || (O == 64 && I == 32) || (O == 32 && I == 64);
+    return (O == 128 && I == 64) || (O == 64 && I == 128) || (O == 64 && I == 32) || (O == 32 && I == 64) ||
+           (O == 96 && I == 48) || (O == 48 && I == 96);
 }
 
 int dense_bwd_pair_supported(int O, int I, int dtype) {
@@ -1197,6 +1243,10 @@ int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* 
 #define PDW_PAIR_T(T)                                           \
     if (O == 128) {                                             \
         if (colsum) PDW_PAIR(T, true, 128, 64); else PDW_PAIR(T, false, 128, 64); \
+    } else if (O == 96) {                                       \
+        if (colsum) PDW_PAIR(T, true, 96, 48); else PDW_PAIR(T, false, 96, 48); \
+    } else if (O == 48) {                                       \
+        PDW_PAIR(T, false, 48, 96);                             \
     } else if (O == 64 && I == 128) {                           \
         if (colsum) PDW_PAIR(T, true, 64, 128); else PDW_PAIR(T, false, 64, 128); \
     } else if (O == 64) {                                       \

@@ -237,7 +237,7 @@ def test_pool_branch(dtype, shape):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,P,K,NO,kmajor", [(3, 64, 128, 64, False), (2, 96, 64, 128, True), (32, 3136, 128, 64, False),
-                                             (1, 32, 128, 8, True)])
+                                             (1, 32, 128, 8, True), (3, 160, 96, 48, False), (8, 12544, 96, 48, False)])
 def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
     """The dense kernel's by-product (sums of x over groups of 32 rows) against a float64 sum, and the mean branch
     computed from it against the one that reads x itself."""
@@ -343,7 +343,7 @@ def test_dense_backward_pair_matches_separate_launches(dtype, N, widths):
     gy = randn(gen, N, O).to(dtype).cuda()
     x = randn(gen, N, I).to(dtype).cuda()
     w = (randn(gen, O, I) / 8).to(dtype).cuda()
-    colsum = N % ops.dense_colsum_rows() == 0 and widths in ((128, 64), (64, 32))   # tile sums: the block's shapes only
+    colsum = N % ops.dense_colsum_rows() == 0 and widths in ((128, 64), (64, 32), (96, 48))   # tile sums: the blocks' shapes only
     if colsum:
         dx0, parts0 = ops.dense_forward(gy, w, w_kmajor=True, colsum=True)
     else:
