@@ -149,13 +149,14 @@ struct WTransposer {
 // whole MFMA steps, and its code has no per-lane predicates and no loop bounds to test: those were a third of the
 // generic kernel's vector-ALU work.
 //
-// POOL (SK = 128, SNO = 64; rows are the pixels of [B, Himg, Wimg] images, Himg % 4 == 0, Wimg % 8 == 0, no rowbias): a
+// POOL (static widths; rows are the pixels of [B, Himg, Wimg] images, Himg % 4 == 0, Wimg % 8 == 0, no rowbias): a
 // tile is a block of 4 image rows x 8 columns instead of 32 consecutive pixels (a load or store instruction still
-// covers 1 KB of consecutive bytes: 4 pixels of K values, 8 pixels of NO), so that it holds 2 x 4 whole windows of
+// covers 1 KB of consecutive bytes of an image row: 4 pixels of 128 values in, 8 pixels of 64 out; with other widths
+// an instruction's 64 chunks run over the end of the tile's image row into its next one), so that it holds 2 x 4 whole windows of
 // the 2x2 average pool of Y, which the kernel writes to `pool` [B, Himg/2, Wimg/2, NO] from the result tile in LDS:
 // (((y00 + y01) + y10) + y11) / 4 in fp32 of the rounded results, as the pooling kernel computes it.
 //
-// MID (SK = 64, SNO = 128, rows = the pixels of [B, Himg, Wimg] images in the 4 x 8 tiles of POOL): the rows are not
+// MID (rows = the pixels of [B, Himg, Wimg] images in the 4 x 8 tiles of POOL; written here for K = 64, NO = 128): the rows are not
 // loaded but made, from the convolution outputs of a two-scale block (conv_block.py:18-21, 41-44): row (b, i, j) =
 // [ gate(cf[b, i, j]) | bilinear resize to Himg x Wimg of gate(ch[b]) at (i, j) ], cf [B, Himg, Wimg, 64] the full
 // scale, ch [B, Himg/2, Wimg/2, 64] the half scale, gate(v) = v[:32] * v[32:] * gs rounded to T.  A tile's resized
@@ -216,7 +217,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                                                 uint32_t* dsm, T* __restrict__ pool = nullptr, int Himg = 0,
                                                 int Wimg = 0, const MidRows* mid = nullptr) {
     constexpr bool STATIC = SK > 0 && SNO > 0;
-    static_assert(!POOL || (SK == 128 && SNO == 64 && !KMAJOR), "pooled output: the 128 -> 64 layer");
+    static_assert(!POOL || (STATIC && !KMAJOR), "pooled output: layers with their extents as constants");
     static_assert(MID == 0 || (((STATIC && SK <= 64) || (SK == 0 && SNO == 0)) && !KMAJOR && !COLSUM && !POOL),
                   "made rows: a layer with its extents as constants (inner width up to 64), or any covered widths");
     // POOL: first pixel of a tile and first pixel of its part of the pooled tensor (two 32-bit divisions per tile,
@@ -283,6 +284,22 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
             }
         }
     }
+    // POOL / MID with widths whose passes of 64 chunks are not whole pixels: where in global memory, relative to the
+    // tile's first pixel, this lane's chunk i*64 + lane = (pixel, 8 values) of a tile of 4 x 8 pixels lies (lane
+    // constants; input rows of K values, output rows of NO)
+    [[maybe_unused]] int gin[LP], gout[2 * kNT];
+    if constexpr (STATIC && (POOL || MID != 0)) {
+#pragma unroll
+        for (int i = 0; i < LP; ++i) {
+            const int cidx = i * 64 + lane, pix = cidx / (SK / 8), cc = cidx - pix * (SK / 8);
+            gin[i] = ((pix >> 3) * Wimg + (pix & 7)) * SK + 8 * cc;
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * kNT; ++i) {
+            const int cidx = i * 64 + lane, pix = cidx / (SNO / 8), cc = cidx - pix * (SNO / 8);
+            gout[i] = ((pix >> 3) * Wimg + (pix & 7)) * SNO + 8 * cc;
+        }
+    }
     [[maybe_unused]] Frag fa[2], fb[2], ha[2], hb[2];
     [[maybe_unused]] auto mid_load = [&](long long t) {
         const int b = tile_pixel(t);
@@ -312,9 +329,23 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
         } else if constexpr (POOL) {
             tile_pixel(t);
             base = X + (long long)px_next * K;
+            if constexpr (SK == 128) {
 #pragma unroll
-            for (int i = 0; i < LP; ++i)   // chunks i*64 .. of the tile: its pixels 4 i .. 4 i + 3 = image row i / 2, 4 columns
-                raw[i] = *reinterpret_cast<const Frag*>(base + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * K + lane * 8);
+                for (int i = 0; i < LP; ++i)   // chunks i*64 .. of the tile: its pixels 4 i .. 4 i + 3 = image row i / 2, 4 columns
+                    raw[i] = *reinterpret_cast<const Frag*>(base + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * K + lane * 8);
+            } else {
+#pragma unroll
+                for (int i = 0; i < LP; ++i) {   // chunk i*64 + lane = (pixel, 8 values) of the tile; whole passes (K % 16 == 0)
+                    // (built from its four words: copied as a whole, an array that nothing reads word by word stays
+                    // in scratch memory)
+                    if (i * 64 < 32 * (SK / 8)) {
+                        const uint4 u = *reinterpret_cast<const uint4*>(base + gin[i]);
+                        raw[i] = Frag{{u.x, u.y, u.z, u.w}};
+                    } else {
+                        raw[i] = Frag{{0u, 0u, 0u, 0u}};
+                    }
+                }
+            }
         } else if (STATIC && rows_left >= 32) {
 #pragma unroll
             for (int i = 0; i < LP; ++i) {
@@ -601,13 +632,25 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                 for (int i = 0; i < LO; ++i)
                     if (i * 64 < 32 * cpr) of[i] = *reinterpret_cast<const Frag*>(tl + oout[i]);
                 // the lane's window of the pool (2 x 4 per tile) and 8 of its features
-                const int wr = lane >> 5, wc = (lane >> 3) & 3, ch = (lane & 7) * 8;
+                constexpr int CPR = SNO / 8;
+                int wr = lane >> 5, wc = (lane >> 3) & 3, ch = (lane & 7) * 8;
+                if constexpr (CPR != 8) {
+                    const int win = min(lane / CPR, 7);
+                    wr = win >> 2, wc = win & 3, ch = (lane - (lane / CPR) * CPR) * 8;
+                }
+                const bool wok = CPR == 8 || lane < 8 * CPR;
                 const T* p00 = tl + (16 * wr + 2 * wc) * ldt + ch;
                 const Frag q00 = *reinterpret_cast<const Frag*>(p00), q01 = *reinterpret_cast<const Frag*>(p00 + ldt);
                 const Frag q10 = *reinterpret_cast<const Frag*>(p00 + 8 * ldt), q11 = *reinterpret_cast<const Frag*>(p00 + 9 * ldt);
+                if constexpr (SNO == 64) {
 #pragma unroll
-                for (int i = 0; i < LO; ++i)   // chunks i*64 .. = image row i of the tile, 8 pixels
-                    if (i * 64 < 32 * cpr) *reinterpret_cast<Frag*>(yb + (long long)i * Wimg * NO + lane * 8) = of[i];
+                    for (int i = 0; i < LO; ++i)   // chunks i*64 .. = image row i of the tile, 8 pixels
+                        if (i * 64 < 32 * cpr) *reinterpret_cast<Frag*>(yb + (long long)i * Wimg * NO + lane * 8) = of[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < LO; ++i)   // whole passes (NO % 16 == 0)
+                        if (i * 64 < 32 * CPR) *reinterpret_cast<Frag*>(yb + gout[i]) = of[i];
+                }
                 Frag o;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -620,7 +663,7 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                     o.v[j] = *reinterpret_cast<const uint32_t*>(&pv);
                 }
                 T* pb = pool + ((long long)pp_cur + wr * (Wimg >> 1) + wc) * NO + ch;
-                *reinterpret_cast<Frag*>(pb) = o;
+                if (wok) *reinterpret_cast<Frag*>(pb) = o;
             } else if constexpr (MID != 0) {
                 yb = Y + (long long)px_cur * NO;
                 Frag of[LO];
@@ -632,12 +675,8 @@ __device__ __forceinline__ void dense_rows_body(const T* __restrict__ X, const T
                         *reinterpret_cast<Frag*>(yb + (long long)((i >> 1) * Wimg + 4 * (i & 1)) * NO + lane * 8) = of[i];
                 } else if constexpr (STATIC) {
 #pragma unroll
-                    for (int i = 0; i < LO; ++i) {   // whole passes (NO % 16 == 0), divisions by constants
-                        if (i * 64 < 32 * (SNO / 8)) {
-                            const int cidx = i * 64 + lane, pix = cidx / (SNO / 8), cc = cidx - pix * (SNO / 8);
-                            *reinterpret_cast<Frag*>(yb + (long long)((pix >> 3) * Wimg + (pix & 7)) * NO + 8 * cc) = of[i];
-                        }
-                    }
+                    for (int i = 0; i < LO; ++i)   // whole passes (NO % 16 == 0)
+                        if (i * 64 < 32 * (SNO / 8)) *reinterpret_cast<Frag*>(yb + gout[i]) = of[i];
                 } else {
 #pragma unroll
                     for (int i = 0; i < LO; ++i)
@@ -690,14 +729,14 @@ __global__ __launch_bounds__(256, 2) void dense_rows_k(const T* __restrict__ X, 
 
 // The 128 -> 64 layer over the pixels of [B, Himg, Wimg] images with the tile sums of X and the 2x2 average pool of Y
 // (dense_rows_body, POOL).
-template <typename T>
+template <typename T, int SK, int SNO>
 __global__ __launch_bounds__(256, 2) void dense_rows_pool_k(const T* __restrict__ X, const T* __restrict__ W,
                                                          const T* __restrict__ bias, T* __restrict__ Y,
                                                          float* __restrict__ colsum, T* __restrict__ pool, long long N,
                                                          int Himg, int Wimg) {
     extern __shared__ uint32_t dsm[];
-    dense_rows_body<T, false, true, 128, 64, true>(X, W, bias, nullptr, Y, colsum, N, 128, 64, 1, 8, 2, blockIdx.x,
-                                                   gridDim.x, dsm, pool, Himg, Wimg);
+    dense_rows_body<T, false, true, SK, SNO, true>(X, W, bias, nullptr, Y, colsum, N, SK, SNO, 1, SK / 16,
+                                                   (SNO + 31) / 32, blockIdx.x, gridDim.x, dsm, pool, Himg, Wimg);
 }
 
 // The 64 -> 128 layer on rows made from the two scales of a pyramid block (dense_rows_body, MID).
@@ -1050,12 +1089,14 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     return check_launch("dense_rows");
 }
 
-// y = x W^T (+ bias) for the pixels of [B, H, W] images with K = 128 features in and NO = 64 out, the sums of x over
+// y = x W^T (+ bias) for the pixels of [B, H, W] images with (K, NO) = (128, 64) or (96, 48) features in / out (conv_up
+// of a pyramid block of 128 or 96 features), the sums of x over
 // each 32-pixel tile (tiles of 4 rows x 8 columns here: still H * W / 32 per image, image after image) and the 2x2
 // average pool of y.  -1: not covered (other widths, extents that are not multiples of 4 x 8, fp32).
 int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
                            int H, int W, int K, int NO, int dtype, hipStream_t s) {
-    if (dtype == kF32 || K != 128 || NO != 64 || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
+    const bool s128 = K == 128 && NO == 64, s96 = K == 96 && NO == 48;
+    if (dtype == kF32 || !(s128 || s96) || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
     if (tune_env("PDW_DENSE_GENERIC") || tune_env("PDW_NO_DENSE_POOL")) return -1;
     const long long N = (long long)B * H * W;
     if (N > 0x7fffffffLL) return -1;
@@ -1066,13 +1107,17 @@ int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void*
     long long blocks = (ntiles + 3) / 4;
     const int cap = tune_env("PDW_DENSE_BLOCKS") ? atoi(tune_env("PDW_DENSE_BLOCKS")) : 512;
     if (blocks > cap) blocks = cap;
-    const size_t lds = ((size_t)2 * 32 * (128 + 8) + 4 * 32 * (128 + 8)) * 2 + (bias ? (size_t)4 * 2 * 2 * 32 * sizeof(float) : 0);
-    if (dtype == kF16)
-        hipLaunchKernelGGL(dense_rows_pool_k<f16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const f16_t*)x, (const f16_t*)w,
-                           (const f16_t*)bias, (f16_t*)y, colsum, (f16_t*)pool, N, H, W);
-    else
-        hipLaunchKernelGGL(dense_rows_pool_k<bf16_t>, dim3((unsigned)blocks), dim3(256), lds, s, (const bf16_t*)x,
-                           (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, colsum, (bf16_t*)pool, N, H, W);
+    // (weights as 2 feature tiles x 128 padded inner values, four tile buffers of 32 rows x (K + 8), the bias table)
+    const size_t lds = ((size_t)2 * 32 * (128 + 8) + 4 * 32 * (K + 8)) * 2 + (bias ? (size_t)4 * 2 * 2 * 32 * sizeof(float) : 0);
+#define PDW_POOL(T, SK, SNO)                                                                                         \
+    hipLaunchKernelGGL((dense_rows_pool_k<T, SK, SNO>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x,       \
+                       (const T*)w, (const T*)bias, (T*)y, colsum, (T*)pool, N, H, W)
+    if (dtype == kF16) {
+        if (s128) PDW_POOL(f16_t, 128, 64); else PDW_POOL(f16_t, 96, 48);
+    } else {
+        if (s128) PDW_POOL(bf16_t, 128, 64); else PDW_POOL(bf16_t, 96, 48);
+    }
+#undef PDW_POOL
     return check_launch("dense_rows_pool");
 }
 

@@ -266,7 +266,8 @@ def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("case", [(32, 56, 56, 128, 64), (3, 8, 16, 128, 64), (1, 4, 8, 128, 64), (2, 12, 40, 128, 64),
-                                  (2, 10, 16, 128, 64), (2, 8, 12, 128, 64), (2, 8, 16, 64, 32), (5, 36, 24, 128, 64)])
+                                  (2, 10, 16, 128, 64), (2, 8, 12, 128, 64), (2, 8, 16, 64, 32), (5, 36, 24, 128, 64),
+                                  (8, 112, 112, 96, 48), (1, 4, 8, 96, 48), (3, 12, 40, 96, 48), (2, 8, 12, 96, 48)])
 def test_dense_forward_pool_is_the_layer_then_the_pool(dtype, case):
     """pdw_dense_fwd_colsum_pool: the layer's result bitwise that of pdw_dense_fwd, its 2x2 average pool bitwise that of
     pdw_avgpool_fwd on it, and per-image sums of x from the tile sums (tiles of 4 rows x 8 columns) equal to a float64
@@ -278,7 +279,7 @@ def test_dense_forward_pool_is_the_layer_then_the_pool(dtype, case):
     x = randn(gen, B, H, W, K).to(dtype).cuda()
     w = (randn(gen, NO, K) / 8).to(dtype).cuda()
     got = ops.dense_forward_pool(x, w)
-    covered = dtype != torch.float32 and (K, NO) == (128, 64) and H % 4 == 0 and W % 8 == 0
+    covered = dtype != torch.float32 and (K, NO) in ((128, 64), (96, 48)) and H % 4 == 0 and W % 8 == 0
     assert (got is not None) == covered
     if got is None:
         return
