@@ -350,8 +350,8 @@ int pdw_dense_fwd_colsum(const void *x, const void *w, int w_kmajor, const void 
  * pool[B,H/2,W/2,NO] = what pdw_avgpool_fwd makes of y (conv_block.py:37 together with the pooling of conv_block.py:16
  * for the second scale: the convolutions of both scales can then start together, pdw_dwconv_fwd2).  The kernel's row
  * tiles are blocks of 4 image rows x 8 columns, so colsum[t] are the sums of x over such blocks (still H*W/32 per
- * image, image after image).  Status 3 (nothing launched) where not covered: 16-bit types, (K, NO) = (128, 64) or
- * (96, 48), H % 4 == 0, W % 8 == 0 only. */
+ * image, image after image).  Status 3 (nothing launched) where not covered: 16-bit types, (K, NO) = (128, 64),
+ * (96, 48) or (64, 32), H % 4 == 0, W % 8 == 0 only. */
 int pdw_dense_fwd_colsum_pool(const void *x, const void *w, const void *bias, void *y, float *colsum, void *pool, int B,
                               int H, int W, int K, int NO, int dtype, void *stream);
 
@@ -399,8 +399,8 @@ int pdw_dense_bwd_pair(const void *gy, const void *w, const void *x, void *dx, f
  * launches and one summation launch)
  * without a host interpreter between them.  Covered when pdw_convblock_supported: 16-bit dtype, even H, W >= 4 with
  * H*W a multiple of pdw_dense_colsum_rows(), layer widths D (block), I (inner, a multiple of 16) that the dense
- * kernels and pdw_dense_bwd_pair cover (multiples of 8 up to 128; D = 128, I = 64 and D = 96, I = 48 run variants with
- * compile-time extents throughout, D = 64, I = 32 in the backward), odd K.  All tensors channels-last and contiguous, all
+ * kernels and pdw_dense_bwd_pair cover (multiples of 8 up to 128; D = 128, 96 and 64 with I = D / 2 run variants with
+ * compile-time extents), odd K.  All tensors channels-last and contiguous, all
  * parameters in `dtype`: x, y[B,H,W,D]; w_up[I,D]; w_dw0, w_dw1[K,K,I]; w_pool[D,D]; w_out[D,I]; b_pool, b_out[D] or
  * NULL.  The forward writes what the backward reads again: a = conv_up(x), c0 = conv(a), xp = pool(a)[B,H/2,W/2,I],
  * c1 = conv(xp), cat[B,H,W,I] (the gated scales), m[B,D] (per-image mean of x).  The backward overwrites dx and the

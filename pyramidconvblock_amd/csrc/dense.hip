@@ -1074,9 +1074,11 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     } else {                              \
         PDW_GO_S(T, KM, false);           \
     }
-    // conv_up of a 96-feature pyramid block (with the tile sums): its extents as constants, too
+    // conv_up of a 96- or 64-feature pyramid block (with the tile sums): its extents as constants, too
     if (K == 96 && NO == 48 && colsum && !w_kmajor && !tune_env("PDW_DENSE_GENERIC")) {
         if (dtype == kF16) PDW_GO(f16_t, false, true, 96, 48); else PDW_GO(bf16_t, false, true, 96, 48);
+    } else if (K == 64 && NO == 32 && colsum && !w_kmajor && !tune_env("PDW_DENSE_GENERIC")) {
+        if (dtype == kF16) PDW_GO(f16_t, false, true, 64, 32); else PDW_GO(bf16_t, false, true, 64, 32);
     } else
     if (dtype == kF16) {
         if (w_kmajor) { PDW_GO2(f16_t, true) } else { PDW_GO2(f16_t, false) }
@@ -1089,14 +1091,14 @@ int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bi
     return check_launch("dense_rows");
 }
 
-// y = x W^T (+ bias) for the pixels of [B, H, W] images with (K, NO) = (128, 64) or (96, 48) features in / out (conv_up
-// of a pyramid block of 128 or 96 features), the sums of x over
+// y = x W^T (+ bias) for the pixels of [B, H, W] images with (K, NO) = (128, 64), (96, 48) or (64, 32) features in / out
+// (conv_up of a pyramid block of 128, 96 or 64 features), the sums of x over
 // each 32-pixel tile (tiles of 4 rows x 8 columns here: still H * W / 32 per image, image after image) and the 2x2
 // average pool of y.  -1: not covered (other widths, extents that are not multiples of 4 x 8, fp32).
 int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void* y, float* colsum, void* pool, int B,
                            int H, int W, int K, int NO, int dtype, hipStream_t s) {
-    const bool s128 = K == 128 && NO == 64, s96 = K == 96 && NO == 48;
-    if (dtype == kF32 || !(s128 || s96) || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
+    const bool s128 = K == 128 && NO == 64, s96 = K == 96 && NO == 48, s64 = K == 64 && NO == 32;
+    if (dtype == kF32 || !(s128 || s96 || s64) || H % 4 != 0 || W % 8 != 0 || B < 1 || H < 4 || W < 8) return -1;
     if (tune_env("PDW_DENSE_GENERIC") || tune_env("PDW_NO_DENSE_POOL")) return -1;
     const long long N = (long long)B * H * W;
     if (N > 0x7fffffffLL) return -1;
@@ -1107,15 +1109,18 @@ int dense_rows_pool_launch(const void* x, const void* w, const void* bias, void*
     long long blocks = (ntiles + 3) / 4;
     const int cap = tune_env("PDW_DENSE_BLOCKS") ? atoi(tune_env("PDW_DENSE_BLOCKS")) : 512;
     if (blocks > cap) blocks = cap;
-    // (weights as 2 feature tiles x 128 padded inner values, four tile buffers of 32 rows x (K + 8), the bias table)
-    const size_t lds = ((size_t)2 * 32 * (128 + 8) + 4 * 32 * (K + 8)) * 2 + (bias ? (size_t)4 * 2 * 2 * 32 * sizeof(float) : 0);
+    // (weights as whole feature tiles x 64 or 128 padded inner values, four tile buffers of 32 rows x (K + 8), the
+    // bias table)
+    const int nnt = cdiv(NO, 32);
+    const size_t lds = ((size_t)nnt * 32 * ((K > 64 ? 128 : 64) + 8) + 4 * 32 * (K + 8)) * 2 +
+                       (bias ? (size_t)4 * 2 * nnt * 32 * sizeof(float) : 0);
 #define PDW_POOL(T, SK, SNO)                                                                                         \
     hipLaunchKernelGGL((dense_rows_pool_k<T, SK, SNO>), dim3((unsigned)blocks), dim3(256), lds, s, (const T*)x,       \
                        (const T*)w, (const T*)bias, (T*)y, colsum, (T*)pool, N, H, W)
     if (dtype == kF16) {
-        if (s128) PDW_POOL(f16_t, 128, 64); else PDW_POOL(f16_t, 96, 48);
+        if (s128) PDW_POOL(f16_t, 128, 64); else if (s96) PDW_POOL(f16_t, 96, 48); else PDW_POOL(f16_t, 64, 32);
     } else {
-        if (s128) PDW_POOL(bf16_t, 128, 64); else PDW_POOL(bf16_t, 96, 48);
+        if (s128) PDW_POOL(bf16_t, 128, 64); else if (s96) PDW_POOL(bf16_t, 96, 48); else PDW_POOL(bf16_t, 64, 32);
     }
 #undef PDW_POOL
     return check_launch("dense_rows_pool");
@@ -1143,6 +1148,7 @@ int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void*
     if (N > 0x7fffffffLL / 128) return -1;
     const bool exact = I == 64 && D == 128 && !tune_env("PDW_DENSE_GENERIC");
     const bool exact96 = I == 48 && D == 96 && !tune_env("PDW_DENSE_GENERIC");
+    const bool exact64 = I == 32 && D == 64 && !tune_env("PDW_DENSE_GENERIC");
     const int nnt = cdiv(D, 32);
     for (const void* p : {cf, ch, w, (const void*)y})
         if (!p || (reinterpret_cast<uintptr_t>(p) & 15)) return -1;
@@ -1164,6 +1170,8 @@ int dense_mid_rows_launch(const void* cf, const void* ch, void* cat, const void*
         PDW_MID(T, M, 64, 128);    \
     else if (exact96)              \
         PDW_MID(T, M, 48, 96);     \
+    else if (exact64)              \
+        PDW_MID(T, M, 32, 64);     \
     else                           \
         PDW_MID(T, M, 0, 0)
     if (dtype == kF16) {

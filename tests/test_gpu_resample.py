@@ -237,7 +237,8 @@ def test_pool_branch(dtype, shape):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,P,K,NO,kmajor", [(3, 64, 128, 64, False), (2, 96, 64, 128, True), (32, 3136, 128, 64, False),
-                                             (1, 32, 128, 8, True), (3, 160, 96, 48, False), (8, 12544, 96, 48, False)])
+                                             (1, 32, 128, 8, True), (3, 160, 96, 48, False), (8, 12544, 96, 48, False),
+                                             (5, 96, 64, 32, False)])
 def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
     """The dense kernel's by-product (sums of x over groups of 32 rows) against a float64 sum, and the mean branch
     computed from it against the one that reads x itself."""
@@ -267,7 +268,8 @@ def test_dense_colsum_feeds_pool_branch(dtype, B, P, K, NO, kmajor):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("case", [(32, 56, 56, 128, 64), (3, 8, 16, 128, 64), (1, 4, 8, 128, 64), (2, 12, 40, 128, 64),
                                   (2, 10, 16, 128, 64), (2, 8, 12, 128, 64), (2, 8, 16, 64, 32), (5, 36, 24, 128, 64),
-                                  (8, 112, 112, 96, 48), (1, 4, 8, 96, 48), (3, 12, 40, 96, 48), (2, 8, 12, 96, 48)])
+                                  (8, 112, 112, 96, 48), (1, 4, 8, 96, 48), (3, 12, 40, 96, 48), (2, 8, 12, 96, 48),
+                                  (3, 20, 24, 64, 32), (16, 56, 56, 64, 32), (2, 8, 16, 32, 16)])
 def test_dense_forward_pool_is_the_layer_then_the_pool(dtype, case):
     """pdw_dense_fwd_colsum_pool: the layer's result bitwise that of pdw_dense_fwd, its 2x2 average pool bitwise that of
     pdw_avgpool_fwd on it, and per-image sums of x from the tile sums (tiles of 4 rows x 8 columns) equal to a float64
@@ -279,7 +281,7 @@ def test_dense_forward_pool_is_the_layer_then_the_pool(dtype, case):
     x = randn(gen, B, H, W, K).to(dtype).cuda()
     w = (randn(gen, NO, K) / 8).to(dtype).cuda()
     got = ops.dense_forward_pool(x, w)
-    covered = dtype != torch.float32 and (K, NO) in ((128, 64), (96, 48)) and H % 4 == 0 and W % 8 == 0
+    covered = dtype != torch.float32 and (K, NO) in ((128, 64), (96, 48), (64, 32)) and H % 4 == 0 and W % 8 == 0
     assert (got is not None) == covered
     if got is None:
         return
@@ -394,7 +396,8 @@ def test_sum_parts_is_the_fp32_sum_rounded_once(shape, dtype):
 @pytest.mark.parametrize("case", [(32, 56, 56, 64, 128), (1, 4, 8, 64, 128), (3, 8, 16, 64, 128), (2, 12, 40, 64, 128),
                                   (2, 64, 8, 64, 128), (5, 36, 24, 64, 128), (2, 10, 16, 64, 128), (2, 8, 16, 32, 64),
                                   (70, 8, 8, 64, 128), (8, 112, 112, 48, 96), (3, 8, 24, 16, 32), (2, 12, 16, 64, 96),
-                                  (2, 8, 8, 32, 128), (2, 8, 8, 48, 56), (2, 8, 8, 96, 128), (2, 8, 8, 24, 48)])
+                                  (2, 8, 8, 32, 128), (2, 8, 8, 48, 56), (2, 8, 8, 96, 128), (2, 8, 8, 24, 48),
+                                  (16, 56, 56, 32, 64), (3, 12, 24, 48, 96)])
 def test_dense_forward_gated_is_the_gates_then_the_layer(oracle, dtype, with_cat, case):
     """pdw_dense_fwd_gated (the block's output layer on rows it makes from the two convolution outputs: both gates and
     the resize where the tile is staged) gives bitwise what the gate launch followed by the plain layer gives, with
