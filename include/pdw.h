@@ -324,8 +324,11 @@ int pdw_block_mid_infer(const void *xh, void *y, int B, int H, int W, int h, int
                         const float *parts, int nparts, const void *w_pool, const void *b_pool, const void *b_out,
                         void *m, float *rowbias, int P, int D, int dtype, void *stream);
 
-/* Dense layers of the block on the matrix cores (bf16/fp16, K <= 128, NO <= 128, K % 8 == 0, NO % 8 == 0;
- * pdw_dense_supported says whether a shape is covered - callers use a library GEMM otherwise).
+/* Dense layers of the block on the matrix cores.  bf16/fp16 with K <= 128, NO <= 128, K % 8 == 0, NO % 8 == 0 run the
+ * tiled kernels (persistent workgroups, weights in LDS, a 32-row tile per wavefront over all features); fp32 and
+ * every other width with K % 4 == 0, NO % 4 == 0, K <= 256 run one 32 x 32 result tile per wavefront
+ * (v_mfma_f32_32x32x2_f32 in fp32), forward, input gradient and weight gradient alike.  pdw_dense_supported says
+ * whether a shape is covered - callers use a library GEMM otherwise.
  *   y[n,o] = sum_k x[n,k] * W(o,k) + bias[o] + rowbias[n / P][o]        x[N,K] -> y[N,NO]
  * W(o,k) = w[o*K + k] (w_kmajor == 0, the nn.Linear layout) or w[k*NO + o] (w_kmajor != 0, which gives the
  * input gradient of a layer from its own weight without a transpose).  bias (element type) and rowbias

@@ -992,7 +992,8 @@ static bool dense_dims_ok(int K, int NO, int dtype) {
     return dtype != kF32 && K >= 8 && K <= 16 * kKT && K % 8 == 0 && NO >= 8 && NO <= 32 * kNT && NO % 8 == 0;
 }
 
-int dense_rows_supported(int K, int NO, int dtype) { return dense_dims_ok(K, NO, dtype) ? 1 : 0; }
+// (the tiled kernels of this file, or the one-tile-per-wavefront kernels of dense_any.hip: fp32, other widths)
+int dense_rows_supported(int K, int NO, int dtype) { return (dense_dims_ok(K, NO, dtype) || dense_any_dims_ok(K, NO)) ? 1 : 0; }
 
 int dense_colsum_rows() { return 32; }
 
@@ -1001,7 +1002,14 @@ int dense_colsum_supported(int K, int NO, int dtype) { return dense_dims_ok(K, N
 int dense_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
                       long long N, int K, int NO, int P, int dtype, hipStream_t s, float* colsum,
                       const ReduceJobs* rider) {
-    if (!dense_dims_ok(K, NO, dtype)) return -1;
+    if (!dense_dims_ok(K, NO, dtype)) {
+        // fp32 and the widths the tiled kernels do not take: no tile sums there, and summations that were to ride
+        // in this launch get one of their own
+        if (colsum || !dense_any_dims_ok(K, NO)) return -1;
+        if (rider)
+            if (int e = reduce_jobs_launch(*rider, s)) return e;
+        return dense_any_rows_launch(x, w, w_kmajor, bias, rowbias, y, N, K, NO, P, dtype, s);
+    }
     if (rider && colsum) return -1;
     if (colsum && (!dense_colsum_supported(K, NO, dtype) || (reinterpret_cast<uintptr_t>(colsum) & 15))) return -1;
     if (N == 0) return 0;
@@ -1195,10 +1203,14 @@ static void dense_wgrad_plan(long long N, int* blocks, int* stages_per_block) {
     if (*blocks < 1) *blocks = 1;
 }
 
-int dense_wgrad_supported(int M, int NO, int dtype) {
+// the staged kernel of this file
+static bool dense_wgrad_tiled_ok(int M, int NO, int dtype) {
     const int mt = cdiv(M, 32), nt = cdiv(NO, 32);
-    return (dtype != kF32 && M >= 8 && NO >= 8 && M % 8 == 0 && NO % 8 == 0 && mt <= 4 && nt <= 4 && mt * nt <= 8) ? 1
-                                                                                                                  : 0;
+    return dtype != kF32 && M >= 8 && NO >= 8 && M % 8 == 0 && NO % 8 == 0 && mt <= 4 && nt <= 4 && mt * nt <= 8;
+}
+
+int dense_wgrad_supported(int M, int NO, int dtype) {
+    return (dense_wgrad_tiled_ok(M, NO, dtype) || dense_any_wgrad_dims_ok(M, NO)) ? 1 : 0;
 }
 
 size_t dense_wgrad_workspace(long long N, int M, int NO) {
@@ -1242,7 +1254,11 @@ static int dense_wgrad_t(const void* a, const void* b, void* dw, void* ws, long 
 
 int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,
                        hipStream_t s) {
-    if (!dense_wgrad_supported(M, NO, dtype)) return -1;
+    if (!dense_wgrad_tiled_ok(M, NO, dtype)) {   // fp32, other widths: at most as many partials as the workspace holds
+        int blocks, spb;
+        dense_wgrad_plan(N, &blocks, &spb);
+        return dense_any_wgrad_launch(a, b, dw, ws, N, M, NO, dtype, blocks, s);
+    }
     if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15)) return -1;
     if (dtype == kF16) return dense_wgrad_t<f16_t>(a, b, dw, ws, N, M, NO, s);
     return dense_wgrad_t<bf16_t>(a, b, dw, ws, N, M, NO, s);
@@ -1257,7 +1273,7 @@ int dense_bwd_pair_supported(int O, int I, int dtype) {
     if (dtype == kF32) return 0;
     if (pair_exact(O, I)) return 1;
     // any widths both bodies cover: the row product with K = O, NO = I and the weight gradient with M = O, NO = I
-    return (dense_dims_ok(O, I, dtype) && dense_wgrad_supported(O, I, dtype)) ? 1 : 0;
+    return (dense_dims_ok(O, I, dtype) && dense_wgrad_tiled_ok(O, I, dtype)) ? 1 : 0;
 }
 
 // with the 32-row tile sums of gy (the `colsum` argument of the launch)

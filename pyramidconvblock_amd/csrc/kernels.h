@@ -122,6 +122,13 @@ size_t dense_wgrad_workspace(long long N, int M, int NO);
 int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,
                        hipStream_t s);
 // input gradient (optionally with the column sums of gy) and weight gradient of a layer W[O][I] in one launch
+// dense_any.hip: one 32 x 32 tile per wavefront, any dtype, widths that are multiples of 4 (inner width <= 256)
+bool dense_any_dims_ok(int K, int NO);
+int dense_any_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
+                          long long N, int K, int NO, int P, int dtype, hipStream_t s);
+bool dense_any_wgrad_dims_ok(int M, int NO);
+int dense_any_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,
+                           int max_chunks, hipStream_t s);
 int dense_bwd_pair_supported(int O, int I, int dtype);
 int dense_bwd_pair_colsum_supported(int O, int I, int dtype);
 int dense_bwd_pair_launch(const void* gy, const void* w, const void* xin, void* dx, float* colsum, void* dw, void* ws,

@@ -233,8 +233,10 @@ def add_rowbias_(y, v):
 
 
 def dense_supported(K, NO, dtype):
-    """True when the matrix-core dense kernels cover an inner size K, output size NO layer of this dtype."""
-    if dtype not in (torch.float16, torch.bfloat16):
+    """True when the matrix-core dense kernels cover an inner size K, output size NO layer of this dtype (forward,
+    input gradient and weight gradient): 16-bit layers up to 128 wide in the tiled kernels, and fp32 or other widths
+    (multiples of 4, inner width up to 256) one result tile per wavefront."""
+    if dtype not in _lib._DTYPES:
         return False
     return bool(_lib.lib().pdw_dense_supported(int(K), int(NO), _lib.dtype_code(dtype)))
 

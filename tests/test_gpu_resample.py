@@ -211,6 +211,34 @@ def test_dense_layers(dtype, K, NO, N, P):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("K,NO", [(200, 100), (100, 200), (128, 64), (64, 128), (256, 132), (4, 4), (36, 52), (12, 256)])
+@pytest.mark.parametrize("N,P", [(3 * 35, 35), (1, 1), (3 * 3477, 3477), (100, 33), (50, 7), (96, 32), (130, 64)])
+def test_dense_layers_any_width_and_fp32(dtype, K, NO, N, P):
+    """The dense entry points on fp32 and on widths the tiled kernels do not take (multiples of 4, wider than 128: the
+    ragged block's 200 / 100), against float64: forward in both weight layouts with bias and per-image rows (images
+    that end inside a 32-row tile, images shorter than a tile, a last image cut short) and the weight gradient."""
+    from pyramidconvblock_amd import ops
+
+    assert ops.dense_supported(K, NO, dtype) and ops.dense_supported(NO, K, dtype)
+    gen = torch.Generator().manual_seed(K * 1000 + NO + N)
+    x = randn(gen, N, K).to(dtype)
+    w = (randn(gen, NO, K) / K ** 0.5).to(dtype)
+    b = randn(gen, NO).to(dtype)
+    rb = randn(gen, (N + P - 1) // P, NO)
+    ref = x.double() @ w.double().t() + b.double() + rb.double().repeat_interleave(P, 0)[:N]
+    y = ops.dense_forward(x.cuda(), w.cuda(), bias=b.cuda(), rowbias=rb.cuda(), rows_per_image=P)
+    assert_close(y, ref.numpy(), dtype, "dense fwd")
+    y0 = ops.dense_forward(x.cuda(), w.cuda())
+    assert_close(y0, (x.double() @ w.double().t()).numpy(), dtype, "dense fwd, no bias")
+    g = randn(gen, N, NO).to(dtype)
+    dx = ops.dense_forward(g.cuda(), w.cuda(), w_kmajor=True)         # g @ w : [N,NO] x [NO,K]
+    assert_close(dx, (g.double() @ w.double()).numpy(), dtype, "dense dgrad")
+    dw = ops.dense_wgrad(g.cuda(), x.cuda())                           # g^T @ x : [NO, K]
+    assert_close(dw, (g.double().t() @ x.double()).numpy(), dtype, "dense wgrad")
+    assert not ops.dense_supported(K + 2, NO, dtype) and not ops.dense_supported(260, NO, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(4, 9, 7, 24), (32, 56, 56, 128), (3, 57, 61, 200)])
 def test_pool_branch(dtype, shape):
     """Global-mean branch (conv_block.py:46-47) forward and backward against float64."""
