@@ -9,10 +9,11 @@ names, parameter shapes and ``[B,H,W,C]`` in/out contract
 convolutions, gates and upsampling go through libpdw.so, the gate outputs are written straight
 into the halves of the concatenated buffer (no ``torch.cat``), the pooled branch is added in
 place, and the backward reuses one per-image column sum for both bias gradients and the
-gradient of the mean.  For 16-bit types and widths up to 128 the dense layers run on the
-matrix-core kernels of libpdw.so (bias / broadcast add fused into the store, deterministic
-split reduction for the weight gradients); other shapes use library GEMMs, with the weight
-gradients as a batched split-K product.
+gradient of the mean.  The dense layers run on the matrix-core kernels of libpdw.so (bias /
+broadcast add fused into the store, deterministic split reduction for the weight gradients):
+16-bit layers up to 128 wide in the tiled kernels, fp32 and other widths that are multiples of
+4 (inner width up to 256) one result tile per wavefront; anything else uses library GEMMs, with
+the weight gradients as a batched split-K product.
 """
 from __future__ import annotations
 
