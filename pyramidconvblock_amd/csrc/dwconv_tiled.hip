@@ -111,6 +111,10 @@ int dwconv_tiled_launch(const void* x, const void* w, void* y, int B, int H, int
         const int r = dwconv_mfma_launch(x, w, add, pool, y, B, H, W, C, KH, KW, PH, PW, flip, dtype, s);
         if (r != -1 || add || pool) return r;   // only the matrix-core kernel has the fused forms
     }
+    if (dtype == kF32) {   // fp32 matrix cores (square odd filters 5 .. 17, C % 4 == 0)
+        const int r = dwconv_f32m_launch(x, w, y, B, H, W, C, KH, KW, PH, PW, flip, s);
+        if (r != -1) return r;
+    }
     switch (KW) {
         case 3: return dwconv_tiled_kw3(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);
         case 5: return dwconv_tiled_kw5(x, w, y, B, H, W, C, KH, PH, PW, flip, dtype, s);

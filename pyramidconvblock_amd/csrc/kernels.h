@@ -122,6 +122,9 @@ size_t dense_wgrad_workspace(long long N, int M, int NO);
 int dense_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,
                        hipStream_t s);
 // input gradient (optionally with the column sums of gy) and weight gradient of a layer W[O][I] in one launch
+// dwconv_f32m.hip: fp32 forward / input gradient on the fp32 matrix cores; -1 = not covered
+int dwconv_f32m_launch(const void* x, const void* w, void* y, int B, int H, int W, int C, int KH, int KW, int PH, int PW,
+                       bool flip, hipStream_t s);
 // dense_any.hip: one 32 x 32 tile per wavefront, any dtype, widths that are multiples of 4 (inner width <= 256)
 bool dense_any_dims_ok(int K, int NO);
 int dense_any_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,

@@ -65,6 +65,17 @@ def test_kernel_larger_than_image(oracle):
     _run(oracle, (1, 6, 5, 8), 13, torch.bfloat16)
 
 
+@pytest.mark.parametrize("case", [((3, 57, 61, 100), 15, None), ((2, 40, 70, 12), 17, None), ((1, 33, 35, 4), 11, None),
+                                  ((2, 24, 64, 20), 13, None), ((3, 20, 90, 36), 17, (8, 8)), ((2, 37, 41, 8), 17, (3, 11)),
+                                  ((1, 70, 130, 16), 13, (0, 6)), ((2, 56, 56, 128), 17, None)])
+def test_fp32_matrix_core_forward_and_input_gradient(oracle, case):
+    """Shapes on which the fp32 forward / input gradient take the fp32 matrix-core kernel (the largest filter on
+    images wider than 32 columns, filters from 11 on small tensors): ragged channel counts, extents off the 16 x 64
+    tiles, paddings other than k // 2 (the input gradient then runs at padding k - 1 - p), against the oracle."""
+    shape, k, pad = case
+    _run(oracle, shape, k, torch.float32, padding=pad, seed=k)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("k", [9, 15])
 def test_config5_ragged(oracle, dtype, k):
