@@ -40,7 +40,9 @@ CASES = [
     ((4, 28, 28, 64), 13, torch.bfloat16),   # two images side by side in one instruction
     ((2, 57, 61, 24), 9, torch.bfloat16),
     ((2, 30, 33, 100), 9, torch.bfloat16),   # C % 8 != 0: vector kernel, 16-bit dot products
-    ((2, 30, 33, 20), 13, torch.float32),    # fp32 vector kernel
+    ((2, 30, 33, 20), 13, torch.float32),    # fp32, small tensor: matrix-core kernel
+    ((2, 40, 44, 8), 17, torch.float32),     # fp32 matrix-core kernel
+    ((2, 30, 33, 20), 7, torch.float32),     # fp32 vector kernel
     ((1, 24, 25, 16), 17, torch.float16),
 ]
 PLANTS = [(0, 17, 19, 5, float("inf")), (1, 2, 1, 3, float("nan")), (0, 23, 0, 7, float("-inf"))]
