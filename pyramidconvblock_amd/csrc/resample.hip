@@ -311,11 +311,11 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
     const T* gb = gy + b * H * W * ldg + c;
-    // The candidate ranges are generous (up to 10 wide when the output is twice the input); the destinations
+    // The candidate ranges are generous (up to 11 wide when the output is about twice the input); the destinations
     // that really weigh in are a contiguous run of about 2 * out/in.  Up to NS of them per axis are handled
     // without branches: weights beyond the run are zero and addresses clamped, so the NS loads of a row are issued
     // together (a load behind a per-lane `continue` is a trip to memory of its own).
-    constexpr int NC = 10, NS = 5;
+    constexpr int NC = 12, NS = 5;
     int i0 = ihi + 1, i1 = ilo - 1, j0 = jhi + 1, j1 = jlo - 1;
     if (ihi - ilo < NC && jhi - jlo < NC) {
 #pragma unroll
