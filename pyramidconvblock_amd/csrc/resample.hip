@@ -774,6 +774,13 @@ __device__ __forceinline__ float chunk_column_sum(const float* __restrict__ pp, 
 #pragma unroll
     for (int j = 0; j < 8; ++j) s[j] = 0.f;
     int q = 0;
+    for (; q + 32 <= nchunks; q += 32) {   // 32 loads in flight, added in the order of the 8-wide loop below
+        float v[32];
+#pragma unroll
+        for (int j = 0; j < 32; ++j) v[j] = pp[(long long)(q + j) * D];
+#pragma unroll
+        for (int j = 0; j < 32; ++j) s[j & 7] += v[j];
+    }
     for (; q + 8 <= nchunks; q += 8) {
         float v[8];
 #pragma unroll
@@ -781,7 +788,14 @@ __device__ __forceinline__ float chunk_column_sum(const float* __restrict__ pp, 
 #pragma unroll
         for (int j = 0; j < 8; ++j) s[j] += v[j];
     }
-    for (; q < nchunks; ++q) s[0] += pp[(long long)q * D];
+    {   // the last, partial group: requested together, added to s[0] one after the other
+        float v[7];
+#pragma unroll
+        for (int j = 0; j < 7; ++j) v[j] = q + j < nchunks ? pp[(long long)(q + j) * D] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 7; ++j)
+            if (q + j < nchunks) s[0] += v[j];
+    }
     return ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
 }
 
@@ -827,10 +841,40 @@ __global__ __launch_bounds__(256) void pool_branch_bwd_a_k(const float* __restri
     const int b = blockIdx.x;
     for (int c = threadIdx.x; c < D; c += 256) {
         const float s = chunk_column_sum(part + (long long)b * nchunks * D + c, nchunks, D);
-        gs[(long long)b * D + c] = s;
+        if (blockIdx.y == 0) gs[(long long)b * D + c] = s;
         sm[c] = s;
     }
     __syncthreads();
+    if (gridDim.y > 1) {
+        // wide layers (D > 128): gridDim.y slices of 32 columns of dmean (every slice forms the column sums again: a
+        // few KB from L2), 8 row lanes per column with 32 loads in flight each, combined through LDS
+        const int cl = threadIdx.x & 31, ol = threadIdx.x >> 5, c = blockIdx.y * 32 + cl;
+        float* pr = sm + D;   // [8][32]
+        float a4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (c < D) {
+            for (int o = ol; o < D; o += 256) {   // 32 loads in flight: one round for D <= 256
+                float wv[32], sv[32];
+#pragma unroll
+                for (int j = 0; j < 32; ++j) {
+                    const int oo = o + 8 * j;
+                    const bool ok = oo < D;
+                    wv[j] = ok ? to_f32(wp[(long long)oo * D + c]) : 0.f;
+                    sv[j] = ok ? sm[oo] : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < 32; ++j) a4[j & 3] = fmaf(sv[j], wv[j], a4[j & 3]);
+            }
+        }
+        pr[ol * 32 + cl] = (a4[0] + a4[1]) + (a4[2] + a4[3]);
+        __syncthreads();
+        if (ol == 0 && c < D) {
+            float t = 0.f;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) t += pr[q * 32 + cl];
+            dmean[(long long)b * D + c] = t * inv_p;
+        }
+        return;
+    }
     // thread (ol, c): rows o = ol, ol+OL, ...  of Wp, coalesced over c; OL row lanes combined through LDS
     const int OL = D <= 128 ? 256 / (D < 32 ? 32 : D) : 1;   // row lanes when D <= 128
     float* prod = sm + D;
@@ -1587,7 +1631,8 @@ int pool_branch_bwd_launch(const void* gy, const void* m, const void* wp, void* 
         return check_launch("pool_branch_bwd");
     }
 #define PDW_PB(T)                                                                                                  \
-    hipLaunchKernelGGL((pool_branch_bwd_a_k<T>), dim3(B), dim3(256), lds, s, ws, n, D, inv_p, (const T*)wp, gs, dmean); \
+    hipLaunchKernelGGL((pool_branch_bwd_a_k<T>), dim3(B, D > 128 ? (D + 31) / 32 : 1), dim3(256), lds, s, ws, n, D,    \
+                       inv_p, (const T*)wp, gs, dmean);                                                            \
     if (int e = check_launch("pool_branch_bwd_a")) return e;                                                       \
     hipLaunchKernelGGL((pool_branch_bwd_b_k<T>), dim3(D), dim3(256), ldsb, s, gs, (const T*)m, B, D, (T*)gbias,    \
                        (T*)gbias2, (T*)gwp);
