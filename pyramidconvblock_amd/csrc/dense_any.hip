@@ -384,9 +384,10 @@ static int any_wgrad_chunks(long long N, int M, int NO, int max_chunks) {
 int dense_any_wgrad_launch(const void* a, const void* b, void* dw, void* ws, long long N, int M, int NO, int dtype,
                            int max_chunks, hipStream_t s) {
     if (!dense_any_wgrad_dims_ok(M, NO) || N > 0x7fffffffLL || max_chunks < 1) return -1;
-    if (N == 0) {   // an empty sum
-        if (hipMemsetAsync(dw, 0, (size_t)M * NO * (dtype == kF32 ? 4 : 2), s) != hipSuccess) return 1;
-        return 0;
+    if (N == 0) {   // an empty sum: the summation of no partials writes the zeros (a kernel, so that it can be captured)
+        if (dtype == kF32) return wgrad_reduce_launch<float>((const float*)ws, dw, 0, M * NO, s);
+        if (dtype == kF16) return wgrad_reduce_launch<f16_t>((const float*)ws, dw, 0, M * NO, s);
+        return wgrad_reduce_launch<bf16_t>((const float*)ws, dw, 0, M * NO, s);
     }
     const int chunks0 = any_wgrad_chunks(N, M, NO, max_chunks);
     const int ks = dtype == kF32 ? 8 : 16;

@@ -239,6 +239,21 @@ def test_dense_layers_any_width_and_fp32(dtype, K, NO, N, P):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("K,NO", [(200, 100), (128, 64)])
+def test_dense_layers_on_no_rows(dtype, K, NO):
+    """An empty batch: the forward returns an empty tensor, the weight gradient zeros."""
+    from pyramidconvblock_amd import ops
+
+    x = torch.zeros(0, K, dtype=dtype, device="cuda")
+    g = torch.zeros(0, NO, dtype=dtype, device="cuda")
+    w = torch.ones(NO, K, dtype=dtype, device="cuda")
+    assert tuple(ops.dense_forward(x, w).shape) == (0, NO)
+    dw = ops.dense_wgrad(g, x)
+    torch.cuda.synchronize()
+    assert tuple(dw.shape) == (NO, K) and not dw.any()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(4, 9, 7, 24), (32, 56, 56, 128), (3, 57, 61, 200)])
 def test_pool_branch(dtype, shape):
     """Global-mean branch (conv_block.py:46-47) forward and backward against float64."""
