@@ -330,13 +330,13 @@ int any_rows_go(const void* x, const void* w, const void* bias, const float* row
 
 bool dense_any_dims_ok(int K, int NO) { return K >= 4 && NO >= 4 && K % 4 == 0 && NO % 4 == 0 && K <= kAnyMaxK; }
 
-// -1: not covered (widths, alignment, more than 2^31 - 1 bytes of x).
+// -1: not covered (widths, alignment, more than 2^31 - 1 rows).
 int dense_any_rows_launch(const void* x, const void* w, int w_kmajor, const void* bias, const float* rowbias, void* y,
                           long long N, int K, int NO, int P, int dtype, hipStream_t s) {
     if (!dense_any_dims_ok(K, NO)) return -1;
     if (N == 0) return 0;
     const int es = dtype == kF32 ? 4 : 2;
-    if (N > 0x7fffffffLL || N * K * es > 0x7fffffffLL) return -1;   // (32-bit byte offsets into x)
+    if (N > 0x7fffffffLL) return -1;   // (descriptors are per 32-row tile: no limit on the bytes of x)
     const uintptr_t amask = es == 4 ? 15 : 7;   // groups of 4 values
     if ((reinterpret_cast<uintptr_t>(x) & amask) || (reinterpret_cast<uintptr_t>(w) & amask)) return -1;
     if (rowbias && P < 32) {
