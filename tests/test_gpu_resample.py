@@ -238,6 +238,24 @@ def test_dense_layers_any_width_and_fp32(dtype, K, NO, N, P):
     assert not ops.dense_supported(K + 2, NO, dtype) and not ops.dense_supported(260, NO, torch.float32)
 
 
+def test_dense_fp32_rows_beyond_two_gigabytes():
+    """x of more than 2^31 bytes in fp32 (32-bit byte offsets would wrap at row 4 194 304): rows at the start, around
+    that row and at the end against float64."""
+    from pyramidconvblock_amd import ops
+
+    K, NO, N = 128, 64, 4_300_000
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(N, K, device="cuda", generator=gen)
+    w = torch.randn(NO, K, device="cuda", generator=gen) / K ** 0.5
+    y = ops.dense_forward(x, w)
+    torch.cuda.synchronize()
+    for lo in (0, (1 << 31) // (K * 4) - 40, N - 70):
+        sl = slice(lo, lo + 70)
+        ref = x[sl].double().cpu() @ w.double().cpu().t()
+        assert_close(y[sl], ref.numpy(), torch.float32, f"rows from {lo}")
+    del x, y
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("K,NO", [(200, 100), (128, 64)])
 def test_dense_layers_on_no_rows(dtype, K, NO):
