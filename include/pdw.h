@@ -259,8 +259,9 @@ int pdw_bilinear_gate_bwd(const void *gy, const void *x, void *gx, int B, int h,
  * torch.cat of conv_block.py:43 written directly (conv_block.py:18-21 for both entries of self.gates). */
 int pdw_gate_pair_fwd(const void *xf, const void *xh, void *y, int B, int H, int W, int h, int w, int I, int ldy,
                       int dtype, void *stream);
-/* Its gradient for exactly doubled extents (anything else is an error; the caller then uses the single-branch
- * entry points): gy[B,H,W,2G] (pixels ldgy apart) -> gxf[B,H,W,I], gxh[B,h,w,I]. */
+/* Its gradient, one launch for any extents (exactly doubled ones take a kernel with fixed taps): gy[B,H,W,2G] (pixels
+ * ldgy apart) -> gxf[B,H,W,I], gxh[B,h,w,I]; the same bits as pdw_gate_bwd on the first half and pdw_bilinear_bwd +
+ * pdw_gate_bwd on the second. */
 int pdw_gate_pair_bwd(const void *gy, const void *xf, const void *xh, void *gxf, void *gxh, int B, int H, int W,
                       int h, int w, int I, int ldgy, int dtype, void *stream);
 

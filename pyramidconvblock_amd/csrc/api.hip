@@ -450,12 +450,11 @@ int pdw_gate_pair_bwd(const void* gy, const void* xf, const void* xh, void* gxf,
     if (int e = check_resample("pdw_gate_pair_bwd", gy, gxh, B, H, W, I, h, w, dtype)) return e;
     if (I < 2 || (I & 1)) return set_error("pdw_gate_pair_bwd: need even I >= 2 (I=%d)", I), 1;
     if (B > 0 && (!xf || !xh || !gxf)) return set_error("pdw_gate_pair_bwd: null pointer"), 1;
-    if (H != 2 * h || W != 2 * w || h < 2 || w < 2)
-        return set_error("pdw_gate_pair_bwd: needs H = 2h, W = 2w, h,w >= 2 (h=%d w=%d H=%d W=%d); use "
-                         "pdw_gate_bwd and pdw_bilinear_bwd + pdw_gate_bwd", h, w, H, W), 1;
     if (ldgy == 0) ldgy = I;
     if (ldgy < I) return set_error("pdw_gate_pair_bwd: ldgy=%d smaller than I=%d", ldgy, I), 1;
-    return gate_pair_bwd_launch(gy, xf, xh, gxf, gxh, B, H, W, h, w, I, ldgy, dtype, (hipStream_t)stream);
+    const int r = gate_pair_bwd_launch(gy, xf, xh, gxf, gxh, B, H, W, h, w, I, ldgy, dtype, (hipStream_t)stream);
+    if (r == -1) return set_error("pdw_gate_pair_bwd: case not covered (B=%d H=%d W=%d h=%d w=%d)", B, H, W, h, w), 3;
+    return r;
 }
 
 size_t pdw_spatial_sum_workspace_bytes(int B, int P, int C) {

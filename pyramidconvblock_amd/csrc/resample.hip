@@ -293,24 +293,16 @@ __global__ __launch_bounds__(256) void bilinear_bwd_x2_k(const T* __restrict__ g
     store_f32<T, VEC>(gx + ((b * h + m) * w + n) * C + c, acc);
 }
 
+// acc = the gradient of source (m, n) of one image: the sum over the destinations that read it of their weight times
+// gy (gb: the image's gy at the lane's channels, pixel stride ldg), for any ratio of extents.
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w,
-                                                      int C, int H, int W, int ldg, float sy, float sx,
-                                                      long long total) {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int CV = C / VEC;
-    int cq, n, m;
-    long long b;
-    split_idx(idx, CV, w, h, cq, n, m, b);
-    const int c = cq * VEC;
+__device__ __forceinline__ void bilinear_bwd_gather(const T* __restrict__ gb, int h, int w, int H, int W, int ldg, float sy,
+                                                    float sx, int m, int n, float (&acc)[VEC]) {
     int ilo, ihi, jlo, jhi;
     bl_dst_range(m, sy, H, ilo, ihi);
     bl_dst_range(n, sx, W, jlo, jhi);
-    float acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
-    const T* gb = gy + b * H * W * ldg + c;
     // The candidate ranges are generous (up to 11 wide when the output is about twice the input); the destinations
     // that really weigh in are a contiguous run of about 2 * out/in.  Up to NS of them per axis are handled
     // without branches: weights beyond the run are zero and addresses clamped, so the NS loads of a row are issued
@@ -366,6 +358,21 @@ __global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, 
             }
         }
     }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinear_bwd_k(const T* __restrict__ gy, T* __restrict__ gx, int h, int w,
+                                                      int C, int H, int W, int ldg, float sy, float sx,
+                                                      long long total) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int CV = C / VEC;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, CV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
+    float acc[VEC];
+    bilinear_bwd_gather<T, VEC>(gy + b * H * W * ldg + c, h, w, H, W, ldg, sy, sx, m, n, acc);
     store_f32<T, VEC>(gx + ((b * h + m) * w + n) * C + c, acc);
 }
 
@@ -702,6 +709,43 @@ __global__ __launch_bounds__(256) void gate_pair_bwd_k(const T* __restrict__ gy,
         const long long idx = (long long)(blockIdx.x - nblk_full) * blockDim.x + threadIdx.x;
         if (idx < total_half) bilinear_gate_bwd_x2_item<T, VEC>(gy + I / 2, xh, gxh, h, w, I, ldg, s, idx);
     }
+}
+
+// The same for any ratio of extents: the half-resolution items gather their gradient with bilinear_bwd_gather
+// (rounded to T, as the separate kernel stores it) and apply the gate's gradient.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_pair_bwd_gen_k(const T* __restrict__ gy, const T* __restrict__ xf,
+                                                           const T* __restrict__ xh, T* __restrict__ gxf,
+                                                           T* __restrict__ gxh, int h, int w, int H, int W, int I, int ldg,
+                                                           float s, float sy, float sx, unsigned nblk_full,
+                                                           long long total_full, long long total_half) {
+    if (blockIdx.x < nblk_full) {
+        const long long first = (long long)blockIdx.x * (kGateItems * 256) + threadIdx.x;
+        if (first < total_full) gate_bwd_items<T, VEC, kGateItems>(xf, gy, gxf, I, ldg, s, first, 256, total_full);
+        return;
+    }
+    const long long idx = (long long)(blockIdx.x - nblk_full) * blockDim.x + threadIdx.x;
+    if (idx >= total_half) return;
+    const int G = I / 2, GV = G / VEC;
+    int cq, n, m;
+    long long b;
+    split_idx(idx, GV, w, h, cq, n, m, b);
+    const int c = cq * VEC;
+    const T* xp = xh + ((b * h + m) * w + n) * I + c;
+    const ChanVec<T, VEC> xa = *reinterpret_cast<const ChanVec<T, VEC>*>(xp);
+    const ChanVec<T, VEC> xb = *reinterpret_cast<const ChanVec<T, VEC>*>(xp + G);
+    float acc[VEC];
+    bilinear_bwd_gather<T, VEC>(gy + b * H * W * ldg + G + c, h, w, H, W, ldg, sy, sx, m, n, acc);
+    float ga[VEC], gbv[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        const float g = to_f32(from_f32<T>(acc[v]));
+        ga[v] = gate_f32(g, to_f32(xb.v[v]), s);
+        gbv[v] = gate_f32(g, to_f32(xa.v[v]), s);
+    }
+    T* op = gxh + ((b * h + m) * w + n) * I + c;
+    store_f32<T, VEC>(op, ga);
+    store_f32<T, VEC>(op + G, gbv);
 }
 
 // ---------------------------------------------------------------- per-image column sums and broadcast add
@@ -1362,16 +1406,22 @@ int gate_pair_fwd_launch(const void* xf, const void* xh, void* y, int B, int H, 
 // -1: extents are not exactly doubled (the caller runs the separate kernels).
 int gate_pair_bwd_launch(const void* gy, const void* xf, const void* xh, void* gxf, void* gxh, int B, int H, int W, int h,
                          int w, int I, int ldg, int dtype, hipStream_t s) {
-    if (H != 2 * h || W != 2 * w || h < 2 || w < 2) return -1;
     const void* ptrs[5] = {gy, xf, xh, gxf, gxh};
     const int vec = pick_vec(gcd_int(I / 2, ldg), esize(dtype), ptrs, 5);
     const long long tf = (long long)B * H * W * (I / 2 / vec), th = (long long)B * h * w * (I / 2 / vec);
     unsigned bf, bh;
-    if (tf == 0) return 0;
+    if (tf == 0 || th == 0) return tf == 0 && th == 0 ? 0 : -1;
     if (!grid_for((tf + kGateItems - 1) / kGateItems, &bf) || !grid_for(th, &bh) ||
         (unsigned long long)bf + bh > 0x7fffffffULL)
         return 1;
     const float sc = sqrtf((float)(I / 2));
+    if (H != 2 * h || W != 2 * w || h < 2 || w < 2) {   // any ratio of extents
+        const float sy = (float)h / (float)H, sx = (float)w / (float)W;
+#define CALL(T, V) hipLaunchKernelGGL((gate_pair_bwd_gen_k<T, V>), dim3(bf + bh), dim3(256), 0, s, (const T*)gy, (const T*)xf, (const T*)xh, (T*)gxf, (T*)gxh, h, w, H, W, I, ldg, sc, sy, sx, bf, tf, th);
+        PDW_TYPE_SWITCH(dtype, vec, CALL)
+#undef CALL
+        return check_launch("gate_pair_bwd");
+    }
 #define CALL(T, V) hipLaunchKernelGGL((gate_pair_bwd_k<T, V>), dim3(bf + bh), dim3(256), 0, s, (const T*)gy, (const T*)xf, (const T*)xh, (T*)gxf, (T*)gxh, h, w, I, ldg, sc, bf, tf, th);
     PDW_TYPE_SWITCH(dtype, vec, CALL)
 #undef CALL

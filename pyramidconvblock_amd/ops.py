@@ -152,13 +152,13 @@ def gate_pair_forward(xf, xh, out):
 
 
 def gate_pair_backward(xf, xh, gy):
-    """Gradients (gxf, gxh) of gate_pair_forward; gy [B,H,W,2G] may be a channel slice.  One launch when the
-    extents are exactly doubled, the single-branch kernels otherwise."""
+    """Gradients (gxf, gxh) of gate_pair_forward; gy [B,H,W,2G] may be a channel slice.  One launch
+    (pdw_gate_pair_bwd), whatever the ratio of the extents."""
     dev = _lib.require_device(xf, xh, gy)
     B, H, W, I = xf.shape
     h, w = xh.shape[1], xh.shape[2]
     G = I // 2
-    if H == 2 * h and W == 2 * w and h >= 2 and w >= 2:
+    if xf.numel() and xh.numel():
         gxf, gxh = torch.empty_like(xf), torch.empty_like(xh)
         if xf.numel():
             _launch("pdw_gate_pair_bwd", dev, gy.data_ptr(), xf.data_ptr(), xh.data_ptr(), gxf.data_ptr(),

@@ -142,7 +142,8 @@ def test_gate_bilinear_fused(oracle, dtype, hw, out, I):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hw,out,I", [((5, 6), (10, 12), 24), ((28, 28), (56, 56), 64), ((4, 5), (9, 11), 6),
-                                      ((2, 2), (4, 4), 2), ((3, 7), (6, 14), 20)])
+                                      ((2, 2), (4, 4), 2), ((3, 7), (6, 14), 20), ((28, 30), (57, 61), 100),
+                                      ((1, 1), (3, 2), 8), ((7, 9), (7, 9), 16)])
 def test_gate_pair(oracle, dtype, hw, out, I):
     """Both gates of a two-scale block written into the concatenated tensor by one launch, and their gradients
     taken from it by one launch, against the oracle's gate / bilinear applied branch by branch."""
@@ -165,6 +166,9 @@ def test_gate_pair(oracle, dtype, hw, out, I):
     assert_close(gxf, oracle.gate_bwd(xf.double().numpy(), g[..., 8:8 + G].double().numpy()), dtype, "pair: d full")
     assert_close(gxh, oracle.gate_bwd(xh.double().numpy(), oracle.bilinear_bwd(g[..., 8 + G:].double().numpy(), hw)),
                  dtype, "pair: d pooled")
+    # the same bits as the single-branch kernels, whatever the ratio of the extents
+    assert torch.equal(gxf, ops.gate_backward(xf.cuda(), gs[..., :G]))
+    assert torch.equal(gxh, ops.gate_backward(xh.cuda(), ops.bilinear_backward(gs[..., G:], hw)))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
